@@ -1,0 +1,180 @@
+// Memref-descriptor entry points: what `func.call` sites in lowered COMET host
+// code bind to.  Operands are HOST memrefs, as for the reference's other runtime
+// calls (lib/ExecutionEngine/StatUtils.cpp:89-113,
+// lib/ExecutionEngine/blis_interface.cpp:143-146 in pnnl/COMET); each call
+// uploads, runs the device kernels and copies the result back.  These return
+// void like their counterparts, so a failure prints the message and exits, the
+// reference's own error behaviour (lib/ExecutionEngine/HipGpuUtils.cpp:10-19).
+#include <stdio.h>
+#include <stdlib.h>
+
+#include "common.h"
+
+using namespace comet;
+
+namespace {
+
+[[noreturn]] void die(const char *where)
+{
+    fprintf(stderr, "comet_hip error in %s: %s\n", where, comet_hip_last_error());
+    exit(1);
+}
+
+template <typename T>
+const T *data1(const comet_memref_1d *m, const char *who)
+{
+    if (!m || (m->sizes[0] > 0 && !m->aligned)) {
+        set_error(COMET_HIP_ERR_ARG, "null memref");
+        die(who);
+    }
+    if (m->sizes[0] > 1 && m->strides[0] != 1) {
+        set_error(COMET_HIP_ERR_ARG, "non-contiguous 1-D memref (stride %lld)", (long long)m->strides[0]);
+        die(who);
+    }
+    return (const T *)m->aligned + m->offset;
+}
+
+struct DeviceBuf {
+    int64_t p = 0;
+    explicit DeviceBuf(int64_t bytes) : p(comet_hip_malloc(bytes)) {}
+    ~DeviceBuf() { (void)comet_hip_free(p); }
+};
+
+// result of the "sizes" call, waiting for the "fill" call
+int64_t g_pending_c = 0;
+
+}  // namespace
+
+extern "C" void _mlir_ciface_comet_hip_spmv_csr_f64_i64(comet_memref_1d *pos, comet_memref_1d *crd,
+                                                         comet_memref_1d *val, comet_memref_1d *x, comet_memref_1d *y)
+{
+    const char *who = "comet_hip_spmv_csr_f64_i64";
+    const int64_t nrows = pos->sizes[0] - 1, ncols = x->sizes[0];
+    if (nrows < 0 || y->sizes[0] != nrows) {
+        set_error(COMET_HIP_ERR_ARG, "y has %lld entries, A has %lld rows", (long long)y->sizes[0], (long long)nrows);
+        die(who);
+    }
+    int64_t a = comet_hip_csr_upload_i64(nrows, ncols, data1<int64_t>(pos, who), data1<int64_t>(crd, who),
+                                         data1<double>(val, who));
+    if (!a)
+        die(who);
+    DeviceBuf dx(ncols * 8), dy(nrows * 8);
+    if ((ncols && !dx.p) || (nrows && !dy.p))
+        die(who);
+    double *hy = (double *)data1<double>(y, who);
+    if (comet_hip_memcpy(dx.p, (void *)data1<double>(x, who), ncols * 8, 0) ||
+        comet_hip_memcpy(dy.p, hy, nrows * 8, 0) || comet_hip_spmv_csr_f64(a, dx.p, dy.p, 1) ||
+        comet_hip_memcpy(dy.p, hy, nrows * 8, 1))
+        die(who);
+    (void)comet_hip_csr_destroy(a);
+}
+
+extern "C" void _mlir_ciface_comet_hip_spmm_csr_f64_i64(comet_memref_1d *pos, comet_memref_1d *crd,
+                                                         comet_memref_1d *val, comet_memref_2d *B, comet_memref_2d *C)
+{
+    const char *who = "comet_hip_spmm_csr_f64_i64";
+    if (!B || !C || !B->aligned || !C->aligned) {
+        set_error(COMET_HIP_ERR_ARG, "null memref");
+        die(who);
+    }
+    const int64_t nrows = pos->sizes[0] - 1, ncols = B->sizes[0], K = B->sizes[1];
+    if (nrows < 0 || C->sizes[0] != nrows || C->sizes[1] != K || (K > 1 && (B->strides[1] != 1 || C->strides[1] != 1)) ||
+        (ncols > 1 && B->strides[0] != K) || (nrows > 1 && C->strides[0] != K)) {
+        set_error(COMET_HIP_ERR_ARG, "B/C must be contiguous row-major with matching shapes");
+        die(who);
+    }
+    int64_t a = comet_hip_csr_upload_i64(nrows, ncols, data1<int64_t>(pos, who), data1<int64_t>(crd, who),
+                                         data1<double>(val, who));
+    if (!a)
+        die(who);
+    DeviceBuf db(ncols * K * 8), dc(nrows * K * 8);
+    if ((ncols * K && !db.p) || (nrows * K && !dc.p))
+        die(who);
+    double *hb = (double *)B->aligned + B->offset, *hc = (double *)C->aligned + C->offset;
+    if (comet_hip_memcpy(db.p, hb, ncols * K * 8, 0) || comet_hip_memcpy(dc.p, hc, nrows * K * 8, 0) ||
+        comet_hip_spmm_csr_f64(a, K, db.p, K, dc.p, K, 1) || comet_hip_memcpy(dc.p, hc, nrows * K * 8, 1))
+        die(who);
+    (void)comet_hip_csr_destroy(a);
+}
+
+extern "C" void _mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i64(
+    int64_t nrowsA, int64_t ncolsB, comet_memref_1d *Apos, comet_memref_1d *Acrd, comet_memref_1d *Aval,
+    comet_memref_1d *Bpos, comet_memref_1d *Bcrd, comet_memref_1d *Bval, comet_memref_1d *Mpos,
+    comet_memref_1d *Mcrd, comet_memref_1d *sizes)
+{
+    const char *who = "comet_hip_spgemm_csr_sizes_f64_i64";
+    const int64_t nrowsB = Bpos->sizes[0] - 1;
+    if (Apos->sizes[0] - 1 != nrowsA || !sizes || sizes->sizes[0] < 1) {
+        set_error(COMET_HIP_ERR_ARG, "inconsistent row counts or missing sizes memref");
+        die(who);
+    }
+    if (g_pending_c) {
+        (void)comet_hip_csr_destroy(g_pending_c);
+        g_pending_c = 0;
+    }
+    int64_t a = comet_hip_csr_upload_i64(nrowsA, nrowsB, data1<int64_t>(Apos, who), data1<int64_t>(Acrd, who),
+                                         data1<double>(Aval, who));
+    int64_t b = a ? comet_hip_csr_upload_i64(nrowsB, ncolsB, data1<int64_t>(Bpos, who), data1<int64_t>(Bcrd, who),
+                                             data1<double>(Bval, who))
+                  : 0;
+    int64_t m = 0;
+    if (a && b && Mpos && Mpos->sizes[0] > 0) {
+        // a mask carries structure only; its device value array is all zeros
+        const int64_t mnnz = Mcrd->sizes[0];
+        double *zeros = (double *)calloc((size_t)(mnnz > 0 ? mnnz : 1), sizeof(double));
+        m = comet_hip_csr_upload_i64(nrowsA, ncolsB, data1<int64_t>(Mpos, who), data1<int64_t>(Mcrd, who), zeros);
+        free(zeros);
+        if (!m)
+            die(who);
+    }
+    if (!a || !b)
+        die(who);
+    g_pending_c = comet_hip_spgemm_csr(a, b, m);
+    if (!g_pending_c)
+        die(who);
+    int64_t nnz = 0;
+    (void)comet_hip_csr_dims(g_pending_c, nullptr, nullptr, &nnz);
+    ((int64_t *)sizes->aligned + sizes->offset)[0] = nnz;
+    (void)comet_hip_csr_destroy(a);
+    (void)comet_hip_csr_destroy(b);
+    if (m)
+        (void)comet_hip_csr_destroy(m);
+}
+
+extern "C" void _mlir_ciface_comet_hip_spgemm_csr_fill_f64_i64(comet_memref_1d *Cpos, comet_memref_1d *Ccrd,
+                                                                comet_memref_1d *Cval)
+{
+    const char *who = "comet_hip_spgemm_csr_fill_f64_i64";
+    if (!g_pending_c) {
+        set_error(COMET_HIP_ERR_ARG, "fill called without a preceding sizes call");
+        die(who);
+    }
+    int64_t nrows = 0, nnz = 0;
+    (void)comet_hip_csr_dims(g_pending_c, &nrows, nullptr, &nnz);
+    if (Cpos->sizes[0] < nrows + 1 || Ccrd->sizes[0] < nnz || Cval->sizes[0] < nnz) {
+        set_error(COMET_HIP_ERR_ARG, "output memrefs too small for %lld rows / %lld entries", (long long)nrows,
+                  (long long)nnz);
+        die(who);
+    }
+    if (comet_hip_csr_download_i64(g_pending_c, (int64_t *)data1<int64_t>(Cpos, who),
+                                   (int64_t *)data1<int64_t>(Ccrd, who), (double *)data1<double>(Cval, who)))
+        die(who);
+    (void)comet_hip_csr_destroy(g_pending_c);
+    g_pending_c = 0;
+}
+
+extern "C" double _mlir_ciface_comet_hip_tricount_f64_i64(int64_t ncols, comet_memref_1d *pos, comet_memref_1d *crd,
+                                                           comet_memref_1d *val)
+{
+    const char *who = "comet_hip_tricount_f64_i64";
+    const int64_t nrows = pos->sizes[0] - 1;
+    int64_t l = comet_hip_csr_upload_i64(nrows, ncols, data1<int64_t>(pos, who), data1<int64_t>(crd, who),
+                                         data1<double>(val, who));
+    if (!l)
+        die(who);
+    double out = 0.0;
+    if (comet_hip_spgemm_masked_sum(l, l, l, &out))
+        die(who);
+    (void)comet_hip_csr_destroy(l);
+    return out;
+}

@@ -1,0 +1,75 @@
+// Shared host-side plumbing of the gfx950 runtime: error reporting, the
+// library stream, CSR handles, cached workspaces and per-kernel event timing.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+#include <vector>
+
+#include "../../include/comet_hip_rt.h"
+
+namespace comet {
+
+// One process-wide stream at default priority; every kernel and copy of the
+// library is ordered on it.
+hipStream_t stream();
+int ensure_init();
+int set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int num_cus();
+
+#define COMET_HIPCHK(call)                                                                   \
+    do {                                                                                     \
+        hipError_t e_ = (call);                                                              \
+        if (e_ != hipSuccess)                                                                \
+            return comet::set_error(COMET_HIP_ERR_HIP, "%s failed: %s (%s:%d)", #call,       \
+                                    hipGetErrorString(e_), __FILE__, __LINE__);              \
+    } while (0)
+
+#define COMET_CHK(expr)                \
+    do {                               \
+        int rc_ = (expr);              \
+        if (rc_ != COMET_HIP_OK)       \
+            return rc_;                \
+    } while (0)
+
+// Grow-only device scratch buffer.  `zeroed` buffers are cleared when they are
+// (re)allocated and their users must leave them all-zero on return.
+struct Workspace {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+    int ensure(size_t need, bool zeroed);
+    void release();
+};
+
+struct Csr {
+    int64_t nrows = 0, ncols = 0, nnz = 0;
+    int64_t *pos = nullptr;
+    int32_t *crd = nullptr;
+    double *val = nullptr;
+    bool owns = false;
+    // SpMM plan: row that holds the first nonzero of every fixed-size chunk.
+    int32_t *spmm_chunk_row = nullptr;
+    int64_t spmm_nchunks = 0;
+};
+
+Csr *csr_from_handle(int64_t h);           // nullptr (and error set) if unknown
+int64_t csr_register(Csr *c);              // takes ownership of the struct
+int csr_alloc(Csr *c, int64_t nrows, int64_t ncols, int64_t nnz);   // allocates pos/crd/val, owns = true
+
+// Records an event pair around a kernel launch when profiling is on.
+struct KernelTimer {
+    explicit KernelTimer(const char *name);
+    ~KernelTimer();
+    int slot;
+};
+
+static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// exclusive scan of int64 counts into pos[0..n] (pos[n] = total), on the stream
+int exclusive_scan_i64(const int64_t *counts, int64_t n, int64_t *pos);
+
+// deterministic tree sum of a device array, result copied to the host
+int reduce_sum_device(const double *v, int64_t n, double *out_host);
+
+}  // namespace comet

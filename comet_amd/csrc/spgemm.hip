@@ -1,0 +1,694 @@
+// Gustavson SpGEMM (symbolic + numeric), masked SpGEMM and the fused
+// masked-SpGEMM + SUM used for triangle counting, for gfx950.
+//
+// What is computed is what the reference's workspace lowering computes
+// (lib/Dialect/IndexTree/Transforms/SymbolicCompute.cpp:215-339,
+// lib/Conversion/IndexTreeToSCF/SymbolicDomainConversion.cpp:81-340,
+// lib/Dialect/IndexTree/Transforms/WorkspaceTransforms.cpp:97-276,
+// lib/Conversion/TensorAlgebraToSCF/SparseTensorConversionPass.cpp:595-638,
+// 982-1159; masks: lib/Conversion/IndexTreeToSCF/IndexTreeToSCF.cpp:1083-1148,
+// 1327-1448): every structurally reachable (i,j) is kept, columns come out
+// ascending.  How it is computed is different: one 1024-lane workgroup owns a
+// row at a time and keeps the row's column set as a bitmap in LDS (128 KiB
+// covers 2^20 columns), so counting is a popcount, "sort the touched columns"
+// (the reference's comet_sort call) is reading the bitmap in order, and the
+// mark array / mark value bookkeeping disappears.  Values accumulate with
+// workgroup-scope fp64 atomics into a dense per-workgroup slab in HBM that the
+// extraction step reads back and re-zeroes with an atomic exchange, so every
+// access to the slab is performed at the L2 and no stale L1 line can be seen.
+// The order in which the products of one (i,j) are added is therefore not the
+// reference's ascending-k order: values agree to rounding, structure exactly.
+#include "common.h"
+
+namespace comet {
+
+constexpr int SG_T = 1024;                 // lanes per workgroup
+constexpr int SG_WAVES = SG_T / 64;
+constexpr int SG_LDS_MAX_W = 32;           // words per lane that still fit LDS (32 * 1024 * 4 B = 128 KiB)
+
+__device__ inline int64_t readlane_i64(int64_t v, int lane)
+{
+    int lo = (int)(v & 0xffffffff), hi = (int)(v >> 32);
+    lo = __builtin_amdgcn_readlane(lo, lane);
+    hi = __builtin_amdgcn_readlane(hi, lane);
+    return ((int64_t)hi << 32) | (uint32_t)lo;
+}
+
+__device__ inline double readlane_d(double v, int lane)
+{
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __builtin_amdgcn_readlane(lo, lane);
+    hi = __builtin_amdgcn_readlane(hi, lane);
+    return __hiloint2double(hi, lo);
+}
+
+// Bitmap layout: lane t of the workgroup owns the 32*W consecutive columns
+// [t*32*W, (t+1)*32*W) and its k-th word sits at address k*SG_T + t, so that a
+// sweep over "my words" is conflict-free in LDS (and coalesced in HBM).
+struct BmAddr {
+    int logW;
+    __device__ inline int word(int j) const
+    {
+        const int w = j >> 5;
+        return ((w & ((1 << logW) - 1)) << 10) + (w >> logW);   // SG_T == 1 << 10
+    }
+    __device__ inline uint32_t bit(int j) const { return 1u << (j & 31); }
+};
+static_assert(SG_T == 1024, "BmAddr::word assumes 1024 lanes");
+
+// Visit every product of output row i: f(j, a*b) for k in A_i (ascending per
+// wavefront), j in B_k.  Each wavefront takes 64 entries of A_i at a time (one
+// per lane, coalesced), then walks them one by one with all lanes striding
+// over B_k.
+template <bool VALUES, typename F>
+__device__ inline void for_each_product(int64_t as, int64_t ae, const int32_t *__restrict__ Acrd,
+                                        const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
+                                        const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval, F f)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    for (int64_t base = as + (int64_t)wave * 64; base < ae; base += (int64_t)SG_WAVES * 64) {
+        const int cnt = (int)(ae - base < 64 ? ae - base : 64);
+        int64_t bs = 0, be = 0;
+        double a = 0.0;
+        if (lane < cnt) {
+            const int k = Acrd[base + lane];
+            bs = Bpos[k];
+            be = Bpos[k + 1];
+            if (VALUES)
+                a = Aval[base + lane];
+        }
+        for (int t = 0; t < cnt; ++t) {
+            const int64_t s = readlane_i64(bs, t), e = readlane_i64(be, t);
+            const double at = VALUES ? readlane_d(a, t) : 0.0;
+            for (int64_t q = s + lane; q < e; q += 64) {
+                const int j = Bcrd[q];
+                if (VALUES)
+                    f(j, at * Bval[q]);
+                else
+                    f(j, 0.0);
+            }
+        }
+    }
+}
+
+__device__ inline int wave_sum_i32(int v)
+{
+    for (int d = 32; d > 0; d >>= 1)
+        v += __shfl_down(v, d, 64);
+    return v;
+}
+
+__device__ inline double wave_sum_f64(double v)
+{
+    for (int d = 32; d > 0; d >>= 1)
+        v += __shfl_down(v, d, 64);
+    return v;
+}
+
+// Rows are dealt to workgroups round-robin (row = first + blockIdx.x + n*gridDim.x).
+// The row index is then made of kernel arguments and blockIdx only, so it lives in
+// scalar registers and every branch on it (empty row -> continue, end of loop) is a
+// uniform scalar branch.  That matters because the row loop contains workgroup
+// barriers: a row index that merely happens to be equal in all lanes (for instance
+// one broadcast through LDS from a ticket counter) lets the compiler treat
+// `continue` as divergent and park most lanes in a barrier loop that never
+// advances, which hangs the workgroup.
+extern __shared__ uint32_t sg_dyn_lds[];
+
+// ---------------------------------------------------------------------------
+// Symbolic phase.  Unmasked: set the bit of every reachable column, count the
+// bits that were new.  Masked: the bitmap starts as the mask row; a product
+// clears its bit, and the bits that were still set are the output entries.
+// ---------------------------------------------------------------------------
+template <bool BM_LDS, bool MASKED>
+__global__ __launch_bounds__(SG_T) void spgemm_symbolic_kernel(
+    int64_t nrows, const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd,
+    const int64_t *__restrict__ Bpos, const int32_t *__restrict__ Bcrd, const int64_t *__restrict__ Mpos,
+    const int32_t *__restrict__ Mcrd, int logW, uint32_t *__restrict__ gbm, int64_t *__restrict__ rowcount)
+{
+    __shared__ int wave_cnt[SG_WAVES];
+    uint32_t *bm;
+    if constexpr (BM_LDS)
+        bm = sg_dyn_lds;
+    else
+        bm = gbm + ((size_t)blockIdx.x << (10 + logW));
+    const BmAddr ad{logW};
+    const int nwords = SG_T << logW;
+    if constexpr (BM_LDS) {
+        for (int w = threadIdx.x; w < nwords; w += SG_T)
+            bm[w] = 0;
+    }
+    __syncthreads();
+    for (int64_t i = blockIdx.x; i < nrows; i += gridDim.x) {
+        const int64_t as = Apos[i], ae = Apos[i + 1];
+        if (as == ae) {
+            if (threadIdx.x == 0)
+                rowcount[i] = 0;
+            continue;
+        }
+        if constexpr (MASKED) {
+            const int64_t ms = Mpos[i], me = Mpos[i + 1];
+            if (ms == me) {
+                if (threadIdx.x == 0)
+                    rowcount[i] = 0;
+                continue;
+            }
+            for (int64_t t = ms + threadIdx.x; t < me; t += SG_T)
+                atomicOr(&bm[ad.word(Mcrd[t])], ad.bit(Mcrd[t]));
+            __syncthreads();
+        }
+        int count = 0;
+        for_each_product<false>(as, ae, Acrd, nullptr, Bpos, Bcrd, nullptr, [&](int j, double) {
+            const uint32_t b = ad.bit(j);
+            if constexpr (MASKED) {
+                const uint32_t old = atomicAnd(&bm[ad.word(j)], ~b);
+                count += (old & b) ? 1 : 0;
+            } else {
+                const uint32_t old = atomicOr(&bm[ad.word(j)], b);
+                count += (old & b) ? 0 : 1;
+            }
+        });
+        count = wave_sum_i32(count);
+        if ((threadIdx.x & 63) == 0)
+            wave_cnt[threadIdx.x >> 6] = count;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int total = 0;
+            for (int w = 0; w < SG_WAVES; ++w)
+                total += wave_cnt[w];
+            rowcount[i] = total;
+        }
+        // leave the bitmap all-zero for the next row
+        if constexpr (MASKED) {
+            for (int64_t t = Mpos[i] + threadIdx.x; t < Mpos[i + 1]; t += SG_T)
+                atomicAnd(&bm[ad.word(Mcrd[t])], 0u);
+        } else if constexpr (BM_LDS) {
+            for (int w = threadIdx.x; w < nwords; w += SG_T)
+                bm[w] = 0;
+        } else {
+            for_each_product<false>(as, ae, Acrd, nullptr, Bpos, Bcrd, nullptr,
+                                    [&](int j, double) { atomicAnd(&bm[ad.word(j)], 0u); });
+        }
+        __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Numeric phase for rows [row_begin,row_end).
+// ---------------------------------------------------------------------------
+template <bool BM_LDS, bool MASKED>
+__global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
+    int64_t row_begin, int64_t row_end, int64_t ncols, const int64_t *__restrict__ Apos,
+    const int32_t *__restrict__ Acrd, const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
+    const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval, const int64_t *__restrict__ Mpos,
+    const int32_t *__restrict__ Mcrd, int logW, uint32_t *__restrict__ gbm, uint32_t *__restrict__ gmask,
+    double *__restrict__ slabs, const int64_t *__restrict__ Cpos,
+    int32_t *__restrict__ Ccrd, double *__restrict__ Cval)
+{
+    __shared__ int wave_tot[SG_WAVES];
+    uint32_t *bm;
+    if constexpr (BM_LDS)
+        bm = sg_dyn_lds;
+    else
+        bm = gbm + ((size_t)blockIdx.x << (10 + logW));
+    uint32_t *mbm = MASKED ? gmask + ((size_t)blockIdx.x << (10 + logW)) : nullptr;
+    double *slab = slabs + (size_t)blockIdx.x * (size_t)ncols;
+    const BmAddr ad{logW};
+    const int W = 1 << logW;
+    const int nwords = SG_T << logW;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if constexpr (BM_LDS) {
+        for (int w = threadIdx.x; w < nwords; w += SG_T)
+            bm[w] = 0;
+    }
+    __syncthreads();
+    const int64_t out0 = Cpos[row_begin];
+    for (int64_t i = row_begin + blockIdx.x; i < row_end; i += gridDim.x) {
+        const int64_t as = Apos[i], ae = Apos[i + 1];
+        const int64_t ob = Cpos[i], oe = Cpos[i + 1];
+        if (as == ae || ob == oe)
+            continue;
+        if constexpr (MASKED) {
+            for (int64_t t = Mpos[i] + threadIdx.x; t < Mpos[i + 1]; t += SG_T)
+                atomicOr(&mbm[ad.word(Mcrd[t])], ad.bit(Mcrd[t]));
+            __syncthreads();
+        }
+        for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, Bval, [&](int j, double v) {
+            const int w = ad.word(j);
+            const uint32_t b = ad.bit(j);
+            if constexpr (MASKED) {
+                if (!(atomicOr(&mbm[w], 0u) & b))
+                    return;
+            }
+            atomicOr(&bm[w], b);
+            __hip_atomic_fetch_add(&slab[j], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        });
+        __syncthreads();
+        // extraction: my words hold my columns in ascending order
+        int mine = 0;
+        for (int k = 0; k < W; ++k)
+            mine += __popc(BM_LDS ? bm[(k << 10) + threadIdx.x] : atomicOr(&bm[(k << 10) + threadIdx.x], 0u));
+        int inc = mine;
+        for (int d = 1; d < 64; d <<= 1) {
+            const int o = __shfl_up(inc, d, 64);
+            if (lane >= d)
+                inc += o;
+        }
+        if (lane == 63)
+            wave_tot[wave] = inc;
+        __syncthreads();
+        int64_t off = ob - out0 + (inc - mine);
+        for (int w = 0; w < wave; ++w)
+            off += wave_tot[w];
+        for (int k = 0; k < W; ++k) {
+            uint32_t word;
+            if constexpr (BM_LDS) {
+                word = bm[(k << 10) + threadIdx.x];
+                bm[(k << 10) + threadIdx.x] = 0;
+            } else {
+                word = atomicAnd(&bm[(k << 10) + threadIdx.x], 0u);
+            }
+            const int jbase = (((int)threadIdx.x << logW) + k) << 5;
+            while (word) {
+                const int b = __ffs(word) - 1;
+                word &= word - 1;
+                const int j = jbase + b;
+                Ccrd[off] = j;
+                Cval[off] = __hip_atomic_exchange(&slab[j], 0.0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                ++off;
+            }
+        }
+        if constexpr (MASKED) {
+            for (int64_t t = Mpos[i] + threadIdx.x; t < Mpos[i + 1]; t += SG_T)
+                atomicAnd(&mbm[ad.word(Mcrd[t])], 0u);
+        }
+        __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Masked SpGEMM + SUM without the output: rowsum[i] = sum over products of row
+// i that fall on a stored entry of mask row i.  Per-lane partial sums are
+// combined in a fixed order, so the result does not depend on scheduling.
+// ---------------------------------------------------------------------------
+template <bool BM_LDS>
+__global__ __launch_bounds__(SG_T) void spgemm_masked_sum_kernel(
+    int64_t nrows, const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd,
+    const double *__restrict__ Aval, const int64_t *__restrict__ Bpos, const int32_t *__restrict__ Bcrd,
+    const double *__restrict__ Bval, const int64_t *__restrict__ Mpos, const int32_t *__restrict__ Mcrd,
+    int logW, uint32_t *__restrict__ gbm, double *__restrict__ rowsum)
+{
+    __shared__ double wave_part[SG_WAVES];
+    uint32_t *bm;
+    if constexpr (BM_LDS)
+        bm = sg_dyn_lds;
+    else
+        bm = gbm + ((size_t)blockIdx.x << (10 + logW));
+    const BmAddr ad{logW};
+    const int nwords = SG_T << logW;
+    if constexpr (BM_LDS) {
+        for (int w = threadIdx.x; w < nwords; w += SG_T)
+            bm[w] = 0;
+    }
+    __syncthreads();
+    for (int64_t i = blockIdx.x; i < nrows; i += gridDim.x) {
+        const int64_t as = Apos[i], ae = Apos[i + 1];
+        const int64_t ms = Mpos[i], me = Mpos[i + 1];
+        if (as == ae || ms == me) {
+            if (threadIdx.x == 0)
+                rowsum[i] = 0.0;
+            continue;
+        }
+        for (int64_t t = ms + threadIdx.x; t < me; t += SG_T)
+            atomicOr(&bm[ad.word(Mcrd[t])], ad.bit(Mcrd[t]));
+        __syncthreads();
+        double part = 0.0;
+        for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, Bval, [&](int j, double v) {
+            uint32_t word;
+            if constexpr (BM_LDS)
+                word = bm[ad.word(j)];
+            else
+                word = atomicOr(&bm[ad.word(j)], 0u);
+            if (word & ad.bit(j))
+                part += v;
+        });
+        part = wave_sum_f64(part);
+        if ((threadIdx.x & 63) == 0)
+            wave_part[threadIdx.x >> 6] = part;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            double total = 0.0;
+            for (int w = 0; w < SG_WAVES; ++w)
+                total += wave_part[w];
+            rowsum[i] = total;
+        }
+        for (int64_t t = ms + threadIdx.x; t < me; t += SG_T)
+            atomicAnd(&bm[ad.word(Mcrd[t])], 0u);
+        __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------------------
+// CSR .* CSR -> CSR, one lane per row, two-pointer merge of the sorted rows
+// (lib/Conversion/IndexTreeToSCF/IndexTreeToSCF.cpp:864-1053).
+// ---------------------------------------------------------------------------
+template <bool FILL>
+__global__ void eltwise_mult_kernel(int64_t nrows, const int64_t *__restrict__ Apos,
+                                    const int32_t *__restrict__ Acrd, const double *__restrict__ Aval,
+                                    const int64_t *__restrict__ Bpos, const int32_t *__restrict__ Bcrd,
+                                    const double *__restrict__ Bval, int64_t *__restrict__ rowcount,
+                                    const int64_t *__restrict__ Cpos, int32_t *__restrict__ Ccrd,
+                                    double *__restrict__ Cval)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= nrows)
+        return;
+    int64_t p = Apos[i], q = Bpos[i];
+    const int64_t pe = Apos[i + 1], qe = Bpos[i + 1];
+    int64_t n = 0;
+    int64_t o = FILL ? Cpos[i] : 0;
+    while (p < pe && q < qe) {
+        const int ca = Acrd[p], cb = Bcrd[q];
+        if (ca == cb) {
+            if (FILL) {
+                Ccrd[o] = ca;
+                Cval[o] = Aval[p] * Bval[q];
+                ++o;
+            }
+            ++n;
+        }
+        p += (ca <= cb);
+        q += (cb <= ca);
+    }
+    if (!FILL)
+        rowcount[i] = n;
+}
+
+// ------------------------------------------------------------------ host side
+struct SgScratch {
+    Workspace rowcount;   // int64[nrows] / double[nrows]
+    Workspace gbm;        // global bitmaps (only when the bitmap does not fit LDS)
+    Workspace gmask;      // global mask bitmaps (masked numeric)
+    Workspace slabs;      // dense accumulators, zero between calls
+};
+static SgScratch g_sg;
+
+struct SgGeom {
+    int logW;
+    bool lds;
+    int groups;
+    size_t lds_bytes;
+    size_t bm_words;      // words per workgroup bitmap
+};
+
+static int sg_geometry(int64_t ncols, SgGeom *g)
+{
+    const int64_t words = ceil_div(ncols > 0 ? ncols : 1, 32);
+    int logW = 0;
+    while (((int64_t)SG_T << logW) < words)
+        ++logW;
+    if (logW > 20)
+        return set_error(COMET_HIP_ERR_SIZE, "too many columns (%lld)", (long long)ncols);
+    g->logW = logW;
+    g->lds = (1 << logW) <= SG_LDS_MAX_W;
+    g->bm_words = (size_t)SG_T << logW;
+    g->lds_bytes = g->lds ? g->bm_words * sizeof(uint32_t) : 0;
+    g->groups = num_cus() > 0 ? num_cus() : 256;
+    if (g->lds && g->lds_bytes <= 48 * 1024)
+        g->groups *= 2;          // two workgroups of 16 wavefronts fit a CU when the bitmap is small
+    return COMET_HIP_OK;
+}
+
+template <typename K>
+static int sg_allow_lds(K kernel, size_t bytes)
+{
+    if (bytes > 0)
+        COMET_HIPCHK(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+    return COMET_HIP_OK;
+}
+
+static int check_product_shapes(const Csr *a, const Csr *b, const Csr *m, const char *who)
+{
+    if (a->ncols != b->nrows)
+        return set_error(COMET_HIP_ERR_ARG, "%s: A is %lld x %lld but B is %lld x %lld", who, (long long)a->nrows,
+                         (long long)a->ncols, (long long)b->nrows, (long long)b->ncols);
+    if (m && (m->nrows != a->nrows || m->ncols != b->ncols))
+        return set_error(COMET_HIP_ERR_ARG, "%s: mask is %lld x %lld, product is %lld x %lld", who,
+                         (long long)m->nrows, (long long)m->ncols, (long long)a->nrows, (long long)b->ncols);
+    return COMET_HIP_OK;
+}
+
+static int symbolic_counts(const Csr *a, const Csr *b, const Csr *m, int64_t *rowcount)
+{
+    SgGeom g;
+    COMET_CHK(sg_geometry(b->ncols, &g));
+    uint32_t *gbm = nullptr;
+    if (!g.lds) {
+        COMET_CHK(g_sg.gbm.ensure(sizeof(uint32_t) * g.bm_words * (size_t)g.groups, true));
+        gbm = (uint32_t *)g_sg.gbm.ptr;
+    }
+    const dim3 grid((unsigned)g.groups), block(SG_T);
+#define LAUNCH_SYM(L, M)                                                                                   \
+    do {                                                                                                   \
+        COMET_CHK(sg_allow_lds(spgemm_symbolic_kernel<L, M>, g.lds_bytes));                                \
+        KernelTimer t(M ? "spgemm_symbolic_masked" : "spgemm_symbolic");                                   \
+        spgemm_symbolic_kernel<L, M><<<grid, block, g.lds_bytes, stream()>>>(                              \
+            a->nrows, a->pos, a->crd, b->pos, b->crd, m ? m->pos : nullptr, m ? m->crd : nullptr, g.logW,  \
+            gbm, rowcount);                                                                        \
+    } while (0)
+    if (g.lds) {
+        if (m) LAUNCH_SYM(true, true); else LAUNCH_SYM(true, false);
+    } else {
+        if (m) LAUNCH_SYM(false, true); else LAUNCH_SYM(false, false);
+    }
+#undef LAUNCH_SYM
+    COMET_HIPCHK(hipGetLastError());
+    return COMET_HIP_OK;
+}
+
+static int numeric_rows(const Csr *a, const Csr *b, const Csr *m, const int64_t *Cpos, int64_t rb, int64_t re,
+                        int32_t *Ccrd, double *Cval)
+{
+    SgGeom g;
+    COMET_CHK(sg_geometry(b->ncols, &g));
+    uint32_t *gbm = nullptr, *gmask = nullptr;
+    if (!g.lds) {
+        COMET_CHK(g_sg.gbm.ensure(sizeof(uint32_t) * g.bm_words * (size_t)g.groups, true));
+        gbm = (uint32_t *)g_sg.gbm.ptr;
+    }
+    if (m) {
+        COMET_CHK(g_sg.gmask.ensure(sizeof(uint32_t) * g.bm_words * (size_t)g.groups, true));
+        gmask = (uint32_t *)g_sg.gmask.ptr;
+    }
+    COMET_CHK(g_sg.slabs.ensure(sizeof(double) * (size_t)(b->ncols > 0 ? b->ncols : 1) * (size_t)g.groups, true));
+    const dim3 grid((unsigned)g.groups), block(SG_T);
+#define LAUNCH_NUM(L, M)                                                                                   \
+    do {                                                                                                   \
+        COMET_CHK(sg_allow_lds(spgemm_numeric_kernel<L, M>, g.lds_bytes));                                 \
+        KernelTimer t(M ? "spgemm_numeric_masked" : "spgemm_numeric");                                     \
+        spgemm_numeric_kernel<L, M><<<grid, block, g.lds_bytes, stream()>>>(                               \
+            rb, re, b->ncols, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m ? m->pos : nullptr,        \
+            m ? m->crd : nullptr, g.logW, gbm, gmask, (double *)g_sg.slabs.ptr, Cpos, Ccrd, Cval); \
+    } while (0)
+    if (g.lds) {
+        if (m) LAUNCH_NUM(true, true); else LAUNCH_NUM(true, false);
+    } else {
+        if (m) LAUNCH_NUM(false, true); else LAUNCH_NUM(false, false);
+    }
+#undef LAUNCH_NUM
+    COMET_HIPCHK(hipGetLastError());
+    return COMET_HIP_OK;
+}
+
+}  // namespace comet
+
+using namespace comet;
+
+extern "C" int comet_hip_spgemm_csr_symbolic(int64_t ah, int64_t bh, int64_t mh, int64_t pos_dptr, int64_t *nnz_out)
+{
+    COMET_CHK(ensure_init());
+    Csr *a = csr_from_handle(ah), *b = csr_from_handle(bh), *m = mh ? csr_from_handle(mh) : nullptr;
+    if (!a || !b || (mh && !m))
+        return COMET_HIP_ERR_HANDLE;
+    if (!pos_dptr)
+        return set_error(COMET_HIP_ERR_ARG, "null pos passed to comet_hip_spgemm_csr_symbolic");
+    COMET_CHK(check_product_shapes(a, b, m, "spgemm symbolic"));
+    int64_t *pos = (int64_t *)pos_dptr;
+    if (a->nrows > 0) {
+        COMET_CHK(g_sg.rowcount.ensure(sizeof(int64_t) * (size_t)a->nrows, false));
+        COMET_CHK(symbolic_counts(a, b, m, (int64_t *)g_sg.rowcount.ptr));
+    }
+    COMET_CHK(exclusive_scan_i64((const int64_t *)g_sg.rowcount.ptr, a->nrows, pos));
+    if (nnz_out) {
+        COMET_HIPCHK(hipMemcpyAsync(nnz_out, pos + a->nrows, sizeof(int64_t), hipMemcpyDeviceToHost, stream()));
+        COMET_HIPCHK(hipStreamSynchronize(stream()));
+    }
+    return COMET_HIP_OK;
+}
+
+extern "C" int comet_hip_spgemm_csr_numeric(int64_t ah, int64_t bh, int64_t mh, int64_t pos_dptr, int64_t row_begin,
+                                            int64_t row_end, int64_t crd_dptr, int64_t val_dptr)
+{
+    COMET_CHK(ensure_init());
+    Csr *a = csr_from_handle(ah), *b = csr_from_handle(bh), *m = mh ? csr_from_handle(mh) : nullptr;
+    if (!a || !b || (mh && !m))
+        return COMET_HIP_ERR_HANDLE;
+    COMET_CHK(check_product_shapes(a, b, m, "spgemm numeric"));
+    if (row_begin < 0 || row_end < row_begin || row_end > a->nrows)
+        return set_error(COMET_HIP_ERR_ARG, "row range [%lld,%lld) outside [0,%lld]", (long long)row_begin,
+                         (long long)row_end, (long long)a->nrows);
+    if (!pos_dptr || !crd_dptr || !val_dptr)
+        return set_error(COMET_HIP_ERR_ARG, "null output array passed to comet_hip_spgemm_csr_numeric");
+    if (row_begin == row_end)
+        return COMET_HIP_OK;
+    return numeric_rows(a, b, m, (const int64_t *)pos_dptr, row_begin, row_end, (int32_t *)crd_dptr,
+                        (double *)val_dptr);
+}
+
+extern "C" int64_t comet_hip_spgemm_csr(int64_t ah, int64_t bh, int64_t mh)
+{
+    if (ensure_init() != COMET_HIP_OK)
+        return 0;
+    Csr *a = csr_from_handle(ah), *b = csr_from_handle(bh), *m = mh ? csr_from_handle(mh) : nullptr;
+    if (!a || !b || (mh && !m))
+        return 0;
+    if (check_product_shapes(a, b, m, "spgemm") != COMET_HIP_OK)
+        return 0;
+    int64_t *pos = nullptr;
+    if (hipMalloc((void **)&pos, sizeof(int64_t) * (size_t)(a->nrows + 1)) != hipSuccess) {
+        set_error(COMET_HIP_ERR_HIP, "row pointer allocation failed");
+        return 0;
+    }
+    int64_t nnz = 0;
+    if (comet_hip_spgemm_csr_symbolic(ah, bh, mh, (int64_t)pos, &nnz) != COMET_HIP_OK) {
+        (void)hipFree(pos);
+        return 0;
+    }
+    Csr *c = new Csr();
+    c->nrows = a->nrows;
+    c->ncols = b->ncols;
+    c->nnz = nnz;
+    c->pos = pos;
+    c->owns = true;
+    if (hipMalloc((void **)&c->crd, sizeof(int32_t) * (size_t)(nnz > 0 ? nnz : 1)) != hipSuccess ||
+        hipMalloc((void **)&c->val, sizeof(double) * (size_t)(nnz > 0 ? nnz : 1)) != hipSuccess) {
+        set_error(COMET_HIP_ERR_HIP, "output allocation of %lld entries failed", (long long)nnz);
+        (void)hipFree(c->crd);
+        (void)hipFree(pos);
+        delete c;
+        return 0;
+    }
+    if (nnz > 0 && numeric_rows(a, b, m, pos, 0, a->nrows, c->crd, c->val) != COMET_HIP_OK) {
+        (void)hipFree(c->crd);
+        (void)hipFree(c->val);
+        (void)hipFree(pos);
+        delete c;
+        return 0;
+    }
+    return csr_register(c);
+}
+
+extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, double *out)
+{
+    COMET_CHK(ensure_init());
+    Csr *a = csr_from_handle(ah), *b = csr_from_handle(bh), *m = csr_from_handle(mh);
+    if (!a || !b || !m)
+        return COMET_HIP_ERR_HANDLE;
+    if (!out)
+        return set_error(COMET_HIP_ERR_ARG, "null result pointer");
+    COMET_CHK(check_product_shapes(a, b, m, "masked sum"));
+    if (a->nrows == 0) {
+        *out = 0.0;
+        return COMET_HIP_OK;
+    }
+    SgGeom g;
+    COMET_CHK(sg_geometry(b->ncols, &g));
+    COMET_CHK(g_sg.rowcount.ensure(sizeof(double) * (size_t)a->nrows, false));
+    uint32_t *gbm = nullptr;
+    if (!g.lds) {
+        COMET_CHK(g_sg.gbm.ensure(sizeof(uint32_t) * g.bm_words * (size_t)g.groups, true));
+        gbm = (uint32_t *)g_sg.gbm.ptr;
+    }
+    double *rowsum = (double *)g_sg.rowcount.ptr;
+    const dim3 grid((unsigned)g.groups), block(SG_T);
+    if (g.lds) {
+        COMET_CHK(sg_allow_lds(spgemm_masked_sum_kernel<true>, g.lds_bytes));
+        KernelTimer t("spgemm_masked_sum");
+        spgemm_masked_sum_kernel<true><<<grid, block, g.lds_bytes, stream()>>>(
+            a->nrows, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m->pos, m->crd, g.logW, gbm, rowsum);
+    } else {
+        KernelTimer t("spgemm_masked_sum");
+        spgemm_masked_sum_kernel<false><<<grid, block, 0, stream()>>>(
+            a->nrows, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m->pos, m->crd, g.logW, gbm, rowsum);
+    }
+    COMET_HIPCHK(hipGetLastError());
+    return reduce_sum_device(rowsum, a->nrows, out);
+}
+
+extern "C" int64_t comet_hip_eltwise_mult_csr(int64_t ah, int64_t bh)
+{
+    if (ensure_init() != COMET_HIP_OK)
+        return 0;
+    Csr *a = csr_from_handle(ah), *b = csr_from_handle(bh);
+    if (!a || !b)
+        return 0;
+    if (a->nrows != b->nrows || a->ncols != b->ncols) {
+        set_error(COMET_HIP_ERR_ARG, "element-wise product of %lld x %lld and %lld x %lld", (long long)a->nrows,
+                  (long long)a->ncols, (long long)b->nrows, (long long)b->ncols);
+        return 0;
+    }
+    const int64_t n = a->nrows;
+    int64_t *pos = nullptr;
+    if (hipMalloc((void **)&pos, sizeof(int64_t) * (size_t)(n + 1)) != hipSuccess) {
+        set_error(COMET_HIP_ERR_HIP, "row pointer allocation failed");
+        return 0;
+    }
+    auto fail = [&](Csr *c) -> int64_t {
+        if (c) {
+            (void)hipFree(c->crd);
+            (void)hipFree(c->val);
+            delete c;
+        }
+        (void)hipFree(pos);
+        return 0;
+    };
+    if (g_sg.rowcount.ensure(sizeof(int64_t) * (size_t)(n > 0 ? n : 1), false) != COMET_HIP_OK)
+        return fail(nullptr);
+    int64_t *rowcount = (int64_t *)g_sg.rowcount.ptr;
+    const dim3 grid((unsigned)ceil_div(n > 0 ? n : 1, 256)), block(256);
+    if (n > 0) {
+        KernelTimer t("eltwise_mult_count");
+        eltwise_mult_kernel<false><<<grid, block, 0, stream()>>>(n, a->pos, a->crd, a->val, b->pos, b->crd, b->val,
+                                                                 rowcount, nullptr, nullptr, nullptr);
+    }
+    if (exclusive_scan_i64(rowcount, n, pos) != COMET_HIP_OK)
+        return fail(nullptr);
+    int64_t nnz = 0;
+    if (hipMemcpyAsync(&nnz, pos + n, sizeof(int64_t), hipMemcpyDeviceToHost, stream()) != hipSuccess ||
+        hipStreamSynchronize(stream()) != hipSuccess) {
+        set_error(COMET_HIP_ERR_HIP, "reading nnz failed");
+        return fail(nullptr);
+    }
+    Csr *c = new Csr();
+    c->nrows = n;
+    c->ncols = a->ncols;
+    c->nnz = nnz;
+    c->pos = pos;
+    c->owns = true;
+    if (hipMalloc((void **)&c->crd, sizeof(int32_t) * (size_t)(nnz > 0 ? nnz : 1)) != hipSuccess ||
+        hipMalloc((void **)&c->val, sizeof(double) * (size_t)(nnz > 0 ? nnz : 1)) != hipSuccess) {
+        set_error(COMET_HIP_ERR_HIP, "output allocation failed");
+        return fail(c);
+    }
+    if (n > 0 && nnz > 0) {
+        KernelTimer t("eltwise_mult_fill");
+        eltwise_mult_kernel<true><<<grid, block, 0, stream()>>>(n, a->pos, a->crd, a->val, b->pos, b->crd, b->val,
+                                                                nullptr, pos, c->crd, c->val);
+    }
+    if (hipGetLastError() != hipSuccess) {
+        set_error(COMET_HIP_ERR_HIP, "element-wise kernel launch failed");
+        return fail(c);
+    }
+    return csr_register(c);
+}

@@ -1,0 +1,455 @@
+"""ctypes binding of libcomet_hip_rt.so (include/comet_hip_rt.h) plus thin host
+objects that mirror how COMET's lowered code and its Python front end hold
+tensors: dense tensors as contiguous row-major float64, sparse matrices as the
+(pos, crd, val) CSR tuple (frontends/numpy-scipy/cometpy/MLIRGen/lowering.py:
+298-321 in pnnl/COMET passes exactly these arrays to compiled kernels).
+
+There is no CPU fallback: if the shared library has not been built, or no
+MI355X is present, every entry point raises.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libcomet_hip_rt.so")
+
+
+class CometHipError(RuntimeError):
+    pass
+
+
+class TtgtPlan(C.Structure):
+    _fields_ = [
+        ("rankA", C.c_int32), ("rankB", C.c_int32), ("rankC", C.c_int32),
+        ("a_idx", C.c_int32 * 8), ("b_idx", C.c_int32 * 8), ("c_idx", C.c_int32 * 8),
+        ("permA", C.c_int32 * 8), ("permB", C.c_int32 * 8), ("permC", C.c_int32 * 8),
+        ("transA", C.c_int32), ("transB", C.c_int32), ("transC", C.c_int32), ("swapAB", C.c_int32),
+        ("M", C.c_int64), ("N", C.c_int64), ("K", C.c_int64),
+        ("cost", C.c_double),
+        ("candidate", C.c_int32), ("ncandidates", C.c_int32),
+    ]
+
+
+class Memref1D(C.Structure):
+    _fields_ = [("allocated", C.c_void_p), ("aligned", C.c_void_p), ("offset", C.c_int64),
+                ("sizes", C.c_int64 * 1), ("strides", C.c_int64 * 1)]
+
+
+class Memref2D(C.Structure):
+    _fields_ = [("allocated", C.c_void_p), ("aligned", C.c_void_p), ("offset", C.c_int64),
+                ("sizes", C.c_int64 * 2), ("strides", C.c_int64 * 2)]
+
+
+# name -> (restype, argtypes); every symbol include/comet_hip_rt.h declares
+_i64, _i32, _f64, _vp, _int = C.c_int64, C.c_int32, C.c_double, C.c_void_p, C.c_int
+_pi64 = C.POINTER(C.c_int64)
+_m1, _m2 = C.POINTER(Memref1D), C.POINTER(Memref2D)
+SIGNATURES = {
+    "comet_hip_init": (_int, [_int]),
+    "comet_hip_finalize": (_int, []),
+    "comet_hip_last_error": (C.c_char_p, []),
+    "comet_hip_device_name": (_int, [C.c_char_p, _i64]),
+    "comet_hip_malloc": (_i64, [_i64]),
+    "comet_hip_free": (_int, [_i64]),
+    "comet_hip_memcpy": (_int, [_i64, _vp, _i64, _i64]),
+    "comet_hip_memset": (_int, [_i64, _int, _i64]),
+    "comet_hip_sync": (_int, []),
+    "HipMallocF64": (_i64, [_i64]),
+    "HipMallocI64": (_i64, [_i64]),
+    "HipMallocI32": (_i64, [_i64]),
+    "HipFree": (None, [_i64]),
+    "HipMemcpyF64": (None, [_i64, _vp, _vp, _i64, _i64, _i64, _i64]),
+    "HipMemcpyI64": (None, [_i64, _vp, _vp, _i64, _i64, _i64, _i64]),
+    "HipMemcpyI32": (None, [_i64, _vp, _vp, _i64, _i64, _i64, _i64]),
+    "HipMemcpyIndex": (None, [_i64, _vp, _vp, _i64, _i64, _i64, _i64]),
+    "comet_hip_csr_upload_i64": (_i64, [_i64, _i64, _vp, _vp, _vp]),
+    "comet_hip_csr_upload_i32": (_i64, [_i64, _i64, _vp, _vp, _vp]),
+    "comet_hip_csr_wrap": (_i64, [_i64, _i64, _i64, _i64, _i64, _i64]),
+    "comet_hip_csr_dims": (_int, [_i64, _pi64, _pi64, _pi64]),
+    "comet_hip_csr_arrays": (_int, [_i64, _pi64, _pi64, _pi64]),
+    "comet_hip_csr_download_i64": (_int, [_i64, _vp, _vp, _vp]),
+    "comet_hip_csr_download_i32": (_int, [_i64, _vp, _vp, _vp]),
+    "comet_hip_csr_destroy": (_int, [_i64]),
+    "comet_hip_spmv_csr_f64": (_int, [_i64, _i64, _i64, _int]),
+    "comet_hip_spmm_csr_f64": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
+    "comet_hip_spgemm_csr_symbolic": (_int, [_i64, _i64, _i64, _i64, _pi64]),
+    "comet_hip_spgemm_csr_numeric": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64]),
+    "comet_hip_spgemm_csr": (_i64, [_i64, _i64, _i64]),
+    "comet_hip_spgemm_masked_sum": (_int, [_i64, _i64, _i64, C.POINTER(_f64)]),
+    "comet_hip_reduce_sum_f64": (_int, [_i64, _i64, C.POINTER(_f64)]),
+    "comet_hip_eltwise_mult_csr": (_i64, [_i64, _i64]),
+    "comet_hip_transpose_f64": (_int, [_i32, _vp, _vp, _i64, _i64]),
+    "comet_hip_dgemm_f64": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _f64]),
+    "comet_hip_ttgt_plan": (_int, [_i32, _vp, _i32, _vp, _i32, _vp, _vp, _i32, C.POINTER(TtgtPlan)]),
+    "comet_hip_ttgt_contract": (_int, [C.POINTER(TtgtPlan), _vp, _vp, _vp, _i64, _i64, _i64, _f64]),
+    "comet_hip_timer_start": (_int, []),
+    "comet_hip_timer_stop": (_int, [C.POINTER(_f64)]),
+    "comet_hip_profile_enable": (_int, [_int]),
+    "comet_hip_profile_reset": (_int, []),
+    "comet_hip_profile_query": (_int, [C.c_char_p, _pi64, C.POINTER(_f64)]),
+    "comet_hip_profile_name": (_int, [_i32, C.c_char_p, _i64]),
+    "comet_hip_copy_f64": (_int, [_i64, _i64, _i64]),
+    "_mlir_ciface_comet_hip_spmv_csr_f64_i64": (None, [_m1, _m1, _m1, _m1, _m1]),
+    "_mlir_ciface_comet_hip_spmm_csr_f64_i64": (None, [_m1, _m1, _m1, _m2, _m2]),
+    "_mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i64": (None, [_i64, _i64, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _m1]),
+    "_mlir_ciface_comet_hip_spgemm_csr_fill_f64_i64": (None, [_m1, _m1, _m1]),
+    "_mlir_ciface_comet_hip_tricount_f64_i64": (_f64, [_i64, _m1, _m1, _m1]),
+}
+
+_lib = None
+
+
+def lib():
+    """Load the shared library (never builds, never falls back)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise CometHipError(
+                f"{LIB_PATH} is missing: build it first (python -m comet_amd.build or __graft_entry__.build())")
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def _check(rc, what=""):
+    if rc != 0:
+        raise CometHipError(f"{what}: [{rc}] {lib().comet_hip_last_error().decode()}")
+
+
+def _handle(h, what):
+    if not h:
+        raise CometHipError(f"{what}: {lib().comet_hip_last_error().decode()}")
+    return h
+
+
+def init(device=0):
+    _check(lib().comet_hip_init(device), "comet_hip_init")
+
+
+def device_name():
+    buf = C.create_string_buffer(256)
+    _check(lib().comet_hip_device_name(buf, 256), "comet_hip_device_name")
+    return buf.value.decode()
+
+
+def sync():
+    _check(lib().comet_hip_sync(), "comet_hip_sync")
+
+
+def _vptr(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class DeviceArray:
+    """A contiguous row-major array in HBM."""
+
+    def __init__(self, shape, dtype=np.float64, zero=False):
+        self.shape = tuple(int(s) for s in (shape if np.ndim(shape) else (shape,)))
+        self.dtype = np.dtype(dtype)
+        self.size = int(np.prod(self.shape)) if self.shape else 1
+        self.nbytes = self.size * self.dtype.itemsize
+        self.ptr = _handle(lib().comet_hip_malloc(max(self.nbytes, 1)), "comet_hip_malloc")
+        if zero:
+            self.fill_zero()
+
+    @classmethod
+    def from_numpy(cls, a, dtype=None):
+        a = np.ascontiguousarray(a, dtype=dtype or a.dtype)
+        d = cls(a.shape, a.dtype)
+        if a.size:
+            _check(lib().comet_hip_memcpy(d.ptr, _vptr(a), a.nbytes, 0), "upload")
+        return d
+
+    def to_numpy(self):
+        out = np.empty(self.shape, dtype=self.dtype)
+        if self.size:
+            _check(lib().comet_hip_memcpy(self.ptr, _vptr(out), out.nbytes, 1), "download")
+        return out
+
+    def fill_zero(self):
+        _check(lib().comet_hip_memset(self.ptr, 0, self.nbytes), "memset")
+
+    def free(self):
+        if self.ptr:
+            _check(lib().comet_hip_free(self.ptr), "comet_hip_free")
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            if self.ptr and _lib is not None:
+                _lib.comet_hip_free(self.ptr)
+                self.ptr = 0
+        except Exception:
+            pass
+
+
+class CsrMatrix:
+    """Device CSR matrix: pos int64[nrows+1], crd int32[nnz], val float64[nnz]."""
+
+    def __init__(self, handle):
+        self.handle = handle
+
+    @classmethod
+    def from_arrays(cls, shape, pos, crd, val):
+        nrows, ncols = shape
+        pos = np.asarray(pos)
+        if pos.dtype == np.int32:
+            pos = np.ascontiguousarray(pos, dtype=np.int32)
+            crd = np.ascontiguousarray(crd, dtype=np.int32)
+            fn = lib().comet_hip_csr_upload_i32
+        else:
+            pos = np.ascontiguousarray(pos, dtype=np.int64)
+            crd = np.ascontiguousarray(crd, dtype=np.int64)
+            fn = lib().comet_hip_csr_upload_i64
+        val = np.ascontiguousarray(val, dtype=np.float64)
+        if len(pos) != nrows + 1 or len(crd) != len(val):
+            raise ValueError("inconsistent CSR arrays")
+        return cls(_handle(fn(nrows, ncols, _vptr(pos), _vptr(crd), _vptr(val)), "comet_hip_csr_upload"))
+
+    @classmethod
+    def from_scipy(cls, m):
+        m = m.tocsr()
+        m.sort_indices()
+        return cls.from_arrays(m.shape, m.indptr.astype(np.int64), m.indices.astype(np.int64), m.data)
+
+    def dims(self):
+        r, c, n = C.c_int64(), C.c_int64(), C.c_int64()
+        _check(lib().comet_hip_csr_dims(self.handle, C.byref(r), C.byref(c), C.byref(n)), "comet_hip_csr_dims")
+        return r.value, c.value, n.value
+
+    @property
+    def shape(self):
+        return self.dims()[:2]
+
+    @property
+    def nnz(self):
+        return self.dims()[2]
+
+    def device_arrays(self):
+        p, c, v = C.c_int64(), C.c_int64(), C.c_int64()
+        _check(lib().comet_hip_csr_arrays(self.handle, C.byref(p), C.byref(c), C.byref(v)), "comet_hip_csr_arrays")
+        return p.value, c.value, v.value
+
+    def to_arrays(self, index_dtype=np.int64):
+        nrows, _, nnz = self.dims()
+        idt = np.dtype(index_dtype)
+        pos = np.zeros(nrows + 1, dtype=idt)
+        crd = np.zeros(nnz, dtype=idt)
+        val = np.zeros(nnz, dtype=np.float64)
+        fn = lib().comet_hip_csr_download_i64 if idt == np.int64 else lib().comet_hip_csr_download_i32
+        _check(fn(self.handle, _vptr(pos), _vptr(crd) if nnz else None, _vptr(val) if nnz else None), "csr download")
+        return pos, crd, val
+
+    def free(self):
+        if self.handle:
+            _check(lib().comet_hip_csr_destroy(self.handle), "comet_hip_csr_destroy")
+            self.handle = 0
+
+    def __del__(self):
+        try:
+            if self.handle and _lib is not None:
+                _lib.comet_hip_csr_destroy(self.handle)
+                self.handle = 0
+        except Exception:
+            pass
+
+
+# ----------------------------------------------------------------------------- operators
+def spmv(A, x, y=None, accumulate=None):
+    """y (+)= A @ x on device arrays; returns y.  accumulate defaults to True when y is given
+    (the reference always adds into the output it was handed)."""
+    nrows, ncols = A.shape
+    if x.size != ncols:
+        raise ValueError("x has the wrong length")
+    if y is None:
+        y = DeviceArray(nrows)
+        accumulate = False if accumulate is None else accumulate
+        if accumulate:
+            y.fill_zero()
+    elif accumulate is None:
+        accumulate = True
+    _check(lib().comet_hip_spmv_csr_f64(A.handle, x.ptr, y.ptr, int(accumulate)), "comet_hip_spmv_csr_f64")
+    return y
+
+
+def spmm(A, B, Cm=None, accumulate=None):
+    nrows, ncols = A.shape
+    if B.shape[0] != ncols:
+        raise ValueError("B has the wrong number of rows")
+    K = B.shape[1]
+    if Cm is None:
+        Cm = DeviceArray((nrows, K))
+        accumulate = False if accumulate is None else accumulate
+        if accumulate:
+            Cm.fill_zero()
+    elif accumulate is None:
+        accumulate = True
+    _check(lib().comet_hip_spmm_csr_f64(A.handle, K, B.ptr, K, Cm.ptr, K, int(accumulate)), "comet_hip_spmm_csr_f64")
+    return Cm
+
+
+def spgemm(A, B, mask=None):
+    h = lib().comet_hip_spgemm_csr(A.handle, B.handle, mask.handle if mask is not None else 0)
+    return CsrMatrix(_handle(h, "comet_hip_spgemm_csr"))
+
+
+def spgemm_symbolic(A, B, mask=None):
+    """Returns (device row pointer int64[nrows+1], nnz)."""
+    pos = DeviceArray(A.shape[0] + 1, np.int64)
+    nnz = C.c_int64()
+    _check(lib().comet_hip_spgemm_csr_symbolic(A.handle, B.handle, mask.handle if mask is not None else 0,
+                                               pos.ptr, C.byref(nnz)), "comet_hip_spgemm_csr_symbolic")
+    return pos, nnz.value
+
+
+def spgemm_numeric(A, B, pos, row_begin, row_end, crd, val, mask=None):
+    _check(lib().comet_hip_spgemm_csr_numeric(A.handle, B.handle, mask.handle if mask is not None else 0, pos.ptr,
+                                              row_begin, row_end, crd.ptr, val.ptr), "comet_hip_spgemm_csr_numeric")
+
+
+def spgemm_masked_sum(A, B, mask):
+    out = C.c_double()
+    _check(lib().comet_hip_spgemm_masked_sum(A.handle, B.handle, mask.handle, C.byref(out)),
+           "comet_hip_spgemm_masked_sum")
+    return out.value
+
+
+def triangle_count(L):
+    """SUM(C) for C<L> = L * L with L strictly lower triangular."""
+    return spgemm_masked_sum(L, L, L)
+
+
+def reduce_sum(x, n=None):
+    out = C.c_double()
+    _check(lib().comet_hip_reduce_sum_f64(x.ptr, x.size if n is None else n, C.byref(out)), "comet_hip_reduce_sum_f64")
+    return out.value
+
+
+def sum_values(A):
+    """SUM over the stored values of a sparse matrix (the DSL's SUM(A[i,j]))."""
+    _, _, v = A.device_arrays()
+    out = C.c_double()
+    _check(lib().comet_hip_reduce_sum_f64(v, A.nnz, C.byref(out)), "comet_hip_reduce_sum_f64")
+    return out.value
+
+
+def eltwise_mult(A, B):
+    return CsrMatrix(_handle(lib().comet_hip_eltwise_mult_csr(A.handle, B.handle), "comet_hip_eltwise_mult_csr"))
+
+
+def transpose(x, perm, out=None):
+    perm = np.ascontiguousarray(perm, dtype=np.int32)
+    shape = np.array(x.shape, dtype=np.int64)
+    if out is None:
+        out = DeviceArray([x.shape[p] for p in perm])
+    _check(lib().comet_hip_transpose_f64(len(perm), _vptr(shape), _vptr(perm), x.ptr, out.ptr),
+           "comet_hip_transpose_f64")
+    return out
+
+
+def dgemm(A, B, Cm=None, beta=0.0):
+    M, K = A.shape
+    K2, N = B.shape
+    if K != K2:
+        raise ValueError("inner dimensions differ")
+    if Cm is None:
+        Cm = DeviceArray((M, N))
+        beta = 0.0
+    _check(lib().comet_hip_dgemm_f64(M, N, K, A.ptr, B.ptr, Cm.ptr, beta), "comet_hip_dgemm_f64")
+    return Cm
+
+
+def label_ids(a, b, c):
+    """Label numbering by first appearance in A, B, C (frontends/comet_dsl/mlir/MLIRGen.cpp:2236-2276)."""
+    ids = {}
+    for s in (a, b, c):
+        for ch in s:
+            ids.setdefault(ch, len(ids))
+    conv = lambda s: np.array([ids[ch] for ch in s], dtype=np.int32)
+    return ids, conv(a), conv(b), conv(c)
+
+
+def ttgt_plan(a, b, c, extent, which=-1):
+    ids, al, bl, cl = label_ids(a, b, c)
+    ext = np.zeros(len(ids), dtype=np.int64)
+    for ch, i in ids.items():
+        ext[i] = extent[ch]
+    plan = TtgtPlan()
+    _check(lib().comet_hip_ttgt_plan(len(al), _vptr(al), len(bl), _vptr(bl), len(cl), _vptr(cl), _vptr(ext), which,
+                                     C.byref(plan)), "comet_hip_ttgt_plan")
+    return plan
+
+
+def ttgt_contract(a, b, c, A, B, Cm=None, beta=0.0, which=-1, plan=None):
+    """Cm[c] = beta*Cm + sum A[a]*B[b] through transposes + GEMM.  Returns (Cm, plan)."""
+    extent = {}
+    for s, t in ((a, A), (b, B)):
+        for ch, n in zip(s, t.shape):
+            if extent.setdefault(ch, n) != n:
+                raise ValueError(f"label {ch} has two extents")
+    if plan is None:
+        plan = ttgt_plan(a, b, c, extent, which)
+    cshape = [extent[ch] for ch in c]
+    if Cm is None:
+        Cm = DeviceArray(cshape, zero=True)
+    ash, bsh, csh = (np.array(s, dtype=np.int64) for s in (A.shape, B.shape, cshape))
+    _check(lib().comet_hip_ttgt_contract(C.byref(plan), _vptr(ash), _vptr(bsh), _vptr(csh), A.ptr, B.ptr, Cm.ptr, beta),
+           "comet_hip_ttgt_contract")
+    return Cm, plan
+
+
+# ----------------------------------------------------------------------------- timing
+def timer_start():
+    _check(lib().comet_hip_timer_start(), "comet_hip_timer_start")
+
+
+def timer_stop():
+    ms = C.c_double()
+    _check(lib().comet_hip_timer_stop(C.byref(ms)), "comet_hip_timer_stop")
+    return ms.value
+
+
+def profile_enable(on=True):
+    _check(lib().comet_hip_profile_enable(int(on)), "comet_hip_profile_enable")
+
+
+def profile_reset():
+    _check(lib().comet_hip_profile_reset(), "comet_hip_profile_reset")
+
+
+def profile_report():
+    """{kernel name: (launches, total ms)} measured with HIP events on the library's stream."""
+    n = C.c_int64()
+    _check(lib().comet_hip_profile_query(None, C.byref(n), None), "comet_hip_profile_query")
+    out = {}
+    buf = C.create_string_buffer(256)
+    for i in range(n.value):
+        _check(lib().comet_hip_profile_name(i, buf, 256), "comet_hip_profile_name")
+        cnt, ms = C.c_int64(), C.c_double()
+        _check(lib().comet_hip_profile_query(buf.value, C.byref(cnt), C.byref(ms)), "comet_hip_profile_query")
+        out[buf.value.decode()] = (cnt.value, ms.value)
+    return out
+
+
+def memref1d(a):
+    m = Memref1D()
+    m.allocated = m.aligned = a.ctypes.data
+    m.offset = 0
+    m.sizes[0] = a.shape[0]
+    m.strides[0] = 1
+    return m
+
+
+def memref2d(a):
+    m = Memref2D()
+    m.allocated = m.aligned = a.ctypes.data
+    m.offset = 0
+    m.sizes[0], m.sizes[1] = a.shape
+    m.strides[0], m.strides[1] = a.shape[1], 1
+    return m

@@ -1,0 +1,228 @@
+/*
+ * comet_hip_rt.h -- C ABI of the MI355X (gfx950) device runtime and kernel
+ * library for the kernels COMET's index-tree dialect lowers to.
+ *
+ * Lowered COMET host code calls these entry points where it used to run the
+ * generated scf loop nests (CPU) or launch Triton-generated kernels through the
+ * Hip* glue (GPU).  Conventions follow that glue
+ * (lib/ExecutionEngine/HipGpuUtils.cpp:31-159 in pnnl/COMET):
+ *   - device buffers are opaque int64 handles that hold a device address;
+ *   - host tensors arrive as memref descriptors (the `_mlir_ciface_` forms at
+ *     the end of this file) or as plain pointers + sizes;
+ *   - everything runs on one process-wide HIP stream owned by the library.
+ * Unlike the reference glue, which prints and exit(1)s on any HIP error
+ * (HipGpuUtils.cpp:10-19), every function returns a status (0 = success) and
+ * keeps a message for comet_hip_last_error(); setting the environment variable
+ * COMET_HIP_ABORT_ON_ERROR=1 restores print-and-exit.
+ *
+ * Device layout of a CSR matrix: pos int64[nrows+1], crd int32[nnz] (the index
+ * width the reference selects for GPU targets, frontends/comet_dsl/comet.cpp:
+ * 816-823), val float64[nnz]; columns ascending inside each row.  This is the
+ * A2pos/A2crd/Aval part of the reference's sparse-tensor tuple
+ * (lib/Conversion/TensorAlgebraToSCF/SparseTensorConversionPass.cpp:1281-1333).
+ * Dense operands are contiguous row-major float64.
+ */
+#ifndef COMET_HIP_RT_H
+#define COMET_HIP_RT_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define COMET_HIP_OK 0
+#define COMET_HIP_ERR_ARG 1      /* null / negative / inconsistent argument      */
+#define COMET_HIP_ERR_HIP 2      /* a HIP call failed                            */
+#define COMET_HIP_ERR_HANDLE 3   /* unknown or already destroyed handle          */
+#define COMET_HIP_ERR_SIZE 4     /* size overflows what the kernels index with   */
+#define COMET_HIP_ERR_NOGPU 5    /* no usable device                             */
+
+/* ---- lifetime, errors ------------------------------------------------------
+ * Replaces HipSetModuleImage / HipFinit (HipGpuUtils.cpp:39-47,154-159): the
+ * kernels are linked into this library, there is no module image to load. */
+int comet_hip_init(int device);
+int comet_hip_finalize(void);
+const char *comet_hip_last_error(void);
+int comet_hip_device_name(char *buf, int64_t cap);
+
+/* ---- raw device memory -----------------------------------------------------
+ * Replaces HipMalloc{F64,F32,I64,I32} (HipGpuUtils.cpp:49-71), HipFree (:73-78)
+ * and HipMemcpy* (:80-124; direction 0 = host to device, 1 = device to host). */
+int64_t comet_hip_malloc(int64_t bytes);            /* 0 on failure */
+int comet_hip_free(int64_t dptr);
+int comet_hip_memcpy(int64_t dptr, void *host, int64_t bytes, int64_t direction);
+int comet_hip_memset(int64_t dptr, int byte_value, int64_t bytes);
+int comet_hip_sync(void);
+int64_t HipMallocF64(int64_t n);
+int64_t HipMallocI64(int64_t n);
+int64_t HipMallocI32(int64_t n);
+void HipFree(int64_t dptr);
+void HipMemcpyF64(int64_t dptr, void *ptr, void *aligned, int64_t offset, int64_t size, int64_t stride, int64_t dir);
+void HipMemcpyI64(int64_t dptr, void *ptr, void *aligned, int64_t offset, int64_t size, int64_t stride, int64_t dir);
+void HipMemcpyI32(int64_t dptr, void *ptr, void *aligned, int64_t offset, int64_t size, int64_t stride, int64_t dir);
+void HipMemcpyIndex(int64_t dptr, void *ptr, void *aligned, int64_t offset, int64_t size, int64_t stride, int64_t dir);
+
+/* ---- device CSR matrices ---------------------------------------------------
+ * Device-side counterpart of the reader's CSR output (two-call "sizes then
+ * fill" protocol of read_input_sizes_2D_f64 / read_input_2D_f64,
+ * lib/ExecutionEngine/SparseUtils.cpp:1632-1811,1814-2078): upload takes the
+ * host arrays the lowered code already owns; dims + download give them back.
+ * Returns a handle (> 0) or 0 on failure. */
+int64_t comet_hip_csr_upload_i64(int64_t nrows, int64_t ncols, const int64_t *pos,
+                                 const int64_t *crd, const double *val);
+int64_t comet_hip_csr_upload_i32(int64_t nrows, int64_t ncols, const int32_t *pos,
+                                 const int32_t *crd, const double *val);
+/* Wrap device arrays the caller already filled (pos int64, crd int32, val f64);
+ * the handle does not own them. */
+int64_t comet_hip_csr_wrap(int64_t nrows, int64_t ncols, int64_t nnz,
+                           int64_t pos_dptr, int64_t crd_dptr, int64_t val_dptr);
+int comet_hip_csr_dims(int64_t csr, int64_t *nrows, int64_t *ncols, int64_t *nnz);
+int comet_hip_csr_arrays(int64_t csr, int64_t *pos_dptr, int64_t *crd_dptr, int64_t *val_dptr);
+int comet_hip_csr_download_i64(int64_t csr, int64_t *pos, int64_t *crd, double *val);
+int comet_hip_csr_download_i32(int64_t csr, int32_t *pos, int32_t *crd, double *val);
+int comet_hip_csr_destroy(int64_t csr);
+
+/* ---- SpMV  y[i] (+)= sum_p val[p] * x[crd[p]] ------------------------------
+ * Replaces the loop nest of DenseParallelLoopInfo + SparseLoopInfo +
+ * convertCompute (lib/Conversion/IndexTreeToSCF/IndexTreeToSCF.cpp:529-621,
+ * 667-700,1247-1284).  accumulate != 0: y is added to, as the reference does;
+ * accumulate == 0: y is overwritten (the result for a y the caller zero-filled,
+ * without reading it).  x, y are device addresses of float64 vectors. */
+int comet_hip_spmv_csr_f64(int64_t csr, int64_t x_dptr, int64_t y_dptr, int accumulate);
+
+/* ---- SpMM  C[i,:] (+)= sum_p val[p] * B[crd[p],:] --------------------------
+ * Same builders plus the dense inner loop (IndexTreeToSCF.cpp:476-489).
+ * B is ncols x K with row stride ldb, C is nrows x K with row stride ldc
+ * (elements).  accumulate as for SpMV. */
+int comet_hip_spmm_csr_f64(int64_t csr, int64_t K, int64_t b_dptr, int64_t ldb,
+                           int64_t c_dptr, int64_t ldc, int accumulate);
+
+/* ---- SpGEMM  C = A * B, CSR x CSR -> CSR, optional structural mask ---------
+ * Symbolic phase: per-row count of distinct output columns and the row
+ * pointer, replacing the mark-array nest of
+ * lib/Dialect/IndexTree/Transforms/SymbolicCompute.cpp:215-339 as lowered by
+ * lib/Conversion/IndexTreeToSCF/SymbolicDomainConversion.cpp:81-340.
+ * Numeric phase: Gustavson accumulation and sorted row output, replacing the
+ * workspace nest of lib/Dialect/IndexTree/Transforms/WorkspaceTransforms.cpp:
+ * 97-276 as lowered by
+ * lib/Conversion/TensorAlgebraToSCF/SparseTensorConversionPass.cpp:595-638,
+ * 982-1159,261-327 (including its comet_sort call,
+ * lib/ExecutionEngine/SparseUtils.cpp:2600-2626).
+ * mask = 0 for none, else a CSR handle whose pattern restricts the output
+ * (C[i,j] exists only where mask[i,j] is stored): MaskedDomainOp,
+ * lib/Dialect/IndexTree/Transforms/IterationDomainInference.cpp:183-196,
+ * lib/Conversion/IndexTreeToSCF/IndexTreeToSCF.cpp:1083-1148,1327-1448.
+ * The output keeps every structurally reachable entry, also when its value
+ * cancels to 0, with columns ascending per row. */
+/* pos_dptr: device int64[nrows(A)+1], filled; *nnz_out = pos[nrows]. */
+int comet_hip_spgemm_csr_symbolic(int64_t a, int64_t b, int64_t mask,
+                                  int64_t pos_dptr, int64_t *nnz_out);
+/* Rows [row_begin,row_end) of C into crd_dptr (int32) / val_dptr (float64),
+ * written at offset pos[r] - pos[row_begin]; pos_dptr from the symbolic call. */
+int comet_hip_spgemm_csr_numeric(int64_t a, int64_t b, int64_t mask, int64_t pos_dptr,
+                                 int64_t row_begin, int64_t row_end,
+                                 int64_t crd_dptr, int64_t val_dptr);
+/* Both phases; returns a new CSR handle that owns its arrays (0 on failure). */
+int64_t comet_hip_spgemm_csr(int64_t a, int64_t b, int64_t mask);
+
+/* ---- masked SpGEMM + SUM in one pass (triangle counting) -------------------
+ * *out = SUM(C) for C<L> = L * L, the two statements of
+ * test/integration/kernels/triangleCount_SandiaLL_wMasking.ta:18-39, i.e. the
+ * masked numeric phase followed by ReduceOpLowering
+ * (lib/Conversion/TensorAlgebraToSCF/TensorAlgebraToSCF.cpp:417-529), without
+ * materialising C.  a, b, mask may all be the same handle. */
+int comet_hip_spgemm_masked_sum(int64_t a, int64_t b, int64_t mask, double *out);
+
+/* ---- SUM over a device float64 array (ReduceOpLowering, as above) --------- */
+int comet_hip_reduce_sum_f64(int64_t dptr, int64_t n, double *out);
+
+/* ---- CSR .* CSR -> CSR (two-pointer intersection nest,
+ * lib/Conversion/IndexTreeToSCF/IndexTreeToSCF.cpp:864-1053).  New handle. */
+int64_t comet_hip_eltwise_mult_csr(int64_t a, int64_t b);
+
+/* ---- dense tensor transpose, linalg.transpose semantics --------------------
+ * out dim i = in dim perm[i] (how TCtoTTGTDyn.cpp:288-329 builds its
+ * transposes); contiguous row-major float64; rank <= 8. */
+int comet_hip_transpose_f64(int32_t rank, const int64_t *in_shape, const int32_t *perm,
+                            int64_t in_dptr, int64_t out_dptr);
+
+/* ---- row-major DGEMM  C[M,N] = beta*C + A[M,K] * B[K,N] --------------------
+ * Replaces linalg.matmul lowered to loops (frontends/comet_dsl/comet.cpp:
+ * 594-595) and the tiled BLIS micro-kernel path
+ * (_mlir_ciface_linalg_matmul_viewsxs_viewsxs_viewsxs,
+ * lib/ExecutionEngine/blis_interface.cpp:143-181). beta is 0 or 1. */
+int comet_hip_dgemm_f64(int64_t M, int64_t N, int64_t K, int64_t a_dptr, int64_t b_dptr,
+                        int64_t c_dptr, double beta);
+
+/* ---- TTGT contraction ------------------------------------------------------
+ * Plan: index classification, candidate enumeration, cost rule and selection
+ * of include/comet/Dialect/Utils/Utils.h:586-946 and
+ * lib/Dialect/TensorAlgebra/Transforms/TCtoTTGTDyn.cpp:240-272.
+ * x_lab: label id of each dimension in storage order; extent[label] its size;
+ * which = -1 selects by cost (first strict minimum), >= 0 forces a candidate
+ * (--perm-num). */
+typedef struct {
+    int32_t rankA, rankB, rankC;
+    int32_t a_idx[8], b_idx[8], c_idx[8];    /* label order after the transposes      */
+    int32_t permA[8], permB[8], permC[8];    /* linalg.transpose permutations         */
+    int32_t transA, transB, transC, swapAB;  /* which transposes run; operand swap    */
+    int64_t M, N, K;
+    double cost;
+    int32_t candidate, ncandidates;
+} comet_ttgt_plan;
+int comet_hip_ttgt_plan(int32_t rankA, const int32_t *a_lab, int32_t rankB, const int32_t *b_lab,
+                        int32_t rankC, const int32_t *c_lab, const int64_t *extent, int32_t which,
+                        comet_ttgt_plan *plan);
+/* Execute: transposes -> DGEMM -> inverse transpose (TCtoTTGTDyn.cpp:280-672).
+ * a/b/c are device float64 tensors in their declared layouts; workspace for the
+ * transposed copies is owned and cached by the library. */
+int comet_hip_ttgt_contract(const comet_ttgt_plan *plan, const int64_t *a_shape,
+                            const int64_t *b_shape, const int64_t *c_shape,
+                            int64_t a_dptr, int64_t b_dptr, int64_t c_dptr, double beta);
+
+/* ---- timing ----------------------------------------------------------------
+ * HIP events on the library's stream (the reference's getTime /
+ * printElapsedTime, lib/ExecutionEngine/StatUtils.cpp:42-59, measure host wall
+ * clock and cannot see asynchronous kernels).
+ * timer_start/stop bracket a region; kernel profiling, when enabled, records an
+ * event pair around every kernel launch and sums them per kernel name. */
+int comet_hip_timer_start(void);
+int comet_hip_timer_stop(double *ms);
+int comet_hip_profile_enable(int on);
+int comet_hip_profile_reset(void);
+/* name == NULL: number of distinct kernel names recorded so far. */
+int comet_hip_profile_query(const char *name, int64_t *launches, double *total_ms);
+int comet_hip_profile_name(int32_t index, char *buf, int64_t cap);
+/* Plain device-to-device copy kernel (used to calibrate hardware counters). */
+int comet_hip_copy_f64(int64_t dst_dptr, int64_t src_dptr, int64_t n);
+
+/* ---- memref-descriptor forms ----------------------------------------------
+ * What `func.call` sites in lowered code bind to (llvm.emit_c_interface):
+ * pointers to StridedMemRefType<T,N> {T* allocated; T* aligned; int64 offset;
+ * int64 sizes[N]; int64 strides[N]} holding HOST data, exactly as the
+ * reference's other runtime calls receive them
+ * (lib/ExecutionEngine/StatUtils.cpp:89-113, blis_interface.cpp:143-146).
+ * They upload, run the kernel, and copy the result back. */
+typedef struct { void *allocated; void *aligned; int64_t offset; int64_t sizes[1]; int64_t strides[1]; } comet_memref_1d;
+typedef struct { void *allocated; void *aligned; int64_t offset; int64_t sizes[2]; int64_t strides[2]; } comet_memref_2d;
+
+void _mlir_ciface_comet_hip_spmv_csr_f64_i64(comet_memref_1d *pos, comet_memref_1d *crd, comet_memref_1d *val,
+                                             comet_memref_1d *x, comet_memref_1d *y);
+void _mlir_ciface_comet_hip_spmm_csr_f64_i64(comet_memref_1d *pos, comet_memref_1d *crd, comet_memref_1d *val,
+                                             comet_memref_2d *B, comet_memref_2d *C);
+/* SpGEMM in the reader's two-call style: sizes first (nnz of C into
+ * sizes[0]; keeps the device result cached), then fill. */
+void _mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i64(int64_t nrowsA, int64_t ncolsB,
+        comet_memref_1d *Apos, comet_memref_1d *Acrd, comet_memref_1d *Aval,
+        comet_memref_1d *Bpos, comet_memref_1d *Bcrd, comet_memref_1d *Bval,
+        comet_memref_1d *Mpos, comet_memref_1d *Mcrd, comet_memref_1d *sizes);
+void _mlir_ciface_comet_hip_spgemm_csr_fill_f64_i64(comet_memref_1d *Cpos, comet_memref_1d *Ccrd,
+                                                    comet_memref_1d *Cval);
+double _mlir_ciface_comet_hip_tricount_f64_i64(int64_t ncols, comet_memref_1d *pos, comet_memref_1d *crd,
+                                               comet_memref_1d *val);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COMET_HIP_RT_H */

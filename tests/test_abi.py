@@ -1,0 +1,94 @@
+"""CPU-side checks of the C-ABI library: it loads, exports what the header declares,
+reports errors instead of crashing, and its host-only logic (the TTGT plan) agrees with
+the checker.  No kernel is launched here."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from comet_amd import runtime as rt
+from oracle import oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "comet_hip_rt.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"\b((?:comet_hip_|_mlir_ciface_comet_hip_|Hip)[A-Za-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = rt.lib()
+    names = _declared_symbols()
+    assert len(names) >= 45
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in comet_hip_rt.h but not exported"
+    assert set(names) == set(rt.SIGNATURES), set(names) ^ set(rt.SIGNATURES)
+
+
+def test_plan_struct_layout_matches_header():
+    # 3 ranks + 6*8 index slots + 4 flags = 55 int32 -> padded to 224 bytes, 3 int64, 1 double, 2 int32
+    assert C.sizeof(rt.TtgtPlan) == 224 + 24 + 8 + 8
+
+
+def _no_gpu():
+    try:
+        rt.init(0)
+        return False
+    except rt.CometHipError:
+        return True
+
+
+def test_errors_are_reported_not_fatal():
+    if not _no_gpu():
+        pytest.skip("GPU present: covered by the gpu tests")
+    with pytest.raises(rt.CometHipError) as e:
+        rt.init(0)
+    assert "no HIP device" in str(e.value) or "failed" in str(e.value)
+    # every compute entry point refuses to run instead of falling back to the CPU
+    assert rt.lib().comet_hip_malloc(16) == 0
+    assert rt.lib().comet_hip_spmv_csr_f64(1, 0, 0, 0) != 0
+    assert rt.lib().comet_hip_spmm_csr_f64(1, 4, 0, 4, 0, 4, 0) != 0
+    assert rt.lib().comet_hip_dgemm_f64(4, 4, 4, 0, 0, 0, 0.0) != 0
+    pos = np.array([0, 1], dtype=np.int64)
+    crd = np.array([0], dtype=np.int64)
+    val = np.array([1.0])
+    assert rt.lib().comet_hip_csr_upload_i64(1, 1, pos.ctypes.data, crd.ctypes.data, val.ctypes.data) == 0
+    assert rt.lib().comet_hip_last_error()
+
+
+CASES = [("aebf", "dfce", "abcd"), ("cima", "mc", "ia"), ("icmn", "mnca", "ia"), ("ca", "ic", "ia"),
+         ("aedf", "bfce", "abcd"), ("ab", "bc", "ac"), ("ba", "cb", "ca")]
+
+
+@pytest.mark.parametrize("a,b,c", CASES)
+def test_ttgt_plan_matches_checker(a, b, c):
+    sizes = dict(zip("abcdefimn", [2, 3, 4, 5, 3, 2, 3, 4, 2]))
+    ref, chosen, ncand, _ = orc.ttgt_plan(a, b, c, sizes)
+    for which in [-1] + list(range(ncand)):
+        ref, chosen, _, _ = orc.ttgt_plan(a, b, c, sizes, which)
+        got = rt.ttgt_plan(a, b, c, sizes, which)
+        assert got.candidate == chosen and got.ncandidates == ncand
+        for f in ("rankA", "rankB", "rankC", "transA", "transB", "transC", "swapAB", "M", "N", "K"):
+            assert getattr(got, f) == getattr(ref, f), (which, f)
+        assert got.cost == ref.cost
+        for f in ("a_idx", "b_idx", "c_idx", "permA", "permB", "permC"):
+            assert list(getattr(got, f)) == list(getattr(ref, f)), (which, f)
+
+
+def test_ttgt_plan_for_the_benchmark_contraction():
+    p = rt.ttgt_plan("aebf", "dfce", "abcd", {ch: 64 for ch in "abcdef"})
+    assert (p.candidate, p.ncandidates) == (4, 16)
+    assert (p.transA, p.transB, p.transC, p.swapAB) == (1, 1, 0, 0)
+    assert (p.M, p.N, p.K) == (4096, 4096, 4096)
+
+
+def test_ttgt_plan_rejects_non_gemm_expressions():
+    with pytest.raises(rt.CometHipError):
+        rt.ttgt_plan("ab", "ab", "ab", {"a": 2, "b": 2})        # element-wise: label in A, B and C
+    with pytest.raises(rt.CometHipError):
+        rt.ttgt_plan("ab", "bc", "ac", {"a": 2, "b": 2, "c": 2}, which=99)

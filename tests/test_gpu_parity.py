@@ -1,0 +1,446 @@
+"""Parity of the HIP path (called through the C ABI) against the CPU checker on identical
+seeded inputs, the reference's golden vectors, and size-independent properties.
+
+Bars: row pointers, column indices and triangle counts bit-exact; fp64 values within
+1e-12 relative.  Where a value is a sum of signed products the tolerance is taken
+relative to sum(|a||b|) of that entry (the bound summation-order changes obey):
+|got - want| <= 1e-12 * sum|a*b|."""
+import os
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+from comet_amd import gen
+from comet_amd import runtime as rt
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-12
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _device():
+    rt.init(0)
+    print("device:", rt.device_name(), flush=True)
+    yield
+    rt.sync()
+
+
+def _mtx(golden_dir, name, mode=1):
+    return orc.read_mtx_csr(os.path.join(golden_dir, name), mode)
+
+
+def _rand_csr(rng, n, m, density, signed=True):
+    A = sp.random(n, m, density=density, random_state=rng, format="csr",
+                  data_rvs=lambda k: rng.uniform(-1, 1, k) if signed else rng.uniform(0.1, 1, k))
+    A.sort_indices()
+    return A.indptr.astype(np.int64), A.indices.astype(np.int64), A.data.copy()
+
+
+def _abs_csr(pos, crd, val):
+    return pos, crd, np.abs(val)
+
+
+# ----------------------------------------------------------------- runtime plumbing
+def test_upload_download_roundtrip_both_index_widths():
+    rng = np.random.default_rng(0)
+    pos, crd, val = _rand_csr(rng, 300, 200, 0.05)
+    A = rt.CsrMatrix.from_arrays((300, 200), pos, crd, val)
+    assert A.dims() == (300, 200, len(crd))
+    for idt in (np.int64, np.int32):
+        p, c, v = A.to_arrays(idt)
+        assert np.array_equal(p, pos) and np.array_equal(c, crd) and np.array_equal(v, val)
+    B = rt.CsrMatrix.from_arrays((300, 200), pos.astype(np.int32), crd.astype(np.int32), val)
+    p, c, v = B.to_arrays()
+    assert np.array_equal(p, pos) and np.array_equal(c, crd) and np.array_equal(v, val)
+
+
+def test_bad_inputs_are_rejected():
+    pos = np.array([0, 2, 1], dtype=np.int64)
+    with pytest.raises(rt.CometHipError):
+        rt.CsrMatrix.from_arrays((2, 2), pos, np.zeros(1, dtype=np.int64), np.zeros(1))
+    with pytest.raises(rt.CometHipError):      # column out of range
+        rt.CsrMatrix.from_arrays((1, 2), np.array([0, 1]), np.array([5]), np.ones(1))
+    assert rt.lib().comet_hip_spmv_csr_f64(12345, 0, 0, 0) != 0      # unknown handle
+    A = rt.CsrMatrix.from_arrays((1, 2), np.array([0, 1]), np.array([1]), np.ones(1))
+    B = rt.CsrMatrix.from_arrays((3, 2), np.array([0, 0, 0, 0]), np.zeros(0, dtype=np.int64), np.zeros(0))
+    with pytest.raises(rt.CometHipError):      # inner dimensions differ
+        rt.spgemm(A, B)
+
+
+def test_scan_and_reduce():
+    rng = np.random.default_rng(1)
+    v = rng.integers(0, 1000, 100_003).astype(np.float64)
+    d = rt.DeviceArray.from_numpy(v)
+    assert rt.reduce_sum(d) == v.sum()            # integers: exact whatever the order
+    w = rng.uniform(-1, 1, 1_000_003)
+    got = rt.reduce_sum(rt.DeviceArray.from_numpy(w))
+    assert abs(got - orc.reduce_sum(w)) <= RTOL * np.abs(w).sum()
+    assert rt.reduce_sum(rt.DeviceArray(0), 0) == 0.0
+
+
+# ----------------------------------------------------------------- SpMV
+def test_spmv_golden(golden, golden_dir):
+    g = golden["spmv_csr"]
+    (nr, nc), pos, crd, val = _mtx(golden_dir, g["matrix"])
+    A = rt.CsrMatrix.from_arrays((nr, nc), pos, crd, val)
+    y = rt.DeviceArray.from_numpy(np.full(nr, g["y_fill"]))
+    rt.spmv(A, rt.DeviceArray.from_numpy(np.full(nc, g["x_fill"])), y)
+    assert orc.format_f64(y.to_numpy()) == g["printed"]
+
+
+@pytest.mark.parametrize("n,m,density,seed", [(1000, 777, 0.01, 0), (4097, 5000, 0.002, 1), (300, 300, 0.2, 2)])
+def test_spmv_bit_exact_vs_checker(n, m, density, seed):
+    rng = np.random.default_rng(seed)
+    pos, crd, val = _rand_csr(rng, n, m, density)
+    x = rng.uniform(-1, 1, m)
+    y0 = rng.uniform(-1, 1, n)
+    A = rt.CsrMatrix.from_arrays((n, m), pos, crd, val)
+    dx = rt.DeviceArray.from_numpy(x)
+    got_acc = rt.spmv(A, dx, rt.DeviceArray.from_numpy(y0)).to_numpy()
+    assert np.array_equal(got_acc, orc.spmv(pos, crd, val, x, y0))
+    got = rt.spmv(A, dx).to_numpy()
+    assert np.array_equal(got, orc.spmv(pos, crd, val, x))
+
+
+def test_spmv_poisson_shape_scaled_down():
+    pos, crd, val = gen.poisson_csr(n=200_000, mean=10.0, seed=1)
+    x = gen.dense(200_000, seed=11)
+    A = rt.CsrMatrix.from_arrays((200_000, 200_000), pos, crd, val)
+    got = rt.spmv(A, rt.DeviceArray.from_numpy(x)).to_numpy()
+    assert np.array_equal(got, orc.spmv(pos, crd, val, x))
+
+
+def test_spmv_edge_cases():
+    # empty matrix rows, one very long row (longer than an LDS pass), trailing empty rows
+    n, m = 600, 9000
+    pos = np.zeros(n + 1, dtype=np.int64)
+    pos[5:] = 7000
+    pos[300:] = 7003
+    crd = np.concatenate([np.arange(7000), np.array([1, 5, 8999])]).astype(np.int64)
+    rng = np.random.default_rng(3)
+    val = rng.uniform(-1, 1, len(crd))
+    x = rng.uniform(-1, 1, m)
+    A = rt.CsrMatrix.from_arrays((n, m), pos, crd, val)
+    got = rt.spmv(A, rt.DeviceArray.from_numpy(x)).to_numpy()
+    assert np.array_equal(got, orc.spmv(pos, crd, val, x))
+    Z = rt.CsrMatrix.from_arrays((3, 3), np.zeros(4, dtype=np.int64), np.zeros(0, dtype=np.int64), np.zeros(0))
+    y = rt.spmv(Z, rt.DeviceArray.from_numpy(np.ones(3)), rt.DeviceArray.from_numpy(np.array([1.0, 2.0, 3.0])))
+    assert y.to_numpy().tolist() == [1.0, 2.0, 3.0]
+    assert rt.spmv(Z, rt.DeviceArray.from_numpy(np.ones(3))).to_numpy().tolist() == [0.0, 0.0, 0.0]
+
+
+# ----------------------------------------------------------------- SpMM
+def test_spmm_golden(golden, golden_dir):
+    g = golden["spmm_csr"]
+    (nr, nc), pos, crd, val = _mtx(golden_dir, g["matrix"])
+    A = rt.CsrMatrix.from_arrays((nr, nc), pos, crd, val)
+    Cm = rt.DeviceArray.from_numpy(np.full((nr, g["K"]), g["C_fill"]))
+    rt.spmm(A, rt.DeviceArray.from_numpy(np.full((nc, g["K"]), g["B_fill"])), Cm)
+    assert orc.format_f64(Cm.to_numpy()) == g["printed"]
+
+
+def _spmm_check(pos, crd, val, B, C0=None):
+    n = len(pos) - 1
+    A = rt.CsrMatrix.from_arrays((n, B.shape[0]), pos, crd, val)
+    dB = rt.DeviceArray.from_numpy(B)
+    if C0 is None:
+        got = rt.spmm(A, dB).to_numpy()
+    else:
+        got = rt.spmm(A, dB, rt.DeviceArray.from_numpy(C0)).to_numpy()
+    want = orc.spmm(pos, crd, val, B, C0)
+    lens = np.diff(pos)
+    # rows that fit inside one 256-nonzero chunk are computed in the checker's order: bit-exact
+    first_chunk, last_chunk = pos[:-1] // 256, (np.maximum(pos[1:], pos[:-1] + 1) - 1) // 256
+    inside = (first_chunk == last_chunk) | (lens == 0)
+    assert np.array_equal(got[inside], want[inside])
+    bound = orc.spmm(pos, crd, np.abs(val), np.abs(B), None if C0 is None else np.abs(C0))
+    assert np.all(np.abs(got - want) <= RTOL * bound + 0.0)
+    return got, want
+
+
+@pytest.mark.parametrize("n,m,K,density,seed", [(500, 400, 64, 0.02, 0), (1000, 1000, 64, 0.3, 1),
+                                                (257, 129, 7, 0.1, 2), (64, 64, 130, 0.2, 3)])
+def test_spmm_vs_checker(n, m, K, density, seed):
+    rng = np.random.default_rng(seed)
+    pos, crd, val = _rand_csr(rng, n, m, density)
+    B = rng.uniform(-1, 1, (m, K))
+    _spmm_check(pos, crd, val, B)
+    _spmm_check(pos, crd, val, B, rng.uniform(-1, 1, (n, K)))
+
+
+def test_spmm_zipf_shape_scaled_down():
+    pos, crd, val = gen.zipf_csr(n=50_000, mean=16.0, cap=4096, seed=2)
+    B = gen.dense((50_000, 64), seed=12)
+    got, want = _spmm_check(pos, crd, val, B)
+    assert np.diff(pos).max() > 1024     # really has rows that span several chunks
+
+
+def test_spmm_edge_cases():
+    rng = np.random.default_rng(5)
+    # leading, interior and trailing empty rows; a row ending exactly on a chunk boundary; one huge row
+    lens = np.array([0, 0, 256, 0, 1, 255, 0, 1000, 0, 0, 3, 0], dtype=np.int64)
+    m = 2000
+    pos = np.zeros(len(lens) + 1, dtype=np.int64)
+    np.cumsum(lens, out=pos[1:])
+    crd = np.concatenate([np.sort(rng.choice(m, l, replace=False)) for l in lens]).astype(np.int64)
+    val = rng.uniform(-1, 1, len(crd))
+    B = rng.uniform(-1, 1, (m, 64))
+    got, want = _spmm_check(pos, crd, val, B)
+    assert np.all(got[lens == 0] == 0.0)
+    C0 = rng.uniform(-1, 1, (len(lens), 64))
+    got, want = _spmm_check(pos, crd, val, B, C0)
+    assert np.array_equal(got[lens == 0], C0[lens == 0])
+    # no nonzeros at all
+    Z = rt.CsrMatrix.from_arrays((4, 5), np.zeros(5, dtype=np.int64), np.zeros(0, dtype=np.int64), np.zeros(0))
+    out = rt.spmm(Z, rt.DeviceArray.from_numpy(np.ones((5, 3))), rt.DeviceArray.from_numpy(np.ones((4, 3))),
+                  accumulate=False)
+    assert np.all(out.to_numpy() == 0.0)
+
+
+def test_spmm_linearity_at_full_width():
+    # size-independent property: A(B1 + B2) == AB1 + AB2 up to rounding, on a bigger power-law matrix
+    pos, crd, val = gen.zipf_csr(n=100_000, mean=16.0, cap=4096, seed=7)
+    A = rt.CsrMatrix.from_arrays((100_000, 100_000), pos, crd, val)
+    B1, B2 = gen.dense((100_000, 64), seed=21), gen.dense((100_000, 64), seed=22)
+    c1 = rt.spmm(A, rt.DeviceArray.from_numpy(B1)).to_numpy()
+    c2 = rt.spmm(A, rt.DeviceArray.from_numpy(B2)).to_numpy()
+    c12 = rt.spmm(A, rt.DeviceArray.from_numpy(B1 + B2)).to_numpy()
+    scale = np.abs(c1) + np.abs(c2) + 1.0
+    assert np.all(np.abs(c12 - (c1 + c2)) <= 1e-9 * scale)
+
+
+# ----------------------------------------------------------------- SpGEMM
+def test_spgemm_golden(golden, golden_dir):
+    for key, masked in (("spgemm_csr", False), ("spgemm_csr_masked", True)):
+        g = golden[key]
+        (nr, nc), pos, crd, val = _mtx(golden_dir, g["A"])
+        A = rt.CsrMatrix.from_arrays((nr, nc), pos, crd, val)
+        Cm = rt.spgemm(A, A, A if masked else None)
+        p, c, v = Cm.to_arrays()
+        assert p.tolist() == g["pos"] and c.tolist() == g["crd"]
+        assert orc.format_f64(v) == g["printed_val"]
+
+
+def _spgemm_check(a, b, ncolsB, mask=None):
+    (apos, acrd, aval), (bpos, bcrd, bval) = a, b
+    n, kdim = len(apos) - 1, len(bpos) - 1
+    A = rt.CsrMatrix.from_arrays((n, kdim), apos, acrd, aval)
+    B = rt.CsrMatrix.from_arrays((kdim, ncolsB), bpos, bcrd, bval)
+    Mk = None if mask is None else rt.CsrMatrix.from_arrays((n, ncolsB), mask[0], mask[1], np.ones(len(mask[1])))
+    Cm = rt.spgemm(A, B, Mk)
+    p, c, v = Cm.to_arrays()
+    wp, wc, wv = orc.spgemm(apos, acrd, aval, bpos, bcrd, bval, ncolsB, mask=mask)
+    assert np.array_equal(p, wp), "row pointers differ"
+    assert np.array_equal(c, wc), "column indices differ"
+    _, _, bound = orc.spgemm(apos, acrd, np.abs(aval), bpos, bcrd, np.abs(bval), ncolsB, mask=mask)
+    assert np.all(np.abs(v - wv) <= RTOL * bound)
+    return p, c, v
+
+
+@pytest.mark.parametrize("n,k,m,density,seed,signed", [(300, 200, 250, 0.05, 0, True), (1000, 1000, 1000, 0.01, 1, False),
+                                                       (64, 64, 40_000, 0.05, 2, True), (2000, 50, 33, 0.3, 3, True)])
+def test_spgemm_vs_checker(n, k, m, density, seed, signed):
+    rng = np.random.default_rng(seed)
+    a = _rand_csr(rng, n, k, density, signed)
+    b = _rand_csr(rng, k, m, density, signed)
+    _spgemm_check(a, b, m)
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_spgemm_masked_vs_checker(seed):
+    rng = np.random.default_rng(seed)
+    a = _rand_csr(rng, 400, 400, 0.04, signed=False)
+    mk = _rand_csr(rng, 400, 400, 0.1, signed=False)
+    _spgemm_check(a, a, 400, mask=(mk[0], mk[1]))
+
+
+def test_spgemm_wide_matrix_uses_global_bitmap():
+    # more than 2^20 columns: the row bitmap no longer fits LDS
+    rng = np.random.default_rng(4)
+    ncols = (1 << 20) + 4097
+    a = _rand_csr(rng, 50, 60, 0.2, signed=False)
+    bpos = np.arange(0, 61 * 40, 40, dtype=np.int64)
+    bcrd = np.concatenate([np.sort(rng.choice(ncols, 40, replace=False)) for _ in range(60)]).astype(np.int64)
+    bval = rng.uniform(0.1, 1, len(bcrd))
+    _spgemm_check(a, (bpos, bcrd, bval), ncols)
+    rows = [np.unique(rng.choice(bcrd, 30)) for _ in range(50)]     # mask rows drawn from reachable columns
+    mk_pos = np.zeros(51, dtype=np.int64)
+    np.cumsum([len(r) for r in rows], out=mk_pos[1:])
+    _spgemm_check(a, (bpos, bcrd, bval), ncols, mask=(mk_pos, np.concatenate(rows)))
+
+
+def test_spgemm_row_blocks_equal_whole():
+    pos, crd, val = gen.rmat_symmetric_csr(scale=11, edge_factor=8, seed=5)
+    n = 1 << 11
+    A = rt.CsrMatrix.from_arrays((n, n), pos, crd, val)
+    dpos, nnz = rt.spgemm_symbolic(A, A)
+    wp, wc, wv = orc.spgemm(pos, crd, val, pos, crd, val, n)
+    hp = dpos.to_numpy()
+    assert np.array_equal(hp, wp) and nnz == wp[-1]
+    for rb, re in ((0, 7), (7, 1024), (1024, n)):
+        cnt = int(hp[re] - hp[rb])
+        dc, dv = rt.DeviceArray(max(cnt, 1), np.int32), rt.DeviceArray(max(cnt, 1))
+        rt.spgemm_numeric(A, A, dpos, rb, re, dc, dv)
+        c, v = dc.to_numpy()[:cnt], dv.to_numpy()[:cnt]
+        assert np.array_equal(c, wc[hp[rb]:hp[re]])
+        assert np.all(np.abs(v - wv[hp[rb]:hp[re]]) <= RTOL * np.abs(wv[hp[rb]:hp[re]]))
+
+
+def test_spgemm_empty_and_repeatable():
+    Z = rt.CsrMatrix.from_arrays((3, 3), np.zeros(4, dtype=np.int64), np.zeros(0, dtype=np.int64), np.zeros(0))
+    p, c, v = rt.spgemm(Z, Z).to_arrays()
+    assert p.tolist() == [0, 0, 0, 0] and len(c) == 0
+    # the dense slabs and bitmaps must be left clean: a second product gives the same answer
+    rng = np.random.default_rng(9)
+    a = _rand_csr(rng, 500, 500, 0.03, signed=False)
+    first = _spgemm_check(a, a, 500)
+    second = _spgemm_check(a, a, 500)
+    assert np.array_equal(first[1], second[1])
+
+
+# ----------------------------------------------------------------- triangle counting / SUM / eltwise
+def test_triangle_count_golden(golden, golden_dir):
+    g = golden["triangle_count"]
+    (nr, nc), pos, crd, val = _mtx(golden_dir, g["matrix"], g["read_mode"])
+    L = rt.CsrMatrix.from_arrays((nr, nc), pos, crd, val)
+    assert rt.triangle_count(L) == g["count"]
+    # the two-statement program: C<L> = L*L ; SUM(C)
+    assert rt.sum_values(rt.spgemm(L, L, L)) == g["count"]
+    # the unmasked program: SUM((L*L) .* L)
+    E = rt.eltwise_mult(rt.spgemm(L, L), L)
+    assert E.to_arrays()[2].sum() == g["count"]
+
+
+@pytest.mark.parametrize("scale,ef,seed", [(10, 8, 1), (13, 16, 2)])
+def test_triangle_count_rmat_vs_checker_and_trace(scale, ef, seed):
+    pos, crd, val = gen.rmat_symmetric_csr(scale=scale, edge_factor=ef, seed=seed, values="ones")
+    lpos, lcrd, lval = gen.strictly_lower(pos, crd, val)
+    n = 1 << scale
+    L = rt.CsrMatrix.from_arrays((n, n), lpos, lcrd, lval)
+    got = rt.triangle_count(L)
+    assert got == orc.tricount_masked(lpos, lcrd, lval)
+    if scale <= 10:
+        Adj = sp.csr_matrix((val, crd, pos), shape=(n, n))
+        assert got == (Adj @ Adj @ Adj).diagonal().sum() / 6
+    # invariant: the upper-triangular formulation counts the same triangles
+    U = sp.csr_matrix((lval, lcrd, lpos), shape=(n, n)).T.tocsr()
+    U.sort_indices()
+    Ud = rt.CsrMatrix.from_scipy(U)
+    assert rt.triangle_count(Ud) == got
+
+
+def test_masked_sum_general_values():
+    rng = np.random.default_rng(3)
+    a = _rand_csr(rng, 300, 300, 0.05)
+    mk = _rand_csr(rng, 300, 300, 0.2)
+    A = rt.CsrMatrix.from_arrays((300, 300), *a)
+    Mk = rt.CsrMatrix.from_arrays((300, 300), *mk)
+    got = rt.spgemm_masked_sum(A, A, Mk)
+    wp, wc, wv = orc.spgemm(*a, *a, 300, mask=(mk[0], mk[1]))
+    _, _, bound = orc.spgemm(a[0], a[1], np.abs(a[2]), a[0], a[1], np.abs(a[2]), 300, mask=(mk[0], mk[1]))
+    assert abs(got - orc.reduce_sum(wv)) <= RTOL * bound.sum()
+
+
+def test_eltwise_golden_and_random(golden, golden_dir):
+    g = golden["eltwise_mult_csr"]
+    (nr, nc), pos, crd, val = _mtx(golden_dir, g["A"])
+    A = rt.CsrMatrix.from_arrays((nr, nc), pos, crd, val)
+    p, c, v = rt.eltwise_mult(A, A).to_arrays()
+    assert p.tolist() == g["pos"] and c.tolist() == g["crd"] and orc.format_f64(v) == g["printed_val"]
+    rng = np.random.default_rng(2)
+    a, b = _rand_csr(rng, 500, 300, 0.1), _rand_csr(rng, 500, 300, 0.1)
+    p, c, v = rt.eltwise_mult(rt.CsrMatrix.from_arrays((500, 300), *a), rt.CsrMatrix.from_arrays((500, 300), *b)).to_arrays()
+    wp, wc, wv = orc.eltwise_mult(*a, *b)
+    assert np.array_equal(p, wp) and np.array_equal(c, wc) and np.array_equal(v, wv)
+
+
+# ----------------------------------------------------------------- transposes, GEMM, TTGT
+@pytest.mark.parametrize("shape,perm", [((3, 4, 5, 2), (0, 2, 1, 3)), ((3, 4, 5, 2), (3, 1, 2, 0)),
+                                        ((7, 9), (1, 0)), ((16, 33, 65), (2, 0, 1)), ((4, 1, 6, 1, 5), (4, 3, 2, 1, 0)),
+                                        ((5, 6, 7), (0, 1, 2)), ((64, 3, 64), (2, 1, 0))])
+def test_transpose_matches_checker(shape, perm):
+    rng = np.random.default_rng(0)
+    x = rng.uniform(-1, 1, shape)
+    got = rt.transpose(rt.DeviceArray.from_numpy(x), perm).to_numpy()
+    assert np.array_equal(got, orc.transpose(x, perm))
+    assert np.array_equal(got, np.transpose(x, perm))
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 16), (256, 384, 128), (100, 70, 33), (1, 5, 9), (130, 129, 1), (16, 16, 4)])
+def test_dgemm_vs_checker(M, N, K):
+    rng = np.random.default_rng(M + N + K)
+    A, B, C0 = rng.uniform(-1, 1, (M, K)), rng.uniform(-1, 1, (K, N)), rng.uniform(-1, 1, (M, N))
+    dA, dB = rt.DeviceArray.from_numpy(A), rt.DeviceArray.from_numpy(B)
+    bound = np.abs(A) @ np.abs(B)
+    got = rt.dgemm(dA, dB).to_numpy()
+    assert np.all(np.abs(got - orc.gemm_ijk(A, B)) <= RTOL * bound)
+    got1 = rt.dgemm(dA, dB, rt.DeviceArray.from_numpy(C0), beta=1.0).to_numpy()
+    assert np.all(np.abs(got1 - orc.gemm_ijk(A, B, C0)) <= RTOL * (bound + np.abs(C0)))
+
+
+def test_ttgt_goldens(golden):
+    for g in golden["ttgt"]:
+        A = np.full([g["extent"][ch] for ch in g["A"]], g["A_fill"])
+        B = np.full([g["extent"][ch] for ch in g["B"]], g["B_fill"])
+        Cm, plan = rt.ttgt_contract(g["A"], g["B"], g["C"], rt.DeviceArray.from_numpy(A), rt.DeviceArray.from_numpy(B))
+        assert orc.format_f64(Cm.to_numpy()) == g["printed"], g["source"]
+
+
+@pytest.mark.parametrize("a,b,c", [("aebf", "dfce", "abcd"), ("cima", "mc", "ia"), ("icmn", "mnca", "ia")])
+def test_ttgt_every_candidate_vs_checker(a, b, c):
+    rng = np.random.default_rng(4)
+    sizes = dict(zip("abcdefimn", [4, 3, 8, 5, 6, 7, 3, 4, 2]))
+    A = rng.uniform(-1, 1, [sizes[ch] for ch in a])
+    B = rng.uniform(-1, 1, [sizes[ch] for ch in b])
+    dA, dB = rt.DeviceArray.from_numpy(A), rt.DeviceArray.from_numpy(B)
+    bound = np.einsum(f"{a},{b}->{c}", np.abs(A), np.abs(B))
+    ncand = rt.ttgt_plan(a, b, c, sizes).ncandidates
+    C0 = rng.uniform(-1, 1, bound.shape)
+    for which in [-1] + list(range(ncand)):
+        want, _, chosen = orc.ttgt_contract(a, b, c, A, B, which=which)
+        Cm, plan = rt.ttgt_contract(a, b, c, dA, dB, which=which)
+        assert plan.candidate == chosen
+        assert np.all(np.abs(Cm.to_numpy() - want) <= RTOL * bound), which
+        want1, _, _ = orc.ttgt_contract(a, b, c, A, B, C0=C0, beta=1.0, which=which)
+        Cm1, _ = rt.ttgt_contract(a, b, c, dA, dB, Cm=rt.DeviceArray.from_numpy(C0), beta=1.0, which=which)
+        assert np.all(np.abs(Cm1.to_numpy() - want1) <= RTOL * (bound + np.abs(C0))), which
+
+
+def test_ttgt_benchmark_contraction_scaled_down():
+    # same index pattern as the 64^4 contraction at extent 16: GEMM 256 x 256 x 256
+    rng = np.random.default_rng(6)
+    A, B = rng.uniform(-1, 1, (16,) * 4), rng.uniform(-1, 1, (16,) * 4)
+    Cm, plan = rt.ttgt_contract("aebf", "dfce", "abcd", rt.DeviceArray.from_numpy(A), rt.DeviceArray.from_numpy(B))
+    assert plan.candidate == 4
+    want, _, _ = orc.ttgt_contract("aebf", "dfce", "abcd", A, B)
+    bound = np.einsum("aebf,dfce->abcd", np.abs(A), np.abs(B))
+    assert np.all(np.abs(Cm.to_numpy() - want) <= RTOL * bound)
+    assert np.allclose(Cm.to_numpy(), np.einsum("aebf,dfce->abcd", A, B), rtol=0, atol=1e-11)
+
+
+# ----------------------------------------------------------------- memref entry points
+def test_mlir_ciface_entry_points(golden, golden_dir):
+    (nr, nc), pos, crd, val = _mtx(golden_dir, "test_rank2.mtx")
+    L = rt.lib()
+    x, y = np.full(nc, 1.7), np.zeros(nr)
+    L._mlir_ciface_comet_hip_spmv_csr_f64_i64(rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val), rt.memref1d(x),
+                                              rt.memref1d(y))
+    assert orc.format_f64(y) == golden["spmv_csr"]["printed"]
+    B, Cm = np.full((nc, 4), 1.7), np.zeros((nr, 4))
+    L._mlir_ciface_comet_hip_spmm_csr_f64_i64(rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val), rt.memref2d(B),
+                                              rt.memref2d(Cm))
+    assert orc.format_f64(Cm) == golden["spmm_csr"]["printed"]
+    sizes = np.zeros(1, dtype=np.int64)
+    empty = np.zeros(0, dtype=np.int64)
+    L._mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i64(nr, nc, rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val),
+                                                      rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val),
+                                                      rt.memref1d(empty), rt.memref1d(empty), rt.memref1d(sizes))
+    assert sizes[0] == 9
+    cp, cc, cv = np.zeros(nr + 1, dtype=np.int64), np.zeros(9, dtype=np.int64), np.zeros(9)
+    L._mlir_ciface_comet_hip_spgemm_csr_fill_f64_i64(rt.memref1d(cp), rt.memref1d(cc), rt.memref1d(cv))
+    g = golden["spgemm_csr"]
+    assert cp.tolist() == g["pos"] and cc.tolist() == g["crd"] and orc.format_f64(cv) == g["printed_val"]
+    (tr, tc), tpos, tcrd, tval = _mtx(golden_dir, "tc.mtx", 2)
+    assert L._mlir_ciface_comet_hip_tricount_f64_i64(tc, rt.memref1d(tpos), rt.memref1d(tcrd), rt.memref1d(tval)) == 5.0
