@@ -1,0 +1,396 @@
+#!/usr/bin/env python3
+"""Benchmark of the index-tree kernel path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload spmm|spmv|ttgt|tricount|spgemm]
+
+A step is one pass of the kernel over one batch of seeded synthetic input that is already
+resident in HBM.  The default workload is the one the headline metric is quoted on: CSR SpMM,
+A 500,000 x 500,000 with power-law rows (mean 16, cap 4096), B 500,000 x 64 fp64.
+Prints ONE JSON line.  `roofline` describes the dominant kernel: algorithmic bytes (or flops)
+per launch divided by that kernel's average duration, measured here with HIP events on the
+library's stream.  `cpu_baseline` is the CPU checker (oracle/, a restatement of the loop nests
+COMET generates) timed on this machine's host cores on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+FP64_MFMA_PEAK_TFLOPS = 78.6  # MI355X dense fp64 matrix, published
+
+
+def host_threads():
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit():
+        return int(env)
+    try:
+        return len(os.sched_getaffinity(0))
+    except AttributeError:
+        return os.cpu_count() or 1
+
+
+def timed_steps(rt, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    rt.sync()
+    t0 = time.perf_counter()
+    rt.timer_start()
+    for _ in range(steps):
+        fn()
+    dev_ms = rt.timer_stop()
+    rt.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return wall_ms / steps, dev_ms / steps
+
+
+def kernel_times(rt, fn, steps):
+    """Average duration per launch of every kernel `fn` starts, from event pairs."""
+    rt.profile_reset()
+    rt.profile_enable(True)
+    for _ in range(steps):
+        fn()
+    rt.sync()
+    rep = rt.profile_report()
+    rt.profile_enable(False)
+    return {k: {"launches": n, "avg_ms": ms / max(n, 1)} for k, (n, ms) in rep.items()}
+
+
+def cpu_time(fn, budget_s=20.0, min_reps=1, max_reps=5):
+    best = None
+    t_start = time.perf_counter()
+    reps = 0
+    while reps < max_reps and (reps < min_reps or time.perf_counter() - t_start < budget_s):
+        t0 = time.perf_counter()
+        fn()
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+        reps += 1
+        if dt > budget_s / 2:
+            break
+    return best, reps
+
+
+# ----------------------------------------------------------------------------- workloads
+def bench_spmm(rt, orc, gen, args):
+    n, K = args.n or 500_000, 64
+    pos, crd, val = gen.zipf_csr(n=n, mean=16.0, cap=4096, seed=2)
+    nnz = len(crd)
+    B = gen.dense((n, K), seed=3)
+    A = rt.CsrMatrix.from_arrays((n, n), pos, crd, val)
+    dB = rt.DeviceArray.from_numpy(B)
+    dC = rt.DeviceArray((n, K))
+    step = lambda: rt.spmm(A, dB, dC, accumulate=False)
+    step()
+    rt.sync()
+    wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
+    kt = kernel_times(rt, step, args.steps)
+    flops = 2.0 * nnz * K
+    ib = 4
+    alg_bytes = nnz * (8 + ib) + (n + 1) * ib + 8 * n * K + 8 * n * K
+    dom = "spmm_csr_nnzsplit"
+    dom_ms = kt[dom]["avg_ms"]
+    # parity of what was just timed, on a sample of rows (full check lives in tests/)
+    got = dC.to_numpy()
+    rows = np.random.default_rng(0).choice(n, 2000, replace=False)
+    sub_pos = np.zeros(len(rows) + 1, dtype=np.int64)
+    np.cumsum(pos[rows + 1] - pos[rows], out=sub_pos[1:])
+    sel = np.concatenate([np.arange(pos[r], pos[r + 1]) for r in rows])
+    want = orc.spmm(sub_pos, crd[sel], val[sel], B)
+    bound = orc.spmm(sub_pos, crd[sel], np.abs(val[sel]), np.abs(B))
+    parity_ok = bool(np.all(np.abs(got[rows] - want) <= 1e-12 * bound))
+    cpu = None
+    if not args.no_cpu:
+        Cc = np.zeros((n, K))
+        t, reps = cpu_time(lambda: orc.lib().oracle_spmm_csr(n, K, pos, crd, val, B, Cc), budget_s=20.0, min_reps=2)
+        cpu = {"value": flops / t / 1e9, "unit": "GFLOP/s", "cores": host_threads(), "kind": "port",
+               "sample": f"the full workload, best of {reps} runs, {t * 1e3:.1f} ms each (OpenMP over rows)"}
+    lens = np.diff(pos)
+    return {
+        "metric": "CSR SpMM GFLOP/s (+ achieved HBM GB/s as % of roofline) on 1 MI355X",
+        "value": flops / (dev_ms * 1e-3) / 1e9, "unit": "GFLOP/s", "ms_per_step": dev_ms,
+        "dtype": "f64",
+        "config": {"workload": "spmm_csr_zipf", "rows": n, "cols": n, "nnz": int(nnz), "dense_cols": K,
+                   "row_lengths": "Zipf s=1.5 rescaled to mean 16, cap 4096 (untruncated draw, scale, clip)",
+                   "max_row": int(lens.max()), "rows_len1_frac": float((lens == 1).mean()), "seed": 2,
+                   "index_bytes": ib, "accumulate": False},
+        "roofline": {"bound": "hbm", "achieved": alg_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": alg_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": dom, "kernel_avg_ms": dom_ms, "algorithmic_bytes": int(alg_bytes),
+                     "gather_inclusive_bytes": int(nnz * 8 * K + nnz * (8 + ib) + 8 * n * K)},
+        "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
+    }
+
+
+def bench_spmv(rt, orc, gen, args):
+    n = args.n or 1_000_000
+    pos, crd, val = gen.poisson_csr(n=n, mean=10.0, seed=1)
+    nnz = len(crd)
+    x = gen.dense(n, seed=4)
+    A = rt.CsrMatrix.from_arrays((n, n), pos, crd, val)
+    dx = rt.DeviceArray.from_numpy(x)
+    dy = rt.DeviceArray(n)
+    step = lambda: rt.spmv(A, dx, dy, accumulate=False)
+    step()
+    wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
+    kt = kernel_times(rt, step, args.steps)
+    parity_ok = bool(np.array_equal(dy.to_numpy(), orc.spmv(pos, crd, val, x)))
+    flops = 2.0 * nnz
+    ib = 4
+    alg_bytes = nnz * (8 + ib) + (n + 1) * ib + 8 * n + 8 * n
+    dom = "spmv_csr_stream"
+    dom_ms = kt[dom]["avg_ms"]
+    cpu = None
+    if not args.no_cpu:
+        y = np.zeros(n)
+        t, reps = cpu_time(lambda: orc.lib().oracle_spmv_csr(n, pos, crd, val, x, y), budget_s=10.0, min_reps=3)
+        cpu = {"value": flops / t / 1e9, "unit": "GFLOP/s", "cores": host_threads(), "kind": "port",
+               "sample": f"the full workload, best of {reps} runs, {t * 1e3:.1f} ms each (OpenMP over rows)"}
+    return {
+        "metric": "CSR SpMV GFLOP/s (+ achieved HBM GB/s as % of roofline) on 1 MI355X",
+        "value": flops / (dev_ms * 1e-3) / 1e9, "unit": "GFLOP/s", "ms_per_step": dev_ms, "dtype": "f64",
+        "config": {"workload": "spmv_csr_poisson", "rows": n, "cols": n, "nnz": int(nnz), "seed": 1, "index_bytes": ib},
+        "roofline": {"bound": "hbm", "achieved": alg_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": alg_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": dom, "kernel_avg_ms": dom_ms, "algorithmic_bytes": int(alg_bytes)},
+        "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
+    }
+
+
+def bench_ttgt(rt, orc, gen, args):
+    e = args.n or 64
+    A = gen.dense((e,) * 4, seed=5)
+    Bt = gen.dense((e,) * 4, seed=6)
+    dA, dB = rt.DeviceArray.from_numpy(A), rt.DeviceArray.from_numpy(Bt)
+    dC = rt.DeviceArray((e,) * 4, zero=True)
+    plan = rt.ttgt_plan("aebf", "dfce", "abcd", {ch: e for ch in "abcdef"}, which=args.candidate)
+    step = lambda: rt.ttgt_contract("aebf", "dfce", "abcd", dA, dB, dC, beta=0.0, plan=plan)
+    step()
+    wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
+    kt = kernel_times(rt, step, args.steps)
+    M = N = K = e * e
+    flops = 2.0 * M * N * K
+    dom = "dgemm_mfma_kernel"
+    dom_ms = kt[dom]["avg_ms"]
+    # parity on a slab of the output: C[a0,b0,:,:] against the checker's GEMM order is too slow at e = 64,
+    # so compare with numpy's einsum on a few (a,b) pairs, tolerance relative to sum |a||b|
+    got = dC.to_numpy()
+    parity_ok = True
+    for (a0, b0) in ((0, 0), (e // 2, 1), (e - 1, e - 1)):
+        want = np.einsum("ef,dfce->cd", A[a0, :, b0, :], Bt)
+        bound = np.einsum("ef,dfce->cd", np.abs(A[a0, :, b0, :]), np.abs(Bt))
+        parity_ok &= bool(np.all(np.abs(got[a0, b0] - want) <= 1e-12 * bound))
+    cpu = None
+    if not args.no_cpu:
+        # the default lowering runs a naive i-j-k loop nest; time it at a reduced extent and scale by flops
+        m = 768
+        Ac, Bc, Cc = gen.dense((m, m), seed=7), gen.dense((m, m), seed=8), np.zeros((m, m))
+        t, reps = cpu_time(lambda: orc.lib().oracle_gemm_ijk(m, m, m, Ac, Bc, Cc), budget_s=15.0, min_reps=1)
+        cpu = {"value": 2.0 * m ** 3 / t / 1e12, "unit": "TFLOP/s", "cores": host_threads(), "kind": "port",
+               "sample": f"naive i-j-k GEMM {m}^3 (OpenMP over i), best of {reps} runs, {t:.2f} s each; the 4096^3 "
+                         f"GEMM would take about {2.0 * 4096 ** 3 / (2.0 * m ** 3 / t):.0f} s at that rate"}
+    perm_bytes = 2 * 8 * e ** 4 * (plan.transA + plan.transB + plan.transC)
+    return {
+        "metric": "TTGT contraction TFLOP/s (fp64 MFMA GEMM + LDS-tiled transposes) on 1 MI355X",
+        "value": flops / (dev_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": dev_ms, "dtype": "f64",
+        "config": {"workload": "ttgt_aebf_dfce_abcd", "extent": e, "gemm": [M, N, K], "candidate": plan.candidate,
+                   "transposes": {"A": plan.transA, "B": plan.transB, "C": plan.transC}, "beta": 0.0},
+        "roofline": {"bound": "mfma", "achieved": flops / (dom_ms * 1e-3) / 1e12, "peak": FP64_MFMA_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": flops / (dom_ms * 1e-3) / 1e12 / FP64_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "kernel": dom, "kernel_avg_ms": dom_ms, "transpose_bytes": int(perm_bytes)},
+        "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
+    }
+
+
+def _row_products(pos, crd):
+    """Products per output row of A*A: sum over k in A_i of nnz(A_k)."""
+    deg = np.diff(pos)
+    w = deg[crd]
+    out = np.zeros(len(pos) - 1, dtype=np.int64)
+    nz = deg > 0
+    out[nz] = np.add.reduceat(w, pos[:-1][nz])
+    return out
+
+
+def bench_tricount(rt, orc, gen, args):
+    scale = args.scale or 20
+    n = 1 << scale
+    pos, crd, val = gen.rmat_symmetric_csr(scale=scale, edge_factor=16, seed=20, values="ones")
+    lpos, lcrd, lval = gen.strictly_lower(pos, crd, val)
+    del pos, crd, val
+    nnzL = len(lcrd)
+    deg = np.diff(lpos)
+    nprod = int(deg[lcrd].sum())
+    L = rt.CsrMatrix.from_arrays((n, n), lpos, lcrd, lval)
+    out = {}
+    step = lambda: out.__setitem__("count", rt.triangle_count(L))
+    step()
+    wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
+    kt = kernel_times(rt, step, args.steps)
+    dom = "spgemm_masked_sum"
+    dom_ms = kt[dom]["avg_ms"]
+    flops = 2.0 * nprod
+    ib = 4
+    alg_bytes = nnzL * (ib + 8) + (n + 1) * ib + 8
+    cpu = None
+    parity = None
+    if not args.no_cpu:
+        t0 = time.perf_counter()
+        want = orc.tricount_masked(lpos, lcrd, lval)
+        t = time.perf_counter() - t0
+        parity = bool(want == out["count"])
+        cpu = {"value": flops / t / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
+               "sample": f"the full workload once, {t:.1f} s, single thread (the reference never parallelises "
+                         f"sparse-output loops)", "count": want}
+    return {
+        "metric": "masked SpGEMM triangle count GFLOP/s (2 flops per masked-candidate product) on 1 MI355X",
+        "value": flops / (dev_ms * 1e-3) / 1e9, "unit": "GFLOP/s", "ms_per_step": dev_ms, "dtype": "f64",
+        "config": {"workload": "tricount_rmat", "scale": scale, "edge_factor": 16, "nnz_L": int(nnzL),
+                   "products": nprod, "triangles": out["count"], "seed": 20},
+        "roofline": {"bound": "hbm", "achieved": alg_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": alg_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": dom,
+                     "kernel_avg_ms": dom_ms, "algorithmic_bytes": int(alg_bytes)},
+        "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity,
+    }
+
+
+def bench_spgemm(rt, orc, gen, args):
+    """C = A*A on the symmetrised R-MAT graph.  The symbolic phase runs over all rows; the numeric
+    phase runs in row blocks sized to a fixed output budget, each block is checksummed and dropped
+    (at scale 20 the whole of C is larger than HBM)."""
+    scale = args.scale or 20
+    n = 1 << scale
+    pos, crd, val = gen.rmat_symmetric_csr(scale=scale, edge_factor=16, seed=20)
+    nnzA = len(crd)
+    rowprod = _row_products(pos, crd)
+    nprod = int(rowprod.sum())
+    A = rt.CsrMatrix.from_arrays((n, n), pos, crd, val)
+    budget = int(args.budget_gb * (1 << 30)) // 12          # entries per block
+    state = {}
+
+    def step():
+        dpos, nnzC = rt.spgemm_symbolic(A, A)
+        hpos = dpos.to_numpy()
+        maxrow = int(np.diff(hpos).max()) if n else 0
+        if maxrow > budget:
+            raise RuntimeError("a single row exceeds the block budget; raise --budget-gb")
+        cap = max(min(budget, int(nnzC)), 1)
+        if state.get("cap") != cap:        # output block buffers are allocated once and reused
+            state["dcrd"], state["dval"] = rt.DeviceArray(cap, np.int32), rt.DeviceArray(cap)
+            state["cap"] = cap
+        dcrd, dval = state["dcrd"], state["dval"]
+        rb, blocks, vsum = 0, 0, 0.0
+        while rb < n:
+            re = int(np.searchsorted(hpos, hpos[rb] + cap, side="right")) - 1
+            re = min(max(re, rb + 1), n)
+            rt.spgemm_numeric(A, A, dpos, rb, re, dcrd, dval)
+            vsum += rt.reduce_sum(dval, int(hpos[re] - hpos[rb]))
+            rb = re
+            blocks += 1
+        state.update(nnzC=int(nnzC), blocks=blocks, vsum=vsum, hpos=hpos, dpos=dpos)
+
+    step()
+    wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
+    kt = kernel_times(rt, step, max(1, min(args.steps, 2)))
+    nnzC = state["nnzC"]
+    flops = 2.0 * nprod
+    ib = 4
+    alg_bytes = nnzA * (8 + ib) + (n + 1) * ib + nnzC * (8 + ib) + 8 * (n + 1)
+    sym_ms = kt["spgemm_symbolic"]["avg_ms"] * kt["spgemm_symbolic"]["launches"] / max(1, min(args.steps, 2))
+    num_ms = kt["spgemm_numeric"]["avg_ms"] * kt["spgemm_numeric"]["launches"] / max(1, min(args.steps, 2))
+    # sum of all values is a size-independent invariant: sum(C) = sum_k colsum(A)[k] * rowsum(A)[k]
+    rowsum = np.add.reduceat(val, pos[:-1][np.diff(pos) > 0])
+    rs = np.zeros(n)
+    rs[np.diff(pos) > 0] = rowsum
+    cs = np.bincount(crd, weights=val, minlength=n)
+    invariant = float(np.dot(cs, rs))
+    cpu = None
+    parity = {"sum_values_rel_err": abs(state["vsum"] - invariant) / invariant}
+    if not args.no_cpu:
+        # CPU checker on a row sample holding about args.cpu_products products, both phases, single thread
+        rng = np.random.default_rng(0)
+        target = args.cpu_products
+        picks, acc = [], 0
+        order = rng.permutation(n // 256)
+        for b in order:
+            r0, r1 = b * 256, (b + 1) * 256
+            p = int(rowprod[r0:r1].sum())
+            if p == 0 or acc + p > 1.5 * target:
+                continue
+            picks.append((r0, r1))
+            acc += p
+            if acc >= target:
+                break
+        t = 0.0
+        struct_ok = True
+        hpos = state["hpos"]
+        for (r0, r1) in picks:
+            t0 = time.perf_counter()
+            cp, cc, cv = orc.spgemm(pos, crd, val, pos, crd, val, n, rows=(r0, r1))
+            t += time.perf_counter() - t0
+            struct_ok &= bool(np.array_equal(cp, hpos[r0:r1 + 1] - hpos[r0]))
+            cnt = int(hpos[r1] - hpos[r0])
+            if cnt <= state["cap"]:
+                rt.spgemm_numeric(A, A, state["dpos"], r0, r1, state["dcrd"], state["dval"])
+                gc, gv = state["dcrd"].to_numpy()[:cnt], state["dval"].to_numpy()[:cnt]
+                struct_ok &= bool(np.array_equal(gc, cc)) and bool(np.all(np.abs(gv - cv) <= 1e-12 * np.abs(cv)))
+        parity["sampled_blocks_bit_exact_structure_and_1e-12_values"] = struct_ok
+        cpu = {"value": 2.0 * acc / t / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
+               "sample": f"{len(picks)} blocks of 256 rows holding {acc} of {nprod} products, symbolic + numeric, "
+                         f"{t:.1f} s, single thread; extrapolated whole-job time {t * nprod / acc:.0f} s"}
+    return {
+        "metric": "Gustavson SpGEMM GFLOP/s (2 flops per product, symbolic + numeric) on 1 MI355X",
+        "value": flops / (dev_ms * 1e-3) / 1e9, "unit": "GFLOP/s", "ms_per_step": dev_ms, "dtype": "f64",
+        "config": {"workload": "spgemm_rmat_AxA", "scale": scale, "edge_factor": 16, "nnz_A": int(nnzA),
+                   "products": nprod, "nnz_C": nnzC, "row_blocks": state["blocks"], "block_budget_gb": args.budget_gb,
+                   "seed": 20},
+        "roofline": {"bound": "hbm", "achieved": alg_bytes / ((sym_ms + num_ms) * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": alg_bytes / ((sym_ms + num_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "kernel": "spgemm_symbolic + spgemm_numeric", "kernel_avg_ms": sym_ms + num_ms,
+                     "symbolic_ms": sym_ms, "numeric_ms": num_ms, "algorithmic_bytes": int(alg_bytes)},
+        "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity,
+    }
+
+
+WORKLOADS = {"spmm": bench_spmm, "spmv": bench_spmv, "ttgt": bench_ttgt, "tricount": bench_tricount,
+             "spgemm": bench_spgemm}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="spmm")
+    ap.add_argument("--n", type=int, default=0, help="override the problem size (rows, or extent for ttgt)")
+    ap.add_argument("--scale", type=int, default=0, help="R-MAT scale for tricount / spgemm (default 20)")
+    ap.add_argument("--candidate", type=int, default=-1, help="force a TTGT candidate (default: cost rule)")
+    ap.add_argument("--budget-gb", type=float, default=48.0, help="spgemm: output bytes per numeric row block")
+    ap.add_argument("--cpu-products", type=int, default=1_500_000_000, help="spgemm: products in the CPU sample")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (every kernel is single-device; see DESIGN.md "
+                 "for how the path would shard); rerun with --gpus 1")
+    from comet_amd import gen, runtime as rt
+    from oracle import oracle as orc
+    rt.init(0)
+    res = WORKLOADS[args.workload](rt, orc, gen, args)
+    line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"), "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": res.pop("ms_per_step"),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": res.pop("dtype"),
+            "data": "synthetic (seeded numpy PCG64, generated on the host, resident in HBM before timing)",
+            "config": res.pop("config"), "roofline": res.pop("roofline"), "cpu_baseline": res.pop("cpu_baseline"),
+            "device": rt.device_name()}
+    line.update(res)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
