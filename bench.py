@@ -358,7 +358,29 @@ def bench_spgemm(rt, orc, gen, args):
     }
 
 
-WORKLOADS = {"spmm": bench_spmm, "spmv": bench_spmv, "ttgt": bench_ttgt, "tricount": bench_tricount,
+def bench_copy(rt, orc, gen, args):
+    """Plain device-to-device copy of a known size: the yardstick the FETCH_SIZE / WRITE_SIZE counters
+    of the other kernels are scaled by."""
+    n = args.n or (1 << 27)            # 1 GiB read + 1 GiB written
+    src = rt.DeviceArray(n, zero=True)
+    dst = rt.DeviceArray(n)
+    step = lambda: rt._check(rt.lib().comet_hip_copy_f64(dst.ptr, src.ptr, n), "comet_hip_copy_f64")
+    step()
+    wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
+    kt = kernel_times(rt, step, args.steps)
+    dom_ms = kt["copy_f64_kernel"]["avg_ms"]
+    nbytes = 16.0 * n
+    return {
+        "metric": "device copy GB/s (counter calibration)", "value": nbytes / (dev_ms * 1e-3) / 1e9, "unit": "GB/s",
+        "ms_per_step": dev_ms, "dtype": "f64", "config": {"workload": "copy_f64", "elements": n},
+        "roofline": {"bound": "hbm", "achieved": nbytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": nbytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": "copy_f64_kernel",
+                     "kernel_avg_ms": dom_ms, "algorithmic_bytes": int(nbytes)},
+        "cpu_baseline": None, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": None,
+    }
+
+
+WORKLOADS = {"copy": bench_copy, "spmm": bench_spmm, "spmv": bench_spmv, "ttgt": bench_ttgt, "tricount": bench_tricount,
              "spgemm": bench_spgemm}
 
 

@@ -24,7 +24,7 @@ namespace comet {
 
 constexpr int SG_T = 1024;                 // lanes per workgroup
 constexpr int SG_WAVES = SG_T / 64;
-constexpr int SG_LDS_MAX_W = 32;           // words per lane that still fit LDS (32 * 1024 * 4 B = 128 KiB)
+constexpr int SG_LDS_MAX_W = 32;           // words per lane that still fit LDS (33 * 1024 * 4 B = 132 KiB)
 
 __device__ inline int64_t readlane_i64(int64_t v, int lane)
 {
@@ -42,52 +42,62 @@ __device__ inline double readlane_d(double v, int lane)
     return __hiloint2double(hi, lo);
 }
 
-// Bitmap layout: lane t of the workgroup owns the 32*W consecutive columns
-// [t*32*W, (t+1)*32*W) and its k-th word sits at address k*SG_T + t, so that a
-// sweep over "my words" is conflict-free in LDS (and coalesced in HBM).
+// Bitmap layout: word w = j/32 sits at address w + w/W, i.e. one padding word
+// after every W words, W = words per lane.  Random probes of neighbouring
+// columns land in neighbouring LDS banks, and the extraction sweep, in which
+// lane t reads its own words t*W .. t*W+W-1 at addresses t*(W+1)+k, is
+// conflict-free too because W+1 is odd.
 struct BmAddr {
     int logW;
     __device__ inline int word(int j) const
     {
         const int w = j >> 5;
-        return ((w & ((1 << logW) - 1)) << 10) + (w >> logW);   // SG_T == 1 << 10
+        return w + (w >> logW);
     }
     __device__ inline uint32_t bit(int j) const { return 1u << (j & 31); }
 };
-static_assert(SG_T == 1024, "BmAddr::word assumes 1024 lanes");
 
-// Visit every product of output row i: f(j, a*b) for k in A_i (ascending per
-// wavefront), j in B_k.  Each wavefront takes 64 entries of A_i at a time (one
-// per lane, coalesced), then walks them one by one with all lanes striding
-// over B_k.
+// Visit every product of output row i: f(j, q, a) for k in A_i, q over the
+// entries of B_k, j = Bcrd[q], a = A's value (the visitor loads Bval[q] itself,
+// and only if it needs it).  The entries of A_i are dealt to the 16 wavefronts
+// one at a time (entry p goes to wavefront p mod 16), because in a sorted row
+// the neighbours with long rows sit next to each other and would otherwise all
+// land on one wavefront.  A wavefront fetches 64 of its entries at once (one per
+// lane), then walks them one by one with all lanes striding over B_k, four
+// loads in flight per lane.
 template <bool VALUES, typename F>
 __device__ inline void for_each_product(int64_t as, int64_t ae, const int32_t *__restrict__ Acrd,
                                         const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
-                                        const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval, F f)
+                                        const int32_t *__restrict__ Bcrd, F f)
 {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    for (int64_t base = as + (int64_t)wave * 64; base < ae; base += (int64_t)SG_WAVES * 64) {
-        const int cnt = (int)(ae - base < 64 ? ae - base : 64);
+    for (int64_t base = as + wave; base < ae; base += (int64_t)SG_WAVES * 64) {
+        const int64_t left = (ae - base + SG_WAVES - 1) / SG_WAVES;     // my entries from here on
+        const int cnt = (int)(left < 64 ? left : 64);
         int64_t bs = 0, be = 0;
         double a = 0.0;
         if (lane < cnt) {
-            const int k = Acrd[base + lane];
+            const int64_t p = base + (int64_t)lane * SG_WAVES;
+            const int k = Acrd[p];
             bs = Bpos[k];
             be = Bpos[k + 1];
             if (VALUES)
-                a = Aval[base + lane];
+                a = Aval[p];
         }
         for (int t = 0; t < cnt; ++t) {
             const int64_t s = readlane_i64(bs, t), e = readlane_i64(be, t);
             const double at = VALUES ? readlane_d(a, t) : 0.0;
-            for (int64_t q = s + lane; q < e; q += 64) {
-                const int j = Bcrd[q];
-                if (VALUES)
-                    f(j, at * Bval[q]);
-                else
-                    f(j, 0.0);
+            int64_t q = s + lane;
+            for (; q + 192 < e; q += 256) {
+                const int j0 = Bcrd[q], j1 = Bcrd[q + 64], j2 = Bcrd[q + 128], j3 = Bcrd[q + 192];
+                f(j0, q, at);
+                f(j1, q + 64, at);
+                f(j2, q + 128, at);
+                f(j3, q + 192, at);
             }
+            for (; q < e; q += 64)
+                f(Bcrd[q], q, at);
         }
     }
 }
@@ -106,14 +116,27 @@ __device__ inline double wave_sum_f64(double v)
     return v;
 }
 
-// Rows are dealt to workgroups round-robin (row = first + blockIdx.x + n*gridDim.x).
-// The row index is then made of kernel arguments and blockIdx only, so it lives in
-// scalar registers and every branch on it (empty row -> continue, end of loop) is a
-// uniform scalar branch.  That matters because the row loop contains workgroup
-// barriers: a row index that merely happens to be equal in all lanes (for instance
-// one broadcast through LDS from a ticket counter) lets the compiler treat
-// `continue` as divergent and park most lanes in a barrier loop that never
-// advances, which hangs the workgroup.
+// Rows are handed out through a global ticket counter, because row costs differ
+// by six orders of magnitude and follow the bit pattern of the row id in R-MAT
+// graphs (a fixed row -> workgroup map leaves some workgroups with ten times the
+// work of others).  Lane 0 draws the ticket, LDS broadcasts it, and the value is
+// read back through readfirstlane so that it lives in scalar registers: every
+// branch on the row index is then a uniform scalar branch.  That matters because
+// the row loop contains workgroup barriers.  The loop must also keep a single
+// back edge with the draw at its end (no `continue`): with a draw at the top and
+// a `continue` below it the compiler splits the loop per lane and parks lanes
+// 1..1023 in a barrier loop that never draws again, which hangs the workgroup.
+__device__ inline int64_t draw_row(unsigned long long *ticket, int64_t first, int64_t *slot)
+{
+    if (threadIdx.x == 0)
+        *slot = first + (int64_t)atomicAdd(ticket, 1ull);
+    __syncthreads();
+    const int64_t r = *slot;
+    __syncthreads();
+    const int lo = __builtin_amdgcn_readfirstlane((int)(r & 0xffffffff));
+    const int hi = __builtin_amdgcn_readfirstlane((int)(r >> 32));
+    return ((int64_t)hi << 32) | (uint32_t)lo;
+}
 extern __shared__ uint32_t sg_dyn_lds[];
 
 // ---------------------------------------------------------------------------
@@ -125,41 +148,42 @@ template <bool BM_LDS, bool MASKED>
 __global__ __launch_bounds__(SG_T) void spgemm_symbolic_kernel(
     int64_t nrows, const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd,
     const int64_t *__restrict__ Bpos, const int32_t *__restrict__ Bcrd, const int64_t *__restrict__ Mpos,
-    const int32_t *__restrict__ Mcrd, int logW, uint32_t *__restrict__ gbm, int64_t *__restrict__ rowcount)
+    const int32_t *__restrict__ Mcrd, int logW, uint32_t *__restrict__ gbm, unsigned long long *ticket,
+    int64_t *__restrict__ rowcount)
 {
+    __shared__ int64_t row_slot;
     __shared__ int wave_cnt[SG_WAVES];
     uint32_t *bm;
     if constexpr (BM_LDS)
         bm = sg_dyn_lds;
     else
-        bm = gbm + ((size_t)blockIdx.x << (10 + logW));
+        bm = gbm + (size_t)blockIdx.x * (size_t)(SG_T * ((1 << logW) + 1));
     const BmAddr ad{logW};
-    const int nwords = SG_T << logW;
+    const int nwords = SG_T * ((1 << logW) + 1);
     if constexpr (BM_LDS) {
         for (int w = threadIdx.x; w < nwords; w += SG_T)
             bm[w] = 0;
     }
     __syncthreads();
-    for (int64_t i = blockIdx.x; i < nrows; i += gridDim.x) {
+    int64_t i = draw_row(ticket, 0, &row_slot);
+    while (i < nrows) {
         const int64_t as = Apos[i], ae = Apos[i + 1];
-        if (as == ae) {
-            if (threadIdx.x == 0)
-                rowcount[i] = 0;
-            continue;
-        }
+        int64_t ms = 0, me = 1;
         if constexpr (MASKED) {
-            const int64_t ms = Mpos[i], me = Mpos[i + 1];
-            if (ms == me) {
-                if (threadIdx.x == 0)
-                    rowcount[i] = 0;
-                continue;
-            }
+            ms = Mpos[i];
+            me = Mpos[i + 1];
+        }
+        const bool work = as != ae && ms != me;
+        if (!work && threadIdx.x == 0)
+            rowcount[i] = 0;
+        if (work) {
+        if constexpr (MASKED) {
             for (int64_t t = ms + threadIdx.x; t < me; t += SG_T)
                 atomicOr(&bm[ad.word(Mcrd[t])], ad.bit(Mcrd[t]));
             __syncthreads();
         }
         int count = 0;
-        for_each_product<false>(as, ae, Acrd, nullptr, Bpos, Bcrd, nullptr, [&](int j, double) {
+        for_each_product<false>(as, ae, Acrd, nullptr, Bpos, Bcrd, [&](int j, int64_t, double) {
             const uint32_t b = ad.bit(j);
             if constexpr (MASKED) {
                 const uint32_t old = atomicAnd(&bm[ad.word(j)], ~b);
@@ -187,10 +211,11 @@ __global__ __launch_bounds__(SG_T) void spgemm_symbolic_kernel(
             for (int w = threadIdx.x; w < nwords; w += SG_T)
                 bm[w] = 0;
         } else {
-            for_each_product<false>(as, ae, Acrd, nullptr, Bpos, Bcrd, nullptr,
-                                    [&](int j, double) { atomicAnd(&bm[ad.word(j)], 0u); });
+            for_each_product<false>(as, ae, Acrd, nullptr, Bpos, Bcrd,
+                                    [&](int j, int64_t, double) { atomicAnd(&bm[ad.word(j)], 0u); });
         }
-        __syncthreads();
+        }   // work
+        i = draw_row(ticket, 0, &row_slot);     // its barriers also close this row's bitmap clean-up
     }
 }
 
@@ -203,20 +228,21 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
     const int32_t *__restrict__ Acrd, const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
     const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval, const int64_t *__restrict__ Mpos,
     const int32_t *__restrict__ Mcrd, int logW, uint32_t *__restrict__ gbm, uint32_t *__restrict__ gmask,
-    double *__restrict__ slabs, const int64_t *__restrict__ Cpos,
+    double *__restrict__ slabs, unsigned long long *ticket, const int64_t *__restrict__ Cpos,
     int32_t *__restrict__ Ccrd, double *__restrict__ Cval)
 {
+    __shared__ int64_t row_slot;
     __shared__ int wave_tot[SG_WAVES];
     uint32_t *bm;
     if constexpr (BM_LDS)
         bm = sg_dyn_lds;
     else
-        bm = gbm + ((size_t)blockIdx.x << (10 + logW));
-    uint32_t *mbm = MASKED ? gmask + ((size_t)blockIdx.x << (10 + logW)) : nullptr;
+        bm = gbm + (size_t)blockIdx.x * (size_t)(SG_T * ((1 << logW) + 1));
+    uint32_t *mbm = MASKED ? gmask + (size_t)blockIdx.x * (size_t)(SG_T * ((1 << logW) + 1)) : nullptr;
     double *slab = slabs + (size_t)blockIdx.x * (size_t)ncols;
     const BmAddr ad{logW};
     const int W = 1 << logW;
-    const int nwords = SG_T << logW;
+    const int nwords = SG_T * ((1 << logW) + 1);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     if constexpr (BM_LDS) {
         for (int w = threadIdx.x; w < nwords; w += SG_T)
@@ -224,17 +250,17 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
     }
     __syncthreads();
     const int64_t out0 = Cpos[row_begin];
-    for (int64_t i = row_begin + blockIdx.x; i < row_end; i += gridDim.x) {
+    int64_t i = draw_row(ticket, row_begin, &row_slot);
+    while (i < row_end) {
         const int64_t as = Apos[i], ae = Apos[i + 1];
         const int64_t ob = Cpos[i], oe = Cpos[i + 1];
-        if (as == ae || ob == oe)
-            continue;
+        if (as != ae && ob != oe) {
         if constexpr (MASKED) {
             for (int64_t t = Mpos[i] + threadIdx.x; t < Mpos[i + 1]; t += SG_T)
                 atomicOr(&mbm[ad.word(Mcrd[t])], ad.bit(Mcrd[t]));
             __syncthreads();
         }
-        for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, Bval, [&](int j, double v) {
+        for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, [&](int j, int64_t q, double a) {
             const int w = ad.word(j);
             const uint32_t b = ad.bit(j);
             if constexpr (MASKED) {
@@ -242,13 +268,13 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
                     return;
             }
             atomicOr(&bm[w], b);
-            __hip_atomic_fetch_add(&slab[j], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            __hip_atomic_fetch_add(&slab[j], a * Bval[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         });
         __syncthreads();
         // extraction: my words hold my columns in ascending order
         int mine = 0;
         for (int k = 0; k < W; ++k)
-            mine += __popc(BM_LDS ? bm[(k << 10) + threadIdx.x] : atomicOr(&bm[(k << 10) + threadIdx.x], 0u));
+            mine += __popc(BM_LDS ? bm[threadIdx.x * (W + 1) + k] : atomicOr(&bm[threadIdx.x * (W + 1) + k], 0u));
         int inc = mine;
         for (int d = 1; d < 64; d <<= 1) {
             const int o = __shfl_up(inc, d, 64);
@@ -264,10 +290,10 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
         for (int k = 0; k < W; ++k) {
             uint32_t word;
             if constexpr (BM_LDS) {
-                word = bm[(k << 10) + threadIdx.x];
-                bm[(k << 10) + threadIdx.x] = 0;
+                word = bm[threadIdx.x * (W + 1) + k];
+                bm[threadIdx.x * (W + 1) + k] = 0;
             } else {
-                word = atomicAnd(&bm[(k << 10) + threadIdx.x], 0u);
+                word = atomicAnd(&bm[threadIdx.x * (W + 1) + k], 0u);
             }
             const int jbase = (((int)threadIdx.x << logW) + k) << 5;
             while (word) {
@@ -283,7 +309,8 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
             for (int64_t t = Mpos[i] + threadIdx.x; t < Mpos[i + 1]; t += SG_T)
                 atomicAnd(&mbm[ad.word(Mcrd[t])], 0u);
         }
-        __syncthreads();
+        }   // row with output
+        i = draw_row(ticket, row_begin, &row_slot);     // its barriers also close this row's clean-up
     }
 }
 
@@ -297,41 +324,42 @@ __global__ __launch_bounds__(SG_T) void spgemm_masked_sum_kernel(
     int64_t nrows, const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd,
     const double *__restrict__ Aval, const int64_t *__restrict__ Bpos, const int32_t *__restrict__ Bcrd,
     const double *__restrict__ Bval, const int64_t *__restrict__ Mpos, const int32_t *__restrict__ Mcrd,
-    int logW, uint32_t *__restrict__ gbm, double *__restrict__ rowsum)
+    int logW, uint32_t *__restrict__ gbm, unsigned long long *ticket, double *__restrict__ rowsum)
 {
+    __shared__ int64_t row_slot;
     __shared__ double wave_part[SG_WAVES];
     uint32_t *bm;
     if constexpr (BM_LDS)
         bm = sg_dyn_lds;
     else
-        bm = gbm + ((size_t)blockIdx.x << (10 + logW));
+        bm = gbm + (size_t)blockIdx.x * (size_t)(SG_T * ((1 << logW) + 1));
     const BmAddr ad{logW};
-    const int nwords = SG_T << logW;
+    const int nwords = SG_T * ((1 << logW) + 1);
     if constexpr (BM_LDS) {
         for (int w = threadIdx.x; w < nwords; w += SG_T)
             bm[w] = 0;
     }
     __syncthreads();
-    for (int64_t i = blockIdx.x; i < nrows; i += gridDim.x) {
+    int64_t i = draw_row(ticket, 0, &row_slot);
+    while (i < nrows) {
         const int64_t as = Apos[i], ae = Apos[i + 1];
         const int64_t ms = Mpos[i], me = Mpos[i + 1];
-        if (as == ae || ms == me) {
-            if (threadIdx.x == 0)
-                rowsum[i] = 0.0;
-            continue;
-        }
+        const bool work = as != ae && ms != me;
+        if (!work && threadIdx.x == 0)
+            rowsum[i] = 0.0;
+        if (work) {
         for (int64_t t = ms + threadIdx.x; t < me; t += SG_T)
             atomicOr(&bm[ad.word(Mcrd[t])], ad.bit(Mcrd[t]));
         __syncthreads();
         double part = 0.0;
-        for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, Bval, [&](int j, double v) {
+        for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, [&](int j, int64_t q, double a) {
             uint32_t word;
             if constexpr (BM_LDS)
                 word = bm[ad.word(j)];
             else
                 word = atomicOr(&bm[ad.word(j)], 0u);
             if (word & ad.bit(j))
-                part += v;
+                part += a * Bval[q];     // the value is fetched for hits only
         });
         part = wave_sum_f64(part);
         if ((threadIdx.x & 63) == 0)
@@ -345,7 +373,8 @@ __global__ __launch_bounds__(SG_T) void spgemm_masked_sum_kernel(
         }
         for (int64_t t = ms + threadIdx.x; t < me; t += SG_T)
             atomicAnd(&bm[ad.word(Mcrd[t])], 0u);
-        __syncthreads();
+        }   // work
+        i = draw_row(ticket, 0, &row_slot);     // its barriers also close this row's bitmap clean-up
     }
 }
 
@@ -387,6 +416,7 @@ __global__ void eltwise_mult_kernel(int64_t nrows, const int64_t *__restrict__ A
 
 // ------------------------------------------------------------------ host side
 struct SgScratch {
+    Workspace ticket;     // one 64-bit row counter
     Workspace rowcount;   // int64[nrows] / double[nrows]
     Workspace gbm;        // global bitmaps (only when the bitmap does not fit LDS)
     Workspace gmask;      // global mask bitmaps (masked numeric)
@@ -412,7 +442,7 @@ static int sg_geometry(int64_t ncols, SgGeom *g)
         return set_error(COMET_HIP_ERR_SIZE, "too many columns (%lld)", (long long)ncols);
     g->logW = logW;
     g->lds = (1 << logW) <= SG_LDS_MAX_W;
-    g->bm_words = (size_t)SG_T << logW;
+    g->bm_words = (size_t)SG_T * ((size_t)(1 << logW) + 1);
     g->lds_bytes = g->lds ? g->bm_words * sizeof(uint32_t) : 0;
     g->groups = num_cus() > 0 ? num_cus() : 256;
     if (g->lds && g->lds_bytes <= 48 * 1024)
@@ -425,6 +455,13 @@ static int sg_allow_lds(K kernel, size_t bytes)
 {
     if (bytes > 0)
         COMET_HIPCHK(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+    return COMET_HIP_OK;
+}
+
+static int sg_reset_ticket()
+{
+    COMET_CHK(g_sg.ticket.ensure(sizeof(unsigned long long), false));
+    COMET_HIPCHK(hipMemsetAsync(g_sg.ticket.ptr, 0, sizeof(unsigned long long), stream()));
     return COMET_HIP_OK;
 }
 
@@ -443,6 +480,7 @@ static int symbolic_counts(const Csr *a, const Csr *b, const Csr *m, int64_t *ro
 {
     SgGeom g;
     COMET_CHK(sg_geometry(b->ncols, &g));
+    COMET_CHK(sg_reset_ticket());
     uint32_t *gbm = nullptr;
     if (!g.lds) {
         COMET_CHK(g_sg.gbm.ensure(sizeof(uint32_t) * g.bm_words * (size_t)g.groups, true));
@@ -455,7 +493,7 @@ static int symbolic_counts(const Csr *a, const Csr *b, const Csr *m, int64_t *ro
         KernelTimer t(M ? "spgemm_symbolic_masked" : "spgemm_symbolic");                                   \
         spgemm_symbolic_kernel<L, M><<<grid, block, g.lds_bytes, stream()>>>(                              \
             a->nrows, a->pos, a->crd, b->pos, b->crd, m ? m->pos : nullptr, m ? m->crd : nullptr, g.logW,  \
-            gbm, rowcount);                                                                        \
+            gbm, (unsigned long long *)g_sg.ticket.ptr, rowcount);                                                                        \
     } while (0)
     if (g.lds) {
         if (m) LAUNCH_SYM(true, true); else LAUNCH_SYM(true, false);
@@ -472,6 +510,7 @@ static int numeric_rows(const Csr *a, const Csr *b, const Csr *m, const int64_t 
 {
     SgGeom g;
     COMET_CHK(sg_geometry(b->ncols, &g));
+    COMET_CHK(sg_reset_ticket());
     uint32_t *gbm = nullptr, *gmask = nullptr;
     if (!g.lds) {
         COMET_CHK(g_sg.gbm.ensure(sizeof(uint32_t) * g.bm_words * (size_t)g.groups, true));
@@ -489,7 +528,8 @@ static int numeric_rows(const Csr *a, const Csr *b, const Csr *m, const int64_t 
         KernelTimer t(M ? "spgemm_numeric_masked" : "spgemm_numeric");                                     \
         spgemm_numeric_kernel<L, M><<<grid, block, g.lds_bytes, stream()>>>(                               \
             rb, re, b->ncols, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m ? m->pos : nullptr,        \
-            m ? m->crd : nullptr, g.logW, gbm, gmask, (double *)g_sg.slabs.ptr, Cpos, Ccrd, Cval); \
+            m ? m->crd : nullptr, g.logW, gbm, gmask, (double *)g_sg.slabs.ptr, (unsigned long long *)g_sg.ticket.ptr, Cpos,   \
+            Ccrd, Cval); \
     } while (0)
     if (g.lds) {
         if (m) LAUNCH_NUM(true, true); else LAUNCH_NUM(true, false);
@@ -604,6 +644,7 @@ extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, d
     }
     SgGeom g;
     COMET_CHK(sg_geometry(b->ncols, &g));
+    COMET_CHK(sg_reset_ticket());
     COMET_CHK(g_sg.rowcount.ensure(sizeof(double) * (size_t)a->nrows, false));
     uint32_t *gbm = nullptr;
     if (!g.lds) {
@@ -616,11 +657,13 @@ extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, d
         COMET_CHK(sg_allow_lds(spgemm_masked_sum_kernel<true>, g.lds_bytes));
         KernelTimer t("spgemm_masked_sum");
         spgemm_masked_sum_kernel<true><<<grid, block, g.lds_bytes, stream()>>>(
-            a->nrows, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m->pos, m->crd, g.logW, gbm, rowsum);
+            a->nrows, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m->pos, m->crd, g.logW, gbm,
+            (unsigned long long *)g_sg.ticket.ptr, rowsum);
     } else {
         KernelTimer t("spgemm_masked_sum");
         spgemm_masked_sum_kernel<false><<<grid, block, 0, stream()>>>(
-            a->nrows, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m->pos, m->crd, g.logW, gbm, rowsum);
+            a->nrows, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m->pos, m->crd, g.logW, gbm,
+            (unsigned long long *)g_sg.ticket.ptr, rowsum);
     }
     COMET_HIPCHK(hipGetLastError());
     return reduce_sum_device(rowsum, a->nrows, out);
