@@ -26,6 +26,14 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP64_MFMA_PEAK_TFLOPS = 78.6  # MI355X dense fp64 matrix, published
 
 
+_T0 = time.perf_counter()
+
+
+def log(msg):
+    """Progress line on stderr (the JSON result is the only thing printed on stdout)."""
+    print(f"[bench {time.perf_counter() - _T0:7.1f}s] {msg}", file=sys.stderr, flush=True)
+
+
 def host_threads():
     env = os.environ.get("OMP_NUM_THREADS")
     if env and env.isdigit():
@@ -221,6 +229,7 @@ def _row_products(pos, crd):
 def bench_tricount(rt, orc, gen, args):
     scale = args.scale or 20
     n = 1 << scale
+    log(f"generating R-MAT scale {scale}")
     pos, crd, val = gen.rmat_symmetric_csr(scale=scale, edge_factor=16, seed=20, values="ones")
     lpos, lcrd, lval = gen.strictly_lower(pos, crd, val)
     del pos, crd, val
@@ -241,6 +250,7 @@ def bench_tricount(rt, orc, gen, args):
     cpu = None
     parity = None
     if not args.no_cpu:
+        log("CPU checker, full workload")
         t0 = time.perf_counter()
         want = orc.tricount_masked(lpos, lcrd, lval)
         t = time.perf_counter() - t0
@@ -266,16 +276,19 @@ def bench_spgemm(rt, orc, gen, args):
     (at scale 20 the whole of C is larger than HBM)."""
     scale = args.scale or 20
     n = 1 << scale
+    log(f"generating R-MAT scale {scale}")
     pos, crd, val = gen.rmat_symmetric_csr(scale=scale, edge_factor=16, seed=20)
     nnzA = len(crd)
     rowprod = _row_products(pos, crd)
     nprod = int(rowprod.sum())
+    log(f"nnz(A) = {nnzA}, products = {nprod}; uploading")
     A = rt.CsrMatrix.from_arrays((n, n), pos, crd, val)
     budget = int(args.budget_gb * (1 << 30)) // 12          # entries per block
     state = {}
 
     def step():
         dpos, nnzC = rt.spgemm_symbolic(A, A)
+        log(f"symbolic done: nnz(C) = {nnzC}")
         hpos = dpos.to_numpy()
         maxrow = int(np.diff(hpos).max()) if n else 0
         if maxrow > budget:
@@ -291,19 +304,26 @@ def bench_spgemm(rt, orc, gen, args):
             re = min(max(re, rb + 1), n)
             rt.spgemm_numeric(A, A, dpos, rb, re, dcrd, dval)
             vsum += rt.reduce_sum(dval, int(hpos[re] - hpos[rb]))
+            log(f"numeric rows [{rb},{re}): {int(hpos[re] - hpos[rb])} entries")
             rb = re
             blocks += 1
         state.update(nnzC=int(nnzC), blocks=blocks, vsum=vsum, hpos=hpos, dpos=dpos)
 
-    step()
-    wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
-    kt = kernel_times(rt, step, max(1, min(args.steps, 2)))
+    # every step is seconds long: per-kernel event timing stays on during the timed steps
+    for _ in range(args.warmup):
+        step()
+    rt.profile_reset()
+    rt.profile_enable(True)
+    wall_ms, dev_ms = timed_steps(rt, step, args.steps, 0)
+    rep = rt.profile_report()
+    rt.profile_enable(False)
+    kt = {k: {"launches": c, "avg_ms": ms / max(c, 1)} for k, (c, ms) in rep.items()}
     nnzC = state["nnzC"]
     flops = 2.0 * nprod
     ib = 4
     alg_bytes = nnzA * (8 + ib) + (n + 1) * ib + nnzC * (8 + ib) + 8 * (n + 1)
-    sym_ms = kt["spgemm_symbolic"]["avg_ms"] * kt["spgemm_symbolic"]["launches"] / max(1, min(args.steps, 2))
-    num_ms = kt["spgemm_numeric"]["avg_ms"] * kt["spgemm_numeric"]["launches"] / max(1, min(args.steps, 2))
+    sym_ms = kt["spgemm_symbolic"]["avg_ms"] * kt["spgemm_symbolic"]["launches"] / args.steps
+    num_ms = kt["spgemm_numeric"]["avg_ms"] * kt["spgemm_numeric"]["launches"] / args.steps
     # sum of all values is a size-independent invariant: sum(C) = sum_k colsum(A)[k] * rowsum(A)[k]
     rowsum = np.add.reduceat(val, pos[:-1][np.diff(pos) > 0])
     rs = np.zeros(n)
@@ -330,6 +350,7 @@ def bench_spgemm(rt, orc, gen, args):
         t = 0.0
         struct_ok = True
         hpos = state["hpos"]
+        log(f"CPU checker on {len(picks)} row blocks ({acc} products)")
         for (r0, r1) in picks:
             t0 = time.perf_counter()
             cp, cc, cv = orc.spgemm(pos, crd, val, pos, crd, val, n, rows=(r0, r1))
@@ -338,8 +359,9 @@ def bench_spgemm(rt, orc, gen, args):
             cnt = int(hpos[r1] - hpos[r0])
             if cnt <= state["cap"]:
                 rt.spgemm_numeric(A, A, state["dpos"], r0, r1, state["dcrd"], state["dval"])
-                gc, gv = state["dcrd"].to_numpy()[:cnt], state["dval"].to_numpy()[:cnt]
+                gc, gv = state["dcrd"].to_numpy(cnt), state["dval"].to_numpy(cnt)
                 struct_ok &= bool(np.array_equal(gc, cc)) and bool(np.all(np.abs(gv - cv) <= 1e-12 * np.abs(cv)))
+            log(f"  rows [{r0},{r1}): {cnt} entries checked, CPU time so far {t:.1f} s, ok = {struct_ok}")
         parity["sampled_blocks_bit_exact_structure_and_1e-12_values"] = struct_ok
         cpu = {"value": 2.0 * acc / t / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
                "sample": f"{len(picks)} blocks of 256 rows holding {acc} of {nprod} products, symbolic + numeric, "

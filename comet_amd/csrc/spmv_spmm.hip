@@ -131,9 +131,9 @@ __global__ __launch_bounds__(SPMM_WAVES * 64) void spmm_csr_nnzsplit(
         const int cnt = (int)(e - base < 64 ? e - base : 64);
         int my_crd = 0;
         double my_val = 0.0;
-        if (lane < cnt) {
-            my_crd = crd[base + lane];
-            my_val = val[base + lane];
+        if (lane < cnt) {      // A is streamed once: keep it from displacing B in the caches
+            my_crd = __builtin_nontemporal_load(crd + base + lane);
+            my_val = __builtin_nontemporal_load(val + base + lane);
         }
         for (int t0 = 0; t0 < cnt; t0 += SPMM_U) {
             double b[SPMM_U];
@@ -158,8 +158,8 @@ __global__ __launch_bounds__(SPMM_WAVES * 64) void spmm_csr_nnzsplit(
                         if (active) {
                             if (first_piece && head)
                                 carry0[lane] = acc;
-                            else
-                                C[r * ldc + col] = acc;
+                            else     // C is written once and not read again by this kernel
+                                __builtin_nontemporal_store(acc, C + r * ldc + col);
                         }
                         first_piece = false;
                         open = false;

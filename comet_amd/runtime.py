@@ -166,9 +166,15 @@ class DeviceArray:
             _check(lib().comet_hip_memcpy(d.ptr, _vptr(a), a.nbytes, 0), "upload")
         return d
 
-    def to_numpy(self):
-        out = np.empty(self.shape, dtype=self.dtype)
-        if self.size:
+    def to_numpy(self, count=None):
+        """Copy to the host: the whole array, or its first `count` elements (flat)."""
+        if count is None:
+            out = np.empty(self.shape, dtype=self.dtype)
+        else:
+            if count < 0 or count > self.size:
+                raise ValueError("count outside the array")
+            out = np.empty(count, dtype=self.dtype)
+        if out.size:
             _check(lib().comet_hip_memcpy(self.ptr, _vptr(out), out.nbytes, 1), "download")
         return out
 
