@@ -71,9 +71,18 @@ __global__ __launch_bounds__(SPMV_T) void spmv_csr_stream(const int64_t *__restr
 // in an earlier chunk, [1] a piece whose row goes on into the next) and the
 // fix-up kernel adds the pieces in chunk order.
 // ============================================================================
-constexpr int SPMM_CH = 256;   // nonzeros per wavefront
-constexpr int SPMM_U = 16;     // B-row loads in flight per wavefront
-constexpr int SPMM_WAVES = 4;  // wavefronts per workgroup
+#ifndef COMET_SPMM_CH
+#define COMET_SPMM_CH 256
+#endif
+#ifndef COMET_SPMM_U
+#define COMET_SPMM_U 16
+#endif
+#ifndef COMET_SPMM_WAVES
+#define COMET_SPMM_WAVES 4
+#endif
+constexpr int SPMM_CH = COMET_SPMM_CH;        // nonzeros per wavefront
+constexpr int SPMM_U = COMET_SPMM_U;          // B-row loads in flight per wavefront
+constexpr int SPMM_WAVES = COMET_SPMM_WAVES;  // wavefronts per workgroup
 
 // chunk_row[c] = the row r with pos[r] <= c*SPMM_CH < pos[r+1]
 __global__ void spmm_chunk_rows(const int64_t *__restrict__ pos, int64_t nrows, int64_t nchunks,

@@ -215,14 +215,27 @@ static int transpose_device(int rank, const int64_t *in_shape, const int32_t *pe
 // A[l%16][l/16] and B[l/16][l%16] and receives D[4*v + l/16][l%16], v = 0..3
 // (measured on gfx950 with one-hot operands).
 // ============================================================================
-constexpr int GM_BM = 128, GM_BN = 128, GM_BK = 16;
-constexpr int GM_LDA = GM_BM + 4;   // padded leading dimensions (doubles)
-constexpr int GM_LDB = GM_BN + 4;
+#ifndef COMET_GM_BK
+#define COMET_GM_BK 16
+#endif
+#ifndef COMET_GM_PAD
+#define COMET_GM_PAD 4
+#endif
+#ifndef COMET_GM_OCC
+#define COMET_GM_OCC 2
+#endif
+// Measured on the 4096^3 product: 2 wavefronts per SIMD (register budget 256) lifts the kernel from 62 % to
+// 90 % of the fp64 MFMA peak; a deeper K tile (32) does not fit two workgroups' LDS and falls back to 59 %.
+constexpr int GM_BM = 128, GM_BN = 128, GM_BK = COMET_GM_BK;
+constexpr int GM_LDA = GM_BM + COMET_GM_PAD;   // padded leading dimensions (doubles)
+constexpr int GM_LDB = GM_BN + COMET_GM_PAD;
+constexpr int GM_EA = GM_BM * GM_BK / 256;     // doubles each lane stages per tile of A (along k)
+constexpr int GM_EB = GM_BK * GM_BN / 256;     // ... and of B (along n)
 
 typedef double double4_t __attribute__((ext_vector_type(4)));
 
 template <bool GUARD>
-__global__ __launch_bounds__(256) void dgemm_mfma_kernel(int64_t M, int64_t N, int64_t K,
+__global__ __launch_bounds__(256, COMET_GM_OCC) void dgemm_mfma_kernel(int64_t M, int64_t N, int64_t K,
                                                          const double *__restrict__ A,
                                                          const double *__restrict__ B, double *__restrict__ C,
                                                          int use_c)
@@ -235,16 +248,17 @@ __global__ __launch_bounds__(256) void dgemm_mfma_kernel(int64_t M, int64_t N, i
     const int64_t bm = blockIdx.y, bn = blockIdx.x;
     const int64_t m0 = bm * GM_BM, n0 = bn * GM_BN;
 
-    // global -> register staging: A tile 128 x 16 (row tid/2, k half tid%2), B tile 16 x 128 (k tid/16, 8 cols)
-    const int a_row = tid >> 1, a_k = (tid & 1) * 8;
-    const int b_k = tid >> 4, b_col = (tid & 15) * 8;
-    double ra[8], rb[8];
+    // global -> register staging: A tile 128 x BK (two lanes per row, GM_EA consecutive k each),
+    // B tile BK x 128 (GM_EB consecutive columns per lane)
+    const int a_row = tid / (GM_BK / GM_EA), a_k = (tid % (GM_BK / GM_EA)) * GM_EA;
+    const int b_k = tid / (GM_BN / GM_EB), b_col = (tid % (GM_BN / GM_EB)) * GM_EB;
+    double ra[GM_EA], rb[GM_EB];
 
     auto load_tiles = [&](int64_t k0) {
         const int64_t gm = m0 + a_row;
         const double *ap = A + gm * K + k0 + a_k;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
+        for (int e = 0; e < GM_EA; ++e) {
             if (GUARD)
                 ra[e] = (gm < M && k0 + a_k + e < K) ? ap[e] : 0.0;
             else
@@ -253,7 +267,7 @@ __global__ __launch_bounds__(256) void dgemm_mfma_kernel(int64_t M, int64_t N, i
         const int64_t gk = k0 + b_k;
         const double *bp = B + gk * N + n0 + b_col;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
+        for (int e = 0; e < GM_EB; ++e) {
             if (GUARD)
                 rb[e] = (gk < K && n0 + b_col + e < N) ? bp[e] : 0.0;
             else
@@ -262,10 +276,10 @@ __global__ __launch_bounds__(256) void dgemm_mfma_kernel(int64_t M, int64_t N, i
     };
     auto store_tiles = [&](int buf) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
+        for (int e = 0; e < GM_EA; ++e)
             As[buf][a_k + e][a_row] = ra[e];
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
+        for (int e = 0; e < GM_EB; ++e)
             Bs[buf][b_k][b_col + e] = rb[e];
     };
 

@@ -13,7 +13,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libcomet_hip_rt.so")
+# COMET_HIP_LIB points at an alternative build of the same library (used when tuning kernel parameters)
+LIB_PATH = os.environ.get("COMET_HIP_LIB") or os.path.join(_HERE, "libcomet_hip_rt.so")
 
 
 class CometHipError(RuntimeError):
