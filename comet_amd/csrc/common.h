@@ -51,6 +51,19 @@ struct Csr {
     // SpMM plan: row that holds the first nonzero of every fixed-size chunk.
     int32_t *spmm_chunk_row = nullptr;
     int64_t spmm_nchunks = 0;
+    // SpMV plan: the matrix re-stored as `spmv_nb` column blocks (block-major copy of crd/val, one row
+    // pointer array per block) so that the slice of x a pass gathers from stays inside one L2.
+    // spmv_nb == 0: not decided yet; 1: run on the original arrays.
+    int spmv_nb = 0;
+    int64_t *spmv_bpos = nullptr;            // [spmv_nb][nrows + 1], relative to the block's base
+    int32_t *spmv_bcrd = nullptr;
+    double *spmv_bval = nullptr;
+    std::vector<int64_t> spmv_base;          // first entry of each block in spmv_bcrd / spmv_bval
+    // SpGEMM plan for the right-hand operand: sg_blkptr[cb * nrows + k] = number of entries of row k whose
+    // column is below cb * 2^14, for cb = 0..sg_nblk, so that the slice of a row inside one block of 16384
+    // columns is found without searching.
+    int32_t *sg_blkptr = nullptr;
+    int sg_nblk = 0;
 };
 
 Csr *csr_from_handle(int64_t h);           // nullptr (and error set) if unknown

@@ -136,6 +136,14 @@ static void csr_release(Csr *c)
     }
     if (c->spmm_chunk_row)
         (void)hipFree(c->spmm_chunk_row);
+    if (c->sg_blkptr)
+        (void)hipFree(c->sg_blkptr);
+    if (c->spmv_bpos)
+        (void)hipFree(c->spmv_bpos);
+    if (c->spmv_bcrd)
+        (void)hipFree(c->spmv_bcrd);
+    if (c->spmv_bval)
+        (void)hipFree(c->spmv_bval);
     delete c;
 }
 

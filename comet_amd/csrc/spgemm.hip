@@ -228,8 +228,9 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
     const int32_t *__restrict__ Acrd, const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
     const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval, const int64_t *__restrict__ Mpos,
     const int32_t *__restrict__ Mcrd, int logW, uint32_t *__restrict__ gbm, uint32_t *__restrict__ gmask,
-    double *__restrict__ slabs, unsigned long long *ticket, const int64_t *__restrict__ Cpos,
-    int32_t *__restrict__ Ccrd, double *__restrict__ Cval)
+    double *__restrict__ slabs, unsigned long long *ticket, const int64_t *__restrict__ rowprod,
+    int64_t dense_threshold, const int64_t *__restrict__ Cpos, int32_t *__restrict__ Ccrd,
+    double *__restrict__ Cval)
 {
     __shared__ int64_t row_slot;
     __shared__ int wave_tot[SG_WAVES];
@@ -254,7 +255,9 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
     while (i < row_end) {
         const int64_t as = Apos[i], ae = Apos[i + 1];
         const int64_t ob = Cpos[i], oe = Cpos[i + 1];
-        if (as != ae && ob != oe) {
+        // rows with many products are left to spgemm_numeric_dense_kernel
+        const bool mine_to_do = rowprod == nullptr || rowprod[i - row_begin] < dense_threshold;
+        if (as != ae && ob != oe && mine_to_do) {
         if constexpr (MASKED) {
             for (int64_t t = Mpos[i] + threadIdx.x; t < Mpos[i + 1]; t += SG_T)
                 atomicOr(&mbm[ad.word(Mcrd[t])], ad.bit(Mcrd[t]));
@@ -311,6 +314,200 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
         }
         }   // row with output
         i = draw_row(ticket, row_begin, &row_slot);     // its barriers also close this row's clean-up
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Numeric phase for rows with many products: the L2 performs only ~20 G atomic
+// line operations per second, so the slab path above costs one of those per
+// product.  Here a row is swept in blocks of 16384 columns whose accumulators
+// (128 KiB of doubles) and bitmap live in LDS; the products of one block are
+// found through the per-row block pointers of B's plan.  Blocks are visited in
+// ascending order and each is emitted in bitmap order, so the row still comes
+// out sorted.
+// ---------------------------------------------------------------------------
+constexpr int SG_CB_LOG = 14;
+constexpr int SG_CB = 1 << SG_CB_LOG;                                 // columns per block
+constexpr size_t SG_DENSE_LDS = (size_t)SG_CB * 8 + (size_t)SG_CB / 8;  // accumulators + bitmap
+
+// products[i - row_begin] = sum over k in A_i of nnz(B_k); one wavefront per row
+__global__ __launch_bounds__(256) void spgemm_row_products(int64_t row_begin, int64_t row_end,
+                                                           const int64_t *__restrict__ Apos,
+                                                           const int32_t *__restrict__ Acrd,
+                                                           const int64_t *__restrict__ Bpos,
+                                                           int64_t *__restrict__ products)
+{
+    const int64_t i = row_begin + (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= row_end)
+        return;
+    const int lane = threadIdx.x & 63;
+    int64_t s = 0;
+    for (int64_t p = Apos[i] + lane; p < Apos[i + 1]; p += 64) {
+        const int k = Acrd[p];
+        s += Bpos[k + 1] - Bpos[k];
+    }
+    for (int d = 32; d > 0; d >>= 1)
+        s += __shfl_down(s, d, 64);
+    if (lane == 0)
+        products[i - row_begin] = s;
+}
+
+// blkptr[cb * nrows + k] = entries of row k with column < cb * SG_CB
+__global__ void spgemm_block_pointers(int64_t nrows, const int64_t *__restrict__ pos,
+                                      const int32_t *__restrict__ crd, int nblk, int32_t *__restrict__ blkptr)
+{
+    const int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= nrows)
+        return;
+    const int64_t s = pos[k], e = pos[k + 1];
+    int64_t lo = s;
+    blkptr[k] = 0;
+    for (int cb = 1; cb <= nblk; ++cb) {
+        const int64_t bound = (int64_t)cb << SG_CB_LOG;
+        int64_t hi = e;
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (crd[mid] < bound)
+                lo = mid + 1;
+            else
+                hi = mid;
+        }
+        blkptr[(int64_t)cb * nrows + k] = (int32_t)(lo - s);
+    }
+}
+
+__global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
+    int64_t row_begin, int64_t row_end, int64_t nrowsB, const int64_t *__restrict__ Apos,
+    const int32_t *__restrict__ Acrd, const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
+    const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval, const int32_t *__restrict__ blkptr, int nblk,
+    unsigned long long *ticket, const int64_t *__restrict__ rowprod, int64_t dense_threshold,
+    const int64_t *__restrict__ Cpos, int32_t *__restrict__ Ccrd, double *__restrict__ Cval)
+{
+    __shared__ int64_t row_slot;
+    __shared__ int wave_tot[SG_WAVES];
+    double *acc = reinterpret_cast<double *>(sg_dyn_lds);
+    uint32_t *bm = sg_dyn_lds + SG_CB * 2;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    for (int j = threadIdx.x; j < SG_CB; j += SG_T)
+        acc[j] = 0.0;
+    if (threadIdx.x < SG_CB / 32)
+        bm[threadIdx.x] = 0;
+    __syncthreads();
+    const int64_t out0 = Cpos[row_begin];
+    int64_t i = draw_row(ticket, row_begin, &row_slot);
+    while (i < row_end) {
+        const int64_t as = Apos[i], ae = Apos[i + 1];
+        if (as != ae && rowprod[i - row_begin] >= dense_threshold) {
+            int64_t off = Cpos[i] - out0;
+            for (int cb = 0; cb < nblk; ++cb) {
+                const int32_t *bp0 = blkptr + (int64_t)cb * nrowsB, *bp1 = bp0 + nrowsB;
+                const int col0 = cb << SG_CB_LOG;
+                for (int64_t base = as + wave; base < ae; base += (int64_t)SG_WAVES * 64) {
+                    const int64_t left = (ae - base + SG_WAVES - 1) / SG_WAVES;
+                    const int cnt = (int)(left < 64 ? left : 64);
+                    int64_t lo = 0, hi = 0;
+                    double a = 0.0;
+                    if (lane < cnt) {
+                        const int64_t p = base + (int64_t)lane * SG_WAVES;
+                        const int k = Acrd[p];
+                        const int64_t b0 = Bpos[k];
+                        lo = b0 + bp0[k];
+                        hi = b0 + bp1[k];
+                        a = Aval[p];
+                    }
+                    // long slices take the whole wavefront, one at a time; short ones (a slice of one block
+                    // often holds a dozen entries) are handed to the four 16-lane quarters, four at a time
+                    unsigned long long big = __ballot(hi - lo >= 32);
+                    unsigned long long todo = __ballot(lo < hi && hi - lo < 32);
+                    while (big) {
+                        const int t = __builtin_ctzll(big);
+                        big &= big - 1;
+                        const int64_t s = readlane_i64(lo, t), e = readlane_i64(hi, t);
+                        const double at = readlane_d(a, t);
+                        int64_t q = s + lane;
+                        for (; q + 192 < e; q += 256) {      // four loads in flight per lane
+                            const int j0 = Bcrd[q] - col0, j1 = Bcrd[q + 64] - col0;
+                            const int j2 = Bcrd[q + 128] - col0, j3 = Bcrd[q + 192] - col0;
+                            const double v0 = Bval[q], v1 = Bval[q + 64], v2 = Bval[q + 128], v3 = Bval[q + 192];
+                            atomicOr(&bm[j0 >> 5], 1u << (j0 & 31));
+                            atomicOr(&bm[j1 >> 5], 1u << (j1 & 31));
+                            atomicOr(&bm[j2 >> 5], 1u << (j2 & 31));
+                            atomicOr(&bm[j3 >> 5], 1u << (j3 & 31));
+                            __hip_atomic_fetch_add(&acc[j0], at * v0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                            __hip_atomic_fetch_add(&acc[j1], at * v1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                            __hip_atomic_fetch_add(&acc[j2], at * v2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                            __hip_atomic_fetch_add(&acc[j3], at * v3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        }
+                        for (; q < e; q += 64) {
+                            const int j = Bcrd[q] - col0;
+                            atomicOr(&bm[j >> 5], 1u << (j & 31));
+                            __hip_atomic_fetch_add(&acc[j], at * Bval[q], __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+                        }
+                    }
+                    const int quarter = lane >> 4, sub = lane & 15;
+                    while (todo) {
+                        int pick = -1;
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            const int t = todo ? __builtin_ctzll(todo) : -1;
+                            todo = todo ? (todo & (todo - 1)) : 0;
+                            pick = quarter == g ? t : pick;
+                        }
+                        const int src = pick < 0 ? lane : pick;
+                        const int64_t s = ((int64_t)__shfl((int)(lo >> 32), src, 64) << 32) |
+                                          (uint32_t)__shfl((int)(lo & 0xffffffff), src, 64);
+                        const int64_t e = ((int64_t)__shfl((int)(hi >> 32), src, 64) << 32) |
+                                          (uint32_t)__shfl((int)(hi & 0xffffffff), src, 64);
+                        const double at = __hiloint2double(__shfl(__double2hiint(a), src, 64),
+                                                           __shfl(__double2loint(a), src, 64));
+                        if (pick >= 0) {
+                            for (int64_t q = s + sub; q < e; q += 16) {
+                                const int j = Bcrd[q] - col0;
+                                atomicOr(&bm[j >> 5], 1u << (j & 31));
+                                __hip_atomic_fetch_add(&acc[j], at * Bval[q], __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_WORKGROUP);
+                            }
+                        }
+                    }
+                }
+                __syncthreads();
+                // emit this block: lane t < 512 owns bitmap word t, i.e. 32 consecutive columns
+                uint32_t word = threadIdx.x < SG_CB / 32 ? bm[threadIdx.x] : 0u;
+                const int mine = __popc(word);
+                int inc = mine;
+                for (int d = 1; d < 64; d <<= 1) {
+                    const int o = __shfl_up(inc, d, 64);
+                    if (lane >= d)
+                        inc += o;
+                }
+                if (lane == 63)
+                    wave_tot[wave] = inc;
+                __syncthreads();
+                int64_t o = off + (inc - mine);
+                int total = 0;
+                for (int w = 0; w < SG_WAVES; ++w) {
+                    if (w < wave)
+                        o += wave_tot[w];
+                    total += wave_tot[w];
+                }
+                const int jbase = (int)threadIdx.x << 5;
+                while (word) {
+                    const int b = __ffs(word) - 1;
+                    word &= word - 1;
+                    Ccrd[o] = col0 + jbase + b;
+                    Cval[o] = acc[jbase + b];
+                    acc[jbase + b] = 0.0;
+                    ++o;
+                }
+                if (threadIdx.x < SG_CB / 32)
+                    bm[threadIdx.x] = 0;
+                off += total;
+                __syncthreads();
+            }
+        }
+        i = draw_row(ticket, row_begin, &row_slot);
     }
 }
 
@@ -421,6 +618,7 @@ struct SgScratch {
     Workspace gbm;        // global bitmaps (only when the bitmap does not fit LDS)
     Workspace gmask;      // global mask bitmaps (masked numeric)
     Workspace slabs;      // dense accumulators, zero between calls
+    Workspace rowprod;    // products per row of the current row range
 };
 static SgScratch g_sg;
 
@@ -505,12 +703,55 @@ static int symbolic_counts(const Csr *a, const Csr *b, const Csr *m, int64_t *ro
     return COMET_HIP_OK;
 }
 
-static int numeric_rows(const Csr *a, const Csr *b, const Csr *m, const int64_t *Cpos, int64_t rb, int64_t re,
+constexpr int SG_DENSE_MAX_BLOCKS = 64;        // the dense path serves matrices of up to 2^20 columns
+#ifndef COMET_SG_DENSE_PER_BLOCK
+#define COMET_SG_DENSE_PER_BLOCK 128
+#endif
+constexpr int64_t SG_DENSE_PER_BLOCK = COMET_SG_DENSE_PER_BLOCK;   // products per column block from which a block sweep pays
+
+// Per-row block pointers of the right-hand operand, built once per matrix.
+static int sg_plan_blocks(Csr *b)
+{
+    const int nblk = (int)ceil_div(b->ncols > 0 ? b->ncols : 1, SG_CB);
+    if (b->sg_blkptr && b->sg_nblk == nblk)
+        return COMET_HIP_OK;
+    if (b->sg_blkptr) {
+        COMET_HIPCHK(hipStreamSynchronize(stream()));
+        COMET_HIPCHK(hipFree(b->sg_blkptr));
+        b->sg_blkptr = nullptr;
+    }
+    COMET_HIPCHK(hipMalloc((void **)&b->sg_blkptr,
+                           sizeof(int32_t) * (size_t)(nblk + 1) * (size_t)(b->nrows > 0 ? b->nrows : 1)));
+    b->sg_nblk = nblk;
+    if (b->nrows > 0) {
+        KernelTimer t("spgemm_block_pointers");
+        spgemm_block_pointers<<<dim3((unsigned)ceil_div(b->nrows, 256)), dim3(256), 0, stream()>>>(
+            b->nrows, b->pos, b->crd, nblk, b->sg_blkptr);
+    }
+    COMET_HIPCHK(hipGetLastError());
+    return COMET_HIP_OK;
+}
+
+static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos, int64_t rb, int64_t re,
                         int32_t *Ccrd, double *Cval)
 {
     SgGeom g;
     COMET_CHK(sg_geometry(b->ncols, &g));
     COMET_CHK(sg_reset_ticket());
+    // rows with many products go to the LDS-accumulator kernel (unmasked products only)
+    const int nblk = (int)ceil_div(b->ncols > 0 ? b->ncols : 1, SG_CB);
+    const bool dense = !m && nblk <= SG_DENSE_MAX_BLOCKS;
+    const int64_t dense_threshold = SG_DENSE_PER_BLOCK * nblk;
+    int64_t *rowprod = nullptr;
+    if (dense) {
+        COMET_CHK(sg_plan_blocks(b));
+        COMET_CHK(g_sg.rowprod.ensure(sizeof(int64_t) * (size_t)(re - rb), false));
+        rowprod = (int64_t *)g_sg.rowprod.ptr;
+        KernelTimer t("spgemm_row_products");
+        spgemm_row_products<<<dim3((unsigned)ceil_div(re - rb, 4)), dim3(256), 0, stream()>>>(rb, re, a->pos, a->crd,
+                                                                                              b->pos, rowprod);
+        COMET_HIPCHK(hipGetLastError());
+    }
     uint32_t *gbm = nullptr, *gmask = nullptr;
     if (!g.lds) {
         COMET_CHK(g_sg.gbm.ensure(sizeof(uint32_t) * g.bm_words * (size_t)g.groups, true));
@@ -528,8 +769,8 @@ static int numeric_rows(const Csr *a, const Csr *b, const Csr *m, const int64_t 
         KernelTimer t(M ? "spgemm_numeric_masked" : "spgemm_numeric");                                     \
         spgemm_numeric_kernel<L, M><<<grid, block, g.lds_bytes, stream()>>>(                               \
             rb, re, b->ncols, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m ? m->pos : nullptr,        \
-            m ? m->crd : nullptr, g.logW, gbm, gmask, (double *)g_sg.slabs.ptr, (unsigned long long *)g_sg.ticket.ptr, Cpos,   \
-            Ccrd, Cval); \
+            m ? m->crd : nullptr, g.logW, gbm, gmask, (double *)g_sg.slabs.ptr,                            \
+            (unsigned long long *)g_sg.ticket.ptr, rowprod, dense_threshold, Cpos, Ccrd, Cval);            \
     } while (0)
     if (g.lds) {
         if (m) LAUNCH_NUM(true, true); else LAUNCH_NUM(true, false);
@@ -538,6 +779,16 @@ static int numeric_rows(const Csr *a, const Csr *b, const Csr *m, const int64_t 
     }
 #undef LAUNCH_NUM
     COMET_HIPCHK(hipGetLastError());
+    if (dense) {
+        COMET_CHK(sg_reset_ticket());
+        COMET_CHK(sg_allow_lds(spgemm_numeric_dense_kernel, SG_DENSE_LDS));
+        KernelTimer t("spgemm_numeric_dense");
+        spgemm_numeric_dense_kernel<<<dim3((unsigned)(num_cus() > 0 ? num_cus() : 256)), block, SG_DENSE_LDS,
+                                      stream()>>>(rb, re, b->nrows, a->pos, a->crd, a->val, b->pos, b->crd, b->val,
+                                                  b->sg_blkptr, nblk, (unsigned long long *)g_sg.ticket.ptr, rowprod,
+                                                  dense_threshold, Cpos, Ccrd, Cval);
+        COMET_HIPCHK(hipGetLastError());
+    }
     return COMET_HIP_OK;
 }
 

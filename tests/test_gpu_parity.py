@@ -112,6 +112,20 @@ def test_spmv_poisson_shape_scaled_down():
     assert np.array_equal(got, orc.spmv(pos, crd, val, x))
 
 
+def test_spmv_column_blocked_plan_is_bit_exact():
+    # x larger than an L2: the library re-stores A in column blocks and runs one pass per block;
+    # the additions must still happen in the checker's order
+    n = 600_000
+    pos, crd, val = gen.poisson_csr(n=n, mean=4.0, seed=5)
+    assert len(crd) > (1 << 20)
+    x, y0 = gen.dense(n, seed=15), gen.dense(n, seed=16)
+    A = rt.CsrMatrix.from_arrays((n, n), pos, crd, val)
+    dx = rt.DeviceArray.from_numpy(x)
+    assert np.array_equal(rt.spmv(A, dx).to_numpy(), orc.spmv(pos, crd, val, x))
+    assert np.array_equal(rt.spmv(A, dx, rt.DeviceArray.from_numpy(y0)).to_numpy(), orc.spmv(pos, crd, val, x, y0))
+    assert np.array_equal(rt.spmv(A, dx).to_numpy(), orc.spmv(pos, crd, val, x))      # plan reused
+
+
 def test_spmv_edge_cases():
     # empty matrix rows, one very long row (longer than an LDS pass), trailing empty rows
     n, m = 600, 9000
