@@ -24,6 +24,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP64_MFMA_PEAK_TFLOPS = 78.6  # MI355X dense fp64 matrix, published
+# HBM bytes per launch of spmm_csr_nnzsplit on the default workload, from rocprofv3 --pmc FETCH_SIZE (x 2.000) and
+# WRITE_SIZE (x 1.000), factors from a 1 GiB copy kernel; see profiles/spmm_csr_nnzsplit__spmm_zipf_500k_k64.txt
+SPMM_TRAFFIC_BYTES = int((2_017_117 * 2.000 + 264_614 * 1.000) * 1024)
 
 
 _T0 = time.perf_counter()
@@ -129,7 +132,8 @@ def bench_spmm(rt, orc, gen, args):
                    "max_row": int(lens.max()), "rows_len1_frac": float((lens == 1).mean()), "seed": 2,
                    "index_bytes": ib, "accumulate": False},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": alg_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "unit": "GB/s", "frac": alg_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": SPMM_TRAFFIC_BYTES if (n, K) == (500_000, 64) else None,
                      "kernel": dom, "kernel_avg_ms": dom_ms, "algorithmic_bytes": int(alg_bytes),
                      "gather_inclusive_bytes": int(nnz * 8 * K + nnz * (8 + ib) + 8 * n * K)},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
@@ -154,7 +158,9 @@ def bench_spmv(rt, orc, gen, args):
     alg_bytes = nnz * (8 + ib) + (n + 1) * ib + 8 * n + 8 * n
     dom = "spmv_csr_stream"     # one launch per column block of the plan: a step is all of them
     passes = kt[dom]["launches"] // args.steps
-    dom_ms = kt[dom]["avg_ms"] * passes
+    # the passes are ~20 us each, short enough for an event pair per launch to add 25 % of its own; the step
+    # holds nothing but these passes, so the event pair around the timed steps is the kernel time
+    dom_ms = dev_ms
     cpu = None
     if not args.no_cpu:
         y = np.zeros(n)
@@ -168,7 +174,8 @@ def bench_spmv(rt, orc, gen, args):
                    "column_block_passes": passes},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": alg_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": dom, "kernel_avg_ms": dom_ms, "algorithmic_bytes": int(alg_bytes)},
+                     "kernel": dom, "kernel_avg_ms": dom_ms, "launches_per_step": passes,
+                     "algorithmic_bytes": int(alg_bytes)},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
     }
 
@@ -325,7 +332,8 @@ def bench_spgemm(rt, orc, gen, args):
     ib = 4
     alg_bytes = nnzA * (8 + ib) + (n + 1) * ib + nnzC * (8 + ib) + 8 * (n + 1)
     sym_ms = kt["spgemm_symbolic"]["avg_ms"] * kt["spgemm_symbolic"]["launches"] / args.steps
-    num_ms = kt["spgemm_numeric"]["avg_ms"] * kt["spgemm_numeric"]["launches"] / args.steps
+    num_ms = sum(kt[k]["avg_ms"] * kt[k]["launches"] for k in
+                 ("spgemm_numeric", "spgemm_numeric_dense", "spgemm_row_products") if k in kt) / args.steps
     # sum of all values is a size-independent invariant: sum(C) = sum_k colsum(A)[k] * rowsum(A)[k]
     rowsum = np.add.reduceat(val, pos[:-1][np.diff(pos) > 0])
     rs = np.zeros(n)
@@ -376,7 +384,8 @@ def bench_spgemm(rt, orc, gen, args):
                    "seed": 20},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / ((sym_ms + num_ms) * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": alg_bytes / ((sym_ms + num_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": None, "kernel": "spgemm_symbolic + spgemm_numeric", "kernel_avg_ms": sym_ms + num_ms,
+                     "traffic": None, "kernel": "spgemm_symbolic + spgemm_numeric + spgemm_numeric_dense",
+                     "kernel_avg_ms": sym_ms + num_ms,
                      "symbolic_ms": sym_ms, "numeric_ms": num_ms, "algorithmic_bytes": int(alg_bytes)},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity,
     }

@@ -59,10 +59,10 @@ struct Csr {
     int32_t *spmv_bcrd = nullptr;
     double *spmv_bval = nullptr;
     std::vector<int64_t> spmv_base;          // first entry of each block in spmv_bcrd / spmv_bval
-    // SpGEMM plan for the right-hand operand: sg_blkptr[cb * nrows + k] = number of entries of row k whose
-    // column is below cb * 2^14, for cb = 0..sg_nblk, so that the slice of a row inside one block of 16384
-    // columns is found without searching.
-    int32_t *sg_blkptr = nullptr;
+    // SpGEMM plan for the right-hand operand: sg_blkptr[k * (sg_nblk + 1) + cb] = position of the first entry
+    // of row k whose column is >= cb * 2^14, so that the slice of a row inside one block of 16384 columns is
+    // found without searching.
+    int64_t *sg_blkptr = nullptr;
     int sg_nblk = 0;
 };
 

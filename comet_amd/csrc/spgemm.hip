@@ -352,16 +352,18 @@ __global__ __launch_bounds__(256) void spgemm_row_products(int64_t row_begin, in
         products[i - row_begin] = s;
 }
 
-// blkptr[cb * nrows + k] = entries of row k with column < cb * SG_CB
+// blkptr[k * (nblk + 1) + cb] = position in crd/val of the first entry of row k whose column is >= cb * SG_CB
+// (cb = nblk gives the end of the row): the slice of row k inside block cb is one 16-byte load away.
 __global__ void spgemm_block_pointers(int64_t nrows, const int64_t *__restrict__ pos,
-                                      const int32_t *__restrict__ crd, int nblk, int32_t *__restrict__ blkptr)
+                                      const int32_t *__restrict__ crd, int nblk, int64_t *__restrict__ blkptr)
 {
     const int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (k >= nrows)
         return;
     const int64_t s = pos[k], e = pos[k + 1];
+    int64_t *out = blkptr + k * (nblk + 1);
     int64_t lo = s;
-    blkptr[k] = 0;
+    out[0] = s;
     for (int cb = 1; cb <= nblk; ++cb) {
         const int64_t bound = (int64_t)cb << SG_CB_LOG;
         int64_t hi = e;
@@ -372,19 +374,20 @@ __global__ void spgemm_block_pointers(int64_t nrows, const int64_t *__restrict__
             else
                 hi = mid;
         }
-        blkptr[(int64_t)cb * nrows + k] = (int32_t)(lo - s);
+        out[cb] = lo;
     }
 }
 
 __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
-    int64_t row_begin, int64_t row_end, int64_t nrowsB, const int64_t *__restrict__ Apos,
-    const int32_t *__restrict__ Acrd, const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
-    const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval, const int32_t *__restrict__ blkptr, int nblk,
+    int64_t row_begin, int64_t row_end, const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd,
+    const double *__restrict__ Aval, const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval,
+    const int64_t *__restrict__ blkptr, int nblk,
     unsigned long long *ticket, const int64_t *__restrict__ rowprod, int64_t dense_threshold,
     const int64_t *__restrict__ Cpos, int32_t *__restrict__ Ccrd, double *__restrict__ Cval)
 {
     __shared__ int64_t row_slot;
     __shared__ int wave_tot[SG_WAVES];
+    __shared__ int block_touched;
     double *acc = reinterpret_cast<double *>(sg_dyn_lds);
     uint32_t *bm = sg_dyn_lds + SG_CB * 2;
     const int lane = threadIdx.x & 63;
@@ -393,6 +396,8 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
         acc[j] = 0.0;
     if (threadIdx.x < SG_CB / 32)
         bm[threadIdx.x] = 0;
+    if (threadIdx.x == 0)
+        block_touched = 0;
     __syncthreads();
     const int64_t out0 = Cpos[row_begin];
     int64_t i = draw_row(ticket, row_begin, &row_slot);
@@ -401,8 +406,8 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
         if (as != ae && rowprod[i - row_begin] >= dense_threshold) {
             int64_t off = Cpos[i] - out0;
             for (int cb = 0; cb < nblk; ++cb) {
-                const int32_t *bp0 = blkptr + (int64_t)cb * nrowsB, *bp1 = bp0 + nrowsB;
                 const int col0 = cb << SG_CB_LOG;
+                int touched = 0;     // did this wavefront add anything to the block
                 for (int64_t base = as + wave; base < ae; base += (int64_t)SG_WAVES * 64) {
                     const int64_t left = (ae - base + SG_WAVES - 1) / SG_WAVES;
                     const int cnt = (int)(left < 64 ? left : 64);
@@ -410,16 +415,16 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                     double a = 0.0;
                     if (lane < cnt) {
                         const int64_t p = base + (int64_t)lane * SG_WAVES;
-                        const int k = Acrd[p];
-                        const int64_t b0 = Bpos[k];
-                        lo = b0 + bp0[k];
-                        hi = b0 + bp1[k];
+                        const int64_t *bp = blkptr + (int64_t)Acrd[p] * (nblk + 1) + cb;
+                        lo = bp[0];
+                        hi = bp[1];
                         a = Aval[p];
                     }
                     // long slices take the whole wavefront, one at a time; short ones (a slice of one block
                     // often holds a dozen entries) are handed to the four 16-lane quarters, four at a time
                     unsigned long long big = __ballot(hi - lo >= 32);
                     unsigned long long todo = __ballot(lo < hi && hi - lo < 32);
+                    touched |= (big | todo) != 0;
                     while (big) {
                         const int t = __builtin_ctzll(big);
                         big &= big - 1;
@@ -472,7 +477,14 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                         }
                     }
                 }
+                // one barrier tells everybody whether the block received anything (an LDS flag that the
+                // emitting path resets); the value is made scalar so that the branch on it is uniform,
+                // because the block body below holds barriers
+                if (touched && lane == 0)
+                    block_touched = 1;
                 __syncthreads();
+                const int any = __builtin_amdgcn_readfirstlane(block_touched);
+                if (any) {
                 // emit this block: lane t < 512 owns bitmap word t, i.e. 32 consecutive columns
                 uint32_t word = threadIdx.x < SG_CB / 32 ? bm[threadIdx.x] : 0u;
                 const int mine = __popc(word);
@@ -503,8 +515,11 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                 }
                 if (threadIdx.x < SG_CB / 32)
                     bm[threadIdx.x] = 0;
+                if (threadIdx.x == 0)
+                    block_touched = 0;
                 off += total;
                 __syncthreads();
+                }   // block received products
             }
         }
         i = draw_row(ticket, row_begin, &row_slot);
@@ -721,7 +736,7 @@ static int sg_plan_blocks(Csr *b)
         b->sg_blkptr = nullptr;
     }
     COMET_HIPCHK(hipMalloc((void **)&b->sg_blkptr,
-                           sizeof(int32_t) * (size_t)(nblk + 1) * (size_t)(b->nrows > 0 ? b->nrows : 1)));
+                           sizeof(int64_t) * (size_t)(nblk + 1) * (size_t)(b->nrows > 0 ? b->nrows : 1)));
     b->sg_nblk = nblk;
     if (b->nrows > 0) {
         KernelTimer t("spgemm_block_pointers");
@@ -784,8 +799,7 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
         COMET_CHK(sg_allow_lds(spgemm_numeric_dense_kernel, SG_DENSE_LDS));
         KernelTimer t("spgemm_numeric_dense");
         spgemm_numeric_dense_kernel<<<dim3((unsigned)(num_cus() > 0 ? num_cus() : 256)), block, SG_DENSE_LDS,
-                                      stream()>>>(rb, re, b->nrows, a->pos, a->crd, a->val, b->pos, b->crd, b->val,
-                                                  b->sg_blkptr, nblk, (unsigned long long *)g_sg.ticket.ptr, rowprod,
+                                      stream()>>>(rb, re, a->pos, a->crd, a->val, b->crd, b->val, b->sg_blkptr, nblk, (unsigned long long *)g_sg.ticket.ptr, rowprod,
                                                   dense_threshold, Cpos, Ccrd, Cval);
         COMET_HIPCHK(hipGetLastError());
     }
