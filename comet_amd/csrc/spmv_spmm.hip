@@ -318,8 +318,9 @@ __global__ __launch_bounds__(SPMM_WAVES * 64) void spmm_csr_nnzsplit(
                     acc = acc + prod;
                     open = true;
                     const int64_t p = base + t0 + u + 1;
+                    bool holds = true;           // the first turn closes a row that holds nonzeros
                     while (p == rend) {          // row r is complete; also walks over empty rows that follow
-                        if (active) {
+                        if (active && (holds || !ACC)) {     // accumulating leaves empty rows untouched
                             if (first_piece && head)
                                 carry0[lane] = acc;
                             else     // C is written once and not read again by this kernel
@@ -327,13 +328,14 @@ __global__ __launch_bounds__(SPMM_WAVES * 64) void spmm_csr_nnzsplit(
                         }
                         first_piece = false;
                         open = false;
+                        holds = false;
                         ++r;
                         if (r >= nrows)
                             break;
                         rend = pos[r + 1];
                         acc = 0.0;
                         // a row that starts here and ends later keeps its C value for the fix-up instead
-                        if (ACC && active && rend <= e)
+                        if (ACC && active && rend > p && rend <= e)
                             acc = C[r * ldc + col];
                     }
                 }
