@@ -57,9 +57,9 @@ struct BmAddr {
     __device__ inline uint32_t bit(int j) const { return 1u << (j & 31); }
 };
 
-// Visit every product of output row i: f(j, q, a) for k in A_i, q over the
-// entries of B_k, j = Bcrd[q], a = A's value (the visitor loads Bval[q] itself,
-// and only if it needs it).  The entries of A_i are dealt to the 16 wavefronts
+// Visit every product of output row i: f(j, q, a, p, s) for k = Acrd[p] in A_i,
+// q over the entries [s, e) of B_k, j = Bcrd[q], a = A's value (the visitor
+// loads Bval[q] itself, and only if it needs it).  The entries of A_i are dealt to the 16 wavefronts
 // one at a time (entry p goes to wavefront p mod 16), because in a sorted row
 // the neighbours with long rows sit next to each other and would otherwise all
 // land on one wavefront.  A wavefront fetches 64 of its entries at once (one per
@@ -88,16 +88,17 @@ __device__ inline void for_each_product(int64_t as, int64_t ae, const int32_t *_
         for (int t = 0; t < cnt; ++t) {
             const int64_t s = readlane_i64(bs, t), e = readlane_i64(be, t);
             const double at = VALUES ? readlane_d(a, t) : 0.0;
+            const int64_t p = base + (int64_t)t * SG_WAVES;
             int64_t q = s + lane;
             for (; q + 192 < e; q += 256) {
                 const int j0 = Bcrd[q], j1 = Bcrd[q + 64], j2 = Bcrd[q + 128], j3 = Bcrd[q + 192];
-                f(j0, q, at);
-                f(j1, q + 64, at);
-                f(j2, q + 128, at);
-                f(j3, q + 192, at);
+                f(j0, q, at, p, s);
+                f(j1, q + 64, at, p, s);
+                f(j2, q + 128, at, p, s);
+                f(j3, q + 192, at, p, s);
             }
             for (; q < e; q += 64)
-                f(Bcrd[q], q, at);
+                f(Bcrd[q], q, at, p, s);
         }
     }
 }
@@ -136,6 +137,36 @@ __device__ inline int64_t draw_row(unsigned long long *ticket, int64_t first, in
     const int lo = __builtin_amdgcn_readfirstlane((int)(r & 0xffffffff));
     const int hi = __builtin_amdgcn_readfirstlane((int)(r >> 32));
     return ((int64_t)hi << 32) | (uint32_t)lo;
+}
+
+// Semiring operators of C = A @(reduce, mult) B.  The codes are the C ABI's.
+enum { SR_PLUS = 0, SR_MIN = 1, SR_MAX = 2, SR_ANY = 3 };
+__device__ inline double semiring_mult(int op, double a, double b)
+{
+    switch (op) {
+    case 0: return a * b;
+    case 1: return a;
+    case 2: return b;
+    case 3: return 1.0;
+    case 4: return a + b;
+    case 5: return a - b;
+    case 6: return a < b ? a : b;
+    case 7: return a > b ? a : b;
+    default: return a / b;
+    }
+}
+// Order-preserving map of a double onto an unsigned integer and back: min and
+// max become integer atomics whose result does not depend on the order of the
+// products, and an all-zero slot can stand for "nothing stored yet".
+__device__ inline unsigned long long f64_key(double x)
+{
+    const unsigned long long u = (unsigned long long)__double_as_longlong(x);
+    return (u >> 63) ? ~u : (u | 0x8000000000000000ull);
+}
+__device__ inline double key_f64(unsigned long long k)
+{
+    const unsigned long long u = (k >> 63) ? (k & 0x7fffffffffffffffull) : ~k;
+    return __longlong_as_double((long long)u);
 }
 extern __shared__ uint32_t sg_dyn_lds[];
 
@@ -183,7 +214,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_symbolic_kernel(
             __syncthreads();
         }
         int count = 0;
-        for_each_product<false>(as, ae, Acrd, nullptr, Bpos, Bcrd, [&](int j, int64_t, double) {
+        for_each_product<false>(as, ae, Acrd, nullptr, Bpos, Bcrd, [&](int j, int64_t, double, int64_t, int64_t) {
             const uint32_t b = ad.bit(j);
             if constexpr (MASKED) {
                 const uint32_t old = atomicAnd(&bm[ad.word(j)], ~b);
@@ -212,7 +243,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_symbolic_kernel(
                 bm[w] = 0;
         } else {
             for_each_product<false>(as, ae, Acrd, nullptr, Bpos, Bcrd,
-                                    [&](int j, int64_t, double) { atomicAnd(&bm[ad.word(j)], 0u); });
+                                    [&](int j, int64_t, double, int64_t, int64_t) { atomicAnd(&bm[ad.word(j)], 0u); });
         }
         }   // work
         i = draw_row(ticket, 0, &row_slot);     // its barriers also close this row's bitmap clean-up
@@ -222,15 +253,22 @@ __global__ __launch_bounds__(SG_T) void spgemm_symbolic_kernel(
 // ---------------------------------------------------------------------------
 // Numeric phase for rows [row_begin,row_end).
 // ---------------------------------------------------------------------------
-template <bool BM_LDS, bool MASKED>
+// SEMI: any reduction/multiplication pair.  plus adds with the same fp64 atomic;
+// min, max and any keep an integer key in the slab instead of a double and
+// combine with an atomic max, so their results are independent of the order in
+// which the products arrive: min stores the complement of the value's key, max
+// the key itself (and, like the reference, never returns less than 0), any the
+// position (p, q) of the product and so keeps the one a sequential traversal
+// would reach last.  A slot is back to all-zero after extraction in every case.
+template <bool BM_LDS, bool MASKED, bool SEMI>
 __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
     int64_t row_begin, int64_t row_end, int64_t ncols, const int64_t *__restrict__ Apos,
     const int32_t *__restrict__ Acrd, const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
     const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval, const int64_t *__restrict__ Mpos,
     const int32_t *__restrict__ Mcrd, int logW, uint32_t *__restrict__ gbm, uint32_t *__restrict__ gmask,
     double *__restrict__ slabs, unsigned long long *ticket, const int64_t *__restrict__ rowprod,
-    int64_t dense_threshold, const int64_t *__restrict__ Cpos, int32_t *__restrict__ Ccrd,
-    double *__restrict__ Cval)
+    int64_t dense_threshold, int reduce_op, int mult_op, const int64_t *__restrict__ Cpos,
+    int32_t *__restrict__ Ccrd, double *__restrict__ Cval)
 {
     __shared__ int64_t row_slot;
     __shared__ int wave_tot[SG_WAVES];
@@ -263,7 +301,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
                 atomicOr(&mbm[ad.word(Mcrd[t])], ad.bit(Mcrd[t]));
             __syncthreads();
         }
-        for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, [&](int j, int64_t q, double a) {
+        for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, [&](int j, int64_t q, double a, int64_t p, int64_t bs) {
             const int w = ad.word(j);
             const uint32_t b = ad.bit(j);
             if constexpr (MASKED) {
@@ -271,7 +309,22 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
                     return;
             }
             atomicOr(&bm[w], b);
-            __hip_atomic_fetch_add(&slab[j], a * Bval[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if constexpr (SEMI) {
+                unsigned long long *slot = (unsigned long long *)&slab[j];
+                if (reduce_op == SR_ANY) {
+                    const unsigned long long key = ((unsigned long long)(p - as + 1) << 32) | (unsigned long long)(q - bs);
+                    __hip_atomic_fetch_max(slot, key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                } else {
+                    const double e = semiring_mult(mult_op, a, Bval[q]);
+                    if (reduce_op == SR_PLUS)
+                        __hip_atomic_fetch_add(&slab[j], e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    else
+                        __hip_atomic_fetch_max(slot, reduce_op == SR_MIN ? ~f64_key(e) : f64_key(e),
+                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+            } else {
+                __hip_atomic_fetch_add(&slab[j], a * Bval[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
         });
         __syncthreads();
         // extraction: my words hold my columns in ascending order
@@ -304,7 +357,23 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
                 word &= word - 1;
                 const int j = jbase + b;
                 Ccrd[off] = j;
-                Cval[off] = __hip_atomic_exchange(&slab[j], 0.0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                if (SEMI && reduce_op != SR_PLUS) {
+                    const unsigned long long v = __hip_atomic_exchange((unsigned long long *)&slab[j], 0ull,
+                                                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    double out;
+                    if (reduce_op == SR_MIN) {
+                        out = key_f64(~v);
+                    } else if (reduce_op == SR_MAX) {
+                        out = v < f64_key(0.0) ? 0.0 : key_f64(v);
+                    } else {
+                        const int64_t pp = as + (int64_t)(v >> 32) - 1;
+                        const int64_t qq = Bpos[Acrd[pp]] + (int64_t)(v & 0xffffffffull);
+                        out = semiring_mult(mult_op, Aval[pp], Bval[qq]);
+                    }
+                    Cval[off] = out;
+                } else {
+                    Cval[off] = __hip_atomic_exchange(&slab[j], 0.0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
                 ++off;
             }
         }
@@ -564,7 +633,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_masked_sum_kernel(
             atomicOr(&bm[ad.word(Mcrd[t])], ad.bit(Mcrd[t]));
         __syncthreads();
         double part = 0.0;
-        for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, [&](int j, int64_t q, double a) {
+        for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, [&](int j, int64_t q, double a, int64_t, int64_t) {
             uint32_t word;
             if constexpr (BM_LDS)
                 word = bm[ad.word(j)];
@@ -748,14 +817,17 @@ static int sg_plan_blocks(Csr *b)
 }
 
 static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos, int64_t rb, int64_t re,
-                        int32_t *Ccrd, double *Cval)
+                        int32_t *Ccrd, double *Cval, int reduce_op, int mult_op)
 {
+    if (reduce_op < 0 || reduce_op > COMET_SR_ANY || mult_op < 0 || mult_op > COMET_OP_DIV)
+        return set_error(COMET_HIP_ERR_ARG, "unknown semiring (reduce %d, mult %d)", reduce_op, mult_op);
+    const bool semi = reduce_op != COMET_SR_PLUS || mult_op != COMET_OP_TIMES;
     SgGeom g;
     COMET_CHK(sg_geometry(b->ncols, &g));
     COMET_CHK(sg_reset_ticket());
     // rows with many products go to the LDS-accumulator kernel (unmasked products only)
     const int nblk = (int)ceil_div(b->ncols > 0 ? b->ncols : 1, SG_CB);
-    const bool dense = !m && nblk <= SG_DENSE_MAX_BLOCKS;
+    const bool dense = !m && !semi && nblk <= SG_DENSE_MAX_BLOCKS;
     const int64_t dense_threshold = SG_DENSE_PER_BLOCK * nblk;
     int64_t *rowprod = nullptr;
     if (dense) {
@@ -778,20 +850,26 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
     }
     COMET_CHK(g_sg.slabs.ensure(sizeof(double) * (size_t)(b->ncols > 0 ? b->ncols : 1) * (size_t)g.groups, true));
     const dim3 grid((unsigned)g.groups), block(SG_T);
-#define LAUNCH_NUM(L, M)                                                                                   \
+#define LAUNCH_NUM(L, M, S)                                                                                \
     do {                                                                                                   \
-        COMET_CHK(sg_allow_lds(spgemm_numeric_kernel<L, M>, g.lds_bytes));                                 \
-        KernelTimer t(M ? "spgemm_numeric_masked" : "spgemm_numeric");                                     \
-        spgemm_numeric_kernel<L, M><<<grid, block, g.lds_bytes, stream()>>>(                               \
+        COMET_CHK(sg_allow_lds(spgemm_numeric_kernel<L, M, S>, g.lds_bytes));                              \
+        KernelTimer t(S ? "spgemm_numeric_semiring" : M ? "spgemm_numeric_masked" : "spgemm_numeric");    \
+        spgemm_numeric_kernel<L, M, S><<<grid, block, g.lds_bytes, stream()>>>(                            \
             rb, re, b->ncols, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m ? m->pos : nullptr,        \
             m ? m->crd : nullptr, g.logW, gbm, gmask, (double *)g_sg.slabs.ptr,                            \
-            (unsigned long long *)g_sg.ticket.ptr, rowprod, dense_threshold, Cpos, Ccrd, Cval);            \
+            (unsigned long long *)g_sg.ticket.ptr, rowprod, dense_threshold, reduce_op, mult_op, Cpos,     \
+            Ccrd, Cval);                                                                                   \
+    } while (0)
+#define LAUNCH_NUM_S(L, M)                                                                                 \
+    do {                                                                                                   \
+        if (semi) LAUNCH_NUM(L, M, true); else LAUNCH_NUM(L, M, false);                                    \
     } while (0)
     if (g.lds) {
-        if (m) LAUNCH_NUM(true, true); else LAUNCH_NUM(true, false);
+        if (m) LAUNCH_NUM_S(true, true); else LAUNCH_NUM_S(true, false);
     } else {
-        if (m) LAUNCH_NUM(false, true); else LAUNCH_NUM(false, false);
+        if (m) LAUNCH_NUM_S(false, true); else LAUNCH_NUM_S(false, false);
     }
+#undef LAUNCH_NUM_S
 #undef LAUNCH_NUM
     COMET_HIPCHK(hipGetLastError());
     if (dense) {
@@ -835,6 +913,14 @@ extern "C" int comet_hip_spgemm_csr_symbolic(int64_t ah, int64_t bh, int64_t mh,
 extern "C" int comet_hip_spgemm_csr_numeric(int64_t ah, int64_t bh, int64_t mh, int64_t pos_dptr, int64_t row_begin,
                                             int64_t row_end, int64_t crd_dptr, int64_t val_dptr)
 {
+    return comet_hip_spgemm_csr_numeric_semiring(ah, bh, mh, pos_dptr, row_begin, row_end, crd_dptr, val_dptr,
+                                                 COMET_SR_PLUS, COMET_OP_TIMES);
+}
+
+extern "C" int comet_hip_spgemm_csr_numeric_semiring(int64_t ah, int64_t bh, int64_t mh, int64_t pos_dptr,
+                                                     int64_t row_begin, int64_t row_end, int64_t crd_dptr,
+                                                     int64_t val_dptr, int reduce_op, int mult_op)
+{
     COMET_CHK(ensure_init());
     Csr *a = csr_from_handle(ah), *b = csr_from_handle(bh), *m = mh ? csr_from_handle(mh) : nullptr;
     if (!a || !b || (mh && !m))
@@ -848,10 +934,15 @@ extern "C" int comet_hip_spgemm_csr_numeric(int64_t ah, int64_t bh, int64_t mh, 
     if (row_begin == row_end)
         return COMET_HIP_OK;
     return numeric_rows(a, b, m, (const int64_t *)pos_dptr, row_begin, row_end, (int32_t *)crd_dptr,
-                        (double *)val_dptr);
+                        (double *)val_dptr, reduce_op, mult_op);
 }
 
 extern "C" int64_t comet_hip_spgemm_csr(int64_t ah, int64_t bh, int64_t mh)
+{
+    return comet_hip_spgemm_csr_semiring(ah, bh, mh, COMET_SR_PLUS, COMET_OP_TIMES);
+}
+
+extern "C" int64_t comet_hip_spgemm_csr_semiring(int64_t ah, int64_t bh, int64_t mh, int reduce_op, int mult_op)
 {
     if (ensure_init() != COMET_HIP_OK)
         return 0;
@@ -884,7 +975,7 @@ extern "C" int64_t comet_hip_spgemm_csr(int64_t ah, int64_t bh, int64_t mh)
         delete c;
         return 0;
     }
-    if (nnz > 0 && numeric_rows(a, b, m, pos, 0, a->nrows, c->crd, c->val) != COMET_HIP_OK) {
+    if (nnz > 0 && numeric_rows(a, b, m, pos, 0, a->nrows, c->crd, c->val, reduce_op, mult_op) != COMET_HIP_OK) {
         (void)hipFree(c->crd);
         (void)hipFree(c->val);
         (void)hipFree(pos);

@@ -78,6 +78,8 @@ SIGNATURES = {
     "comet_hip_spgemm_csr_symbolic": (_int, [_i64, _i64, _i64, _i64, _pi64]),
     "comet_hip_spgemm_csr_numeric": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64]),
     "comet_hip_spgemm_csr": (_i64, [_i64, _i64, _i64]),
+    "comet_hip_spgemm_csr_numeric_semiring": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int]),
+    "comet_hip_spgemm_csr_semiring": (_i64, [_i64, _i64, _i64, _int, _int]),
     "comet_hip_spgemm_masked_sum": (_int, [_i64, _i64, _i64, C.POINTER(_f64)]),
     "comet_hip_reduce_sum_f64": (_int, [_i64, _i64, C.POINTER(_f64)]),
     "comet_hip_eltwise_mult_csr": (_i64, [_i64, _i64]),
@@ -301,9 +303,26 @@ def spmm(A, B, Cm=None, accumulate=None):
     return Cm
 
 
-def spgemm(A, B, mask=None):
-    h = lib().comet_hip_spgemm_csr(A.handle, B.handle, mask.handle if mask is not None else 0)
-    return CsrMatrix(_handle(h, "comet_hip_spgemm_csr"))
+# operator codes of the C ABI (COMET_SR_* / COMET_OP_*), by the names the .ta language uses
+REDUCE_OPS = {"plus": 0, "+": 0, "min": 1, "max": 2, "any": 3}
+MULT_OPS = {"times": 0, "*": 0, "first": 1, "second": 2, "pair": 3, "plus": 4, "+": 4, "minus": 5, "-": 5,
+            "min": 6, "max": 7, "div": 8, "/": 8}
+
+
+def _semiring_codes(semiring):
+    if semiring is None:
+        return 0, 0
+    reduce_op, mult_op = semiring
+    if reduce_op not in REDUCE_OPS or mult_op not in MULT_OPS:
+        raise ValueError(f"unknown semiring {semiring!r}")
+    return REDUCE_OPS[reduce_op], MULT_OPS[mult_op]
+
+
+def spgemm(A, B, mask=None, semiring=None):
+    """C = A @(reduce, mult) B as a new CsrMatrix; semiring=None is (plus, times)."""
+    r, m = _semiring_codes(semiring)
+    h = lib().comet_hip_spgemm_csr_semiring(A.handle, B.handle, mask.handle if mask is not None else 0, r, m)
+    return CsrMatrix(_handle(h, "comet_hip_spgemm_csr_semiring"))
 
 
 def spgemm_symbolic(A, B, mask=None):
@@ -315,9 +334,11 @@ def spgemm_symbolic(A, B, mask=None):
     return pos, nnz.value
 
 
-def spgemm_numeric(A, B, pos, row_begin, row_end, crd, val, mask=None):
-    _check(lib().comet_hip_spgemm_csr_numeric(A.handle, B.handle, mask.handle if mask is not None else 0, pos.ptr,
-                                              row_begin, row_end, crd.ptr, val.ptr), "comet_hip_spgemm_csr_numeric")
+def spgemm_numeric(A, B, pos, row_begin, row_end, crd, val, mask=None, semiring=None):
+    r, m = _semiring_codes(semiring)
+    _check(lib().comet_hip_spgemm_csr_numeric_semiring(A.handle, B.handle, mask.handle if mask is not None else 0,
+                                                       pos.ptr, row_begin, row_end, crd.ptr, val.ptr, r, m),
+           "comet_hip_spgemm_csr_numeric_semiring")
 
 
 def spgemm_masked_sum(A, B, mask):

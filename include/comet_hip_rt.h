@@ -126,6 +126,29 @@ int comet_hip_spgemm_csr_numeric(int64_t a, int64_t b, int64_t mask, int64_t pos
 /* Both phases; returns a new CSR handle that owns its arrays (0 on failure). */
 int64_t comet_hip_spgemm_csr(int64_t a, int64_t b, int64_t mask);
 
+/* ---- SpGEMM over a semiring  C[a,c] = A[a,b] @(reduce, mult) B[b,c] ---------
+ * The semiring forms of test/integration/semiring/mm_Semiring*_CSRxCSR_oCSR.ta
+ * (frontends/comet_dsl/mlir/MLIRGen.cpp:101-147 for the names the DSL emits).
+ * Per product e = mult(A[i,k], B[k,j]); C[i,j] = reduce over the products,
+ * starting from the value the reference's workspace extract returns for an
+ * untouched column: +inf for min, 0 otherwise - so max never returns less
+ * than 0 (lib/Conversion/IndexTreeToSCF/IndexTreeToSCF.cpp:198-360,1190-1219,
+ * 1249-1284).  "any" keeps the product a sequential traversal reaches last
+ * (IndexTreeToSCF.cpp:346-349).  The structure of C does not depend on the
+ * semiring, so the symbolic call above serves every one of them.  min, max
+ * and any are independent of the order of evaluation and reproduce the
+ * reference bit for bit (up to the sign of a zero); plus rounds like
+ * comet_hip_spgemm_csr_numeric.  (COMET_SR_PLUS, COMET_OP_TIMES) is that
+ * routine itself. */
+enum { COMET_SR_PLUS = 0, COMET_SR_MIN = 1, COMET_SR_MAX = 2, COMET_SR_ANY = 3 };
+enum { COMET_OP_TIMES = 0, COMET_OP_FIRST = 1, COMET_OP_SECOND = 2, COMET_OP_PAIR = 3, COMET_OP_PLUS = 4,
+       COMET_OP_MINUS = 5, COMET_OP_MIN = 6, COMET_OP_MAX = 7, COMET_OP_DIV = 8 };
+int comet_hip_spgemm_csr_numeric_semiring(int64_t a, int64_t b, int64_t mask, int64_t pos_dptr,
+                                          int64_t row_begin, int64_t row_end,
+                                          int64_t crd_dptr, int64_t val_dptr,
+                                          int reduce_op, int mult_op);
+int64_t comet_hip_spgemm_csr_semiring(int64_t a, int64_t b, int64_t mask, int reduce_op, int mult_op);
+
 /* ---- masked SpGEMM + SUM in one pass (triangle counting) -------------------
  * *out = SUM(C) for C<L> = L * L, the two statements of
  * test/integration/kernels/triangleCount_SandiaLL_wMasking.ta:18-39, i.e. the

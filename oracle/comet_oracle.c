@@ -224,6 +224,103 @@ idx_t oracle_spgemm_numeric(idx_t row_begin, idx_t row_end, idx_t ncolsB,
 }
 
 /* ------------------------------------------------------------------------- */
+/* SpGEMM numeric phase over a semiring  C = A @(reduce, mult) B.              */
+/* Per product e = mult(a, b); then W[j] = reduce(w, e) where w is W[j] if the  */
+/* column was already touched in this row and the "zero" of the extract         */
+/* otherwise: +inf for min, 0.0 for every other reduction (also for max):       */
+/*   lib/Conversion/IndexTreeToSCF/IndexTreeToSCF.cpp:198-303 (mult ops),       */
+/*     :307-360 (reduce ops; "any" keeps the new value), :1190-1219 (zero),     */
+/*     :1249-1284 (mult over the operands, extract, reduce, insert)             */
+/*   lib/Conversion/TensorAlgebraToSCF/SparseTensorConversionPass.cpp:849-921   */
+/*     (insert: mark + append the column if new, then store), :925-985          */
+/*     (extract: stored value if marked, else the zero attribute)               */
+/*   frontends/comet_dsl/mlir/MLIRGen.cpp:101-147 (names the DSL can produce)   */
+/* reduce: 0 plusxy, 1 minxy, 2 max, 3 any.                                     */
+/* mult:   0 times, 1 first, 2 second, 3 pairxy, 4 plusxy, 5 minus, 6 minxy,    */
+/*         7 max, 8 div.                                                        */
+/* Returns the number of entries written, or -1 for an unknown operator.        */
+/* ------------------------------------------------------------------------- */
+static double semiring_mult(int op, double a, double b)
+{
+    switch (op) {
+    case 0: return a * b;
+    case 1: return a;
+    case 2: return b;
+    case 3: return 1.0;
+    case 4: return a + b;
+    case 5: return a - b;
+    case 6: return a < b ? a : b;      /* CmpFOp OLT + select */
+    case 7: return a > b ? a : b;      /* CmpFOp OGT + select */
+    default: return a / b;
+    }
+}
+
+static double semiring_reduce(int op, double w, double e)
+{
+    switch (op) {
+    case 0: return w + e;
+    case 1: return w < e ? w : e;
+    case 2: return w > e ? w : e;
+    default: return e;
+    }
+}
+
+idx_t oracle_spgemm_numeric_semiring(idx_t row_begin, idx_t row_end, idx_t ncolsB,
+                                     const idx_t *Apos, const idx_t *Acrd, const double *Aval,
+                                     const idx_t *Bpos, const idx_t *Bcrd, const double *Bval,
+                                     const idx_t *mpos, const idx_t *mcrd,
+                                     int reduce_op, int mult_op,
+                                     idx_t *Ccrd, double *Cval)
+{
+    if (reduce_op < 0 || reduce_op > 3 || mult_op < 0 || mult_op > 8)
+        return -1;
+    size_t n = (size_t)(ncolsB > 0 ? ncolsB : 1);
+    double *W = (double *)malloc(n * sizeof(double));
+    unsigned char *seen = (unsigned char *)calloc(n, 1);
+    idx_t *crds = (idx_t *)malloc(n * sizeof(idx_t));
+    unsigned char *bits = mpos ? (unsigned char *)calloc(n, 1) : NULL;
+    const double zero = reduce_op == 1 ? INFINITY : 0.0;
+    idx_t ipos = 0;
+    for (idx_t i = row_begin; i < row_end; ++i) {
+        idx_t num_crds = 0;
+        if (bits)
+            for (idx_t t = mpos[i]; t < mpos[i + 1]; ++t)
+                bits[mcrd[t]] = 1;
+        for (idx_t p = Apos[i]; p < Apos[i + 1]; ++p) {
+            idx_t k = Acrd[p];
+            for (idx_t q = Bpos[k]; q < Bpos[k + 1]; ++q) {
+                idx_t j = Bcrd[q];
+                if (bits && !bits[j])
+                    continue;
+                double e = semiring_mult(mult_op, Aval[p], Bval[q]);
+                double w = seen[j] ? W[j] : zero;
+                if (!seen[j]) {
+                    seen[j] = 1;
+                    crds[num_crds++] = j;
+                }
+                W[j] = semiring_reduce(reduce_op, w, e);
+            }
+        }
+        if (bits)
+            for (idx_t t = mpos[i]; t < mpos[i + 1]; ++t)
+                bits[mcrd[t]] = 0;
+        qsort(crds, (size_t)num_crds, sizeof(idx_t), cmp_idx);
+        for (idx_t t = 0; t < num_crds; ++t) {
+            idx_t j = crds[t];
+            Ccrd[ipos] = j;
+            Cval[ipos] = W[j];
+            seen[j] = 0;
+            ++ipos;
+        }
+    }
+    free(W);
+    free(seen);
+    free(crds);
+    free(bits);
+    return ipos;
+}
+
+/* ------------------------------------------------------------------------- */
 /* SUM over a value array: acc = val[t] + acc, sequential, acc starts at 0.    */
 /* lib/Conversion/TensorAlgebraToSCF/TensorAlgebraToSCF.cpp:417-529            */
 /* ------------------------------------------------------------------------- */

@@ -58,6 +58,9 @@ def lib():
     L.oracle_spgemm_numeric.argtypes = [C.c_int64, C.c_int64, C.c_int64, i64p, i64p, f64p, i64p, i64p, f64p,
                                         vp, vp, i64p, f64p]
     L.oracle_spgemm_numeric.restype = C.c_int64
+    L.oracle_spgemm_numeric_semiring.argtypes = [C.c_int64, C.c_int64, C.c_int64, i64p, i64p, f64p, i64p, i64p, f64p,
+                                                 vp, vp, C.c_int, C.c_int, i64p, f64p]
+    L.oracle_spgemm_numeric_semiring.restype = C.c_int64
     L.oracle_reduce_sum.argtypes = [f64p, C.c_int64]
     L.oracle_reduce_sum.restype = C.c_double
     L.oracle_eltwise_mult_csr.argtypes = [C.c_int64, i64p, i64p, f64p, i64p, i64p, f64p, i64p, i64p, f64p]
@@ -127,8 +130,13 @@ def spgemm_symbolic(Apos, Acrd, Bpos, Bcrd, ncolsB, mask=None, rows=None):
     return cnt[: r1 - r0], int(total)
 
 
-def spgemm(Apos, Acrd, Aval, Bpos, Bcrd, Bval, ncolsB, mask=None, rows=None):
-    """Symbolic + numeric; returns (pos, crd, val) for rows [r0,r1) with pos starting at 0."""
+REDUCE_OPS = {"plus": 0, "min": 1, "max": 2, "any": 3}
+MULT_OPS = {"times": 0, "first": 1, "second": 2, "pair": 3, "plus": 4, "minus": 5, "min": 6, "max": 7, "div": 8}
+
+
+def spgemm(Apos, Acrd, Aval, Bpos, Bcrd, Bval, ncolsB, mask=None, rows=None, semiring=None):
+    """Symbolic + numeric; returns (pos, crd, val) for rows [r0,r1) with pos starting at 0.
+    semiring = (reduce, mult) names from REDUCE_OPS / MULT_OPS; None is the plain plus-times routine."""
     Apos, Acrd, Aval = _i64(Apos), _i64(Acrd), _f64(Aval)
     Bpos, Bcrd, Bval = _i64(Bpos), _i64(Bcrd), _f64(Bval)
     r0, r1 = (0, len(Apos) - 1) if rows is None else rows
@@ -140,8 +148,13 @@ def spgemm(Apos, Acrd, Aval, Bpos, Bcrd, Bval, ncolsB, mask=None, rows=None):
     mpos = mcrd = None
     if mask is not None:
         mpos, mcrd = _i64(mask[0]), _i64(mask[1])
-    wrote = lib().oracle_spgemm_numeric(r0, r1, ncolsB, Apos, Acrd, Aval, Bpos, Bcrd, Bval,
-                                        _ptr(mpos), _ptr(mcrd), crd, val)
+    if semiring is None:
+        wrote = lib().oracle_spgemm_numeric(r0, r1, ncolsB, Apos, Acrd, Aval, Bpos, Bcrd, Bval,
+                                            _ptr(mpos), _ptr(mcrd), crd, val)
+    else:
+        wrote = lib().oracle_spgemm_numeric_semiring(r0, r1, ncolsB, Apos, Acrd, Aval, Bpos, Bcrd, Bval,
+                                                     _ptr(mpos), _ptr(mcrd), REDUCE_OPS[semiring[0]],
+                                                     MULT_OPS[semiring[1]], crd, val)
     assert wrote == total, (wrote, total)
     return pos, crd[:total], val[:total]
 

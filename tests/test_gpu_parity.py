@@ -237,6 +237,80 @@ def test_spgemm_golden(golden, golden_dir):
         assert orc.format_f64(v) == g["printed_val"]
 
 
+SEMIRING_CASES = ["any_pair", "min_first", "min_plus", "min_second", "plus_first", "plus_pair", "plus_second",
+                  "plus_times"]
+
+
+@pytest.mark.parametrize("name", SEMIRING_CASES)
+def test_spgemm_semiring_golden(golden, golden_dir, name):
+    g = golden["spgemm_csr_semiring"]
+    c = g["cases"][name]
+    (nr, nc), pos, crd, val = _mtx(golden_dir, g["A"])
+    A = rt.CsrMatrix.from_arrays((nr, nc), pos, crd, val)
+    p, cc, v = rt.spgemm(A, A, semiring=(c["reduce"], c["mult"])).to_arrays()
+    assert p.tolist() == g["pos"] and cc.tolist() == g["crd"]
+    assert orc.format_f64(v) == c["printed_val"]
+
+
+@pytest.mark.parametrize("reduce", ["plus", "min", "max", "any"])
+@pytest.mark.parametrize("mult", ["times", "first", "second", "pair", "plus", "minus", "min", "max", "div"])
+def test_spgemm_semiring_vs_checker(reduce, mult):
+    rng = np.random.default_rng(sum(map(ord, reduce + mult)))
+    n, k, m = 300, 257, 2000
+    apos, acrd, aval = _rand_csr(rng, n, k, 0.05)
+    bpos, bcrd, bval = _rand_csr(rng, k, m, 0.04)
+    bval = np.abs(bval) + 0.5          # keeps div finite
+    A = rt.CsrMatrix.from_arrays((n, k), apos, acrd, aval)
+    B = rt.CsrMatrix.from_arrays((k, m), bpos, bcrd, bval)
+    p, c, v = rt.spgemm(A, B, semiring=(reduce, mult)).to_arrays()
+    wp, wc, wv = orc.spgemm(apos, acrd, aval, bpos, bcrd, bval, m, semiring=(reduce, mult))
+    assert np.array_equal(p, wp) and np.array_equal(c, wc)
+    if reduce == "plus":    # sums arrive in any order
+        _, _, count = orc.spgemm(apos, acrd, aval, bpos, bcrd, bval, m, semiring=("plus", "pair"))
+        amax, bmax, bmin = np.abs(aval).max(), bval.max(), bval.min()
+        biggest = max(amax * bmax, amax + bmax, amax / bmin, 1.0)       # no product exceeds this
+        assert np.all(np.abs(v - wv) <= RTOL * count * biggest)
+    else:                   # min, max and any do not depend on the order: bit-exact
+        assert np.array_equal(v, wv)
+
+
+def test_spgemm_semiring_masked_rowblocks_and_reuse():
+    """A masked min-plus product in two row blocks, then plain plus-times on the same handles: the
+    accumulators a semiring leaves behind must not leak into the next call."""
+    rng = np.random.default_rng(12)
+    n = 500
+    pos, crd, val = _rand_csr(rng, n, n, 0.03, signed=False)
+    mpos, mcrd, _ = _rand_csr(rng, n, n, 0.05)
+    A = rt.CsrMatrix.from_arrays((n, n), pos, crd, val)
+    Mk = rt.CsrMatrix.from_arrays((n, n), mpos, mcrd, np.ones(len(mcrd)))
+    cpos, nnz = rt.spgemm_symbolic(A, A, Mk)
+    hp = cpos.to_numpy()
+    wp, wc, wv = orc.spgemm(pos, crd, val, pos, crd, val, n, mask=(mpos, mcrd), semiring=("min", "plus"))
+    assert np.array_equal(hp, wp)
+    for r0, r1 in ((0, 211), (211, n)):
+        cnt = int(hp[r1] - hp[r0])
+        dcrd = rt.DeviceArray(max(cnt, 1), np.int32)
+        dval = rt.DeviceArray(max(cnt, 1))
+        rt.spgemm_numeric(A, A, cpos, r0, r1, dcrd, dval, mask=Mk, semiring=("min", "plus"))
+        assert np.array_equal(dcrd.to_numpy()[:cnt], wc[hp[r0]:hp[r1]])
+        assert np.array_equal(dval.to_numpy()[:cnt], wv[hp[r0]:hp[r1]])
+    for sr in (("max", "times"), ("any", "second"), None):
+        p, c, v = rt.spgemm(A, A, semiring=sr).to_arrays()
+        wp, wc, wv = orc.spgemm(pos, crd, val, pos, crd, val, n, semiring=sr)
+        assert np.array_equal(p, wp) and np.array_equal(c, wc)
+        if sr is None:
+            assert np.allclose(v, wv, rtol=1e-12, atol=0)
+        else:
+            assert np.array_equal(v, wv)
+
+
+def test_spgemm_semiring_rejects_unknown_operator():
+    pos = np.array([0, 1], dtype=np.int64)
+    A = rt.CsrMatrix.from_arrays((1, 1), pos, np.array([0], dtype=np.int64), np.array([1.0]))
+    h = rt.lib().comet_hip_spgemm_csr_semiring(A.handle, A.handle, 0, 9, 0)
+    assert h == 0 and b"semiring" in rt.lib().comet_hip_last_error()
+
+
 def _spgemm_check(a, b, ncolsB, mask=None):
     (apos, acrd, aval), (bpos, bcrd, bval) = a, b
     n, kdim = len(apos) - 1, len(bpos) - 1

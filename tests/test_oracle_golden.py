@@ -97,6 +97,94 @@ def test_spgemm_golden(golden, golden_dir):
     assert orc.format_f64(Cval) == g["printed_val"]
 
 
+SEMIRING_CASES = ["any_pair", "min_first", "min_plus", "min_second", "plus_first", "plus_pair", "plus_second",
+                  "plus_times"]
+
+
+@pytest.mark.parametrize("name", SEMIRING_CASES)
+def test_spgemm_semiring_golden(golden, golden_dir, name):
+    g = golden["spgemm_csr_semiring"]
+    c = g["cases"][name]
+    (nr, nc), pos, crd, val = _mtx(golden_dir, g["A"])
+    Cpos, Ccrd, Cval = orc.spgemm(pos, crd, val, pos, crd, val, nc, semiring=(c["reduce"], c["mult"]))
+    assert Cpos.tolist() == g["pos"]
+    assert Ccrd.tolist() == g["crd"]
+    assert orc.format_f64(Cval) == c["printed_val"]
+
+
+def _semiring_bruteforce(A, B, reduce, mult, mask=None):
+    """Independent statement: gather the products of every (i, j) in traversal order, then fold."""
+    mul = {"times": lambda a, b: a * b, "first": lambda a, b: a, "second": lambda a, b: b,
+           "pair": lambda a, b: 1.0, "plus": lambda a, b: a + b, "minus": lambda a, b: a - b,
+           "min": min, "max": max, "div": lambda a, b: a / b}[mult]
+    out = []
+    for i in range(A.shape[0]):
+        cols = {}
+        for p in range(A.indptr[i], A.indptr[i + 1]):
+            k = A.indices[p]
+            for q in range(B.indptr[k], B.indptr[k + 1]):
+                cols.setdefault(int(B.indices[q]), []).append(mul(float(A.data[p]), float(B.data[q])))
+        row = {}
+        for j, es in cols.items():
+            if mask is not None and not mask[i, j]:
+                continue
+            if reduce == "plus":
+                acc = 0.0
+                for e in es:
+                    acc = acc + e
+            elif reduce == "min":
+                acc = min(es)
+            elif reduce == "max":
+                acc = max([0.0] + es)      # the reference starts max from 0, not from -inf
+            else:
+                acc = es[-1]
+            row[j] = acc
+        out.append(row)
+    return out
+
+
+@pytest.mark.parametrize("reduce", ["plus", "min", "max", "any"])
+@pytest.mark.parametrize("mult", ["times", "first", "second", "pair", "plus", "minus", "min", "max", "div"])
+def test_spgemm_semiring_bruteforce(reduce, mult):
+    rng = np.random.default_rng(sum(map(ord, reduce + mult)))
+    A = sp.random(23, 31, density=0.2, format="csr", random_state=rng, data_rvs=lambda n: rng.uniform(-2, 2, n))
+    B = sp.random(31, 19, density=0.25, format="csr", random_state=rng, data_rvs=lambda n: rng.uniform(0.5, 3, n))
+    A.sort_indices(); B.sort_indices()
+    Cpos, Ccrd, Cval = orc.spgemm(A.indptr, A.indices, A.data, B.indptr, B.indices, B.data, 19,
+                                  semiring=(reduce, mult))
+    want = _semiring_bruteforce(A, B, reduce, mult)
+    for i, row in enumerate(want):
+        got = dict(zip(Ccrd[Cpos[i]:Cpos[i + 1]].tolist(), Cval[Cpos[i]:Cpos[i + 1]].tolist()))
+        assert sorted(got) == sorted(row)
+        assert list(got) == sorted(got)
+        for j in row:
+            assert got[j] == row[j], (i, j, got[j], row[j])
+
+
+def test_spgemm_semiring_masked_bruteforce():
+    rng = np.random.default_rng(77)
+    A = sp.random(20, 20, density=0.3, format="csr", random_state=rng, data_rvs=lambda n: rng.uniform(0.5, 2, n))
+    M = sp.random(20, 20, density=0.3, format="csr", random_state=rng)
+    A.sort_indices(); M.sort_indices()
+    Md = M.toarray() != 0
+    Cpos, Ccrd, Cval = orc.spgemm(A.indptr, A.indices, A.data, A.indptr, A.indices, A.data, 20,
+                                  mask=(M.indptr, M.indices), semiring=("min", "plus"))
+    want = _semiring_bruteforce(A, A, "min", "plus", mask=Md)
+    for i, row in enumerate(want):
+        got = dict(zip(Ccrd[Cpos[i]:Cpos[i + 1]].tolist(), Cval[Cpos[i]:Cpos[i + 1]].tolist()))
+        assert got == row
+
+
+def test_spgemm_semiring_plus_times_is_the_plain_routine():
+    rng = np.random.default_rng(3)
+    A = sp.random(40, 40, density=0.2, format="csr", random_state=rng, data_rvs=lambda n: rng.uniform(-1, 1, n))
+    A.sort_indices()
+    plain = orc.spgemm(A.indptr, A.indices, A.data, A.indptr, A.indices, A.data, 40)
+    semi = orc.spgemm(A.indptr, A.indices, A.data, A.indptr, A.indices, A.data, 40, semiring=("plus", "times"))
+    for x, y in zip(plain, semi):
+        assert np.array_equal(x, y)
+
+
 def test_spgemm_masked_golden(golden, golden_dir):
     g = golden["spgemm_csr_masked"]
     (nr, nc), pos, crd, val = _mtx(golden_dir, g["A"])
