@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the index-tree kernel path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload spmm|spmv|ttgt|tricount|spgemm]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload spmm|spmv|ttgt|tricount|spgemm|coo2csr]
 
 A step is one pass of the kernel over one batch of seeded synthetic input that is already
 resident in HBM.  The default workload is the one the headline metric is quoted on: CSR SpMM,
@@ -413,8 +413,51 @@ def bench_copy(rt, orc, gen, args):
     }
 
 
+def bench_coo2csr(rt, orc, gen, args):
+    """The reader's ordering step: the tuples of the SpMM matrix in shuffled order -> device CSR."""
+    n = args.n or 500_000
+    pos, crd, val = gen.zipf_csr(n=n, mean=16.0, cap=4096, seed=2)
+    nnz = len(crd)
+    row = np.repeat(np.arange(n, dtype=np.int64), np.diff(pos))
+    perm = np.random.Generator(np.random.PCG64(5)).permutation(nnz)
+    row, col, v = row[perm], crd[perm], val[perm]
+    drow = rt.DeviceArray.from_numpy(row.astype(np.int32))
+    dcol = rt.DeviceArray.from_numpy(col.astype(np.int32))
+    dval = rt.DeviceArray.from_numpy(v)
+    out = {}
+
+    def step():
+        out["A"] = rt.CsrMatrix.from_coo_device((n, n), drow, dcol, dval)     # the previous result is freed here
+    step()
+    wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
+    kt = kernel_times(rt, step, args.steps)
+    p, c, vv = out["A"].to_arrays()
+    parity_ok = bool(np.array_equal(p, pos) and np.array_equal(c, crd) and np.array_equal(vv, val))
+    # tuples read once (4 + 4 + 8 B each), CSR written once (4 + 8 B each, 8 B per row pointer)
+    alg_bytes = nnz * 16 + nnz * 12 + 8 * (n + 1)
+    dom = "radix_sort_pairs"
+    dom_ms = kt[dom]["avg_ms"]
+    sort_bytes = nnz * 12 * 2     # one read and one write of (key, position) if the sort were a single pass
+    cpu = None
+    if not args.no_cpu:
+        t, reps = cpu_time(lambda: orc.coo_to_csr(n, row, col, v), budget_s=20.0, min_reps=1)
+        cpu = {"value": nnz / t / 1e6, "unit": "Mtuples/s", "cores": 1, "kind": "port",
+               "sample": f"the full workload, best of {reps} runs, {t:.2f} s each (stable sort by (row, col), "
+                         "filter, row pointers, single thread as in the reference's reader)"}
+    return {
+        "metric": "COO -> CSR ordering Mtuples/s on 1 MI355X", "value": nnz / (dev_ms * 1e-3) / 1e6,
+        "unit": "Mtuples/s", "ms_per_step": dev_ms, "dtype": "u64 keys / f64 values",
+        "config": {"workload": "coo_to_csr_zipf_shuffled", "rows": n, "cols": n, "tuples": int(nnz), "seed": 2},
+        "roofline": {"bound": "hbm", "achieved": sort_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": sort_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": dom + " (rocPRIM, all its passes)", "kernel_avg_ms": dom_ms,
+                     "algorithmic_bytes": int(sort_bytes), "whole_conversion_algorithmic_bytes": int(alg_bytes)},
+        "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
+    }
+
+
 WORKLOADS = {"copy": bench_copy, "spmm": bench_spmm, "spmv": bench_spmv, "ttgt": bench_ttgt, "tricount": bench_tricount,
-             "spgemm": bench_spgemm}
+             "spgemm": bench_spgemm, "coo2csr": bench_coo2csr}
 
 
 def main():

@@ -7,7 +7,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libcomet_hip_rt.so")
-SOURCES = ["runtime.hip", "spmv_spmm.hip", "spgemm.hip", "ttgt.hip", "ciface.hip"]
+SOURCES = ["runtime.hip", "spmv_spmm.hip", "spgemm.hip", "ttgt.hip", "ciface.hip", "formats.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-ffp-contract=off",            # the reference's loops multiply then add, unfused

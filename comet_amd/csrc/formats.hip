@@ -1,0 +1,748 @@
+// Input side of the sparse kernels: MatrixMarket text -> device CSR with the
+// reference's read modes, the SPARSE_FILE_NAME<id> protocol of its reader
+// entry points, and conversion of the other two matrix layouts its tests feed
+// to SpMV/SpMM (COO and DCSR) to and from device CSR, plus CSR transposition.
+//
+// Text is parsed on the host; everything after that - ordering the tuples by
+// (row, column) with ties in file order, dropping the entries a triangular read
+// mode excludes, building the row pointers - runs on the GPU, so a matrix goes
+// from file to a handle the kernels accept without a host-side CSR in between.
+#include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <cstring>
+#include <rocprim/device/device_radix_sort.hpp>
+
+#include <map>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "common.h"
+
+namespace comet {
+
+// ---------------------------------------------------------------------------
+// MatrixMarket text -> unordered tuples (lib/ExecutionEngine/SparseUtils.cpp:
+// 145-356): 1-based indices; a missing value reads as 1.0; the flags come from
+// any line that starts with "%%" (substring tests for "symmetric", "skew",
+// "array"); a symmetric file mirrors every off-diagonal entry right after the
+// entry itself, negated if skew; an array file lists all rows*cols values in
+// column-major order, zeros included.
+// ---------------------------------------------------------------------------
+struct HostCoo {
+    int64_t nrows = 0, ncols = 0;
+    std::vector<int32_t> row, col;
+    std::vector<double> val;
+};
+
+static int parse_mtx(const char *path, HostCoo *out)
+{
+    FILE *f = fopen(path, "rb");
+    if (!f)
+        return set_error(COMET_HIP_ERR_ARG, "cannot open %s", path);
+    std::string text;
+    {
+        char buf[1 << 16];
+        size_t got;
+        while ((got = fread(buf, 1, sizeof buf, f)) > 0)
+            text.append(buf, got);
+        fclose(f);
+    }
+    bool array = false, symmetric = false, skew = false, have_sizes = false;
+    int64_t declared = 0, array_seen = 0;
+    const char *p = text.c_str(), *end = p + text.size();
+    int64_t lineno = 0;
+    while (p < end) {
+        const char *eol = (const char *)memchr(p, '\n', (size_t)(end - p));
+        const char *next = eol ? eol + 1 : end;
+        if (!eol)
+            eol = end;
+        ++lineno;
+        std::string line(p, (size_t)(eol - p));
+        p = next;
+        if (!line.empty() && line[0] == '%') {
+            if (line.size() > 1 && line[1] == '%') {
+                symmetric = line.find("symmetric") != std::string::npos;
+                skew = line.find("skew") != std::string::npos;
+                array = line.find("array") != std::string::npos;
+            }
+            continue;
+        }
+        const char *l = line.c_str();
+        char *t = nullptr;
+        if (!have_sizes) {
+            long long a = 0, b = 0, c = 0;
+            const int n = sscanf(l, "%lld %lld %lld", &a, &b, &c);
+            if (n < 2)
+                continue;      // blank line in front of the size line
+            if ((!array && n != 3) || (array && n != 2))
+                return set_error(COMET_HIP_ERR_ARG, "%s:%lld: invalid size line", path, (long long)lineno);
+            if (a < 0 || b < 0 || c < 0 || a >= (1ll << 31) || b >= (1ll << 31))
+                return set_error(COMET_HIP_ERR_SIZE, "%s: dimensions %lld x %lld not supported", path, a, b);
+            if (array && symmetric)
+                return set_error(COMET_HIP_ERR_ARG, "%s: symmetric array files are not supported", path);
+            out->nrows = a;
+            out->ncols = b;
+            declared = array ? a * b : (symmetric ? 2 * c : c);
+            out->row.reserve((size_t)declared);
+            out->col.reserve((size_t)declared);
+            out->val.reserve((size_t)declared);
+            have_sizes = true;
+            continue;
+        }
+        if (array) {
+            const double v = strtod(l, &t);
+            if (t == l)
+                continue;
+            if (array_seen >= declared)
+                return set_error(COMET_HIP_ERR_ARG, "%s: more than %lld values", path, (long long)declared);
+            out->row.push_back((int32_t)(array_seen % out->nrows));
+            out->col.push_back((int32_t)(array_seen / out->nrows));
+            out->val.push_back(v);
+            ++array_seen;
+            continue;
+        }
+        const long long r = strtoll(l, &t, 0);
+        if (t == l)
+            continue;          // blank line
+        l = t;
+        const long long c = strtoll(l, &t, 0);
+        if (t == l)
+            return set_error(COMET_HIP_ERR_ARG, "%s:%lld: badly formed column", path, (long long)lineno);
+        l = t;
+        double v = strtod(l, &t);
+        if (t == l)
+            v = 1.0;
+        if (r < 1 || r > out->nrows || c < 1 || c > out->ncols)
+            return set_error(COMET_HIP_ERR_ARG, "%s:%lld: entry (%lld,%lld) outside %lld x %lld", path,
+                             (long long)lineno, r, c, (long long)out->nrows, (long long)out->ncols);
+        if ((int64_t)out->row.size() + ((symmetric && r != c) ? 2 : 1) > declared)
+            return set_error(COMET_HIP_ERR_ARG, "%s: more than the declared %lld entries", path,
+                             (long long)declared);
+        out->row.push_back((int32_t)(r - 1));
+        out->col.push_back((int32_t)(c - 1));
+        out->val.push_back(v);
+        if (symmetric && r != c) {
+            out->row.push_back((int32_t)(c - 1));
+            out->col.push_back((int32_t)(r - 1));
+            out->val.push_back(skew ? -v : v);
+        }
+    }
+    if (!have_sizes)
+        return set_error(COMET_HIP_ERR_ARG, "%s: no size line", path);
+    return COMET_HIP_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Device tuples -> CSR.  key = row << 32 | col; a radix sort of (key, original
+// position) is stable, so equal (row, col) pairs keep file order exactly as the
+// reference's std::stable_sort does (SparseUtils.cpp:404-424; duplicates are
+// kept, never merged).  Entries are then filtered by read mode (:458-507: 2
+// strictly lower, 3 lower, 4 strictly upper, 5 upper, anything else all),
+// compacted in order, and row r's pointer is the position of the first kept
+// entry whose row is >= r.
+// ---------------------------------------------------------------------------
+__global__ void coo_make_keys(int64_t n, const int32_t *__restrict__ row, const int32_t *__restrict__ col,
+                              uint64_t *__restrict__ keys, uint32_t *__restrict__ idx)
+{
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < n) {
+        keys[e] = ((uint64_t)(uint32_t)row[e] << 32) | (uint32_t)col[e];
+        idx[e] = (uint32_t)e;
+    }
+}
+
+__device__ inline bool keep_entry(int mode, uint32_t r, uint32_t c)
+{
+    switch (mode) {
+    case COMET_READ_LOWER_TRI_STRICT: return r > c;
+    case COMET_READ_LOWER_TRI: return r >= c;
+    case COMET_READ_UPPER_TRI_STRICT: return r < c;
+    case COMET_READ_UPPER_TRI: return r <= c;
+    default: return true;
+    }
+}
+
+__global__ void coo_flag(int64_t n, const uint64_t *__restrict__ keys, int mode, int64_t *__restrict__ flag)
+{
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < n)
+        flag[e] = keep_entry(mode, (uint32_t)(keys[e] >> 32), (uint32_t)keys[e]) ? 1 : 0;
+}
+
+__global__ void coo_compact(int64_t n, const uint64_t *__restrict__ keys, const uint32_t *__restrict__ idx,
+                            const int64_t *__restrict__ off, const double *__restrict__ val_in,
+                            int32_t *__restrict__ crow, int32_t *__restrict__ crd, double *__restrict__ val)
+{
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < n && off[e + 1] != off[e]) {
+        const int64_t o = off[e];
+        crow[o] = (int32_t)(keys[e] >> 32);
+        crd[o] = (int32_t)(uint32_t)keys[e];
+        val[o] = val_in[idx[e]];
+    }
+}
+
+// pos[r] = number of kept entries whose row is < r, for r in [0, nrows]
+__global__ void rows_to_pos(int64_t nrows, int64_t kept, const int32_t *__restrict__ crow, int64_t *__restrict__ pos)
+{
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r > nrows)
+        return;
+    int64_t lo = 0, hi = kept;
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (crow[mid] < r)
+            lo = mid + 1;
+        else
+            hi = mid;
+    }
+    pos[r] = lo;
+}
+
+// rowid[e] = the row whose range [pos[r], pos[r+1]) holds entry e
+__global__ void csr_expand_rows(int64_t nrows, int64_t nnz, const int64_t *__restrict__ pos,
+                                int32_t *__restrict__ rowid)
+{
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= nnz)
+        return;
+    int64_t lo = 0, hi = nrows;     // last r with pos[r] <= e
+    while (lo < hi) {
+        const int64_t mid = (lo + hi + 1) >> 1;
+        if (pos[mid] <= e)
+            lo = mid;
+        else
+            hi = mid - 1;
+    }
+    rowid[e] = (int32_t)lo;
+}
+
+__global__ void widen_i32(int64_t n, const int32_t *__restrict__ in, int64_t *__restrict__ out)
+{
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < n)
+        out[e] = in[e];
+}
+
+// flag[r] = 1 if row r stores anything
+__global__ void row_nonempty(int64_t nrows, const int64_t *__restrict__ pos, int64_t *__restrict__ flag)
+{
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r < nrows)
+        flag[r] = pos[r + 1] != pos[r] ? 1 : 0;
+}
+
+__global__ void dcsr_compact_rows(int64_t nrows, const int64_t *__restrict__ pos, const int64_t *__restrict__ off,
+                                  int64_t *__restrict__ a1crd, int64_t *__restrict__ a2pos)
+{
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r < nrows && off[r + 1] != off[r]) {
+        a1crd[off[r]] = r;
+        a2pos[off[r]] = pos[r];
+    }
+    if (r == nrows)
+        a2pos[off[nrows]] = pos[nrows];
+}
+
+struct DevBuf {
+    void *p = nullptr;
+    ~DevBuf() { if (p) (void)hipFree(p); }
+    int alloc(size_t bytes)
+    {
+        COMET_HIPCHK(hipMalloc(&p, bytes ? bytes : 1));
+        return COMET_HIP_OK;
+    }
+    template <typename T> T *as() { return (T *)p; }
+};
+
+struct CachedBuf {
+    Workspace w;
+    void *p = nullptr;
+    int alloc(size_t bytes)
+    {
+        COMET_CHK(w.ensure(bytes ? bytes : 1, false));
+        p = w.ptr;
+        return COMET_HIP_OK;
+    }
+    template <typename T> T *as() { return (T *)p; }
+};
+
+static inline dim3 grid_for(int64_t n) { return dim3((unsigned)(n > 0 ? ceil_div(n, 256) : 1)); }
+
+// row/col/val are device arrays of n tuples in input order; returns a new registered handle or 0
+static int64_t coo_device_to_csr(int64_t nrows, int64_t ncols, int64_t n, const int32_t *row, const int32_t *col,
+                                 const double *val, int mode)
+{
+    Csr *c = new Csr();
+    c->nrows = nrows;
+    c->ncols = ncols;
+    c->owns = true;
+    auto fail = [&]() -> int64_t {
+        (void)hipFree(c->pos);
+        (void)hipFree(c->crd);
+        (void)hipFree(c->val);
+        delete c;
+        return 0;
+    };
+    if (hipMalloc((void **)&c->pos, sizeof(int64_t) * (size_t)(nrows + 1)) != hipSuccess) {
+        set_error(COMET_HIP_ERR_HIP, "row pointer allocation failed");
+        return fail();
+    }
+    // temporaries live in grow-only buffers kept for the life of the process: a conversion of a few million
+    // tuples takes less time than the allocations would
+    static CachedBuf keys_in, keys_out, idx_in, idx_out, flag, off, crow, tmp;
+    int64_t kept = 0;
+    if (n > 0) {
+        if (keys_in.alloc(8 * (size_t)n) || keys_out.alloc(8 * (size_t)n) || idx_in.alloc(4 * (size_t)n) ||
+            idx_out.alloc(4 * (size_t)n) || flag.alloc(8 * (size_t)n) || off.alloc(8 * (size_t)(n + 1)))
+            return fail();
+        {
+            KernelTimer t("coo_make_keys");
+            coo_make_keys<<<grid_for(n), dim3(256), 0, stream()>>>(n, row, col, keys_in.as<uint64_t>(),
+                                                                  idx_in.as<uint32_t>());
+        }
+        int row_bits = 1;
+        while (row_bits < 31 && (1ll << row_bits) < nrows)
+            ++row_bits;
+        size_t tmp_bytes = 0;
+        if (rocprim::radix_sort_pairs(nullptr, tmp_bytes, keys_in.as<uint64_t>(), keys_out.as<uint64_t>(),
+                                      idx_in.as<uint32_t>(), idx_out.as<uint32_t>(), (size_t)n, 0u,
+                                      (unsigned)(32 + row_bits), stream()) != hipSuccess ||
+            tmp.alloc(tmp_bytes)) {
+            set_error(COMET_HIP_ERR_HIP, "sort workspace query failed");
+            return fail();
+        }
+        {
+            KernelTimer t("radix_sort_pairs");
+            if (rocprim::radix_sort_pairs(tmp.p, tmp_bytes, keys_in.as<uint64_t>(), keys_out.as<uint64_t>(),
+                                          idx_in.as<uint32_t>(), idx_out.as<uint32_t>(), (size_t)n, 0u,
+                                          (unsigned)(32 + row_bits), stream()) != hipSuccess) {
+                set_error(COMET_HIP_ERR_HIP, "sorting %lld tuples failed", (long long)n);
+                return fail();
+            }
+        }
+        {
+            KernelTimer t("coo_flag");
+            coo_flag<<<grid_for(n), dim3(256), 0, stream()>>>(n, keys_out.as<uint64_t>(), mode, flag.as<int64_t>());
+        }
+        if (exclusive_scan_i64(flag.as<int64_t>(), n, off.as<int64_t>()) != COMET_HIP_OK)
+            return fail();
+        if (hipMemcpyAsync(&kept, off.as<int64_t>() + n, sizeof(int64_t), hipMemcpyDeviceToHost, stream()) !=
+                hipSuccess ||
+            hipStreamSynchronize(stream()) != hipSuccess) {
+            set_error(COMET_HIP_ERR_HIP, "reading the entry count failed");
+            return fail();
+        }
+    }
+    c->nnz = kept;
+    if (hipMalloc((void **)&c->crd, sizeof(int32_t) * (size_t)(kept > 0 ? kept : 1)) != hipSuccess ||
+        hipMalloc((void **)&c->val, sizeof(double) * (size_t)(kept > 0 ? kept : 1)) != hipSuccess ||
+        crow.alloc(4 * (size_t)(kept > 0 ? kept : 1))) {
+        set_error(COMET_HIP_ERR_HIP, "allocation of %lld entries failed", (long long)kept);
+        return fail();
+    }
+    if (n > 0) {
+        KernelTimer t("coo_compact");
+        coo_compact<<<grid_for(n), dim3(256), 0, stream()>>>(n, keys_out.as<uint64_t>(), idx_out.as<uint32_t>(),
+                                                            off.as<int64_t>(), val, crow.as<int32_t>(), c->crd,
+                                                            c->val);
+    }
+    {
+        KernelTimer t("rows_to_pos");
+        rows_to_pos<<<grid_for(nrows + 1), dim3(256), 0, stream()>>>(nrows, kept, crow.as<int32_t>(), c->pos);
+    }
+    if (hipGetLastError() != hipSuccess || hipStreamSynchronize(stream()) != hipSuccess) {
+        set_error(COMET_HIP_ERR_HIP, "building the CSR arrays failed");
+        return fail();
+    }
+    return csr_register(c);
+}
+
+static int64_t coo_host_to_csr(int64_t nrows, int64_t ncols, int64_t n, const int32_t *row, const int32_t *col,
+                               const double *val, int mode)
+{
+    DevBuf drow, dcol, dval;
+    if (drow.alloc(4 * (size_t)n) || dcol.alloc(4 * (size_t)n) || dval.alloc(8 * (size_t)n))
+        return 0;
+    if (n > 0 &&
+        (hipMemcpyAsync(drow.p, row, 4 * (size_t)n, hipMemcpyHostToDevice, stream()) != hipSuccess ||
+         hipMemcpyAsync(dcol.p, col, 4 * (size_t)n, hipMemcpyHostToDevice, stream()) != hipSuccess ||
+         hipMemcpyAsync(dval.p, val, 8 * (size_t)n, hipMemcpyHostToDevice, stream()) != hipSuccess ||
+         hipStreamSynchronize(stream()) != hipSuccess)) {
+        set_error(COMET_HIP_ERR_HIP, "uploading %lld tuples failed", (long long)n);
+        return 0;
+    }
+    return coo_device_to_csr(nrows, ncols, n, drow.as<int32_t>(), dcol.as<int32_t>(), dval.as<double>(), mode);
+}
+
+static bool known_mode(int mode) { return mode >= COMET_READ_DEFAULT && mode <= COMET_READ_UPPER_TRI; }
+
+// ---------------------------------------------------------------------------
+// The reader's file-id protocol (SparseUtils.cpp:1425-1600): id 0..9998 names
+// the environment variable SPARSE_FILE_NAME<id>, 9999 plain SPARSE_FILE_NAME.
+// The sizes call reads the file and keeps the result; the read call that
+// follows consumes it.  What is kept here is the finished device CSR.
+// ---------------------------------------------------------------------------
+static std::map<std::pair<int32_t, int32_t>, int64_t> g_pending_reads;
+
+static int file_name_of(int32_t file_id, std::string *out)
+{
+    const char *v = nullptr;
+    if (file_id >= 0 && file_id < 9999)
+        v = getenv(("SPARSE_FILE_NAME" + std::to_string(file_id)).c_str());
+    else if (file_id == 9999)
+        v = getenv("SPARSE_FILE_NAME");
+    if (!v || !*v)
+        return set_error(COMET_HIP_ERR_ARG, "SPARSE_FILE_NAME%s is not set",
+                         file_id == 9999 ? "" : std::to_string(file_id).c_str());
+    *out = v;
+    if (out->find(".mtx") == std::string::npos)
+        return set_error(COMET_HIP_ERR_ARG, "%s is not a Matrix Market file", v);
+    return COMET_HIP_OK;
+}
+
+static int64_t pending_read(int32_t file_id, int32_t mode, bool take)
+{
+    const int32_t m = known_mode(mode) ? mode : COMET_READ_DEFAULT;   // getMatrixReadOption, SparseUtils.cpp:50-64
+    auto key = std::make_pair(file_id, m);
+    auto it = g_pending_reads.find(key);
+    int64_t h = 0;
+    if (it != g_pending_reads.end()) {
+        h = it->second;
+    } else {
+        std::string name;
+        if (file_name_of(file_id, &name) != COMET_HIP_OK)
+            return 0;
+        h = comet_hip_mtx_read_csr(name.c_str(), m);
+        if (!h)
+            return 0;
+        g_pending_reads[key] = h;
+    }
+    if (take)
+        g_pending_reads.erase(key);
+    return h;
+}
+
+static void die_reader(const char *who)
+{
+    fprintf(stderr, "%s: %s\n", who, comet_hip_last_error());
+    exit(1);
+}
+
+enum Layout { LAYOUT_CSR, LAYOUT_COO, LAYOUT_DCSR, LAYOUT_OTHER };
+static Layout layout_of(int32_t a1, int32_t a1_tile, int32_t a2, int32_t a2_tile)
+{
+    (void)a2_tile;
+    if (a1 == COMET_FMT_COMPRESSED_NONUNIQUE && a2 == COMET_FMT_SINGLETON)
+        return LAYOUT_COO;
+    if (a1 == COMET_FMT_DENSE && a2 == COMET_FMT_COMPRESSED_UNIQUE)
+        return LAYOUT_CSR;
+    if (a1 == COMET_FMT_COMPRESSED_UNIQUE && a2 == COMET_FMT_COMPRESSED_UNIQUE)
+        return LAYOUT_DCSR;
+    (void)a1_tile;
+    return LAYOUT_OTHER;
+}
+
+template <typename T>
+static T *memref_data(void *desc)
+{
+    auto *m = (comet_memref_1d *)desc;
+    return m && m->aligned ? (T *)m->aligned + m->offset : nullptr;
+}
+
+}  // namespace comet
+
+using namespace comet;
+
+extern "C" int64_t comet_hip_mtx_read_csr(const char *path, int read_mode)
+{
+    if (ensure_init() != COMET_HIP_OK)
+        return 0;
+    if (!path) {
+        set_error(COMET_HIP_ERR_ARG, "null path passed to comet_hip_mtx_read_csr");
+        return 0;
+    }
+    if (!known_mode(read_mode)) {
+        set_error(COMET_HIP_ERR_ARG, "unknown read mode %d", read_mode);
+        return 0;
+    }
+    HostCoo coo;
+    if (parse_mtx(path, &coo) != COMET_HIP_OK)
+        return 0;
+    return coo_host_to_csr(coo.nrows, coo.ncols, (int64_t)coo.row.size(), coo.row.data(), coo.col.data(),
+                           coo.val.data(), read_mode);
+}
+
+extern "C" int64_t comet_hip_csr_from_coo_i64(int64_t nrows, int64_t ncols, int64_t nnz, const int64_t *row,
+                                              const int64_t *col, const double *val, int read_mode)
+{
+    if (ensure_init() != COMET_HIP_OK)
+        return 0;
+    if (nrows < 0 || ncols < 0 || nnz < 0 || nrows >= (1ll << 31) || ncols >= (1ll << 31) || nnz >= (1ll << 32) ||
+        (nnz > 0 && (!row || !col || !val)) || !known_mode(read_mode)) {
+        set_error(COMET_HIP_ERR_ARG, "bad arguments to comet_hip_csr_from_coo_i64 (%lld x %lld, %lld entries, mode %d)",
+                  (long long)nrows, (long long)ncols, (long long)nnz, read_mode);
+        return 0;
+    }
+    std::vector<int32_t> r32((size_t)nnz), c32((size_t)nnz);
+    for (int64_t e = 0; e < nnz; ++e) {
+        if (row[e] < 0 || row[e] >= nrows || col[e] < 0 || col[e] >= ncols) {
+            set_error(COMET_HIP_ERR_ARG, "tuple %lld = (%lld,%lld) lies outside %lld x %lld", (long long)e,
+                      (long long)row[e], (long long)col[e], (long long)nrows, (long long)ncols);
+            return 0;
+        }
+        r32[(size_t)e] = (int32_t)row[e];
+        c32[(size_t)e] = (int32_t)col[e];
+    }
+    return coo_host_to_csr(nrows, ncols, nnz, r32.data(), c32.data(), val, read_mode);
+}
+
+extern "C" int64_t comet_hip_csr_from_coo_device(int64_t nrows, int64_t ncols, int64_t nnz, int64_t row_dptr,
+                                                 int64_t col_dptr, int64_t val_dptr, int read_mode)
+{
+    if (ensure_init() != COMET_HIP_OK)
+        return 0;
+    if (nrows < 0 || ncols < 0 || nnz < 0 || nrows >= (1ll << 31) || ncols >= (1ll << 31) || nnz >= (1ll << 32) ||
+        (nnz > 0 && (!row_dptr || !col_dptr || !val_dptr)) || !known_mode(read_mode)) {
+        set_error(COMET_HIP_ERR_ARG, "bad arguments to comet_hip_csr_from_coo_device (%lld x %lld, %lld entries, mode %d)",
+                  (long long)nrows, (long long)ncols, (long long)nnz, read_mode);
+        return 0;
+    }
+    return coo_device_to_csr(nrows, ncols, nnz, (const int32_t *)row_dptr, (const int32_t *)col_dptr,
+                             (const double *)val_dptr, read_mode);
+}
+
+extern "C" int64_t comet_hip_csr_from_dcsr_i64(int64_t nrows, int64_t ncols, int64_t nrows_stored,
+                                               const int64_t *a1crd, const int64_t *a2pos, const int64_t *a2crd,
+                                               const double *aval)
+{
+    if (ensure_init() != COMET_HIP_OK)
+        return 0;
+    if (nrows < 0 || nrows_stored < 0 || nrows_stored > nrows || !a2pos || (nrows_stored > 0 && !a1crd)) {
+        set_error(COMET_HIP_ERR_ARG, "bad arguments to comet_hip_csr_from_dcsr_i64");
+        return 0;
+    }
+    // expand the stored-row list into one pointer per row; the arrays of the second level are CSR's already
+    std::vector<int64_t> pos((size_t)nrows + 1, 0);
+    int64_t prev = -1;
+    for (int64_t s = 0; s < nrows_stored; ++s) {
+        const int64_t r = a1crd[s];
+        if (r <= prev || r >= nrows || a2pos[s + 1] < a2pos[s]) {
+            set_error(COMET_HIP_ERR_ARG, "stored row %lld (row id %lld) is out of order or out of range",
+                      (long long)s, (long long)r);
+            return 0;
+        }
+        for (int64_t q = prev + 1; q <= r; ++q)
+            pos[(size_t)q] = a2pos[s];
+        prev = r;
+    }
+    for (int64_t q = prev + 1; q <= nrows; ++q)
+        pos[(size_t)q] = a2pos[nrows_stored];
+    if (pos[0] != 0) {
+        set_error(COMET_HIP_ERR_ARG, "the second-level pointers must start at 0");
+        return 0;
+    }
+    return comet_hip_csr_upload_i64(nrows, ncols, pos.data(), a2crd, aval);
+}
+
+extern "C" int comet_hip_csr_to_coo_i64(int64_t h, int64_t *row, int64_t *col, double *val)
+{
+    COMET_CHK(ensure_init());
+    Csr *a = csr_from_handle(h);
+    if (!a)
+        return COMET_HIP_ERR_HANDLE;
+    if (a->nnz == 0)
+        return COMET_HIP_OK;
+    if (!row || !col || !val)
+        return set_error(COMET_HIP_ERR_ARG, "null output passed to comet_hip_csr_to_coo_i64");
+    DevBuf r32, wide;
+    COMET_CHK(r32.alloc(4 * (size_t)a->nnz));
+    COMET_CHK(wide.alloc(8 * (size_t)a->nnz));
+    {
+        KernelTimer t("csr_expand_rows");
+        csr_expand_rows<<<grid_for(a->nnz), dim3(256), 0, stream()>>>(a->nrows, a->nnz, a->pos, r32.as<int32_t>());
+    }
+    widen_i32<<<grid_for(a->nnz), dim3(256), 0, stream()>>>(a->nnz, r32.as<int32_t>(), wide.as<int64_t>());
+    COMET_HIPCHK(hipMemcpyAsync(row, wide.p, 8 * (size_t)a->nnz, hipMemcpyDeviceToHost, stream()));
+    widen_i32<<<grid_for(a->nnz), dim3(256), 0, stream()>>>(a->nnz, a->crd, wide.as<int64_t>());
+    COMET_HIPCHK(hipMemcpyAsync(col, wide.p, 8 * (size_t)a->nnz, hipMemcpyDeviceToHost, stream()));
+    COMET_HIPCHK(hipMemcpyAsync(val, a->val, 8 * (size_t)a->nnz, hipMemcpyDeviceToHost, stream()));
+    COMET_HIPCHK(hipStreamSynchronize(stream()));
+    return COMET_HIP_OK;
+}
+
+extern "C" int comet_hip_csr_to_dcsr_i64(int64_t h, int64_t *nrows_stored, int64_t *a1crd, int64_t *a2pos,
+                                         int64_t *a2crd, double *aval)
+{
+    COMET_CHK(ensure_init());
+    Csr *a = csr_from_handle(h);
+    if (!a)
+        return COMET_HIP_ERR_HANDLE;
+    if (!nrows_stored)
+        return set_error(COMET_HIP_ERR_ARG, "null count passed to comet_hip_csr_to_dcsr_i64");
+    DevBuf flag, off, d1, d2, wide;
+    COMET_CHK(flag.alloc(8 * (size_t)(a->nrows + 1)));
+    COMET_CHK(off.alloc(8 * (size_t)(a->nrows + 1)));
+    int64_t stored = 0;
+    if (a->nrows > 0) {
+        row_nonempty<<<grid_for(a->nrows), dim3(256), 0, stream()>>>(a->nrows, a->pos, flag.as<int64_t>());
+        COMET_CHK(exclusive_scan_i64(flag.as<int64_t>(), a->nrows, off.as<int64_t>()));
+        COMET_HIPCHK(hipMemcpyAsync(&stored, off.as<int64_t>() + a->nrows, 8, hipMemcpyDeviceToHost, stream()));
+        COMET_HIPCHK(hipStreamSynchronize(stream()));
+    }
+    *nrows_stored = stored;
+    if (!a1crd && !a2pos && !a2crd && !aval)
+        return COMET_HIP_OK;            // size query
+    if (!a1crd || !a2pos || (a->nnz > 0 && (!a2crd || !aval)))
+        return set_error(COMET_HIP_ERR_ARG, "null output passed to comet_hip_csr_to_dcsr_i64");
+    if (a->nrows == 0) {
+        a2pos[0] = 0;
+        return COMET_HIP_OK;
+    }
+    COMET_CHK(d1.alloc(8 * (size_t)stored));
+    COMET_CHK(d2.alloc(8 * (size_t)(stored + 1)));
+    {
+        KernelTimer t("dcsr_compact_rows");
+        dcsr_compact_rows<<<grid_for(a->nrows + 1), dim3(256), 0, stream()>>>(a->nrows, a->pos, off.as<int64_t>(),
+                                                                             d1.as<int64_t>(), d2.as<int64_t>());
+    }
+    COMET_HIPCHK(hipMemcpyAsync(a1crd, d1.p, 8 * (size_t)stored, hipMemcpyDeviceToHost, stream()));
+    COMET_HIPCHK(hipMemcpyAsync(a2pos, d2.p, 8 * (size_t)(stored + 1), hipMemcpyDeviceToHost, stream()));
+    if (a->nnz > 0) {
+        COMET_CHK(wide.alloc(8 * (size_t)a->nnz));
+        widen_i32<<<grid_for(a->nnz), dim3(256), 0, stream()>>>(a->nnz, a->crd, wide.as<int64_t>());
+        COMET_HIPCHK(hipMemcpyAsync(a2crd, wide.p, 8 * (size_t)a->nnz, hipMemcpyDeviceToHost, stream()));
+        COMET_HIPCHK(hipMemcpyAsync(aval, a->val, 8 * (size_t)a->nnz, hipMemcpyDeviceToHost, stream()));
+    }
+    COMET_HIPCHK(hipStreamSynchronize(stream()));
+    return COMET_HIP_OK;
+}
+
+extern "C" int64_t comet_hip_csr_transpose(int64_t h)
+{
+    if (ensure_init() != COMET_HIP_OK)
+        return 0;
+    Csr *a = csr_from_handle(h);
+    if (!a)
+        return 0;
+    DevBuf rowid;
+    if (rowid.alloc(4 * (size_t)a->nnz))
+        return 0;
+    if (a->nnz > 0) {
+        KernelTimer t("csr_expand_rows");
+        csr_expand_rows<<<grid_for(a->nnz), dim3(256), 0, stream()>>>(a->nrows, a->nnz, a->pos, rowid.as<int32_t>());
+    }
+    // the tuples of the transpose are (column, row, value): order them by (column, row)
+    return coo_device_to_csr(a->ncols, a->nrows, a->nnz, a->crd, rowid.as<int32_t>(), a->val, COMET_READ_DEFAULT);
+}
+
+extern "C" int64_t comet_hip_read_input_2D_handle(int32_t file_id, int32_t read_mode)
+{
+    if (ensure_init() != COMET_HIP_OK)
+        return 0;
+    return pending_read(file_id, read_mode, true);
+}
+
+extern "C" void comet_hip_read_input_sizes_2D_f64(int32_t file_id, int32_t a1format, int32_t a1_tile_format,
+                                                  int32_t a2format, int32_t a2_tile_format, int sizes_rank,
+                                                  void *sizes_desc, int32_t read_mode)
+{
+    const char *who = "comet_hip_read_input_sizes_2D_f64";
+    (void)sizes_rank;
+    int64_t *s = memref_data<int64_t>(sizes_desc);
+    const Layout lay = layout_of(a1format, a1_tile_format, a2format, a2_tile_format);
+    if (!s || lay == LAYOUT_OTHER) {
+        set_error(COMET_HIP_ERR_ARG, "only CSR, COO and DCSR layouts are read (formats %d,%d)", a1format, a2format);
+        die_reader(who);
+    }
+    if (ensure_init() != COMET_HIP_OK)
+        die_reader(who);
+    const int64_t h = pending_read(file_id, read_mode, false);
+    if (!h)
+        die_reader(who);
+    int64_t nrows = 0, ncols = 0, nnz = 0;
+    (void)comet_hip_csr_dims(h, &nrows, &ncols, &nnz);
+    for (int i = 0; i < 8; ++i)
+        s[i] = 0;
+    if (lay == LAYOUT_COO) {            // SparseUtils.cpp:1643-1659
+        s[0] = 2;
+        s[1] = nnz;
+        s[4] = 1;
+        s[5] = nnz;
+    } else if (lay == LAYOUT_CSR) {     // :1672-1687
+        s[0] = 1;
+        s[1] = 1;
+        s[4] = nrows + 1;
+        s[5] = nnz;
+    } else {                            // DCSR, :1731-1749 with the array sizes of :669-735
+        int64_t stored = 0;
+        if (comet_hip_csr_to_dcsr_i64(h, &stored, nullptr, nullptr, nullptr, nullptr))
+            die_reader(who);
+        s[0] = 2;
+        s[1] = stored;
+        s[4] = stored + 1;
+        s[5] = nnz;
+    }
+    s[8] = nnz;
+    s[9] = nrows;
+    s[10] = ncols;
+}
+
+extern "C" void comet_hip_read_input_2D_f64_i64(int32_t file_id, int32_t a1format, int32_t a1_tile_format,
+                                                int32_t a2format, int32_t a2_tile_format, int a1pos_rank,
+                                                void *a1pos_desc, int a1crd_rank, void *a1crd_desc,
+                                                int a1tile_pos_rank, void *a1tile_pos_desc, int a1tile_crd_rank,
+                                                void *a1tile_crd_desc, int a2pos_rank, void *a2pos_desc,
+                                                int a2crd_rank, void *a2crd_desc, int a2tile_pos_rank,
+                                                void *a2tile_pos_desc, int a2tile_crd_rank, void *a2tile_crd_desc,
+                                                int aval_rank, void *aval_desc, int32_t read_mode)
+{
+    const char *who = "comet_hip_read_input_2D_f64_i64";
+    (void)a1pos_rank; (void)a1crd_rank; (void)a1tile_pos_rank; (void)a1tile_crd_rank; (void)a2pos_rank;
+    (void)a2crd_rank; (void)a2tile_pos_rank; (void)a2tile_crd_rank; (void)aval_rank;
+    int64_t *a1pos = memref_data<int64_t>(a1pos_desc), *a1crd = memref_data<int64_t>(a1crd_desc);
+    int64_t *a2pos = memref_data<int64_t>(a2pos_desc), *a2crd = memref_data<int64_t>(a2crd_desc);
+    double *aval = memref_data<double>(aval_desc);
+    const Layout lay = layout_of(a1format, a1_tile_format, a2format, a2_tile_format);
+    if (lay == LAYOUT_OTHER || !a1pos || !a1crd || !a2pos || !a2crd || !aval) {
+        set_error(COMET_HIP_ERR_ARG, "only CSR, COO and DCSR layouts are read (formats %d,%d), all arrays required",
+                  a1format, a2format);
+        die_reader(who);
+    }
+    if (ensure_init() != COMET_HIP_OK)
+        die_reader(who);
+    // arrays a layout does not use hold -1 in their first element (SparseUtils.cpp:1840-1848)
+    void *all[8] = {a1pos_desc, a1crd_desc, a2pos_desc, a2crd_desc,
+                    a1tile_pos_desc, a1tile_crd_desc, a2tile_pos_desc, a2tile_crd_desc};
+    for (void *d : all) {
+        int64_t *p = memref_data<int64_t>(d);
+        if (p && ((comet_memref_1d *)d)->sizes[0] > 0)
+            p[0] = -1;
+    }
+    const int64_t h = pending_read(file_id, read_mode, true);
+    if (!h)
+        die_reader(who);
+    int64_t nrows = 0, nnz = 0;
+    (void)comet_hip_csr_dims(h, &nrows, nullptr, &nnz);
+    int rc = COMET_HIP_OK;
+    if (lay == LAYOUT_CSR) {            // :1898-1936
+        a1pos[0] = nrows;
+        rc = comet_hip_csr_download_i64(h, a2pos, a2crd, aval);
+    } else if (lay == LAYOUT_COO) {     // :1855-1896
+        a1pos[0] = 0;
+        a1pos[1] = nnz;
+        rc = comet_hip_csr_to_coo_i64(h, a1crd, a2crd, aval);
+    } else {                            // DCSR :1983-2010
+        int64_t stored = 0;
+        rc = comet_hip_csr_to_dcsr_i64(h, &stored, a1crd, a2pos, a2crd, aval);
+        a1pos[0] = 0;
+        a1pos[1] = stored;
+    }
+    (void)comet_hip_csr_destroy(h);
+    if (rc)
+        die_reader(who);
+}

@@ -80,6 +80,16 @@ SIGNATURES = {
     "comet_hip_spgemm_csr": (_i64, [_i64, _i64, _i64]),
     "comet_hip_spgemm_csr_numeric_semiring": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int]),
     "comet_hip_spgemm_csr_semiring": (_i64, [_i64, _i64, _i64, _int, _int]),
+    "comet_hip_mtx_read_csr": (_i64, [C.c_char_p, _int]),
+    "comet_hip_read_input_sizes_2D_f64": (None, [_i32, _i32, _i32, _i32, _i32, _int, _vp, _i32]),
+    "comet_hip_read_input_2D_f64_i64": (None, [_i32, _i32, _i32, _i32, _i32] + [_int, _vp] * 9 + [_i32]),
+    "comet_hip_read_input_2D_handle": (_i64, [_i32, _i32]),
+    "comet_hip_csr_from_coo_i64": (_i64, [_i64, _i64, _i64, _vp, _vp, _vp, _int]),
+    "comet_hip_csr_from_coo_device": (_i64, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
+    "comet_hip_csr_from_dcsr_i64": (_i64, [_i64, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "comet_hip_csr_to_coo_i64": (_int, [_i64, _vp, _vp, _vp]),
+    "comet_hip_csr_to_dcsr_i64": (_int, [_i64, _pi64, _vp, _vp, _vp, _vp]),
+    "comet_hip_csr_transpose": (_i64, [_i64]),
     "comet_hip_spgemm_masked_sum": (_int, [_i64, _i64, _i64, C.POINTER(_f64)]),
     "comet_hip_reduce_sum_f64": (_int, [_i64, _i64, C.POINTER(_f64)]),
     "comet_hip_eltwise_mult_csr": (_i64, [_i64, _i64]),
@@ -226,6 +236,75 @@ class CsrMatrix:
         m = m.tocsr()
         m.sort_indices()
         return cls.from_arrays(m.shape, m.indptr.astype(np.int64), m.indices.astype(np.int64), m.data)
+
+    @classmethod
+    def from_mtx(cls, path, read_mode=1):
+        """MatrixMarket file -> device CSR; read_mode as in comet_read(id, mode): 1 all, 2 strictly lower,
+        3 lower, 4 strictly upper, 5 upper."""
+        return cls(_handle(lib().comet_hip_mtx_read_csr(os.fsencode(path), int(read_mode)), "comet_hip_mtx_read_csr"))
+
+    @classmethod
+    def from_file_id(cls, file_id, read_mode=1):
+        """comet_read(file_id, read_mode): the file named by SPARSE_FILE_NAME<file_id>."""
+        return cls(_handle(lib().comet_hip_read_input_2D_handle(int(file_id), int(read_mode)),
+                           "comet_hip_read_input_2D_handle"))
+
+    @classmethod
+    def from_coo(cls, shape, row, col, val, read_mode=1):
+        """Tuples in any order (ordered on the GPU by (row, col), ties in input order)."""
+        row = np.ascontiguousarray(row, dtype=np.int64)
+        col = np.ascontiguousarray(col, dtype=np.int64)
+        val = np.ascontiguousarray(val, dtype=np.float64)
+        if not (len(row) == len(col) == len(val)):
+            raise ValueError("row, col and val must have one entry per tuple")
+        h = lib().comet_hip_csr_from_coo_i64(int(shape[0]), int(shape[1]), len(val), _vptr(row), _vptr(col),
+                                             _vptr(val), int(read_mode))
+        return cls(_handle(h, "comet_hip_csr_from_coo_i64"))
+
+    @classmethod
+    def from_coo_device(cls, shape, row, col, val, read_mode=1):
+        """row, col: int32 DeviceArrays; val: float64 DeviceArray."""
+        if row.dtype != np.int32 or col.dtype != np.int32 or val.dtype != np.float64:
+            raise ValueError("device tuples must be int32 / int32 / float64")
+        h = lib().comet_hip_csr_from_coo_device(int(shape[0]), int(shape[1]), val.size, row.ptr, col.ptr, val.ptr,
+                                                int(read_mode))
+        return cls(_handle(h, "comet_hip_csr_from_coo_device"))
+
+    @classmethod
+    def from_dcsr(cls, shape, a1crd, a2pos, a2crd, aval):
+        """The reference's DCSR arrays: ids of the rows that store anything, then CSR over those rows."""
+        a1crd = np.ascontiguousarray(a1crd, dtype=np.int64)
+        a2pos = np.ascontiguousarray(a2pos, dtype=np.int64)
+        a2crd = np.ascontiguousarray(a2crd, dtype=np.int64)
+        aval = np.ascontiguousarray(aval, dtype=np.float64)
+        if len(a2pos) != len(a1crd) + 1:
+            raise ValueError("a2pos must hold one more entry than a1crd")
+        h = lib().comet_hip_csr_from_dcsr_i64(int(shape[0]), int(shape[1]), len(a1crd), _vptr(a1crd), _vptr(a2pos),
+                                              _vptr(a2crd), _vptr(aval))
+        return cls(_handle(h, "comet_hip_csr_from_dcsr_i64"))
+
+    def to_coo(self):
+        nnz = self.nnz
+        row, col, val = np.zeros(nnz, dtype=np.int64), np.zeros(nnz, dtype=np.int64), np.zeros(nnz)
+        _check(lib().comet_hip_csr_to_coo_i64(self.handle, _vptr(row), _vptr(col), _vptr(val)),
+               "comet_hip_csr_to_coo_i64")
+        return row, col, val
+
+    def to_dcsr(self):
+        """(a1pos, a1crd, a2pos, a2crd, aval) as the reference's reader lays DCSR out."""
+        stored = C.c_int64()
+        _check(lib().comet_hip_csr_to_dcsr_i64(self.handle, C.byref(stored), None, None, None, None),
+               "comet_hip_csr_to_dcsr_i64")
+        nnz = self.nnz
+        a1crd = np.zeros(stored.value, dtype=np.int64)
+        a2pos = np.zeros(stored.value + 1, dtype=np.int64)
+        a2crd, aval = np.zeros(nnz, dtype=np.int64), np.zeros(nnz)
+        _check(lib().comet_hip_csr_to_dcsr_i64(self.handle, C.byref(stored), _vptr(a1crd), _vptr(a2pos),
+                                               _vptr(a2crd), _vptr(aval)), "comet_hip_csr_to_dcsr_i64")
+        return np.array([0, stored.value], dtype=np.int64), a1crd, a2pos, a2crd, aval
+
+    def transpose(self):
+        return CsrMatrix(_handle(lib().comet_hip_csr_transpose(self.handle), "comet_hip_csr_transpose"))
 
     def dims(self):
         r, c, n = C.c_int64(), C.c_int64(), C.c_int64()

@@ -149,6 +149,75 @@ int comet_hip_spgemm_csr_numeric_semiring(int64_t a, int64_t b, int64_t mask, in
                                           int reduce_op, int mult_op);
 int64_t comet_hip_spgemm_csr_semiring(int64_t a, int64_t b, int64_t mask, int reduce_op, int mult_op);
 
+/* ---- input side: MatrixMarket files, read modes, the file-id protocol ---------
+ * Read modes of comet_read(id, mode): lib/ExecutionEngine/SparseUtils.cpp:40-64.
+ * Storage format codes per dimension: include/comet/ExecutionEngine/
+ * RunnerUtils.h:71-77. */
+enum { COMET_READ_DEFAULT = 1, COMET_READ_LOWER_TRI_STRICT = 2, COMET_READ_LOWER_TRI = 3,
+       COMET_READ_UPPER_TRI_STRICT = 4, COMET_READ_UPPER_TRI = 5 };
+enum { COMET_FMT_DENSE = 0, COMET_FMT_COMPRESSED_UNIQUE = 1, COMET_FMT_COMPRESSED_NONUNIQUE = 2,
+       COMET_FMT_SINGLETON = 3 };
+/* Parse a MatrixMarket file (coordinate or array; general, symmetric or skew;
+ * a missing value reads as 1.0) on the host, then order, filter by read mode
+ * and build CSR on the GPU: CooMatrix::InitMarket + CsrMatrix::Init,
+ * SparseUtils.cpp:145-356,404-533.  Duplicates are kept in file order.
+ * Returns a CSR handle (0 on failure). */
+int64_t comet_hip_mtx_read_csr(const char *path, int read_mode);
+/* The reader's two calls, SparseUtils.cpp:1632-1810 (read_input_sizes_2D_f64)
+ * and :1814-2050 (read_input_2D_f64_i64), with their argument lists: file_id
+ * 0..9998 names the environment variable SPARSE_FILE_NAME<id>, 9999
+ * SPARSE_FILE_NAME (:1444-1466); every (rank, descriptor) pair is an unranked
+ * memref whose descriptor is a rank-1 strided memref of int64 (float64 for
+ * Aval).  Layouts read: CSR (Dense, Compressed_unique), COO
+ * (Compressed_nonunique, singleton), DCSR (Compressed_unique,
+ * Compressed_unique); any other prints a message and exits, like every failure
+ * of these two calls in the reference.  sizes[0..10] as in the reference;
+ * arrays a layout does not use get -1 in their first element.  The sizes call
+ * builds the device CSR and keeps it for the read call that follows. */
+void comet_hip_read_input_sizes_2D_f64(int32_t file_id, int32_t a1format, int32_t a1_tile_format,
+                                       int32_t a2format, int32_t a2_tile_format,
+                                       int sizes_rank, void *sizes_desc, int32_t read_mode);
+void comet_hip_read_input_2D_f64_i64(int32_t file_id, int32_t a1format, int32_t a1_tile_format,
+                                     int32_t a2format, int32_t a2_tile_format,
+                                     int a1pos_rank, void *a1pos_desc, int a1crd_rank, void *a1crd_desc,
+                                     int a1tile_pos_rank, void *a1tile_pos_desc,
+                                     int a1tile_crd_rank, void *a1tile_crd_desc,
+                                     int a2pos_rank, void *a2pos_desc, int a2crd_rank, void *a2crd_desc,
+                                     int a2tile_pos_rank, void *a2tile_pos_desc,
+                                     int a2tile_crd_rank, void *a2tile_crd_desc,
+                                     int aval_rank, void *aval_desc, int32_t read_mode);
+/* The same read for lowered code that keeps tensors on the device: the CSR
+ * handle itself (0 on failure), no host arrays.  Consumes what a preceding
+ * sizes call for the same id and mode built, or reads the file now. */
+int64_t comet_hip_read_input_2D_handle(int32_t file_id, int32_t read_mode);
+
+/* ---- the other matrix layouts of the reference's SpMV/SpMM tests ------------
+ * COO = {Compressed_nonunique, singleton}: A1pos = [0, nnz], A1crd = rows,
+ * A2crd = columns (SparseUtils.cpp:1855-1896); DCSR = {Compressed_unique,
+ * Compressed_unique}: A1pos = [0, stored rows], A1crd = ids of the rows that
+ * store anything, A2pos/A2crd/Aval as in CSR over those rows (:669-735).
+ * test/integration/ops/mult_spm{v,m}_{COO,DCSR}xDense.ta run on the CSR
+ * kernels after one of these conversions.  Tuples may come in any order
+ * (ordered on the GPU, ties keep input order); read_mode filters as above. */
+int64_t comet_hip_csr_from_coo_i64(int64_t nrows, int64_t ncols, int64_t nnz, const int64_t *row,
+                                   const int64_t *col, const double *val, int read_mode);
+/* The same for tuples that already sit in HBM: int32 rows and columns, float64
+ * values; indices must lie inside the matrix (not checked). */
+int64_t comet_hip_csr_from_coo_device(int64_t nrows, int64_t ncols, int64_t nnz, int64_t row_dptr,
+                                      int64_t col_dptr, int64_t val_dptr, int read_mode);
+int64_t comet_hip_csr_from_dcsr_i64(int64_t nrows, int64_t ncols, int64_t nrows_stored,
+                                    const int64_t *a1crd, const int64_t *a2pos,
+                                    const int64_t *a2crd, const double *aval);
+/* Host arrays of nnz entries each. */
+int comet_hip_csr_to_coo_i64(int64_t csr, int64_t *row, int64_t *col, double *val);
+/* *nrows_stored is always written; with all four arrays null this is the size
+ * query (a1crd: stored, a2pos: stored + 1, a2crd/aval: nnz). */
+int comet_hip_csr_to_dcsr_i64(int64_t csr, int64_t *nrows_stored, int64_t *a1crd, int64_t *a2pos,
+                              int64_t *a2crd, double *aval);
+/* New handle holding the transpose, columns ascending per row (the CSR -> CSC
+ * reordering of lib/ExecutionEngine/TransposeUtils.cpp done as one device sort). */
+int64_t comet_hip_csr_transpose(int64_t csr);
+
 /* ---- masked SpGEMM + SUM in one pass (triangle counting) -------------------
  * *out = SUM(C) for C<L> = L * L, the two statements of
  * test/integration/kernels/triangleCount_SandiaLL_wMasking.ta:18-39, i.e. the

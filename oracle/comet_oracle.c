@@ -419,7 +419,8 @@ double oracle_tricount_masked(idx_t nrows, idx_t ncols, const idx_t *pos,
 /* lib/ExecutionEngine/SparseUtils.cpp:40-64 (modes: 1 default, 2 strictly     */
 /* lower, 3 lower, 4 strictly upper, 5 upper), :145-356 (parse: 1-based        */
 /* indices, missing value = 1.0, "symmetric" mirrors off-diagonal entries,     */
-/* "skew" negates the mirrored value), :404-533 (stable sort by (row,col),     */
+/* "skew" negates the mirrored value, "array" files list every value column    */
+/* by column), :404-533 (stable sort by (row,col),                             */
 /* duplicates kept, filter by mode, row offsets).                              */
 /* Two-call protocol like read_input_sizes_2D / read_input_2D: call with       */
 /* pos == NULL to get sizes (out_dims[0..2] = rows, cols, nnz after filter),   */
@@ -446,13 +447,47 @@ static int keep_entry(int mode, idx_t r, idx_t c)
     }
 }
 
+/* Order tuples by (row, col) keeping input order among equals, drop what the   */
+/* read mode excludes, lay out CSR (CsrMatrix::Init, SparseUtils.cpp:404-533).  */
+/* pos/crd/val may be NULL to count only.  Returns the number of kept entries.  */
+static idx_t coo_sort_filter(coo_t *coo, idx_t n, idx_t nrows, int mode,
+                             idx_t *pos, idx_t *crd, double *val)
+{
+    qsort(coo, (size_t)n, sizeof(coo_t), cmp_coo);
+    idx_t kept = 0;
+    for (idx_t e = 0; e < n; ++e)
+        kept += keep_entry(mode, coo[e].r, coo[e].c);
+    if (pos) {
+        idx_t w = 0, prev = -1;
+        for (idx_t e = 0; e < n; ++e) {
+            if (!keep_entry(mode, coo[e].r, coo[e].c)) continue;
+            for (idx_t r = prev + 1; r <= coo[e].r; ++r) pos[r] = w;
+            prev = coo[e].r;
+            crd[w] = coo[e].c; val[w] = coo[e].v; ++w;
+        }
+        for (idx_t r = prev + 1; r <= nrows; ++r) pos[r] = kept;
+    }
+    return kept;
+}
+
+/* The same from tuple arrays (the COO -> CSR step without the file).            */
+idx_t oracle_coo_to_csr(idx_t nrows, idx_t n, const idx_t *row, const idx_t *col, const double *v,
+                        int mode, idx_t *pos, idx_t *crd, double *val)
+{
+    coo_t *coo = (coo_t *)malloc(sizeof(coo_t) * (size_t)(n > 0 ? n : 1));
+    for (idx_t e = 0; e < n; ++e) { coo[e].r = row[e]; coo[e].c = col[e]; coo[e].v = v[e]; coo[e].seq = e; }
+    idx_t kept = coo_sort_filter(coo, n, nrows, mode, pos, crd, val);
+    free(coo);
+    return kept;
+}
+
 int oracle_read_mtx_csr(const char *path, int mode, idx_t *out_dims,
                         idx_t *pos, idx_t *crd, double *val)
 {
     FILE *f = fopen(path, "r");
     if (!f) return 1;
     char line[1024];
-    int symmetric = 0, skew = 0, have_header = 0;
+    int symmetric = 0, skew = 0, array = 0, have_header = 0;
     idx_t nrows = 0, ncols = 0, nnz_decl = 0, n = 0;
     coo_t *coo = NULL;
     while (fgets(line, sizeof line, f)) {
@@ -460,18 +495,28 @@ int oracle_read_mtx_csr(const char *path, int mode, idx_t *out_dims,
             if (line[1] == '%') {
                 symmetric = strstr(line, "symmetric") != NULL;
                 skew = strstr(line, "skew") != NULL;
+                array = strstr(line, "array") != NULL;
             }
             continue;
         }
         if (!have_header) {
-            long long a, b, c;
-            if (sscanf(line, "%lld %lld %lld", &a, &b, &c) != 3) { fclose(f); return 2; }
-            nrows = a; ncols = b; nnz_decl = symmetric ? 2 * c : c;
+            long long a, b, c = 0;
+            int got = sscanf(line, "%lld %lld %lld", &a, &b, &c);
+            if (got < 2) continue; /* blank line */
+            if (got != (array ? 2 : 3)) { fclose(f); return 2; }
+            nrows = a; ncols = b; nnz_decl = array ? a * b : (symmetric ? 2 * c : c);
             coo = (coo_t *)malloc(sizeof(coo_t) * (size_t)(nnz_decl > 0 ? nnz_decl : 1));
             have_header = 1;
             continue;
         }
         char *l = line, *t = NULL;
+        if (array) { /* all rows*cols values, column by column (:253-283) */
+            double v = strtod(l, &t);
+            if (t == l) continue;
+            if (n >= nnz_decl) { free(coo); fclose(f); return 4; }
+            coo[n].c = n / nrows; coo[n].r = n - nrows * coo[n].c; coo[n].v = v; coo[n].seq = n; ++n;
+            continue;
+        }
         long r = strtol(l, &t, 0);
         if (t == l) continue; /* blank line */
         l = t;
@@ -488,21 +533,8 @@ int oracle_read_mtx_csr(const char *path, int mode, idx_t *out_dims,
     }
     fclose(f);
     if (!have_header) return 2;
-    qsort(coo, (size_t)n, sizeof(coo_t), cmp_coo);
-    idx_t kept = 0;
-    for (idx_t e = 0; e < n; ++e)
-        kept += keep_entry(mode, coo[e].r, coo[e].c);
+    idx_t kept = coo_sort_filter(coo, n, nrows, mode, pos, crd, val);
     out_dims[0] = nrows; out_dims[1] = ncols; out_dims[2] = kept;
-    if (pos) {
-        idx_t w = 0, prev = -1;
-        for (idx_t e = 0; e < n; ++e) {
-            if (!keep_entry(mode, coo[e].r, coo[e].c)) continue;
-            for (idx_t r = prev + 1; r <= coo[e].r; ++r) pos[r] = w;
-            prev = coo[e].r;
-            crd[w] = coo[e].c; val[w] = coo[e].v; ++w;
-        }
-        for (idx_t r = prev + 1; r <= nrows; ++r) pos[r] = kept;
-    }
     free(coo);
     return 0;
 }

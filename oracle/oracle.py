@@ -67,6 +67,8 @@ def lib():
     L.oracle_eltwise_mult_csr.restype = C.c_int64
     L.oracle_tricount_masked.argtypes = [C.c_int64, C.c_int64, i64p, i64p, f64p]
     L.oracle_tricount_masked.restype = C.c_double
+    L.oracle_coo_to_csr.argtypes = [C.c_int64, C.c_int64, i64p, i64p, f64p, C.c_int, vp, vp, vp]
+    L.oracle_coo_to_csr.restype = C.c_int64
     L.oracle_read_mtx_csr.argtypes = [C.c_char_p, C.c_int, i64p, vp, vp, vp]
     L.oracle_read_mtx_csr.restype = C.c_int
     L.oracle_format_f64.argtypes = [f64p, C.c_int64, C.c_char_p, C.c_int64]
@@ -180,6 +182,40 @@ def tricount_masked(pos, crd, val, ncols=None):
     pos, crd, val = _i64(pos), _i64(crd), _f64(val)
     n = len(pos) - 1
     return float(lib().oracle_tricount_masked(n, n if ncols is None else ncols, pos, crd, val))
+
+
+def coo_layout(pos, crd, val):
+    """The reader's COO arrays for a matrix given as CSR of the kept tuples: A1pos = [0, nnz], A1crd = row
+    of every tuple, A2pos unused (-1), A2crd = columns (lib/ExecutionEngine/SparseUtils.cpp:1855-1896; the
+    tuples are the same stable (row, col) order the CSR arrays hold)."""
+    pos = _i64(pos)
+    rows = np.repeat(np.arange(len(pos) - 1, dtype=np.int64), np.diff(pos))
+    return np.array([0, len(rows)], dtype=np.int64), rows, np.array([-1], dtype=np.int64), _i64(crd), _f64(val)
+
+
+def dcsr_layout(pos, crd, val):
+    """The reader's DCSR arrays (DcsrMatrix::Init, lib/ExecutionEngine/SparseUtils.cpp:686-735): one A1crd
+    entry and one A2pos entry per row that stores anything, a closing A2pos entry, A1pos = [0, stored rows]."""
+    pos = _i64(pos)
+    a1crd, a2pos = [], []
+    for r in range(len(pos) - 1):          # walk the ordered tuples row by row, as the reference does
+        if pos[r + 1] != pos[r]:
+            a1crd.append(r)
+            a2pos.append(int(pos[r]))
+    a2pos.append(int(pos[-1]))
+    return (np.array([0, len(a1crd)], dtype=np.int64), np.array(a1crd, dtype=np.int64),
+            np.array(a2pos, dtype=np.int64), _i64(crd), _f64(val))
+
+
+def coo_to_csr(nrows, row, col, val, mode=1):
+    """Tuples in any order -> (pos, crd, val) the way the reader orders and filters them."""
+    row, col, val = _i64(row), _i64(col), _f64(val)
+    n = len(row)
+    pos = np.zeros(nrows + 1, dtype=np.int64)
+    crd = np.zeros(max(n, 1), dtype=np.int64)
+    out = np.zeros(max(n, 1))
+    kept = lib().oracle_coo_to_csr(nrows, n, row, col, val, mode, _ptr(pos), _ptr(crd), _ptr(out))
+    return pos, crd[:kept], out[:kept]
 
 
 def read_mtx_csr(path, mode=1):

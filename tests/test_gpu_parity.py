@@ -5,6 +5,7 @@ Bars: row pointers, column indices and triangle counts bit-exact; fp64 values wi
 1e-12 relative.  Where a value is a sum of signed products the tolerance is taken
 relative to sum(|a||b|) of that entry (the bound summation-order changes obey):
 |got - want| <= 1e-12 * sum|a*b|."""
+import ctypes as C
 import os
 
 import numpy as np
@@ -532,3 +533,187 @@ def test_mlir_ciface_entry_points(golden, golden_dir):
     assert cp.tolist() == g["pos"] and cc.tolist() == g["crd"] and orc.format_f64(cv) == g["printed_val"]
     (tr, tc), tpos, tcrd, tval = _mtx(golden_dir, "tc.mtx", 2)
     assert L._mlir_ciface_comet_hip_tricount_f64_i64(tc, rt.memref1d(tpos), rt.memref1d(tcrd), rt.memref1d(tval)) == 5.0
+
+
+# ----------------------------------------------------------------- input side and other layouts
+def test_mtx_reader_goldens(golden, golden_dir):
+    for g in golden["read_csr"]:
+        A = rt.CsrMatrix.from_mtx(os.path.join(golden_dir, g["matrix"]), g["mode"])
+        p, c, v = A.to_arrays()
+        assert p.tolist() == g["pos"] and c.tolist() == g["crd"], g["source"]
+        assert orc.format_f64(v) == g["printed_val"], g["source"]
+    for g in golden["read_coo"]:
+        A = rt.CsrMatrix.from_mtx(os.path.join(golden_dir, g["matrix"]), g["mode"])
+        r, c, v = A.to_coo()
+        assert r.tolist() == g["a1crd"] and c.tolist() == g["a2crd"], g["source"]
+        assert orc.format_f64(v) == g["printed_val"], g["source"]
+
+
+def _desc(a):
+    """(descriptor struct, void pointer to it); the struct must stay alive while the pointer is used"""
+    m = rt.memref1d(a)
+    return m, C.cast(C.pointer(m), C.c_void_p)
+
+
+def _memref_i64(n):
+    a = np.full(max(n, 1), 7, dtype=np.int64)
+    return (a,) + _desc(a)
+
+
+@pytest.mark.parametrize("layout", ["CSR", "COO", "DCSR"])
+def test_reader_file_id_protocol(golden, golden_dir, monkeypatch, layout):
+    """The two reader calls with the reference's argument lists, for the three layouts its matrix tests use."""
+    L = rt.lib()
+    monkeypatch.setenv("SPARSE_FILE_NAME3", os.path.join(golden_dir, "test_rank2.mtx"))
+    fmt = {"CSR": (0, 0, 1, 0), "COO": (2, 0, 3, 0), "DCSR": (1, 0, 1, 0)}[layout]
+    for mode in (1, 3):
+        (nr, nc), pos, crd, val = _mtx(golden_dir, "test_rank2.mtx", mode)
+        sizes = np.zeros(13, dtype=np.int64)
+        sizes_m, sizes_p = _desc(sizes)
+        L.comet_hip_read_input_sizes_2D_f64(3, *fmt, 1, sizes_p, mode)
+        want = {"CSR": (None, pos[:0], pos, crd, val), "COO": orc.coo_layout(pos, crd, val),
+                "DCSR": orc.dcsr_layout(pos, crd, val)}[layout]
+        if layout == "CSR":
+            assert sizes[:11].tolist() == [1, 1, 0, 0, nr + 1, len(crd), 0, 0, len(crd), nr, nc]
+        elif layout == "COO":
+            assert sizes[:11].tolist() == [2, len(crd), 0, 0, 1, len(crd), 0, 0, len(crd), nr, nc]
+        else:
+            stored = len(want[1])
+            assert sizes[:11].tolist() == [2, stored, 0, 0, stored + 1, len(crd), 0, 0, len(crd), nr, nc]
+        arrs = [_memref_i64(int(sizes[i])) for i in range(8)]
+        aval = np.zeros(max(int(sizes[8]), 1))
+        args = []
+        for i in (0, 1, 2, 3, 4, 5, 6, 7):
+            args += [1, arrs[i][2]]
+        aval_m, aval_p = _desc(aval)
+        L.comet_hip_read_input_2D_f64_i64(3, *fmt, *args, 1, aval_p, mode)
+        a1pos, a1crd, a2pos, a2crd = (arrs[i][0] for i in (0, 1, 4, 5))
+        assert arrs[2][0][0] == -1 and arrs[3][0][0] == -1 and arrs[6][0][0] == -1 and arrs[7][0][0] == -1
+        assert np.array_equal(aval[:len(val)], val)
+        if layout == "CSR":
+            assert a1pos[0] == nr and a1crd[0] == -1
+            assert np.array_equal(a2pos, pos) and np.array_equal(a2crd[:len(crd)], crd)
+        elif layout == "COO":
+            assert a1pos.tolist() == [0, len(crd)] and a2pos[0] == -1
+            assert np.array_equal(a1crd[:len(crd)], want[1]) and np.array_equal(a2crd[:len(crd)], crd)
+        else:
+            assert a1pos.tolist() == want[0].tolist()
+            assert np.array_equal(a1crd, want[1]) and np.array_equal(a2pos, want[2])
+            assert np.array_equal(a2crd[:len(crd)], crd)
+    # the device-handle form of the same read, and its failure without the variable
+    A = rt.CsrMatrix.from_file_id(3, 5)
+    (nr, nc), pos, crd, val = _mtx(golden_dir, "test_rank2.mtx", 5)
+    p, c, v = A.to_arrays()
+    assert np.array_equal(p, pos) and np.array_equal(c, crd) and np.array_equal(v, val)
+    monkeypatch.delenv("SPARSE_FILE_NAME4", raising=False)
+    assert L.comet_hip_read_input_2D_handle(4, 1) == 0
+    assert b"SPARSE_FILE_NAME4" in L.comet_hip_last_error()
+
+
+def _write_mtx(path, header, size_line, lines):
+    with open(path, "w") as f:
+        f.write(header + "\n% a comment\n" + size_line + "\n" + "\n".join(lines) + "\n")
+
+
+@pytest.mark.parametrize("flavour", ["general", "symmetric", "skew-symmetric", "pattern", "array", "duplicates"])
+@pytest.mark.parametrize("mode", [1, 2, 3, 4, 5])
+def test_mtx_reader_flavours_vs_checker(tmp_path, flavour, mode):
+    rng = np.random.default_rng(len(flavour) * 7 + mode)
+    n, m = 61, 61
+    path = str(tmp_path / "m.mtx")
+    if flavour == "array":
+        m = 17
+        D = rng.uniform(-1, 1, (n, m))
+        _write_mtx(path, "%%MatrixMarket matrix array real general", f"{n} {m}", [repr(float(v)) for v in D.T.ravel()])
+    else:
+        ent = [(i, j) for i in range(n) for j in range(m) if rng.random() < 0.1]
+        if flavour in ("symmetric", "skew-symmetric"):
+            ent = [(i, j) for i, j in ent if (i >= j if flavour == "symmetric" else i > j)]
+        if flavour == "duplicates":
+            ent = ent + ent[::3] + ent[::5]
+        rng.shuffle(ent)
+        vals = rng.uniform(-1, 1, len(ent))
+        if flavour == "pattern":
+            lines = [f"{i + 1} {j + 1}" for i, j in ent]
+        else:
+            lines = [f"{i + 1} {j + 1} {float(v)!r}" for (i, j), v in zip(ent, vals)]
+        lines.insert(len(lines) // 2, "")          # a blank line in the middle is skipped
+        kind = {"pattern": "pattern general", "duplicates": "real general"}.get(flavour, "real " + flavour)
+        _write_mtx(path, "%%MatrixMarket matrix coordinate " + kind, f"{n} {m} {len(ent)}", lines)
+    (nr, nc), pos, crd, val = orc.read_mtx_csr(path, mode)
+    A = rt.CsrMatrix.from_mtx(path, mode)
+    assert A.shape == (nr, nc)
+    p, c, v = A.to_arrays()
+    assert np.array_equal(p, pos) and np.array_equal(c, crd) and np.array_equal(v, val)
+
+
+def test_coo_dcsr_transpose_conversions():
+    rng = np.random.default_rng(21)
+    n, m, nnz = 3000, 1777, 200_000
+    row = rng.integers(0, n, nnz)
+    row[row % 7 == 3] = 5                    # many duplicates of one row, and rows that stay empty
+    col = rng.integers(0, m, nnz)
+    val = rng.uniform(-1, 1, nnz)
+    order = np.lexsort((col, row))           # stable: ties keep input order
+    srow, scol, sval = row[order], col[order], val[order]
+    pos = np.zeros(n + 1, dtype=np.int64)
+    np.cumsum(np.bincount(srow, minlength=n), out=pos[1:])
+    A = rt.CsrMatrix.from_coo((n, m), row, col, val)
+    p, c, v = A.to_arrays()
+    assert np.array_equal(p, pos) and np.array_equal(c, scol) and np.array_equal(v, sval)
+    r2, c2, v2 = A.to_coo()
+    assert np.array_equal(r2, srow) and np.array_equal(c2, scol) and np.array_equal(v2, sval)
+    # read modes filter the ordered tuples
+    keep = srow >= scol
+    L3 = rt.CsrMatrix.from_coo((n, m), row, col, val, read_mode=3)
+    r3, c3, v3 = L3.to_coo()
+    assert np.array_equal(r3, srow[keep]) and np.array_equal(c3, scol[keep]) and np.array_equal(v3, sval[keep])
+    # DCSR out and back
+    a1pos, a1crd, a2pos, a2crd, aval = A.to_dcsr()
+    w = orc.dcsr_layout(pos, scol, sval)
+    for got, want in zip((a1pos, a1crd, a2pos, a2crd, aval), w):
+        assert np.array_equal(got, want)
+    Bm = rt.CsrMatrix.from_dcsr((n, m), a1crd, a2pos, a2crd, aval)
+    for got, want in zip(Bm.to_arrays(), (pos, scol, sval)):
+        assert np.array_equal(got, want)
+    # transpose: ordered by (column, row), ties in the order of the source; twice gives the source back
+    T = A.transpose()
+    assert T.shape == (m, n)
+    torder = np.lexsort((srow, scol))
+    tp, tc, tv = T.to_arrays()
+    tpos = np.zeros(m + 1, dtype=np.int64)
+    np.cumsum(np.bincount(scol, minlength=m), out=tpos[1:])
+    assert np.array_equal(tp, tpos) and np.array_equal(tc, srow[torder]) and np.array_equal(tv, sval[torder])
+    for got, want in zip(T.transpose().to_arrays(), (pos, scol, sval)):
+        assert np.array_equal(got, want)
+    # empty matrix
+    E = rt.CsrMatrix.from_coo((4, 5), [], [], [])
+    assert E.to_arrays()[0].tolist() == [0, 0, 0, 0, 0] and E.transpose().shape == (5, 4)
+    assert E.to_dcsr()[0].tolist() == [0, 0]
+
+
+def test_spmv_spmm_other_layouts_golden(golden, golden_dir):
+    """mult_spmv/spmm_{COO,DCSR}xDense: the file read into the layout's arrays, handed back, same kernels."""
+    path = os.path.join(golden_dir, "test_rank2.mtx")
+    A = rt.CsrMatrix.from_mtx(path)
+    nr, nc = A.shape
+    r, c, v = A.to_coo()
+    a1pos, a1crd, a2pos, a2crd, aval = A.to_dcsr()
+    for M in (rt.CsrMatrix.from_coo((nr, nc), r, c, v), rt.CsrMatrix.from_dcsr((nr, nc), a1crd, a2pos, a2crd, aval)):
+        y = rt.spmv(M, rt.DeviceArray.from_numpy(np.full(nc, 1.7)), rt.DeviceArray(nr, zero=True))
+        assert orc.format_f64(y.to_numpy()) == golden["spmv_other_layouts"]["printed"]
+        Cm = rt.spmm(M, rt.DeviceArray.from_numpy(np.full((nc, 4), 1.7)), rt.DeviceArray((nr, 4), zero=True))
+        assert orc.format_f64(Cm.to_numpy()) == golden["spmm_other_layouts"]["printed"]
+
+
+def test_reader_rejects_bad_input(tmp_path):
+    L = rt.lib()
+    assert L.comet_hip_mtx_read_csr(str(tmp_path / "missing.mtx").encode(), 1) == 0
+    assert b"cannot open" in L.comet_hip_last_error()
+    bad = tmp_path / "bad.mtx"
+    bad.write_text("%%MatrixMarket matrix coordinate real general\n3 3 1\n4 1 2.0\n")
+    assert L.comet_hip_mtx_read_csr(str(bad).encode(), 1) == 0 and b"outside" in L.comet_hip_last_error()
+    assert L.comet_hip_mtx_read_csr(str(bad).encode(), 9) == 0 and b"read mode" in L.comet_hip_last_error()
+    row = np.array([0, 5], dtype=np.int64)
+    h = L.comet_hip_csr_from_coo_i64(3, 3, 2, row.ctypes.data, row.ctypes.data, np.zeros(2).ctypes.data, 1)
+    assert h == 0 and b"outside" in L.comet_hip_last_error()

@@ -398,3 +398,69 @@ def test_ttgt_every_candidate_matches_einsum(a, b, c):
     for which in (0, ncand - 1):
         Ct, _, _ = orc.ttgt_contract(a, b, c, A, B, C0=C0, beta=1.0, which=which)
         np.testing.assert_allclose(Ct, C0 + ref, rtol=0, atol=1e-13)
+
+
+# ----------------------------------------------------------------- reader: other layouts and file flavours
+def test_read_coo_golden(golden, golden_dir):
+    for g in golden["read_coo"]:
+        _, pos, crd, val = _mtx(golden_dir, g["matrix"], g["mode"])
+        a1pos, a1crd, a2pos, a2crd, aval = orc.coo_layout(pos, crd, val)
+        assert a1pos.tolist() == g["a1pos"], g["source"]
+        assert a1crd.tolist() == g["a1crd"], g["source"]
+        assert a2pos.tolist() == g["a2pos"] and a2crd.tolist() == g["a2crd"], g["source"]
+        assert orc.format_f64(aval) == g["printed_val"], g["source"]
+
+
+def test_dcsr_layout_invariants():
+    """No test of the reference prints a DCSR tensor; what fixes the layout is that expanding it gives the
+    CSR arrays back and that only rows with entries are listed, in ascending order."""
+    rng = np.random.default_rng(4)
+    A = sp.random(40, 30, density=0.05, format="csr", random_state=rng)
+    A.sort_indices()
+    a1pos, a1crd, a2pos, a2crd, aval = orc.dcsr_layout(A.indptr, A.indices, A.data)
+    lens = np.diff(A.indptr)
+    assert a1pos.tolist() == [0, int((lens > 0).sum())]
+    assert a1crd.tolist() == np.flatnonzero(lens > 0).tolist()
+    assert np.array_equal(np.diff(a2pos), lens[lens > 0]) and a2pos[0] == 0
+    assert np.array_equal(a2crd, A.indices) and np.array_equal(aval, A.data)
+
+
+def _write_mtx(path, header, size_line, lines):
+    with open(path, "w") as f:
+        f.write(header + "\n% a comment\n" + size_line + "\n" + "\n".join(lines) + "\n")
+
+
+@pytest.mark.parametrize("flavour", ["general", "symmetric", "skew-symmetric", "pattern", "array"])
+def test_reader_flavours_vs_scipy(tmp_path, flavour):
+    import scipy.io
+    rng = np.random.default_rng(len(flavour))
+    n = 9
+    path = str(tmp_path / "m.mtx")
+    if flavour == "array":
+        D = rng.uniform(-1, 1, (n, 6)).round(3)
+        _write_mtx(path, "%%MatrixMarket matrix array real general", f"{n} 6", [repr(float(v)) for v in D.T.ravel()])
+    else:
+        D = np.where(rng.random((n, n)) < 0.3, rng.uniform(-1, 1, (n, n)).round(3), 0.0)
+        if flavour == "symmetric":
+            D = np.tril(D) + np.tril(D, -1).T
+            ent = [(i, j) for i in range(n) for j in range(i + 1) if D[i, j] != 0]
+        elif flavour == "skew-symmetric":
+            D = np.tril(D, -1) - np.tril(D, -1).T
+            ent = [(i, j) for i in range(n) for j in range(i) if D[i, j] != 0]
+        else:
+            ent = [(i, j) for i in range(n) for j in range(n) if D[i, j] != 0]
+        rng.shuffle(ent)
+        if flavour == "pattern":
+            D = (D != 0).astype(float)
+            lines = [f"{i + 1} {j + 1}" for i, j in ent]
+            head = "%%MatrixMarket matrix coordinate pattern general"
+        else:
+            lines = [f"{i + 1} {j + 1} {float(D[i, j])!r}" for i, j in ent]
+            head = "%%MatrixMarket matrix coordinate real " + (flavour if flavour != "general" else "general")
+        _write_mtx(path, head, f"{n} {n} {len(ent)}", lines)
+    (nr, nc), pos, crd, val = orc.read_mtx_csr(path, 1)
+    got = sp.csr_matrix((val, crd, pos), shape=(nr, nc)).toarray()
+    assert np.array_equal(got, D)
+    assert np.array_equal(got, scipy.io.mmread(path).toarray() if flavour != "array" else scipy.io.mmread(path))
+    for r in range(nr):                        # columns ascending inside every row
+        assert np.all(np.diff(crd[pos[r]:pos[r + 1]]) > 0)
