@@ -64,11 +64,23 @@ struct Csr {
     // found without searching.
     int64_t *sg_blkptr = nullptr;
     int sg_nblk = 0;
+    // SpMM plan for long rows (heavy_state: 0 undecided, 1 not worth it, 2 in use): the long rows re-stored as
+    // per-(XCD, wavefront) lists ordered by column for spmm_heavy_sweep, and the rest of the matrix as `light`.
+    int heavy_state = 0;
+    int64_t heavy_nnz = 0;
+    int64_t *heavy_seg = nullptr;            // [8 * 512 + 1] list boundaries
+    int32_t *heavy_col = nullptr;            // column << 4 | first entry of a run << 3 | which of the wavefront's rows
+    double *heavy_val = nullptr;
+    int64_t heavy_rows = 0;
+    int32_t *heavy_row = nullptr;            // [heavy_rows] row ids of the long rows
+    int32_t *heavy_code = nullptr;           // [8][heavy_rows] wavefront * 8 + slot that holds the row on each XCD
+    Csr *light = nullptr;
 };
 
 Csr *csr_from_handle(int64_t h);           // nullptr (and error set) if unknown
 int64_t csr_register(Csr *c);              // takes ownership of the struct
 int csr_alloc(Csr *c, int64_t nrows, int64_t ncols, int64_t nnz);   // allocates pos/crd/val, owns = true
+void csr_release(Csr *c);                  // frees the arrays it owns, its plans and the struct
 
 // Records an event pair around a kernel launch when profiling is on.
 struct KernelTimer {
@@ -81,6 +93,10 @@ static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // exclusive scan of int64 counts into pos[0..n] (pos[n] = total), on the stream
 int exclusive_scan_i64(const int64_t *counts, int64_t n, int64_t *pos);
+
+// stable radix sort of n (key, payload) pairs on the stream, comparing key bits [0, end_bit)
+int sort_pairs_u64_u32(const uint64_t *keys_in, uint64_t *keys_out, const uint32_t *vals_in, uint32_t *vals_out,
+                       int64_t n, int end_bit);
 
 // deterministic tree sum of a device array, result copied to the host
 int reduce_sum_device(const double *v, int64_t n, double *out_host);

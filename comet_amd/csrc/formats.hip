@@ -271,6 +271,24 @@ struct CachedBuf {
     template <typename T> T *as() { return (T *)p; }
 };
 
+int sort_pairs_u64_u32(const uint64_t *keys_in, uint64_t *keys_out, const uint32_t *vals_in, uint32_t *vals_out,
+                       int64_t n, int end_bit)
+{
+    static Workspace tmp;
+    if (n <= 0)
+        return COMET_HIP_OK;
+    size_t tmp_bytes = 0;
+    if (rocprim::radix_sort_pairs(nullptr, tmp_bytes, keys_in, keys_out, vals_in, vals_out, (size_t)n, 0u,
+                                  (unsigned)end_bit, stream()) != hipSuccess)
+        return set_error(COMET_HIP_ERR_HIP, "sort workspace query failed");
+    COMET_CHK(tmp.ensure(tmp_bytes ? tmp_bytes : 1, false));
+    KernelTimer t("radix_sort_pairs");
+    if (rocprim::radix_sort_pairs(tmp.ptr, tmp_bytes, keys_in, keys_out, vals_in, vals_out, (size_t)n, 0u,
+                                  (unsigned)end_bit, stream()) != hipSuccess)
+        return set_error(COMET_HIP_ERR_HIP, "sorting %lld pairs failed", (long long)n);
+    return COMET_HIP_OK;
+}
+
 static inline dim3 grid_for(int64_t n) { return dim3((unsigned)(n > 0 ? ceil_div(n, 256) : 1)); }
 
 // row/col/val are device arrays of n tuples in input order; returns a new registered handle or 0
@@ -294,7 +312,7 @@ static int64_t coo_device_to_csr(int64_t nrows, int64_t ncols, int64_t n, const 
     }
     // temporaries live in grow-only buffers kept for the life of the process: a conversion of a few million
     // tuples takes less time than the allocations would
-    static CachedBuf keys_in, keys_out, idx_in, idx_out, flag, off, crow, tmp;
+    static CachedBuf keys_in, keys_out, idx_in, idx_out, flag, off, crow;
     int64_t kept = 0;
     if (n > 0) {
         if (keys_in.alloc(8 * (size_t)n) || keys_out.alloc(8 * (size_t)n) || idx_in.alloc(4 * (size_t)n) ||
@@ -308,23 +326,9 @@ static int64_t coo_device_to_csr(int64_t nrows, int64_t ncols, int64_t n, const 
         int row_bits = 1;
         while (row_bits < 31 && (1ll << row_bits) < nrows)
             ++row_bits;
-        size_t tmp_bytes = 0;
-        if (rocprim::radix_sort_pairs(nullptr, tmp_bytes, keys_in.as<uint64_t>(), keys_out.as<uint64_t>(),
-                                      idx_in.as<uint32_t>(), idx_out.as<uint32_t>(), (size_t)n, 0u,
-                                      (unsigned)(32 + row_bits), stream()) != hipSuccess ||
-            tmp.alloc(tmp_bytes)) {
-            set_error(COMET_HIP_ERR_HIP, "sort workspace query failed");
+        if (sort_pairs_u64_u32(keys_in.as<uint64_t>(), keys_out.as<uint64_t>(), idx_in.as<uint32_t>(),
+                               idx_out.as<uint32_t>(), n, 32 + row_bits) != COMET_HIP_OK)
             return fail();
-        }
-        {
-            KernelTimer t("radix_sort_pairs");
-            if (rocprim::radix_sort_pairs(tmp.p, tmp_bytes, keys_in.as<uint64_t>(), keys_out.as<uint64_t>(),
-                                          idx_in.as<uint32_t>(), idx_out.as<uint32_t>(), (size_t)n, 0u,
-                                          (unsigned)(32 + row_bits), stream()) != hipSuccess) {
-                set_error(COMET_HIP_ERR_HIP, "sorting %lld tuples failed", (long long)n);
-                return fail();
-            }
-        }
         {
             KernelTimer t("coo_flag");
             coo_flag<<<grid_for(n), dim3(256), 0, stream()>>>(n, keys_out.as<uint64_t>(), mode, flag.as<int64_t>());

@@ -127,8 +127,15 @@ int csr_alloc(Csr *c, int64_t nrows, int64_t ncols, int64_t nnz)
     return COMET_HIP_OK;
 }
 
-static void csr_release(Csr *c)
+void csr_release(Csr *c)
 {
+    if (c->light)
+        csr_release(c->light);
+    (void)hipFree(c->heavy_seg);
+    (void)hipFree(c->heavy_col);
+    (void)hipFree(c->heavy_val);
+    (void)hipFree(c->heavy_row);
+    (void)hipFree(c->heavy_code);
     if (c->owns) {
         (void)hipFree(c->pos);
         (void)hipFree(c->crd);

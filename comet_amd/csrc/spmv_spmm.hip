@@ -9,6 +9,9 @@
 #include <stdlib.h>
 
 #include <algorithm>
+#include <queue>
+#include <utility>
+#include <vector>
 
 #include "common.h"
 
@@ -381,6 +384,124 @@ __global__ __launch_bounds__(SPMM_WAVES * 64) void spmm_csr_fixup(
     C[r * ldc + col] = acc;
 }
 
+// ============================================================================
+// SpMM, long rows: column sweep with the row sums in registers.
+// ============================================================================
+constexpr int SPMM_HW = 16;      // wavefronts per workgroup of the sweep
+constexpr int SPMM_HR = 8;       // rows a wavefront can own
+constexpr int SPMM_HG = 32;      // workgroups per XCD: one per CU, so that all of them sweep together
+constexpr int SPMM_HBINS = SPMM_HG * SPMM_HW;        // wavefronts (= row bins) per XCD
+constexpr int SPMM_HSLOTS = SPMM_HBINS * SPMM_HR;    // long rows the plan can hold
+constexpr int SPMM_HEAVY_MIN_LEN = 256;              // a long row has at least this many nonzeros
+constexpr int SPMM_HCB = 32;                         // column blocks a wavefront's list is cut into
+
+// One workgroup per (XCD x, row group g); workgroup w runs on XCD w % 8.  XCD x
+// sweeps its eighth of the column range in ascending order, so a row of B is
+// pulled into that XCD's L2 once and hit by every long row that uses it.  A
+// wavefront owns up to SPMM_HR rows and keeps their sums in registers.  Its list
+// is cut into 32 column blocks; inside a block the entries of one row follow
+// each other, columns ascending, so a row is still summed in ascending column
+// order, and a run of entries of one row is added into one plain register: the
+// register file is indexed dynamically only where a run begins (entry bit 3).
+// A wavefront holds 64 entries of its list at a time, one per lane, and hands
+// them out with readlane; the next 64 are fetched while these are used, and the
+// gathers of the next 16 entries are in flight while the current 16 are added.
+// Entry = column << 4 | first-of-run << 3 | owned row.
+__device__ inline void heavy_issue(double (&b)[SPMM_U], int ents, int t0, int cnt, const double *__restrict__ B,
+                                   int64_t ldb, int64_t col)
+{
+#pragma unroll
+    for (int u = 0; u < SPMM_U; ++u) {
+        const int t = t0 + u < cnt ? t0 + u : cnt - 1;      // past the end: reload the last one, never used
+        const int64_t j = (int64_t)(__builtin_amdgcn_readlane(ents, t) >> 4);
+        b[u] = B[j * ldb + col];
+    }
+}
+
+__device__ inline void heavy_add(double (&acc)[SPMM_HR], double &run, int &run_slot, const double (&b)[SPMM_U],
+                                 int ents, double vals, int t0, int cnt)
+{
+#pragma unroll
+    for (int u = 0; u < SPMM_U; ++u) {
+        if (t0 + u < cnt) {
+            const int ent = __builtin_amdgcn_readlane(ents, t0 + u);
+            if (ent & 8) {
+                acc[run_slot] = run;
+                run_slot = ent & 7;
+                run = acc[run_slot];
+            }
+            const double prod = readlane_f64(vals, t0 + u) * b[u];
+            run = run + prod;
+        }
+    }
+}
+
+__global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
+    const int64_t *__restrict__ seg, const int32_t *__restrict__ hent, const double *__restrict__ hval,
+    const double *__restrict__ B, int64_t ldb, int64_t K, double *__restrict__ partial)
+{
+    constexpr int G = SPMM_HG;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int x = blockIdx.x & 7, g = blockIdx.x >> 3;
+    int64_t col = (int64_t)blockIdx.y * 64 + lane;
+    const bool active = col < K;
+    if (!active)
+        col = K - 1;            // idle lanes gather a valid address and store nothing
+    double acc[SPMM_HR];
+#pragma unroll
+    for (int r = 0; r < SPMM_HR; ++r)
+        acc[r] = 0.0;
+    const int64_t bin = ((int64_t)x * G + g) * SPMM_HW + wave;
+    const int64_t s = seg[bin], e = seg[bin + 1];
+    if (s < e) {
+        double bA[SPMM_U], bB[SPMM_U];
+        double run = 0.0;
+        int run_slot = 0;
+        int cnt = (int)(e - s < 64 ? e - s : 64);
+        int c_ent = 0;
+        double c_val = 0.0;
+        if (lane < cnt) {
+            c_ent = __builtin_nontemporal_load(hent + s + lane);
+            c_val = __builtin_nontemporal_load(hval + s + lane);
+        }
+        heavy_issue(bA, c_ent, 0, cnt, B, ldb, col);
+        for (int64_t base = s; base < e; base += 64) {
+            const int64_t left = e - base - 64;
+            const int ncnt = (int)(left < 0 ? 0 : (left < 64 ? left : 64));
+            int n_ent = 0;
+            double n_val = 0.0;
+            if (lane < ncnt) {
+                n_ent = __builtin_nontemporal_load(hent + base + 64 + lane);
+                n_val = __builtin_nontemporal_load(hval + base + 64 + lane);
+            }
+            static_assert(SPMM_U == 16, "the sweep is unrolled for four batches of 16 per 64 entries");
+            if (cnt > 16)
+                heavy_issue(bB, c_ent, 16, cnt, B, ldb, col);
+            heavy_add(acc, run, run_slot, bA, c_ent, c_val, 0, cnt);
+            if (cnt > 32)
+                heavy_issue(bA, c_ent, 32, cnt, B, ldb, col);
+            heavy_add(acc, run, run_slot, bB, c_ent, c_val, 16, cnt);
+            if (cnt > 48)
+                heavy_issue(bB, c_ent, 48, cnt, B, ldb, col);
+            heavy_add(acc, run, run_slot, bA, c_ent, c_val, 32, cnt);
+            if (ncnt > 0)
+                heavy_issue(bA, n_ent, 0, ncnt, B, ldb, col);
+            heavy_add(acc, run, run_slot, bB, c_ent, c_val, 48, cnt);
+            c_ent = n_ent;
+            c_val = n_val;
+            cnt = ncnt;
+        }
+        acc[run_slot] = run;
+    }
+    if (active) {
+        double *out = partial + (((int64_t)x * G + g) * SPMM_HW + wave) * SPMM_HR * K;
+#pragma unroll
+        for (int r = 0; r < SPMM_HR; ++r)
+            out[(int64_t)r * K + col] = acc[r];
+    }
+}
+
 __global__ void fill_rows_f64(double *__restrict__ C, int64_t nrows, int64_t K, int64_t ldc, double v)
 {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -412,9 +533,294 @@ static int spmm_plan(Csr *a)
     return COMET_HIP_OK;
 }
 
+
+// ---------------------------------------------------------------------------
+// Plan for the sweep: pick the long rows, deal them to the 512 wavefronts of an
+// XCD so that every wavefront gets the same number of nonzeros, and re-store
+// their nonzeros as one list per (XCD, wavefront), ordered by column.
+// ---------------------------------------------------------------------------
+// cnt[h * 8 + x] = nonzeros of long row h whose column lies in the range XCD x sweeps
+__global__ void heavy_count(int64_t nheavy, const int32_t *__restrict__ hrow, const int64_t *__restrict__ pos,
+                            const int32_t *__restrict__ crd, int64_t xcols, int32_t *__restrict__ cnt)
+{
+    const int64_t h = (int64_t)blockIdx.x * (blockDim.x >> 3) + (threadIdx.x >> 3);
+    const int x = threadIdx.x & 7;
+    if (h >= nheavy)
+        return;
+    const int64_t s = pos[hrow[h]], e = pos[hrow[h] + 1];
+    auto first_at_least = [&](int64_t c) {
+        int64_t lo = s, hi = e;
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (crd[mid] < c)
+                lo = mid + 1;
+            else
+                hi = mid;
+        }
+        return lo;
+    };
+    cnt[h * 8 + x] = (int32_t)(first_at_least((int64_t)(x + 1) * xcols) - first_at_least((int64_t)x * xcols));
+}
+
+__global__ void heavy_make_keys(int64_t nheavy, const int32_t *__restrict__ hrow, const int32_t *__restrict__ hcode,
+                                const int64_t *__restrict__ hstart, const int64_t *__restrict__ pos,
+                                const int32_t *__restrict__ crd, int64_t xcols, uint64_t *__restrict__ keys,
+                                uint32_t *__restrict__ idx)
+{
+    const int64_t h = blockIdx.x;
+    if (h >= nheavy)
+        return;
+    const int64_t ps = pos[hrow[h]], len = pos[hrow[h] + 1] - ps, o = hstart[h];
+    for (int64_t t = threadIdx.x; t < len; t += blockDim.x) {
+        const uint64_t c = (uint64_t)(uint32_t)crd[ps + t];
+        const uint64_t x = c / (uint64_t)xcols;
+        const uint64_t cb = (c - x * (uint64_t)xcols) * SPMM_HCB / (uint64_t)xcols;   // column block inside the range
+        const uint64_t code = (uint64_t)hcode[x * nheavy + h];       // wavefront * 8 + slot on that XCD
+        keys[o + t] = ((((x * SPMM_HBINS + (code >> 3)) * SPMM_HCB + cb) * SPMM_HR + (code & 7)) << 28) | c;
+        idx[o + t] = (uint32_t)(ps + t);
+    }
+}
+
+__global__ void heavy_fill(int64_t n, const uint64_t *__restrict__ keys, const uint32_t *__restrict__ idx,
+                           const double *__restrict__ val, int32_t *__restrict__ hent, double *__restrict__ hval)
+{
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < n) {
+        const uint64_t k = keys[e];
+        const bool first = e == 0 || (keys[e - 1] >> 28) != (k >> 28);     // another row, block or wavefront
+        hent[e] = (int32_t)(((k & 0xfffffffull) << 4) | (first ? 8u : 0u) | ((k >> 28) & 7));
+        hval[e] = val[idx[e]];
+    }
+}
+
+// seg[b] = first list entry whose (XCD, wavefront) number is >= b
+__global__ void heavy_segments(int64_t n, const uint64_t *__restrict__ keys, int64_t *__restrict__ seg)
+{
+    const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b > 8 * SPMM_HBINS)
+        return;
+    int64_t lo = 0, hi = n;
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if ((int64_t)(keys[mid] >> 28) / (SPMM_HCB * SPMM_HR) < b)
+            lo = mid + 1;
+        else
+            hi = mid;
+    }
+    seg[b] = lo;
+}
+
+__global__ void light_lengths(int64_t nrows, const int64_t *__restrict__ pos, const int32_t *__restrict__ rowcode,
+                              int64_t *__restrict__ len)
+{
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r < nrows)
+        len[r] = rowcode[r] >= 0 ? 0 : pos[r + 1] - pos[r];
+}
+
+__global__ void light_copy(int64_t nrows, const int64_t *__restrict__ pos, const int32_t *__restrict__ crd,
+                           const double *__restrict__ val, const int64_t *__restrict__ lpos,
+                           int32_t *__restrict__ lcrd, double *__restrict__ lval)
+{
+    // one 16-lane group per row: the rows copied here are short
+    const int64_t r = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+    const int sub = threadIdx.x & 15;
+    if (r >= nrows)
+        return;
+    const int64_t n = lpos[r + 1] - lpos[r], src = pos[r], dst = lpos[r];
+    for (int64_t t = sub; t < n; t += 16) {
+        lcrd[dst + t] = crd[src + t];
+        lval[dst + t] = val[src + t];
+    }
+}
+
+// C[row] += the eight per-XCD sums of a long row, in XCD (= column) order
+__global__ __launch_bounds__(256) void spmm_heavy_combine(int64_t nheavy, const int32_t *__restrict__ hrow,
+                                                          const int32_t *__restrict__ hcode,
+                                                          const double *__restrict__ partial,
+                                                          double *__restrict__ C, int64_t ldc, int64_t K)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t h = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t col = (int64_t)blockIdx.y * 64 + lane;
+    if (h >= nheavy || col >= K)
+        return;
+    const int64_t row = hrow[h];
+    double acc = C[row * ldc + col];
+    for (int x = 0; x < 8; ++x)
+        acc = acc + partial[((int64_t)x * SPMM_HSLOTS + hcode[x * nheavy + h]) * K + col];
+    C[row * ldc + col] = acc;
+}
+
+static Workspace g_heavy_partial;
+
+static int spmm_heavy_plan(Csr *a)
+{
+    if (a->heavy_state != 0)
+        return COMET_HIP_OK;
+    a->heavy_state = 1;
+    if (a->nnz < (1 << 19) || a->nnz >= (1ll << 32) || a->ncols >= (1ll << 27))
+        return COMET_HIP_OK;        // list entries keep the column in 27 bits
+    const int64_t n = a->nrows;
+    std::vector<int64_t> pos((size_t)n + 1);
+    COMET_HIPCHK(hipMemcpyAsync(pos.data(), a->pos, sizeof(int64_t) * (size_t)(n + 1), hipMemcpyDeviceToHost,
+                                stream()));
+    COMET_HIPCHK(hipStreamSynchronize(stream()));
+    std::vector<std::pair<int64_t, int32_t>> cand;       // (-length, row): sorts longest first, ties by row
+    for (int64_t r = 0; r < n; ++r)
+        if (pos[(size_t)r + 1] - pos[(size_t)r] >= SPMM_HEAVY_MIN_LEN)
+            cand.emplace_back(-(pos[(size_t)r + 1] - pos[(size_t)r]), (int32_t)r);
+    std::sort(cand.begin(), cand.end());
+    if ((int64_t)cand.size() > SPMM_HSLOTS)
+        cand.resize(SPMM_HSLOTS);
+    const int64_t H = (int64_t)cand.size();
+    int64_t hnnz = 0;
+    for (auto &c : cand)
+        hnnz -= c.first;
+    if (H == 0 || hnnz * 4 < a->nnz)
+        return COMET_HIP_OK;        // the long rows hold too little of the matrix to pay for a second kernel
+    std::vector<int32_t> hrow((size_t)H), hcode((size_t)(8 * H)), rowcode((size_t)n, -1), cnt((size_t)(8 * H));
+    std::vector<int64_t> hstart((size_t)H + 1, 0);
+    for (int64_t k = 0; k < H; ++k) {
+        hrow[(size_t)k] = cand[(size_t)k].second;
+        rowcode[(size_t)hrow[(size_t)k]] = 0;
+        hstart[(size_t)k + 1] = hstart[(size_t)k] - cand[(size_t)k].first;
+    }
+    int32_t *d_cnt = nullptr, *d_rowcode = nullptr;
+    int64_t *d_hstart = nullptr, *d_len = nullptr;
+    uint64_t *k_in = nullptr, *k_out = nullptr;
+    uint32_t *i_in = nullptr, *i_out = nullptr;
+    Csr *light = new Csr();
+    auto cleanup = [&](bool failed) {
+        (void)hipFree(d_cnt);
+        (void)hipFree(d_rowcode);
+        (void)hipFree(d_hstart);
+        (void)hipFree(d_len);
+        (void)hipFree(k_in);
+        (void)hipFree(k_out);
+        (void)hipFree(i_in);
+        (void)hipFree(i_out);
+        if (failed) {
+            (void)hipFree(a->heavy_seg);
+            (void)hipFree(a->heavy_col);
+            (void)hipFree(a->heavy_val);
+            (void)hipFree(a->heavy_row);
+            (void)hipFree(a->heavy_code);
+            a->heavy_seg = nullptr;
+            a->heavy_col = a->heavy_row = a->heavy_code = nullptr;
+            a->heavy_val = nullptr;
+            light->owns = true;
+            csr_release(light);
+        }
+    };
+#define HEAVY_TRY(call)                                                                                       \
+    do {                                                                                                      \
+        if ((call) != hipSuccess) {                                                                           \
+            cleanup(true);                                                                                    \
+            return set_error(COMET_HIP_ERR_HIP, "%s failed while planning the long rows", #call);             \
+        }                                                                                                     \
+    } while (0)
+    HEAVY_TRY(hipMalloc((void **)&d_cnt, 4 * (size_t)(8 * H)));
+    HEAVY_TRY(hipMalloc((void **)&d_rowcode, 4 * (size_t)n));
+    HEAVY_TRY(hipMalloc((void **)&d_hstart, 8 * (size_t)(H + 1)));
+    HEAVY_TRY(hipMalloc((void **)&d_len, 8 * (size_t)n));
+    HEAVY_TRY(hipMalloc((void **)&k_in, 8 * (size_t)hnnz));
+    HEAVY_TRY(hipMalloc((void **)&k_out, 8 * (size_t)hnnz));
+    HEAVY_TRY(hipMalloc((void **)&i_in, 4 * (size_t)hnnz));
+    HEAVY_TRY(hipMalloc((void **)&i_out, 4 * (size_t)hnnz));
+    HEAVY_TRY(hipMalloc((void **)&a->heavy_seg, 8 * (size_t)(8 * SPMM_HBINS + 1)));
+    HEAVY_TRY(hipMalloc((void **)&a->heavy_col, 4 * (size_t)hnnz));
+    HEAVY_TRY(hipMalloc((void **)&a->heavy_val, 8 * (size_t)hnnz));
+    HEAVY_TRY(hipMalloc((void **)&a->heavy_row, 4 * (size_t)H));
+    HEAVY_TRY(hipMalloc((void **)&a->heavy_code, 4 * (size_t)(8 * H)));
+    HEAVY_TRY(hipMemcpyAsync(a->heavy_row, hrow.data(), 4 * (size_t)H, hipMemcpyHostToDevice, stream()));
+
+    HEAVY_TRY(hipMemcpyAsync(d_rowcode, rowcode.data(), 4 * (size_t)n, hipMemcpyHostToDevice, stream()));
+    HEAVY_TRY(hipMemcpyAsync(d_hstart, hstart.data(), 8 * (size_t)(H + 1), hipMemcpyHostToDevice, stream()));
+    const int64_t xcols = ceil_div(a->ncols, 8);
+    // Every XCD gets its own assignment of rows to wavefronts, by what the row holds in that XCD's column
+    // range: longest first, each to the least loaded wavefront that still has a free slot.  Wavefronts with
+    // equal lists move through the columns at the same pace, which is what keeps the rows of B they share
+    // inside the L2 between uses.
+    heavy_count<<<dim3((unsigned)ceil_div(H, 32)), dim3(256), 0, stream()>>>(H, a->heavy_row, a->pos, a->crd, xcols,
+                                                                             d_cnt);
+    HEAVY_TRY(hipMemcpyAsync(cnt.data(), d_cnt, 4 * (size_t)(8 * H), hipMemcpyDeviceToHost, stream()));
+    HEAVY_TRY(hipStreamSynchronize(stream()));
+    for (int x = 0; x < 8; ++x) {
+        std::vector<std::pair<int32_t, int32_t>> order((size_t)H);       // (-count, row index)
+        for (int64_t k = 0; k < H; ++k)
+            order[(size_t)k] = {-cnt[(size_t)(k * 8 + x)], (int32_t)k};
+        std::sort(order.begin(), order.end());
+        // (time the wavefront needs for its list so far, wavefront).  The four wavefronts of a SIMD do not
+        // run at the same speed: the older one wins every arbitration, and the measured entry rates of
+        // wavefronts 0-3, 4-7, 8-11, 12-15 of a workgroup are as 1.21 : 1.06 : 0.91 : 0.81.
+        static const double pace[4] = {1.0 / 1.215, 1.0 / 1.059, 1.0 / 0.913, 1.0 / 0.812};
+        std::priority_queue<std::pair<double, int32_t>, std::vector<std::pair<double, int32_t>>,
+                            std::greater<std::pair<double, int32_t>>> bins;
+        std::vector<int32_t> used(SPMM_HBINS, 0);
+        for (int32_t b = 0; b < SPMM_HBINS; ++b)
+            bins.push({0.0, b});
+        for (auto &o : order) {
+            auto top = bins.top();
+            bins.pop();
+            const int32_t b = top.second;
+            hcode[(size_t)(x * H + o.second)] = b * SPMM_HR + used[(size_t)b];
+            if (++used[(size_t)b] < SPMM_HR)
+                bins.push({top.first - o.first * pace[(b % SPMM_HW) / 4], b});
+        }
+    }
+    HEAVY_TRY(hipMemcpyAsync(a->heavy_code, hcode.data(), 4 * (size_t)(8 * H), hipMemcpyHostToDevice, stream()));
+    {
+        KernelTimer t("heavy_make_keys");
+        heavy_make_keys<<<dim3((unsigned)H), dim3(256), 0, stream()>>>(H, a->heavy_row, a->heavy_code, d_hstart,
+                                                                       a->pos, a->crd, xcols, k_in, i_in);
+    }
+    if (sort_pairs_u64_u32(k_in, k_out, i_in, i_out, hnnz, 28 + 3 + 5 + 12) != COMET_HIP_OK) {
+        cleanup(true);
+        return COMET_HIP_ERR_HIP;
+    }
+    {
+        KernelTimer t("heavy_fill");
+        heavy_fill<<<dim3((unsigned)ceil_div(hnnz, 256)), dim3(256), 0, stream()>>>(
+            hnnz, k_out, i_out, a->val, a->heavy_col, a->heavy_val);
+        heavy_segments<<<dim3((unsigned)ceil_div(8 * SPMM_HBINS + 1, 256)), dim3(256), 0, stream()>>>(
+            hnnz, k_out, a->heavy_seg);
+    }
+    // the rest of the matrix, long rows left empty
+    light->nrows = n;
+    light->ncols = a->ncols;
+    light->nnz = a->nnz - hnnz;
+    light->owns = true;
+    HEAVY_TRY(hipMalloc((void **)&light->pos, 8 * (size_t)(n + 1)));
+    HEAVY_TRY(hipMalloc((void **)&light->crd, 4 * (size_t)(light->nnz > 0 ? light->nnz : 1)));
+    HEAVY_TRY(hipMalloc((void **)&light->val, 8 * (size_t)(light->nnz > 0 ? light->nnz : 1)));
+    light_lengths<<<dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, stream()>>>(n, a->pos, d_rowcode, d_len);
+    if (exclusive_scan_i64(d_len, n, light->pos) != COMET_HIP_OK) {
+        cleanup(true);
+        return COMET_HIP_ERR_HIP;
+    }
+    {
+        KernelTimer t("light_copy");
+        light_copy<<<dim3((unsigned)ceil_div(n * 16, 256)), dim3(256), 0, stream()>>>(n, a->pos, a->crd, a->val,
+                                                                                      light->pos, light->crd, light->val);
+    }
+    HEAVY_TRY(hipGetLastError());
+    HEAVY_TRY(hipStreamSynchronize(stream()));
+#undef HEAVY_TRY
+    cleanup(false);
+    light->heavy_state = 1;
+    a->light = light;
+    a->heavy_nnz = hnnz;
+    a->heavy_rows = H;
+    a->heavy_state = 2;
+    return COMET_HIP_OK;
+}
+
 }  // namespace comet
 
 using namespace comet;
+
+static int spmm_chunks(Csr *a, int64_t K, const double *B, int64_t ldb, double *C, int64_t ldc, int accumulate);
 
 extern "C" int comet_hip_spmv_csr_f64(int64_t csr, int64_t x_dptr, int64_t y_dptr, int accumulate)
 {
@@ -460,6 +866,35 @@ extern "C" int comet_hip_spmm_csr_f64(int64_t csr, int64_t K, int64_t b_dptr, in
     if (!c_dptr || (a->nnz > 0 && !b_dptr))
         return set_error(COMET_HIP_ERR_ARG, "null matrix passed to comet_hip_spmm_csr_f64");
     double *C = (double *)c_dptr;
+    const double *B = (const double *)b_dptr;
+    if (ceil_div(K, 64) > 65535)
+        return set_error(COMET_HIP_ERR_SIZE, "K = %lld needs more than 65535 column tiles", (long long)K);
+    // long rows: column sweep with the sums on chip; everything else: one wavefront per 256 nonzeros
+    if (K >= 16 && K <= 2048 && getenv("COMET_SPMM_NO_SWEEP") == nullptr)
+        COMET_CHK(spmm_heavy_plan(a));
+    if (a->heavy_state != 2 || K < 16 || K > 2048 || getenv("COMET_SPMM_NO_SWEEP") != nullptr)
+        return spmm_chunks(a, K, B, ldb, C, ldc, accumulate);
+    // the long rows are empty in `light`: cleared (or, accumulating, left alone) there, then added to below
+    COMET_CHK(spmm_chunks(a->light, K, B, ldb, C, ldc, accumulate));
+    COMET_CHK(g_heavy_partial.ensure(sizeof(double) * 8 * (size_t)SPMM_HSLOTS * (size_t)K, false));
+    const unsigned tiles = (unsigned)ceil_div(K, 64);
+    {
+        KernelTimer t("spmm_heavy_sweep");
+        spmm_heavy_sweep<<<dim3(8 * SPMM_HG, tiles), dim3(SPMM_HW * 64), 0, stream()>>>(
+            a->heavy_seg, a->heavy_col, a->heavy_val, B, ldb, K, (double *)g_heavy_partial.ptr);
+    }
+    {
+        KernelTimer t("spmm_heavy_combine");
+        spmm_heavy_combine<<<dim3((unsigned)ceil_div(a->heavy_rows, 4), tiles), dim3(256), 0, stream()>>>(
+            a->heavy_rows, a->heavy_row, a->heavy_code, (const double *)g_heavy_partial.ptr, C, ldc, K);
+    }
+    COMET_HIPCHK(hipGetLastError());
+    return COMET_HIP_OK;
+}
+
+static int spmm_chunks(Csr *a, int64_t K, const double *B, int64_t ldb, double *C, int64_t ldc, int accumulate)
+{
+    const int64_t b_dptr = (int64_t)B;
     if (a->nnz == 0) {
         if (!accumulate) {
             KernelTimer t("fill_rows_f64");
@@ -472,8 +907,6 @@ extern "C" int comet_hip_spmm_csr_f64(int64_t csr, int64_t K, int64_t b_dptr, in
     COMET_CHK(spmm_plan(a));
     const int64_t nchunks = a->spmm_nchunks;
     const int64_t tiles = ceil_div(K, 64);
-    if (tiles > 65535)
-        return set_error(COMET_HIP_ERR_SIZE, "K = %lld needs more than 65535 column tiles", (long long)K);
     COMET_CHK(g_spmm_carry.ensure(sizeof(double) * (size_t)(tiles * nchunks * 2 * 64), false));
     double *carry = (double *)g_spmm_carry.ptr;
     const dim3 grid((unsigned)ceil_div(nchunks, SPMM_WAVES), (unsigned)tiles);

@@ -156,6 +156,27 @@ def test_spmm_golden(golden, golden_dir):
     assert orc.format_f64(Cm.to_numpy()) == g["printed"]
 
 
+def _long_rows(pos, K):
+    """The rows the library hands to the column sweep (its rule restated): at least 256 nonzeros, at most
+    the 4096 longest (ties: lower row first), and only if they hold a quarter of a matrix of >= 2^19 nonzeros."""
+    lens = np.diff(pos)
+    rows = np.flatnonzero(lens >= 256)
+    rows = rows[np.argsort(-lens[rows], kind="stable")][:4096]
+    if not (16 <= K <= 2048) or pos[-1] < (1 << 19) or 4 * lens[rows].sum() < pos[-1]:
+        return rows[:0]
+    return rows
+
+
+def _bit_exact_rows(pos, K):
+    """Rows summed in the checker's order: those that lie inside one 256-nonzero chunk of the matrix the
+    chunk kernel sees (the matrix without the rows the sweep takes), and empty rows."""
+    lens = np.diff(pos)
+    light = lens.copy()
+    light[_long_rows(pos, K)] = 0
+    lpos = np.concatenate([[0], np.cumsum(light)])
+    return (lens == 0) | ((light > 0) & (lpos[:-1] // 256 == (lpos[1:] - 1) // 256))
+
+
 def _spmm_check(pos, crd, val, B, C0=None):
     n = len(pos) - 1
     A = rt.CsrMatrix.from_arrays((n, B.shape[0]), pos, crd, val)
@@ -165,10 +186,7 @@ def _spmm_check(pos, crd, val, B, C0=None):
     else:
         got = rt.spmm(A, dB, rt.DeviceArray.from_numpy(C0)).to_numpy()
     want = orc.spmm(pos, crd, val, B, C0)
-    lens = np.diff(pos)
-    # rows that fit inside one 256-nonzero chunk are computed in the checker's order: bit-exact
-    first_chunk, last_chunk = pos[:-1] // 256, (np.maximum(pos[1:], pos[:-1] + 1) - 1) // 256
-    inside = (first_chunk == last_chunk) | (lens == 0)
+    inside = _bit_exact_rows(pos, B.shape[1])
     assert np.array_equal(got[inside], want[inside])
     bound = orc.spmm(pos, crd, np.abs(val), np.abs(B), None if C0 is None else np.abs(C0))
     assert np.all(np.abs(got - want) <= RTOL * bound + 0.0)
@@ -717,3 +735,66 @@ def test_reader_rejects_bad_input(tmp_path):
     row = np.array([0, 5], dtype=np.int64)
     h = L.comet_hip_csr_from_coo_i64(3, 3, 2, row.ctypes.data, row.ctypes.data, np.zeros(2).ctypes.data, 1)
     assert h == 0 and b"outside" in L.comet_hip_last_error()
+
+
+# ----------------------------------------------------------------- SpMM: long rows through the column sweep
+def _kernels_of(fn):
+    rt.profile_reset()
+    rt.profile_enable(True)
+    fn()
+    rt.sync()
+    rep = rt.profile_report()
+    rt.profile_enable(False)
+    return rep
+
+
+def _sweep_check(pos, crd, val, B, C0=None, ld_pad=0):
+    """SpMM on a matrix whose long rows take the sweep: every row within the summation-order bound, and the
+    rows that lie inside one 256-nonzero chunk of the matrix without its long rows bit-exact."""
+    n, m = len(pos) - 1, B.shape[0]
+    K = B.shape[1]
+    A = rt.CsrMatrix.from_arrays((n, m), pos, crd, val)
+    Bp = np.zeros((m, K + ld_pad)); Bp[:, :K] = B
+    Cp = np.full((n, K + ld_pad), 123.0)
+    if C0 is not None:
+        Cp[:, :K] = C0
+    dB, dC = rt.DeviceArray.from_numpy(Bp), rt.DeviceArray.from_numpy(Cp)
+    L = rt.lib()
+    run = lambda: rt._check(L.comet_hip_spmm_csr_f64(A.handle, K, dB.ptr, K + ld_pad, dC.ptr, K + ld_pad,
+                                                     int(C0 is not None)), "spmm")
+    rep = _kernels_of(run)
+    assert "spmm_heavy_sweep" in rep and "spmm_csr_nnzsplit" in rep, sorted(rep)
+    out = dC.to_numpy()
+    assert np.all(out[:, K:] == 123.0)             # the padding of C is not touched
+    got = out[:, :K]
+    want = orc.spmm(pos, crd, val, B, C0)
+    bound = orc.spmm(pos, crd, np.abs(val), np.abs(B), None if C0 is None else np.abs(C0))
+    assert np.all(np.abs(got - want) <= RTOL * bound)
+    long_rows = _long_rows(pos, K)
+    inside = _bit_exact_rows(pos, K)
+    assert inside.sum() > 0 and np.array_equal(got[inside], want[inside])
+    # a second call on the same handle reuses the plan and gives the same bits
+    if C0 is None:
+        run(); assert np.array_equal(dC.to_numpy()[:, :K], got)
+    return len(long_rows)
+
+
+@pytest.mark.parametrize("K,acc,pad", [(64, False, 0), (64, True, 0), (20, False, 3), (100, True, 5)])
+def test_spmm_long_rows_sweep(K, acc, pad):
+    pos, crd, val = gen.zipf_csr(n=40_000, mean=16.0, cap=4096, seed=7)
+    assert len(crd) >= 1 << 19
+    B = gen.dense((40_000, K), seed=8)
+    C0 = gen.dense((40_000, K), seed=9) if acc else None
+    assert _sweep_check(pos, crd, val, B, C0, pad) > 100
+
+
+def test_spmm_more_long_rows_than_the_sweep_holds():
+    """5000 rows of 300 nonzeros: the 4096 longest (ties: lowest row ids) sweep, the others stay on the
+    chunk kernel; an empty row and a short row sit between them."""
+    rng = np.random.default_rng(31)
+    n, m = 5002, 3000
+    lens = np.full(n, 300); lens[17] = 0; lens[4000] = 3
+    pos = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    crd = np.concatenate([np.sort(rng.choice(m, l, replace=False)) for l in lens]).astype(np.int64)
+    val = rng.uniform(-1, 1, len(crd))
+    assert _sweep_check(pos, crd, val, gen.dense((m, 64), seed=2)) == 4096
