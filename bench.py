@@ -24,9 +24,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP64_MFMA_PEAK_TFLOPS = 78.6  # MI355X dense fp64 matrix, published
-# HBM bytes per launch of spmm_csr_nnzsplit on the default workload, from rocprofv3 --pmc FETCH_SIZE (x 2.000) and
-# WRITE_SIZE (x 1.000), factors from a 1 GiB copy kernel; see profiles/spmm_csr_nnzsplit__spmm_zipf_500k_k64.txt
-SPMM_TRAFFIC_BYTES = int((2_017_117 * 2.000 + 264_614 * 1.000) * 1024)
+# HBM bytes per SpMM product (all of its kernels) on the default workload, from rocprofv3 --pmc FETCH_SIZE (x 2.000)
+# and WRITE_SIZE (x 1.000), factors from a 1 GiB copy kernel; see profiles/spmm_kernels__spmm_zipf_500k_k64.txt
+SPMM_TRAFFIC_BYTES = int((749_341 * 2.000 + 271_586 * 1.000) * 1024)
 
 
 _T0 = time.perf_counter()
@@ -105,8 +105,12 @@ def bench_spmm(rt, orc, gen, args):
     flops = 2.0 * nnz * K
     ib = 4
     alg_bytes = nnz * (8 + ib) + (n + 1) * ib + 8 * n * K + 8 * n * K
-    dom = "spmm_csr_nnzsplit"
-    dom_ms = kt[dom]["avg_ms"]
+    # one product = the column sweep over the long rows + the chunk kernel over the rest (+ two small
+    # kernels that stitch rows together); the algorithmic bytes are those of the whole product, so the
+    # roofline is taken over the sum of their launch durations
+    parts = [k for k in ("spmm_heavy_sweep", "spmm_csr_nnzsplit", "spmm_heavy_combine", "spmm_csr_fixup") if k in kt]
+    dom = " + ".join(parts)
+    dom_ms = sum(kt[k]["avg_ms"] * kt[k]["launches"] for k in parts) / args.steps
     # parity of what was just timed, on a sample of rows (full check lives in tests/)
     got = dC.to_numpy()
     rows = np.random.default_rng(0).choice(n, 2000, replace=False)

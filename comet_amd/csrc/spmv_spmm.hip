@@ -388,11 +388,19 @@ __global__ __launch_bounds__(SPMM_WAVES * 64) void spmm_csr_fixup(
 // SpMM, long rows: column sweep with the row sums in registers.
 // ============================================================================
 constexpr int SPMM_HW = 16;      // wavefronts per workgroup of the sweep
-constexpr int SPMM_HR = 8;       // rows a wavefront can own
+#ifndef COMET_SPMM_HR_BITS
+#define COMET_SPMM_HR_BITS 3
+#endif
+#ifndef COMET_SPMM_HEAVY_MIN
+#define COMET_SPMM_HEAVY_MIN 128
+#endif
+constexpr int SPMM_HRB = COMET_SPMM_HR_BITS;         // bits of a list entry that name the owned row
+constexpr int SPMM_HR = 1 << SPMM_HRB;               // rows a wavefront can own
+constexpr int SPMM_HCOLB = 28 - SPMM_HRB;            // bits of a list entry left for the column
 constexpr int SPMM_HG = 32;      // workgroups per XCD: one per CU, so that all of them sweep together
 constexpr int SPMM_HBINS = SPMM_HG * SPMM_HW;        // wavefronts (= row bins) per XCD
 constexpr int SPMM_HSLOTS = SPMM_HBINS * SPMM_HR;    // long rows the plan can hold
-constexpr int SPMM_HEAVY_MIN_LEN = 256;              // a long row has at least this many nonzeros
+constexpr int SPMM_HEAVY_MIN_LEN = COMET_SPMM_HEAVY_MIN;              // a long row has at least this many nonzeros
 constexpr int SPMM_HCB = 32;                         // column blocks a wavefront's list is cut into
 
 // One workgroup per (XCD x, row group g); workgroup w runs on XCD w % 8.  XCD x
@@ -406,14 +414,14 @@ constexpr int SPMM_HCB = 32;                         // column blocks a wavefron
 // A wavefront holds 64 entries of its list at a time, one per lane, and hands
 // them out with readlane; the next 64 are fetched while these are used, and the
 // gathers of the next 16 entries are in flight while the current 16 are added.
-// Entry = column << 4 | first-of-run << 3 | owned row.
+// Entry = column << (SPMM_HRB + 1) | first-of-run << SPMM_HRB | owned row.
 __device__ inline void heavy_issue(double (&b)[SPMM_U], int ents, int t0, int cnt, const double *__restrict__ B,
                                    int64_t ldb, int64_t col)
 {
 #pragma unroll
     for (int u = 0; u < SPMM_U; ++u) {
         const int t = t0 + u < cnt ? t0 + u : cnt - 1;      // past the end: reload the last one, never used
-        const int64_t j = (int64_t)(__builtin_amdgcn_readlane(ents, t) >> 4);
+        const int64_t j = (int64_t)((unsigned)__builtin_amdgcn_readlane(ents, t) >> (SPMM_HRB + 1));
         b[u] = B[j * ldb + col];
     }
 }
@@ -425,9 +433,9 @@ __device__ inline void heavy_add(double (&acc)[SPMM_HR], double &run, int &run_s
     for (int u = 0; u < SPMM_U; ++u) {
         if (t0 + u < cnt) {
             const int ent = __builtin_amdgcn_readlane(ents, t0 + u);
-            if (ent & 8) {
+            if (ent & SPMM_HR) {
                 acc[run_slot] = run;
-                run_slot = ent & 7;
+                run_slot = ent & (SPMM_HR - 1);
                 run = acc[run_slot];
             }
             const double prod = readlane_f64(vals, t0 + u) * b[u];
@@ -575,8 +583,9 @@ __global__ void heavy_make_keys(int64_t nheavy, const int32_t *__restrict__ hrow
         const uint64_t c = (uint64_t)(uint32_t)crd[ps + t];
         const uint64_t x = c / (uint64_t)xcols;
         const uint64_t cb = (c - x * (uint64_t)xcols) * SPMM_HCB / (uint64_t)xcols;   // column block inside the range
-        const uint64_t code = (uint64_t)hcode[x * nheavy + h];       // wavefront * 8 + slot on that XCD
-        keys[o + t] = ((((x * SPMM_HBINS + (code >> 3)) * SPMM_HCB + cb) * SPMM_HR + (code & 7)) << 28) | c;
+        const uint64_t code = (uint64_t)hcode[x * nheavy + h];       // wavefront * SPMM_HR + slot on that XCD
+        keys[o + t] = ((((x * SPMM_HBINS + (code >> SPMM_HRB)) * SPMM_HCB + cb) * SPMM_HR + (code & (SPMM_HR - 1)))
+                       << 28) | c;
         idx[o + t] = (uint32_t)(ps + t);
     }
 }
@@ -588,7 +597,8 @@ __global__ void heavy_fill(int64_t n, const uint64_t *__restrict__ keys, const u
     if (e < n) {
         const uint64_t k = keys[e];
         const bool first = e == 0 || (keys[e - 1] >> 28) != (k >> 28);     // another row, block or wavefront
-        hent[e] = (int32_t)(((k & 0xfffffffull) << 4) | (first ? 8u : 0u) | ((k >> 28) & 7));
+        hent[e] = (int32_t)(uint32_t)(((k & 0xfffffffull) << (SPMM_HRB + 1)) | (first ? (uint64_t)SPMM_HR : 0u) |
+                                      ((k >> 28) & (SPMM_HR - 1)));
         hval[e] = val[idx[e]];
     }
 }
@@ -659,8 +669,8 @@ static int spmm_heavy_plan(Csr *a)
     if (a->heavy_state != 0)
         return COMET_HIP_OK;
     a->heavy_state = 1;
-    if (a->nnz < (1 << 19) || a->nnz >= (1ll << 32) || a->ncols >= (1ll << 27))
-        return COMET_HIP_OK;        // list entries keep the column in 27 bits
+    if (a->nnz < (1 << 19) || a->nnz >= (1ll << 32) || a->ncols >= (1ll << SPMM_HCOLB))
+        return COMET_HIP_OK;        // a list entry has SPMM_HCOLB bits for the column
     const int64_t n = a->nrows;
     std::vector<int64_t> pos((size_t)n + 1);
     COMET_HIPCHK(hipMemcpyAsync(pos.data(), a->pos, sizeof(int64_t) * (size_t)(n + 1), hipMemcpyDeviceToHost,
@@ -775,7 +785,7 @@ static int spmm_heavy_plan(Csr *a)
         heavy_make_keys<<<dim3((unsigned)H), dim3(256), 0, stream()>>>(H, a->heavy_row, a->heavy_code, d_hstart,
                                                                        a->pos, a->crd, xcols, k_in, i_in);
     }
-    if (sort_pairs_u64_u32(k_in, k_out, i_in, i_out, hnnz, 28 + 3 + 5 + 12) != COMET_HIP_OK) {
+    if (sort_pairs_u64_u32(k_in, k_out, i_in, i_out, hnnz, 28 + SPMM_HRB + 5 + 12) != COMET_HIP_OK) {
         cleanup(true);
         return COMET_HIP_ERR_HIP;
     }

@@ -157,10 +157,10 @@ def test_spmm_golden(golden, golden_dir):
 
 
 def _long_rows(pos, K):
-    """The rows the library hands to the column sweep (its rule restated): at least 256 nonzeros, at most
+    """The rows the library hands to the column sweep (its rule restated): at least 128 nonzeros, at most
     the 4096 longest (ties: lower row first), and only if they hold a quarter of a matrix of >= 2^19 nonzeros."""
     lens = np.diff(pos)
-    rows = np.flatnonzero(lens >= 256)
+    rows = np.flatnonzero(lens >= 128)
     rows = rows[np.argsort(-lens[rows], kind="stable")][:4096]
     if not (16 <= K <= 2048) or pos[-1] < (1 << 19) or 4 * lens[rows].sum() < pos[-1]:
         return rows[:0]
