@@ -38,6 +38,7 @@ int num_cus();
 struct Workspace {
     void *ptr = nullptr;
     size_t bytes = 0;
+    bool listed = false;
     int ensure(size_t need, bool zeroed);
     void release();
 };

@@ -72,10 +72,17 @@ int ensure_init()
     return do_init(0);
 }
 
+// every workspace that ever held memory, so that comet_hip_finalize can give all of it back
+static std::vector<Workspace *> g_workspaces;
+
 int Workspace::ensure(size_t need, bool zeroed)
 {
     if (need <= bytes)
         return COMET_HIP_OK;
+    if (!listed) {
+        g_workspaces.push_back(this);
+        listed = true;
+    }
     if (ptr) {
         COMET_HIPCHK(hipStreamSynchronize(stream()));
         COMET_HIPCHK(hipFree(ptr));
@@ -451,9 +458,8 @@ int comet_hip_finalize(void)
     for (Csr *c : g_live)
         csr_release(c);
     g_live.clear();
-    g_scan_ws.release();
-    g_red_ws.release();
-    // the other cached workspaces are released by their owners' atexit-free design: they live until process end
+    for (Workspace *w : g_workspaces)
+        w->release();
     (void)hipStreamDestroy(g_stream);
     g_stream = nullptr;
     g_inited = false;

@@ -1,0 +1,270 @@
+"""Runs the hot-path subset of COMET's tensor-algebra language (.ta) on the MI355X library and prints
+results in the text form the reference's runtime prints, so that the CHECK lines of the reference's
+integration tests (test/integration/{ops,semiring,kernels}/*.ta in pnnl/COMET) can be verified with
+FileCheck against this backend:
+
+    SPARSE_FILE_NAME0=a.mtx python -m comet_amd.ta_run program.ta | FileCheck program.ta
+
+It stands where `comet-opt ... | mlir-cpu-runner ...` stands in those tests' RUN lines.  It is an
+interpreter over library calls, not a compiler: every statement maps to one entry point of
+include/comet_hip_rt.h.  Statements it understands (frontends/comet_dsl/include/Parser.h for the grammar):
+
+    IndexLabel [a] = [?];            IndexLabel [c] = [4];
+    Tensor<double> A([a, b], {CSR}); formats Dense, CSR, COO, DCSR
+    A[a, b] = comet_read(0);         A[a, b] = comet_read(0, 3);      (file id, read mode)
+    B[b, c] = 1.7;                   (fill)
+    C[a, c] = A[a, b] * B[b, c];     SpMV, SpMM, SpGEMM, dense contraction (TTGT)
+    C[a, c] = A[a, b] @(min,+) B[b, c];                               (SpGEMM over a semiring)
+    C[i, k]<M, push> = A[i, j] * B[j, k];                             (masked SpGEMM)
+    C[i, j] = A[i, j] .* B[i, j];    (CSR .* CSR)
+    B[j, i] = transpose(A[i, j], {j, i});                             (dense)
+    var s = SUM(C[i, j]);  var t = getTime();  printElapsedTime(t0, t1);  print(C);  print(s);
+
+Anything else raises TaError naming the statement.  Like the generated code, `C = A * B` adds into what C
+holds (the reference's tests fill C with 0.0 first).
+"""
+import re
+import sys
+import time
+
+import numpy as np
+
+from . import runtime as rt
+
+
+class TaError(RuntimeError):
+    pass
+
+
+def format_values(v):
+    """include/comet/ExecutionEngine/RunnerUtils.h:232-266: "data = \\n", every element through an ostream
+    (six significant digits) followed by a comma, then a newline; nothing at all for an empty tensor."""
+    v = np.ravel(v)
+    if v.size == 0:
+        return ""
+    if v.dtype.kind in "iu":
+        body = "".join(f"{int(x)}," for x in v)
+    else:
+        body = "".join(f"{float(x):g}," for x in v)
+    return "data = \n" + body + "\n"
+
+
+_SEMIRING_TOKENS = {"+": "plus", "*": "times", "min": "min", "max": "max", "any": "any", "first": "first",
+                    "second": "second", "pair": "pair", "-": "minus", "plus": "plus", "times": "times",
+                    "minus": "minus", "/": "div"}
+_FORMATS = {"Dense", "CSR", "COO", "DCSR"}
+
+
+class _Tensor:
+    def __init__(self, name, labels, fmt):
+        self.name, self.labels, self.fmt = name, labels, fmt
+        self.value = None        # DeviceArray (Dense) or CsrMatrix (every sparse format)
+
+
+class Program:
+    def __init__(self, out=sys.stdout):
+        self.extent = {}         # index label -> size or None (the '?' of the language)
+        self.order = []          # index labels in declaration order
+        self.tensors = {}
+        self.scalars = {}
+        self.out = out
+
+    # ------------------------------------------------------------------ helpers
+    def _labels(self, text):
+        labs = [t.strip() for t in text.split(",") if t.strip()]
+        for l in labs:
+            if l not in self.extent:
+                raise TaError(f"index label {l} is not declared")
+        return labs
+
+    def _tensor(self, name):
+        if name not in self.tensors:
+            raise TaError(f"tensor {name} is not declared")
+        return self.tensors[name]
+
+    def _shape(self, labels):
+        shape = []
+        for l in labels:
+            if self.extent[l] is None:
+                raise TaError(f"the size of index {l} is not known yet (it is set by reading a sparse tensor)")
+            shape.append(self.extent[l])
+        return shape
+
+    def _bind(self, labels, shape):
+        for l, n in zip(labels, shape):
+            if self.extent[l] is None:
+                self.extent[l] = int(n)
+            elif self.extent[l] != n:
+                raise TaError(f"index {l} has size {self.extent[l]} but the tensor has {n}")
+
+    def _dense(self, t):
+        if t.value is None:       # declared, never filled: the reference allocates without initialising
+            t.value = rt.DeviceArray(self._shape(t.labels), zero=True)
+        return t.value
+
+    def _sparse(self, t):
+        if t.value is None:
+            raise TaError(f"sparse tensor {t.name} is used before it is read or computed")
+        return t.value
+
+    # ------------------------------------------------------------------ statements
+    def run(self, text):
+        body = re.sub(r"#[^\n]*", "", text)
+        m = re.search(r"def\s+main\s*\(\s*\)\s*\{(.*)\}", body, re.S)
+        if not m:
+            raise TaError("no `def main() { ... }`")
+        for stmt in m.group(1).split(";"):
+            stmt = " ".join(stmt.split())
+            if stmt:
+                self._statement(stmt)
+
+    def _statement(self, s):
+        for pattern, handler in self._RULES:
+            m = re.fullmatch(pattern, s)
+            if m:
+                return handler(self, *m.groups())
+        raise TaError(f"statement not supported by this runner: {s}")
+
+    def _index_label(self, name, size):
+        self.extent[name] = None if size == "?" else int(size)
+        if name not in self.order:
+            self.order.append(name)
+
+    def _declare(self, name, labels, fmt):
+        if fmt not in _FORMATS:
+            raise TaError(f"tensor format {fmt} is not supported by this runner")
+        self.tensors[name] = _Tensor(name, self._labels(labels), fmt)
+
+    def _read(self, name, labels, file_id, mode):
+        t = self._tensor(name)
+        if t.fmt == "Dense" or len(t.labels) != 2:
+            raise TaError("comet_read is supported for sparse matrices")
+        t.value = rt.CsrMatrix.from_file_id(int(file_id), int(mode) if mode else 1)
+        self._bind(t.labels, t.value.shape)
+
+    def _fill(self, name, labels, value):
+        t = self._tensor(name)
+        if t.fmt != "Dense":
+            raise TaError("only dense tensors can be filled with a constant")
+        t.value = rt.DeviceArray.from_numpy(np.full(self._shape(t.labels), float(value)))
+
+    def _product(self, cname, clabels, mask, _mode, aname, alabels, op, red, mul, bname, blabels):
+        c, a, b = self._tensor(cname), self._tensor(aname), self._tensor(bname)
+        al, bl, cl = self._labels(alabels), self._labels(blabels), self._labels(clabels)
+        semiring = None
+        if red is not None:
+            try:
+                semiring = (_SEMIRING_TOKENS[red.strip()], _SEMIRING_TOKENS[mul.strip()])
+            except KeyError:
+                raise TaError(f"semiring @({red},{mul}) is not supported") from None
+        if op == ".*":
+            if not (a.fmt == b.fmt == c.fmt == "CSR") or not (al == bl == cl):
+                raise TaError("elementwise .* is supported for CSR .* CSR -> CSR over the same indices")
+            c.value = rt.eltwise_mult(self._sparse(a), self._sparse(b))
+            return
+        if a.fmt != "Dense" and b.fmt == "Dense" and c.fmt == "Dense":
+            if semiring not in (None, ("plus", "times")) or mask:
+                raise TaError("semirings and masks are supported for sparse x sparse products")
+            A = self._sparse(a)
+            self._bind(al, A.shape)
+            if len(al) == 2 and bl == [al[1]] and cl == [al[0]]:
+                rt.spmv(A, self._dense(b), self._dense(c), accumulate=True)
+            elif len(al) == 2 and len(bl) == 2 and bl[0] == al[1] and cl == [al[0], bl[1]]:
+                rt.spmm(A, self._dense(b), self._dense(c), accumulate=True)
+            else:
+                raise TaError("sparse x dense is supported as C[a] = A[a,b]*B[b] and C[a,c] = A[a,b]*B[b,c]")
+            return
+        if a.fmt != "Dense" and b.fmt != "Dense" and c.fmt != "Dense":
+            if not (len(al) == 2 and len(bl) == 2 and bl[0] == al[1] and cl == [al[0], bl[1]]):
+                raise TaError("sparse x sparse is supported as C[a,c] = A[a,b]*B[b,c]")
+            m = self._sparse(self._tensor(mask)) if mask else None
+            c.value = rt.spgemm(self._sparse(a), self._sparse(b), mask=m, semiring=semiring)
+            self._bind(cl, c.value.shape)
+            return
+        if a.fmt == b.fmt == c.fmt == "Dense":
+            if semiring not in (None, ("plus", "times")) or mask:
+                raise TaError("dense contractions are plus-times and unmasked")
+            # one character per label, numbered as the front end does: by first appearance in A, B, C
+            names = {}
+            for l in al + bl + cl:
+                names.setdefault(l, chr(ord("a") + len(names)))
+            sa, sb, sc = ("".join(names[l] for l in ls) for ls in (al, bl, cl))
+            rt.ttgt_contract(sa, sb, sc, self._dense(a), self._dense(b), self._dense(c), beta=1.0)
+            return
+        raise TaError(f"this combination of formats is not supported: {a.fmt} x {b.fmt} -> {c.fmt}")
+
+    def _transpose(self, bname, blabels, aname, alabels, order):
+        a, b = self._tensor(aname), self._tensor(bname)
+        if a.fmt != "Dense" or b.fmt != "Dense":
+            raise TaError("transpose is supported for dense tensors")
+        al, bl = self._labels(alabels), self._labels(blabels)
+        if self._labels(order) != bl or sorted(al) != sorted(bl):
+            raise TaError("the index list of transpose must be the output's")
+        b.value = rt.transpose(self._dense(a), [al.index(l) for l in bl])
+
+    def _sum(self, var, name, _labels):
+        t = self._tensor(name)
+        self.scalars[var] = rt.reduce_sum(self._dense(t)) if t.fmt == "Dense" else rt.sum_values(self._sparse(t))
+
+    def _get_time(self, var):
+        rt.sync()
+        self.scalars[var] = time.perf_counter()
+
+    def _elapsed(self, t0, t1):
+        self.out.write("ELAPSED_TIME = %f\n" % (self.scalars[t1] - self.scalars[t0]))
+
+    def _print(self, name):
+        if name in self.scalars:
+            self.out.write(format_values(np.array([self.scalars[name]])))
+            return
+        t = self._tensor(name)
+        if t.fmt == "Dense":
+            self.out.write(format_values(self._dense(t).to_numpy()))
+            return
+        A = self._sparse(t)
+        unused = np.array([-1], dtype=np.int64)
+        if t.fmt == "CSR":      # A1pos holds the row count, A1crd is unused (SparseUtils.cpp:1898-1936)
+            pos, crd, val = A.to_arrays()
+            parts = [np.array([A.shape[0]], dtype=np.int64), unused, pos, crd, val]
+        elif t.fmt == "COO":
+            row, col, val = A.to_coo()
+            parts = [np.array([0, len(val)], dtype=np.int64), row, unused, col, val]
+        else:
+            parts = list(A.to_dcsr())
+        for p in parts:
+            self.out.write(format_values(p))
+
+    _IDX = r"\[([^\]]*)\]"
+    _RULES = [
+        (r"IndexLabel\s*\[\s*(\w+)\s*\]\s*=\s*\[\s*(\?|\d+)\s*\]", _index_label),
+        (r"Tensor\s*<\s*double\s*>\s*(\w+)\s*\(\s*\[([^\]]*)\]\s*,\s*\{?\s*(\w+)\s*\}?\s*\)", _declare),
+        (r"(\w+)\s*" + _IDX + r"\s*=\s*comet_read\(\s*(\d+)\s*(?:,\s*(\d+)\s*)?\)", _read),
+        (r"(\w+)\s*" + _IDX + r"\s*=\s*([-+]?[0-9.]+(?:[eE][-+]?\d+)?)", _fill),
+        (r"(\w+)\s*" + _IDX + r"\s*(?:<\s*(\w+)\s*,\s*(\w+)\s*>)?\s*=\s*(\w+)\s*" + _IDX +
+         r"\s*(\.\*|\*|@\(\s*([^,()]+),\s*([^,()]+)\))\s*(\w+)\s*" + _IDX, _product),
+        (r"(\w+)\s*" + _IDX + r"\s*=\s*transpose\(\s*(\w+)\s*" + _IDX + r"\s*,\s*\{([^}]*)\}\s*\)", _transpose),
+        (r"var\s+(\w+)\s*=\s*SUM\(\s*(\w+)\s*" + _IDX + r"\s*\)", _sum),
+        (r"var\s+(\w+)\s*=\s*getTime\(\s*\)", _get_time),
+        (r"printElapsedTime\(\s*(\w+)\s*,\s*(\w+)\s*\)", _elapsed),
+        (r"print\(\s*(\w+)\s*\)", _print),
+    ]
+
+
+def run_text(text, out=sys.stdout):
+    rt.init(0)
+    prog = Program(out)
+    prog.run(text)
+    rt.sync()
+    return prog
+
+
+def main(argv=None):
+    argv = sys.argv[1:] if argv is None else argv
+    if len(argv) != 1:
+        sys.exit("usage: python -m comet_amd.ta_run program.ta   (inputs through SPARSE_FILE_NAME<id>)")
+    with open(argv[0]) as f:
+        run_text(f.read())
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,159 @@
+"""The .ta runner against the reference's printed expectations.  The programs are written here from the
+operation each golden entry names (tests/golden/reference_goldens.json cites the reference test it comes
+from); the expectations are turned into CHECK / CHECK-NEXT lines and verified with LLVM's FileCheck when the
+image has it, by exact text comparison otherwise."""
+import io
+import os
+import shutil
+import subprocess
+
+import numpy as np
+import pytest
+
+from comet_amd import ta_run
+
+pytestmark = pytest.mark.gpu
+
+FILECHECK = shutil.which("FileCheck") or "/opt/rocm/lib/llvm/bin/FileCheck"
+
+
+def _run(program, files, tmp_path, monkeypatch, golden_dir):
+    for i, name in enumerate(files):
+        monkeypatch.setenv(f"SPARSE_FILE_NAME{i}", os.path.join(golden_dir, name))
+    out = io.StringIO()
+    ta_run.run_text(program, out)
+    return out.getvalue()
+
+
+def _check(output, expected_text, tmp_path):
+    """expected_text: the printed form, "data = \\n...\\n" blocks in order."""
+    lines = [l for l in expected_text.split("\n") if l != ""]
+    if os.path.exists(FILECHECK):
+        check = tmp_path / "expect.check"
+        check.write_text("\n".join(("# CHECK: " if i == 0 else "# CHECK-NEXT: ") + l for i, l in enumerate(lines)) + "\n")
+        r = subprocess.run([FILECHECK, str(check)], input=output, text=True, capture_output=True)
+        assert r.returncode == 0, r.stderr + "\n--- output ---\n" + output
+    assert [l.rstrip() for l in output.split("\n") if l.strip()] == [l.rstrip() for l in lines]
+
+
+def _decl(fmt_a="CSR"):
+    return f"""
+def main() {{
+    IndexLabel [a] = [?];
+    IndexLabel [b] = [?];
+    IndexLabel [c] = [?];
+    IndexLabel [k4] = [4];
+    Tensor<double> A([a, b], {{{fmt_a}}});
+"""
+
+
+def _ints(v):
+    return "data = \n" + "".join(f"{int(x)}," for x in v) + "\n"
+
+
+@pytest.mark.parametrize("fmt", ["CSR", "COO", "DCSR"])
+def test_spmv_spmm_programs(golden, golden_dir, tmp_path, monkeypatch, fmt):
+    prog = _decl(fmt) + """
+    Tensor<double> x([b], {Dense});
+    Tensor<double> y([a], {Dense});
+    Tensor<double> B([b, k4], {Dense});
+    Tensor<double> C([a, k4], {Dense});
+    A[a, b] = comet_read(0);
+    x[b] = 1.7;   y[a] = 0.0;
+    B[b, k4] = 1.7;   C[a, k4] = 0.0;
+    y[a] = A[a, b] * x[b];
+    C[a, k4] = A[a, b] * B[b, k4];
+    print(y);
+    print(C);
+}
+"""
+    out = _run(prog, ["test_rank2.mtx"], tmp_path, monkeypatch, golden_dir)
+    _check(out, golden["spmv_csr"]["printed"] + golden["spmm_csr"]["printed"], tmp_path)
+
+
+@pytest.mark.parametrize("name", ["plus_times", "min_plus", "any_pair", "plus_second", "min_first"])
+def test_spgemm_semiring_programs(golden, golden_dir, tmp_path, monkeypatch, name):
+    g = golden["spgemm_csr_semiring"]
+    c = g["cases"][name]
+    tok = {"plus": "+", "times": "*"}
+    op = "*" if name == "plus_times" else f"@({tok.get(c['reduce'], c['reduce'])},{tok.get(c['mult'], c['mult'])})"
+    prog = _decl() + f"""
+    Tensor<double> B([b, c], {{CSR}});
+    Tensor<double> C([a, c], {{CSR}});
+    A[a, b] = comet_read(0);
+    B[b, c] = comet_read(1);
+    C[a, c] = A[a, b] {op} B[b, c];
+    print(C);
+}}
+"""
+    out = _run(prog, [g["A"], g["B"]], tmp_path, monkeypatch, golden_dir)
+    want = _ints([len(g["pos"]) - 1]) + _ints([-1]) + _ints(g["pos"]) + _ints(g["crd"]) + c["printed_val"]
+    _check(out, want, tmp_path)
+
+
+def test_triangle_count_program(golden, golden_dir, tmp_path, monkeypatch):
+    prog = """
+def main() {
+    IndexLabel [i] = [?];   IndexLabel [j] = [?];   IndexLabel [k] = [?];
+    Tensor<double> L([i, j], {CSR});
+    Tensor<double> C([i, j], {CSR});
+    L[i, j] = comet_read(0, 2);           # strictly lower triangle
+    C[i, k]<L, push> = L[i, j] * L[j, k];
+    var ntri = SUM(C[i, j]);
+    print(ntri);
+}
+"""
+    out = _run(prog, ["tc.mtx"], tmp_path, monkeypatch, golden_dir)
+    _check(out, "data = \n5,\n", tmp_path)
+
+
+def test_read_modes_and_layout_printing(golden, golden_dir, tmp_path, monkeypatch):
+    for g in golden["read_csr"][2:4]:
+        prog = _decl("CSR") + f"    A[a, b] = comet_read(0, {g['mode']});\n    print(A);\n}}\n"
+        out = _run(prog, [g["matrix"]], tmp_path, monkeypatch, golden_dir)
+        _check(out, _ints([len(g["pos"]) - 1]) + _ints([-1]) + _ints(g["pos"]) + _ints(g["crd"]) + g["printed_val"],
+               tmp_path)
+    for g in golden["read_coo"]:
+        prog = _decl("COO") + f"    A[a, b] = comet_read(0, {g['mode']});\n    print(A);\n}}\n"
+        out = _run(prog, [g["matrix"]], tmp_path, monkeypatch, golden_dir)
+        _check(out, _ints(g["a1pos"]) + _ints(g["a1crd"]) + _ints(g["a2pos"]) + _ints(g["a2crd"]) + g["printed_val"],
+               tmp_path)
+
+
+def test_dense_contraction_sum_transpose_and_elementwise(golden, golden_dir, tmp_path, monkeypatch):
+    prog = """
+def main() {
+    IndexLabel [i] = [3];  IndexLabel [j] = [5];  IndexLabel [k] = [2];  IndexLabel [l] = [4];
+    IndexLabel [r] = [?];  IndexLabel [s] = [?];
+    Tensor<double> A([i, k, j], {Dense});
+    Tensor<double> B([l, k], {Dense});
+    Tensor<double> C([i, j, l], {Dense});
+    Tensor<double> T([j, i, l], {Dense});
+    Tensor<double> S([r, s], {CSR});
+    Tensor<double> P([r, s], {CSR});
+    A[i, k, j] = 2.0;   B[l, k] = 0.25;   C[i, j, l] = 1.5;
+    C[i, j, l] = A[i, k, j] * B[l, k];
+    T[j, i, l] = transpose(C[i, j, l], {j, i, l});
+    var total = SUM(T[j, i, l]);
+    print(total);
+    S[r, s] = comet_read(0);
+    P[r, s] = S[r, s] .* S[r, s];
+    var sq = SUM(P[r, s]);
+    print(sq);
+    var t0 = getTime();
+    var t1 = getTime();
+    printElapsedTime(t0, t1);
+}
+"""
+    out = _run(prog, ["test_rank2.mtx"], tmp_path, monkeypatch, golden_dir)
+    lines = out.strip().split("\n")
+    # every C element: 1.5 + 2 terms of 2.0*0.25 = 2.5; 60 elements
+    assert lines[0].strip() == "data =" and lines[1] == "150,"
+    vals = np.array([1, 1.4, 2, 2.5, 3, 4.1, 4, 5.2, 5])
+    assert lines[3] == f"{(vals * vals).sum():g},"
+    assert lines[4].startswith("ELAPSED_TIME = ")
+
+
+def test_unsupported_statement_is_named():
+    with pytest.raises(ta_run.TaError, match="not supported"):
+        ta_run.Program().run("def main() { IndexLabel [a] = [4]; for (x in a) {} }")
