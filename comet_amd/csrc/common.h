@@ -76,12 +76,15 @@ struct Csr {
     int32_t *heavy_row = nullptr;            // [heavy_rows] row ids of the long rows
     int32_t *heavy_code = nullptr;           // [8][heavy_rows] wavefront * 8 + slot that holds the row on each XCD
     Csr *light = nullptr;
+    // the transpose, built the first time a dense-times-sparse product needs it
+    Csr *transposed = nullptr;
 };
 
 Csr *csr_from_handle(int64_t h);           // nullptr (and error set) if unknown
 int64_t csr_register(Csr *c);              // takes ownership of the struct
 int csr_alloc(Csr *c, int64_t nrows, int64_t ncols, int64_t nnz);   // allocates pos/crd/val, owns = true
 void csr_release(Csr *c);                  // frees the arrays it owns, its plans and the struct
+Csr *csr_transposed_copy(const Csr *a);    // new unregistered struct holding the transpose (nullptr on failure)
 
 // Records an event pair around a kernel launch when profiling is on.
 struct KernelTimer {

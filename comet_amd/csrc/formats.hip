@@ -292,19 +292,30 @@ int sort_pairs_u64_u32(const uint64_t *keys_in, uint64_t *keys_out, const uint32
 static inline dim3 grid_for(int64_t n) { return dim3((unsigned)(n > 0 ? ceil_div(n, 256) : 1)); }
 
 // row/col/val are device arrays of n tuples in input order; returns a new registered handle or 0
+static Csr *coo_device_to_csr_struct(int64_t nrows, int64_t ncols, int64_t n, const int32_t *row,
+                                     const int32_t *col, const double *val, int mode);
+
 static int64_t coo_device_to_csr(int64_t nrows, int64_t ncols, int64_t n, const int32_t *row, const int32_t *col,
                                  const double *val, int mode)
+{
+    Csr *c = coo_device_to_csr_struct(nrows, ncols, n, row, col, val, mode);
+    return c ? csr_register(c) : 0;
+}
+
+// the same, as a struct that no handle names yet (nullptr on failure)
+static Csr *coo_device_to_csr_struct(int64_t nrows, int64_t ncols, int64_t n, const int32_t *row,
+                                     const int32_t *col, const double *val, int mode)
 {
     Csr *c = new Csr();
     c->nrows = nrows;
     c->ncols = ncols;
     c->owns = true;
-    auto fail = [&]() -> int64_t {
+    auto fail = [&]() -> Csr * {
         (void)hipFree(c->pos);
         (void)hipFree(c->crd);
         (void)hipFree(c->val);
         delete c;
-        return 0;
+        return nullptr;
     };
     if (hipMalloc((void **)&c->pos, sizeof(int64_t) * (size_t)(nrows + 1)) != hipSuccess) {
         set_error(COMET_HIP_ERR_HIP, "row pointer allocation failed");
@@ -363,7 +374,7 @@ static int64_t coo_device_to_csr(int64_t nrows, int64_t ncols, int64_t n, const 
         set_error(COMET_HIP_ERR_HIP, "building the CSR arrays failed");
         return fail();
     }
-    return csr_register(c);
+    return c;
 }
 
 static int64_t coo_host_to_csr(int64_t nrows, int64_t ncols, int64_t n, const int32_t *row, const int32_t *col,
@@ -381,6 +392,20 @@ static int64_t coo_host_to_csr(int64_t nrows, int64_t ncols, int64_t n, const in
         return 0;
     }
     return coo_device_to_csr(nrows, ncols, n, drow.as<int32_t>(), dcol.as<int32_t>(), dval.as<double>(), mode);
+}
+
+Csr *csr_transposed_copy(const Csr *a)
+{
+    DevBuf rowid;
+    if (rowid.alloc(4 * (size_t)a->nnz))
+        return nullptr;
+    if (a->nnz > 0) {
+        KernelTimer t("csr_expand_rows");
+        csr_expand_rows<<<grid_for(a->nnz), dim3(256), 0, stream()>>>(a->nrows, a->nnz, a->pos, rowid.as<int32_t>());
+    }
+    // the tuples of the transpose are (column, row, value): order them by (column, row)
+    return coo_device_to_csr_struct(a->ncols, a->nrows, a->nnz, a->crd, rowid.as<int32_t>(), a->val,
+                                    COMET_READ_DEFAULT);
 }
 
 static bool known_mode(int mode) { return mode >= COMET_READ_DEFAULT && mode <= COMET_READ_UPPER_TRI; }
@@ -633,15 +658,8 @@ extern "C" int64_t comet_hip_csr_transpose(int64_t h)
     Csr *a = csr_from_handle(h);
     if (!a)
         return 0;
-    DevBuf rowid;
-    if (rowid.alloc(4 * (size_t)a->nnz))
-        return 0;
-    if (a->nnz > 0) {
-        KernelTimer t("csr_expand_rows");
-        csr_expand_rows<<<grid_for(a->nnz), dim3(256), 0, stream()>>>(a->nrows, a->nnz, a->pos, rowid.as<int32_t>());
-    }
-    // the tuples of the transpose are (column, row, value): order them by (column, row)
-    return coo_device_to_csr(a->ncols, a->nrows, a->nnz, a->crd, rowid.as<int32_t>(), a->val, COMET_READ_DEFAULT);
+    Csr *t = csr_transposed_copy(a);
+    return t ? csr_register(t) : 0;
 }
 
 extern "C" int64_t comet_hip_read_input_2D_handle(int32_t file_id, int32_t read_mode)

@@ -138,6 +138,8 @@ void csr_release(Csr *c)
 {
     if (c->light)
         csr_release(c->light);
+    if (c->transposed)
+        csr_release(c->transposed);
     (void)hipFree(c->heavy_seg);
     (void)hipFree(c->heavy_col);
     (void)hipFree(c->heavy_val);

@@ -695,6 +695,29 @@ __global__ void eltwise_mult_kernel(int64_t nrows, const int64_t *__restrict__ A
         rowcount[i] = n;
 }
 
+// CSR .* Dense: the stored entries of A times the dense values under them.  TO_DENSE writes them into a dense
+// output at their positions and leaves every other element as it was (the nest only visits the entries of
+// A, test/integration/ops/eltwise_mult_CSRxDense_oDense.ta); otherwise they become the values of a CSR with
+// A's structure (eltwise_mult_CSRxDense_oCSR.ta).
+template <bool TO_DENSE>
+__global__ void eltwise_mult_dense_kernel(int64_t nrows, const int64_t *__restrict__ pos,
+                                          const int32_t *__restrict__ crd, const double *__restrict__ val,
+                                          const double *__restrict__ D, int64_t ldd, double *__restrict__ out,
+                                          int64_t ldo)
+{
+    // one 16-lane group per row
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+    if (i >= nrows)
+        return;
+    for (int64_t p = pos[i] + (threadIdx.x & 15); p < pos[i + 1]; p += 16) {
+        const double v = val[p] * D[i * ldd + crd[p]];
+        if (TO_DENSE)
+            out[i * ldo + crd[p]] = v;
+        else
+            out[p] = v;
+    }
+}
+
 // ------------------------------------------------------------------ host side
 struct SgScratch {
     Workspace ticket;     // one 64-bit row counter
@@ -1090,4 +1113,55 @@ extern "C" int64_t comet_hip_eltwise_mult_csr(int64_t ah, int64_t bh)
         return fail(c);
     }
     return csr_register(c);
+}
+
+extern "C" int64_t comet_hip_eltwise_mult_csr_dense_csr(int64_t ah, int64_t d_dptr, int64_t ldd)
+{
+    if (ensure_init() != COMET_HIP_OK)
+        return 0;
+    Csr *a = csr_from_handle(ah);
+    if (!a)
+        return 0;
+    if (ldd < a->ncols || (a->nnz > 0 && !d_dptr)) {
+        set_error(COMET_HIP_ERR_ARG, "bad dense operand passed to comet_hip_eltwise_mult_csr_dense_csr");
+        return 0;
+    }
+    Csr *c = new Csr();
+    if (csr_alloc(c, a->nrows, a->ncols, a->nnz) != COMET_HIP_OK) {
+        delete c;
+        return 0;
+    }
+    bool ok = hipMemcpyAsync(c->pos, a->pos, sizeof(int64_t) * (size_t)(a->nrows + 1), hipMemcpyDeviceToDevice,
+                             stream()) == hipSuccess;
+    if (ok && a->nnz > 0) {
+        ok = hipMemcpyAsync(c->crd, a->crd, sizeof(int32_t) * (size_t)a->nnz, hipMemcpyDeviceToDevice, stream()) ==
+             hipSuccess;
+        KernelTimer t("eltwise_mult_dense");
+        eltwise_mult_dense_kernel<false><<<dim3((unsigned)ceil_div(a->nrows * 16, 256)), dim3(256), 0, stream()>>>(
+            a->nrows, a->pos, a->crd, a->val, (const double *)d_dptr, ldd, c->val, 0);
+    }
+    if (!ok || hipGetLastError() != hipSuccess) {
+        set_error(COMET_HIP_ERR_HIP, "CSR .* Dense failed");
+        csr_release(c);
+        return 0;
+    }
+    return csr_register(c);
+}
+
+extern "C" int comet_hip_eltwise_mult_csr_dense_dense(int64_t ah, int64_t d_dptr, int64_t ldd, int64_t c_dptr,
+                                                      int64_t ldc)
+{
+    COMET_CHK(ensure_init());
+    Csr *a = csr_from_handle(ah);
+    if (!a)
+        return COMET_HIP_ERR_HANDLE;
+    if (ldd < a->ncols || ldc < a->ncols || (a->nnz > 0 && (!d_dptr || !c_dptr)))
+        return set_error(COMET_HIP_ERR_ARG, "bad dense operand passed to comet_hip_eltwise_mult_csr_dense_dense");
+    if (a->nnz == 0)
+        return COMET_HIP_OK;
+    KernelTimer t("eltwise_mult_dense");
+    eltwise_mult_dense_kernel<true><<<dim3((unsigned)ceil_div(a->nrows * 16, 256)), dim3(256), 0, stream()>>>(
+        a->nrows, a->pos, a->crd, a->val, (const double *)d_dptr, ldd, (double *)c_dptr, ldc);
+    COMET_HIPCHK(hipGetLastError());
+    return COMET_HIP_OK;
 }

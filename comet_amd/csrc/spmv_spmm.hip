@@ -831,6 +831,8 @@ static int spmm_heavy_plan(Csr *a)
 using namespace comet;
 
 static int spmm_chunks(Csr *a, int64_t K, const double *B, int64_t ldb, double *C, int64_t ldc, int accumulate);
+static int spmv_run(Csr *a, int64_t x_dptr, int64_t y_dptr, int accumulate);
+static int spmm_run(Csr *a, int64_t K, int64_t b_dptr, int64_t ldb, int64_t c_dptr, int64_t ldc, int accumulate);
 
 extern "C" int comet_hip_spmv_csr_f64(int64_t csr, int64_t x_dptr, int64_t y_dptr, int accumulate)
 {
@@ -838,8 +840,13 @@ extern "C" int comet_hip_spmv_csr_f64(int64_t csr, int64_t x_dptr, int64_t y_dpt
     Csr *a = csr_from_handle(csr);
     if (!a)
         return COMET_HIP_ERR_HANDLE;
+    return spmv_run(a, x_dptr, y_dptr, accumulate);
+}
+
+static int spmv_run(Csr *a, int64_t x_dptr, int64_t y_dptr, int accumulate)
+{
     if ((a->ncols > 0 && !x_dptr) || (a->nrows > 0 && !y_dptr))
-        return set_error(COMET_HIP_ERR_ARG, "null vector passed to comet_hip_spmv_csr_f64");
+        return set_error(COMET_HIP_ERR_ARG, "null vector passed to a sparse matrix-vector product");
     if (a->nrows == 0)
         return COMET_HIP_OK;
     COMET_CHK(spmv_plan(a));
@@ -868,13 +875,18 @@ extern "C" int comet_hip_spmm_csr_f64(int64_t csr, int64_t K, int64_t b_dptr, in
     Csr *a = csr_from_handle(csr);
     if (!a)
         return COMET_HIP_ERR_HANDLE;
+    return spmm_run(a, K, b_dptr, ldb, c_dptr, ldc, accumulate);
+}
+
+static int spmm_run(Csr *a, int64_t K, int64_t b_dptr, int64_t ldb, int64_t c_dptr, int64_t ldc, int accumulate)
+{
     if (K < 0 || ldb < K || ldc < K)
         return set_error(COMET_HIP_ERR_ARG, "bad K/ldb/ldc (%lld, %lld, %lld)", (long long)K, (long long)ldb,
                          (long long)ldc);
     if (K == 0 || a->nrows == 0)
         return COMET_HIP_OK;
     if (!c_dptr || (a->nnz > 0 && !b_dptr))
-        return set_error(COMET_HIP_ERR_ARG, "null matrix passed to comet_hip_spmm_csr_f64");
+        return set_error(COMET_HIP_ERR_ARG, "null matrix passed to a sparse-dense matrix product");
     double *C = (double *)c_dptr;
     const double *B = (const double *)b_dptr;
     if (ceil_div(K, 64) > 65535)
@@ -943,4 +955,94 @@ static int spmm_chunks(Csr *a, int64_t K, const double *B, int64_t ldb, double *
     }
     COMET_HIPCHK(hipGetLastError());
     return COMET_HIP_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Dense operand on the left: y[j] (+)= sum_i x[i] * B[i,j] and
+// C[a,c] (+)= sum_b A[a,b] * B[b,c] with B in CSR.  The reference's nests run
+// over the dense index outermost and scatter into the output
+// (test/integration/ops/mult_DenseVecxCSR.ta, mult_DenseMatxCSR.ta through
+// lib/Conversion/IndexTreeToSCF/IndexTreeToSCF.cpp:529-700,1247-1284), so an
+// output element receives its products in ascending order of the contracted
+// index.  That is the order in which the transpose of B holds them, so both
+// products run as SpMV / SpMM over the transpose (built once, kept in the
+// handle) and round like the reference; the dense matrix operands are turned
+// by a tiled transpose on the way in and out.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void transpose2d_tile(const double *__restrict__ in, int64_t ld_in, int64_t rows,
+                                                        int64_t cols, double *__restrict__ out, int64_t ld_out)
+{
+    __shared__ double tile[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;       // 32 x 8 threads
+    const int64_t r0 = (int64_t)blockIdx.y * 32, c0 = (int64_t)blockIdx.x * 32;
+    for (int k = ty; k < 32; k += 8)
+        if (r0 + k < rows && c0 + tx < cols)
+            tile[k][tx] = in[(r0 + k) * ld_in + c0 + tx];
+    __syncthreads();
+    for (int k = ty; k < 32; k += 8)
+        if (c0 + k < cols && r0 + tx < rows)
+            out[(c0 + k) * ld_out + r0 + tx] = tile[tx][k];
+}
+
+static int transpose2d(const double *in, int64_t ld_in, int64_t rows, int64_t cols, double *out, int64_t ld_out)
+{
+    if (rows == 0 || cols == 0)
+        return COMET_HIP_OK;
+    if (ceil_div(rows, 32) > 65535)
+        return set_error(COMET_HIP_ERR_SIZE, "dense operand with %lld rows is too tall to turn", (long long)rows);
+    KernelTimer t("transpose2d_tile");
+    transpose2d_tile<<<dim3((unsigned)ceil_div(cols, 32), (unsigned)ceil_div(rows, 32)), dim3(256), 0, stream()>>>(
+        in, ld_in, rows, cols, out, ld_out);
+    COMET_HIPCHK(hipGetLastError());
+    return COMET_HIP_OK;
+}
+
+static int transposed_of(Csr *b, Csr **out)
+{
+    if (!b->transposed) {
+        b->transposed = csr_transposed_copy(b);
+        if (!b->transposed)
+            return COMET_HIP_ERR_HIP;
+    }
+    *out = b->transposed;
+    return COMET_HIP_OK;
+}
+
+extern "C" int comet_hip_vecmat_csr_f64(int64_t csr, int64_t x_dptr, int64_t y_dptr, int accumulate)
+{
+    COMET_CHK(ensure_init());
+    Csr *b = csr_from_handle(csr);
+    if (!b)
+        return COMET_HIP_ERR_HANDLE;
+    Csr *t = nullptr;
+    COMET_CHK(transposed_of(b, &t));
+    return spmv_run(t, x_dptr, y_dptr, accumulate);
+}
+
+static Workspace g_left_a, g_left_c;
+
+extern "C" int comet_hip_densemat_csr_f64(int64_t csr, int64_t M, int64_t a_dptr, int64_t lda, int64_t c_dptr,
+                                          int64_t ldc, int accumulate)
+{
+    COMET_CHK(ensure_init());
+    Csr *b = csr_from_handle(csr);
+    if (!b)
+        return COMET_HIP_ERR_HANDLE;
+    if (M < 0 || lda < b->nrows || ldc < b->ncols)
+        return set_error(COMET_HIP_ERR_ARG, "bad M/lda/ldc (%lld, %lld, %lld)", (long long)M, (long long)lda,
+                         (long long)ldc);
+    if (M == 0 || b->ncols == 0)
+        return COMET_HIP_OK;
+    if (!c_dptr || (b->nrows > 0 && !a_dptr))
+        return set_error(COMET_HIP_ERR_ARG, "null matrix passed to comet_hip_densemat_csr_f64");
+    Csr *t = nullptr;
+    COMET_CHK(transposed_of(b, &t));
+    COMET_CHK(g_left_a.ensure(sizeof(double) * (size_t)(b->nrows > 0 ? b->nrows : 1) * (size_t)M, false));
+    COMET_CHK(g_left_c.ensure(sizeof(double) * (size_t)b->ncols * (size_t)M, false));
+    double *at = (double *)g_left_a.ptr, *ct = (double *)g_left_c.ptr;
+    COMET_CHK(transpose2d((const double *)a_dptr, lda, M, b->nrows, at, M));
+    if (accumulate)
+        COMET_CHK(transpose2d((const double *)c_dptr, ldc, M, b->ncols, ct, M));
+    COMET_CHK(spmm_run(t, M, (int64_t)at, M, (int64_t)ct, M, accumulate));
+    return transpose2d(ct, M, b->ncols, M, (double *)c_dptr, ldc);
 }

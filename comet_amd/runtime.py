@@ -80,6 +80,10 @@ SIGNATURES = {
     "comet_hip_spgemm_csr": (_i64, [_i64, _i64, _i64]),
     "comet_hip_spgemm_csr_numeric_semiring": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int]),
     "comet_hip_spgemm_csr_semiring": (_i64, [_i64, _i64, _i64, _int, _int]),
+    "comet_hip_vecmat_csr_f64": (_int, [_i64, _i64, _i64, _int]),
+    "comet_hip_densemat_csr_f64": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
+    "comet_hip_eltwise_mult_csr_dense_csr": (_i64, [_i64, _i64, _i64]),
+    "comet_hip_eltwise_mult_csr_dense_dense": (_int, [_i64, _i64, _i64, _i64, _i64]),
     "comet_hip_mtx_read_csr": (_i64, [C.c_char_p, _int]),
     "comet_hip_read_input_sizes_2D_f64": (None, [_i32, _i32, _i32, _i32, _i32, _int, _vp, _i32]),
     "comet_hip_read_input_2D_f64_i64": (None, [_i32, _i32, _i32, _i32, _i32] + [_int, _vp] * 9 + [_i32]),
@@ -444,6 +448,47 @@ def sum_values(A):
     out = C.c_double()
     _check(lib().comet_hip_reduce_sum_f64(v, A.nnz, C.byref(out)), "comet_hip_reduce_sum_f64")
     return out.value
+
+
+def vecmat(x, B, y=None, accumulate=None):
+    """y (+)= x @ B for a dense vector x and a sparse B."""
+    nrows, ncols = B.shape
+    if x.size != nrows:
+        raise ValueError("x has the wrong length")
+    if y is None:
+        y, accumulate = DeviceArray(ncols), False
+    elif accumulate is None:
+        accumulate = True
+    _check(lib().comet_hip_vecmat_csr_f64(B.handle, x.ptr, y.ptr, int(accumulate)), "comet_hip_vecmat_csr_f64")
+    return y
+
+
+def densemat(A, B, Cm=None, accumulate=None):
+    """C (+)= A @ B for a dense A (M x nrows(B)) and a sparse B."""
+    nrows, ncols = B.shape
+    if len(A.shape) != 2 or A.shape[1] != nrows:
+        raise ValueError("A has the wrong shape")
+    M = A.shape[0]
+    if Cm is None:
+        Cm, accumulate = DeviceArray((M, ncols)), False
+    elif accumulate is None:
+        accumulate = True
+    _check(lib().comet_hip_densemat_csr_f64(B.handle, M, A.ptr, nrows, Cm.ptr, ncols, int(accumulate)),
+           "comet_hip_densemat_csr_f64")
+    return Cm
+
+
+def eltwise_mult_dense(A, D, out=None):
+    """A .* D for a sparse A and a dense D of the same shape: a CsrMatrix with A's structure, or, when a
+    dense `out` is given, written into it at A's stored positions."""
+    if tuple(D.shape) != tuple(A.shape):
+        raise ValueError("operands differ in shape")
+    if out is None:
+        return CsrMatrix(_handle(lib().comet_hip_eltwise_mult_csr_dense_csr(A.handle, D.ptr, A.shape[1]),
+                                 "comet_hip_eltwise_mult_csr_dense_csr"))
+    _check(lib().comet_hip_eltwise_mult_csr_dense_dense(A.handle, D.ptr, A.shape[1], out.ptr, A.shape[1]),
+           "comet_hip_eltwise_mult_csr_dense_dense")
+    return out
 
 
 def eltwise_mult(A, B):

@@ -13,10 +13,10 @@ include/comet_hip_rt.h.  Statements it understands (frontends/comet_dsl/include/
     Tensor<double> A([a, b], {CSR}); formats Dense, CSR, COO, DCSR
     A[a, b] = comet_read(0);         A[a, b] = comet_read(0, 3);      (file id, read mode)
     B[b, c] = 1.7;                   (fill)
-    C[a, c] = A[a, b] * B[b, c];     SpMV, SpMM, SpGEMM, dense contraction (TTGT)
+    C[a, c] = A[a, b] * B[b, c];     SpMV, SpMM, dense x sparse, SpGEMM, dense contraction (TTGT)
     C[a, c] = A[a, b] @(min,+) B[b, c];                               (SpGEMM over a semiring)
     C[i, k]<M, push> = A[i, j] * B[j, k];                             (masked SpGEMM)
-    C[i, j] = A[i, j] .* B[i, j];    (CSR .* CSR)
+    C[i, j] = A[i, j] .* B[i, j];    (CSR .* CSR, CSR .* Dense, Dense .* CSR)
     B[j, i] = transpose(A[i, j], {j, i});                             (dense)
     var s = SUM(C[i, j]);  var t = getTime();  printElapsedTime(t0, t1);  print(C);  print(s);
 
@@ -158,9 +158,32 @@ class Program:
             except KeyError:
                 raise TaError(f"semiring @({red},{mul}) is not supported") from None
         if op == ".*":
-            if not (a.fmt == b.fmt == c.fmt == "CSR") or not (al == bl == cl):
-                raise TaError("elementwise .* is supported for CSR .* CSR -> CSR over the same indices")
-            c.value = rt.eltwise_mult(self._sparse(a), self._sparse(b))
+            if not (al == bl == cl) or len(al) != 2:
+                raise TaError("elementwise .* is supported for matrices over the same indices")
+            if a.fmt == b.fmt == c.fmt == "CSR":
+                c.value = rt.eltwise_mult(self._sparse(a), self._sparse(b))
+                return
+            sp_, de_ = (a, b) if a.fmt == "CSR" else (b, a)
+            if sp_.fmt == "CSR" and de_.fmt == "Dense" and c.fmt in ("CSR", "Dense"):
+                S = self._sparse(sp_)
+                self._bind(al, S.shape)
+                if c.fmt == "CSR":
+                    c.value = rt.eltwise_mult_dense(S, self._dense(de_))
+                else:
+                    rt.eltwise_mult_dense(S, self._dense(de_), self._dense(c))
+                return
+            raise TaError("elementwise .* is supported for CSR .* CSR -> CSR and CSR .* Dense -> CSR or Dense")
+        if a.fmt == "Dense" and b.fmt != "Dense" and c.fmt == "Dense":
+            if semiring not in (None, ("plus", "times")) or mask:
+                raise TaError("semirings and masks are supported for sparse x sparse products")
+            Bm = self._sparse(b)
+            self._bind(bl, Bm.shape)
+            if len(bl) == 2 and al == [bl[0]] and cl == [bl[1]]:
+                rt.vecmat(self._dense(a), Bm, self._dense(c), accumulate=True)
+            elif len(bl) == 2 and len(al) == 2 and al[1] == bl[0] and cl == [al[0], bl[1]]:
+                rt.densemat(self._dense(a), Bm, self._dense(c), accumulate=True)
+            else:
+                raise TaError("dense x sparse is supported as C[b] = A[a]*B[a,b] and C[a,c] = A[a,b]*B[b,c]")
             return
         if a.fmt != "Dense" and b.fmt == "Dense" and c.fmt == "Dense":
             if semiring not in (None, ("plus", "times")) or mask:

@@ -149,6 +149,24 @@ int comet_hip_spgemm_csr_numeric_semiring(int64_t a, int64_t b, int64_t mask, in
                                           int reduce_op, int mult_op);
 int64_t comet_hip_spgemm_csr_semiring(int64_t a, int64_t b, int64_t mask, int reduce_op, int mult_op);
 
+/* ---- dense operand on the left, and CSR .* Dense ------------------------------
+ * y[j] (+)= sum_i x[i]*B[i,j] (test/integration/ops/mult_DenseVecxCSR.ta) and
+ * C[a,c] (+)= sum_b A[a,b]*B[b,c], A: M x nrows(B) row-major with leading
+ * dimension lda, C: M x ncols(B) (mult_DenseMatxCSR.ta); same index-tree lowering
+ * as SpMV/SpMM with the sparse operand second.  An output element receives its
+ * products in ascending order of the contracted index, as in the reference. */
+int comet_hip_vecmat_csr_f64(int64_t csr, int64_t x_dptr, int64_t y_dptr, int accumulate);
+int comet_hip_densemat_csr_f64(int64_t csr, int64_t M, int64_t a_dptr, int64_t lda,
+                               int64_t c_dptr, int64_t ldc, int accumulate);
+/* C = A .* D for A in CSR and D dense (row-major, leading dimension ldd), with
+ * either operand order of the source program (the product commutes): as a new
+ * CSR with A's structure (eltwise_mult_CSRxDense_oCSR.ta), or written into a
+ * dense C at A's stored positions, every other element of C left as it is
+ * (eltwise_mult_CSRxDense_oDense.ta, eltwise_mult_DensexCSR_oDense.ta). */
+int64_t comet_hip_eltwise_mult_csr_dense_csr(int64_t a, int64_t d_dptr, int64_t ldd);
+int comet_hip_eltwise_mult_csr_dense_dense(int64_t a, int64_t d_dptr, int64_t ldd,
+                                           int64_t c_dptr, int64_t ldc);
+
 /* ---- input side: MatrixMarket files, read modes, the file-id protocol ---------
  * Read modes of comet_read(id, mode): lib/ExecutionEngine/SparseUtils.cpp:40-64.
  * Storage format codes per dimension: include/comet/ExecutionEngine/

@@ -89,6 +89,51 @@ void oracle_spmm_csr(idx_t nrows, idx_t K, const idx_t *pos, const idx_t *crd,
 }
 
 /* ------------------------------------------------------------------------- */
+/* Dense operand on the left, sparse on the right (same builders as SpMV/SpMM; */
+/* the dense index is the outer loop and the output is scattered into):        */
+/*   y[crd[p]] = y[crd[p]] + x[i] * val[p]              loop order i -> p       */
+/*     test/integration/ops/mult_DenseVecxCSR.ta                               */
+/*   C[a,crd[p]] = C[a,crd[p]] + A[a,b] * val[p]        loop order a -> b -> p  */
+/*     test/integration/ops/mult_DenseMatxCSR.ta                               */
+/* A is M x nrows, C is M x ncols, both row-major.                             */
+/* ------------------------------------------------------------------------- */
+void oracle_vecmat_csr(idx_t nrows, const idx_t *pos, const idx_t *crd,
+                       const double *val, const double *x, double *y)
+{
+    for (idx_t i = 0; i < nrows; ++i)
+        for (idx_t p = pos[i]; p < pos[i + 1]; ++p) {
+            double prod = x[i] * val[p];
+            y[crd[p]] = y[crd[p]] + prod;
+        }
+}
+
+void oracle_densemat_csr(idx_t M, idx_t nrows, idx_t ncols, const double *A,
+                         const idx_t *pos, const idx_t *crd, const double *val, double *C)
+{
+    for (idx_t a = 0; a < M; ++a)
+        for (idx_t b = 0; b < nrows; ++b)
+            for (idx_t p = pos[b]; p < pos[b + 1]; ++p) {
+                double prod = A[a * nrows + b] * val[p];
+                C[a * ncols + crd[p]] = C[a * ncols + crd[p]] + prod;
+            }
+}
+
+/* ------------------------------------------------------------------------- */
+/* CSR .* Dense: out[p] = val[p] * D[i, crd[p]] over the stored entries of A   */
+/* (the "noop_times" compute of an elementwise statement assigns, it does not  */
+/* accumulate: lib/Conversion/IndexTreeToSCF/IndexTreeToSCF.cpp:346-353,       */
+/* 1249-1284; frontends/comet_dsl/mlir/MLIRGen.cpp:960-990).  The caller puts  */
+/* out[p] into a CSR with A's structure or into a dense C at (i, crd[p]).      */
+/* ------------------------------------------------------------------------- */
+void oracle_eltwise_mult_csr_dense(idx_t nrows, idx_t ncols, const idx_t *pos, const idx_t *crd,
+                                   const double *val, const double *D, double *out)
+{
+    for (idx_t i = 0; i < nrows; ++i)
+        for (idx_t p = pos[i]; p < pos[i + 1]; ++p)
+            out[p] = val[p] * D[i * ncols + crd[p]];
+}
+
+/* ------------------------------------------------------------------------- */
 /* SpGEMM symbolic phase over rows [row_begin,row_end).                        */
 /* Mark-array counting of distinct output columns per row:                     */
 /*   lib/Dialect/IndexTree/Transforms/SymbolicCompute.cpp:215-339 (tree),      */

@@ -53,6 +53,12 @@ def lib():
     L.oracle_spmv_csr.restype = None
     L.oracle_spmm_csr.argtypes = [C.c_int64, C.c_int64, i64p, i64p, f64p, f64p, f64p]
     L.oracle_spmm_csr.restype = None
+    L.oracle_vecmat_csr.argtypes = [C.c_int64, i64p, i64p, f64p, f64p, f64p]
+    L.oracle_vecmat_csr.restype = None
+    L.oracle_densemat_csr.argtypes = [C.c_int64, C.c_int64, C.c_int64, f64p, i64p, i64p, f64p, f64p]
+    L.oracle_densemat_csr.restype = None
+    L.oracle_eltwise_mult_csr_dense.argtypes = [C.c_int64, C.c_int64, i64p, i64p, f64p, f64p, f64p]
+    L.oracle_eltwise_mult_csr_dense.restype = None
     L.oracle_spgemm_symbolic.argtypes = [C.c_int64, C.c_int64, C.c_int64, i64p, i64p, i64p, i64p, vp, vp, i64p]
     L.oracle_spgemm_symbolic.restype = C.c_int64
     L.oracle_spgemm_numeric.argtypes = [C.c_int64, C.c_int64, C.c_int64, i64p, i64p, f64p, i64p, i64p, f64p,
@@ -118,6 +124,28 @@ def spmm(pos, crd, val, B, C0=None):
     Cm = np.zeros((n, K)) if C0 is None else _f64(C0).copy()
     lib().oracle_spmm_csr(n, K, pos, crd, val, B, Cm)
     return Cm
+
+
+def vecmat(x, pos, crd, val, ncols, y0=None):
+    pos, crd, val, x = _i64(pos), _i64(crd), _f64(val), _f64(x)
+    y = np.zeros(ncols) if y0 is None else _f64(y0).copy()
+    lib().oracle_vecmat_csr(len(pos) - 1, pos, crd, val, x, y)
+    return y
+
+
+def densemat(A, pos, crd, val, ncols, C0=None):
+    pos, crd, val, A = _i64(pos), _i64(crd), _f64(val), _f64(A)
+    Cm = np.zeros((A.shape[0], ncols)) if C0 is None else _f64(C0).copy()
+    lib().oracle_densemat_csr(A.shape[0], len(pos) - 1, ncols, A, pos, crd, val, Cm)
+    return Cm
+
+
+def eltwise_mult_dense(pos, crd, val, D):
+    """Values of A .* D at A's stored positions, in storage order."""
+    pos, crd, val, D = _i64(pos), _i64(crd), _f64(val), _f64(D)
+    out = np.zeros(max(len(val), 1))
+    lib().oracle_eltwise_mult_csr_dense(len(pos) - 1, D.shape[1], pos, crd, val, D, out)
+    return out[:len(val)]
 
 
 def spgemm_symbolic(Apos, Acrd, Bpos, Bcrd, ncolsB, mask=None, rows=None):

@@ -798,3 +798,52 @@ def test_spmm_more_long_rows_than_the_sweep_holds():
     crd = np.concatenate([np.sort(rng.choice(m, l, replace=False)) for l in lens]).astype(np.int64)
     val = rng.uniform(-1, 1, len(crd))
     assert _sweep_check(pos, crd, val, gen.dense((m, 64), seed=2)) == 4096
+
+
+# ----------------------------------------------------------------- dense operand on the left, CSR .* Dense
+def test_vecmat_densemat_eltwise_dense_golden(golden, golden_dir):
+    A = rt.CsrMatrix.from_mtx(os.path.join(golden_dir, "test_rank2.mtx"))
+    nr, nc = A.shape
+    g = golden["vecmat_csr"]
+    y = rt.vecmat(rt.DeviceArray.from_numpy(np.full(nr, g["x_fill"])), A, rt.DeviceArray(nc, zero=True))
+    assert orc.format_f64(y.to_numpy()) == g["printed"]
+    g = golden["densemat_csr"]
+    Cm = rt.densemat(rt.DeviceArray.from_numpy(np.full((g["M"], nr), g["a_fill"])), A,
+                     rt.DeviceArray((g["M"], nc), zero=True))
+    assert orc.format_f64(Cm.to_numpy()) == g["printed"]
+    g = golden["eltwise_mult_csr_dense"]
+    D = rt.DeviceArray.from_numpy(np.full((nr, nc), g["d_fill"]))
+    p, c, v = rt.eltwise_mult_dense(A, D).to_arrays()
+    assert p.tolist() == g["pos"] and c.tolist() == g["crd"] and orc.format_f64(v) == g["printed_val"]
+    out = rt.eltwise_mult_dense(A, D, rt.DeviceArray((nr, nc), zero=True))
+    assert orc.format_f64(out.to_numpy()) == g["printed_dense"]
+
+
+@pytest.mark.parametrize("n,m,M,density,seed", [(300, 200, 7, 0.05, 0), (1000, 1500, 64, 0.02, 1), (50, 3000, 33, 0.2, 2)])
+def test_vecmat_densemat_vs_checker(n, m, M, density, seed):
+    rng = np.random.default_rng(seed)
+    pos, crd, val = _rand_csr(rng, n, m, density)
+    B = rt.CsrMatrix.from_arrays((n, m), pos, crd, val)
+    x, y0 = rng.uniform(-1, 1, n), rng.uniform(-1, 1, m)
+    y = rt.vecmat(rt.DeviceArray.from_numpy(x), B, rt.DeviceArray.from_numpy(y0)).to_numpy()
+    assert np.array_equal(y, orc.vecmat(x, pos, crd, val, m, y0))             # same order of additions: bit-exact
+    assert np.array_equal(rt.vecmat(rt.DeviceArray.from_numpy(x), B).to_numpy(), orc.vecmat(x, pos, crd, val, m))
+    A, C0 = rng.uniform(-1, 1, (M, n)), rng.uniform(-1, 1, (M, m))
+    want = orc.densemat(A, pos, crd, val, m, C0)
+    got = rt.densemat(rt.DeviceArray.from_numpy(A), B, rt.DeviceArray.from_numpy(C0)).to_numpy()
+    bound = orc.densemat(np.abs(A), pos, crd, np.abs(val), m, np.abs(C0))
+    assert np.all(np.abs(got - want) <= RTOL * bound)
+    tpos = np.concatenate([[0], np.cumsum(np.bincount(crd, minlength=m))])
+    inside = tpos[:-1] // 256 == (np.maximum(tpos[1:], tpos[:-1] + 1) - 1) // 256   # columns summed by one wavefront
+    assert np.array_equal(got[:, inside], want[:, inside])
+    got0 = rt.densemat(rt.DeviceArray.from_numpy(A), B).to_numpy()
+    assert np.all(np.abs(got0 - orc.densemat(A, pos, crd, val, m)) <= RTOL * bound)
+    # CSR .* Dense
+    D = rng.uniform(-1, 1, (n, m))
+    dD = rt.DeviceArray.from_numpy(D)
+    p, c, v = rt.eltwise_mult_dense(B, dD).to_arrays()
+    assert np.array_equal(p, pos) and np.array_equal(c, crd) and np.array_equal(v, orc.eltwise_mult_dense(pos, crd, val, D))
+    keep = rng.uniform(-1, 1, (n, m))
+    out = rt.eltwise_mult_dense(B, dD, rt.DeviceArray.from_numpy(keep)).to_numpy()
+    keep[np.repeat(np.arange(n), np.diff(pos)), crd] = v
+    assert np.array_equal(out, keep)

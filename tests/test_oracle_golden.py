@@ -464,3 +464,48 @@ def test_reader_flavours_vs_scipy(tmp_path, flavour):
     assert np.array_equal(got, scipy.io.mmread(path).toarray() if flavour != "array" else scipy.io.mmread(path))
     for r in range(nr):                        # columns ascending inside every row
         assert np.all(np.diff(crd[pos[r]:pos[r + 1]]) > 0)
+
+
+# ----------------------------------------------------------------- dense operand on the left, CSR .* Dense
+def test_vecmat_densemat_golden(golden, golden_dir):
+    g = golden["vecmat_csr"]
+    (nr, nc), pos, crd, val = _mtx(golden_dir, g["matrix"])
+    y = orc.vecmat(np.full(nr, g["x_fill"]), pos, crd, val, nc, np.full(nc, g["y_fill"]))
+    assert orc.format_f64(y) == g["printed"]
+    g = golden["densemat_csr"]
+    Cm = orc.densemat(np.full((g["M"], nr), g["a_fill"]), pos, crd, val, nc, np.full((g["M"], nc), g["c_fill"]))
+    assert orc.format_f64(Cm) == g["printed"]
+
+
+def test_vecmat_densemat_order_and_scipy():
+    rng = np.random.default_rng(8)
+    B = sp.random(37, 23, density=0.3, format="csr", random_state=rng, data_rvs=lambda n: rng.uniform(-1, 1, n))
+    B.sort_indices()
+    x, A = rng.uniform(-1, 1, 37), rng.uniform(-1, 1, (5, 37))
+    y0, C0 = rng.uniform(-1, 1, 23), rng.uniform(-1, 1, (5, 23))
+    y = orc.vecmat(x, B.indptr, B.indices, B.data, 23, y0)
+    Cm = orc.densemat(A, B.indptr, B.indices, B.data, 23, C0)
+    assert np.allclose(y, y0 + x @ B.toarray(), rtol=1e-13) and np.allclose(Cm, C0 + A @ B.toarray(), rtol=1e-13)
+    Bd = B.toarray()
+    for j in range(23):                  # ascending contracted index, multiply then add, starting from the output
+        acc = y0[j]
+        for i in range(37):
+            if Bd[i, j] != 0:
+                acc = acc + x[i] * Bd[i, j]
+        assert y[j] == acc
+    acc = C0[3, 7]
+    for i in range(37):
+        if Bd[i, 7] != 0:
+            acc = acc + A[3, i] * Bd[i, 7]
+    assert Cm[3, 7] == acc
+
+
+def test_eltwise_mult_csr_dense_golden(golden, golden_dir):
+    g = golden["eltwise_mult_csr_dense"]
+    (nr, nc), pos, crd, val = _mtx(golden_dir, g["matrix"])
+    v = orc.eltwise_mult_dense(pos, crd, val, np.full((nr, nc), g["d_fill"]))
+    assert pos.tolist() == g["pos"] and crd.tolist() == g["crd"]
+    assert orc.format_f64(v) == g["printed_val"]
+    dense = np.zeros((nr, nc))
+    dense[np.repeat(np.arange(nr), np.diff(pos)), crd] = v
+    assert orc.format_f64(dense) == g["printed_dense"]

@@ -157,3 +157,27 @@ def main() {
 def test_unsupported_statement_is_named():
     with pytest.raises(ta_run.TaError, match="not supported"):
         ta_run.Program().run("def main() { IndexLabel [a] = [4]; for (x in a) {} }")
+
+
+def test_dense_left_and_csr_times_dense_programs(golden, golden_dir, tmp_path, monkeypatch):
+    prog = """
+def main() {
+    IndexLabel [m] = [4];  IndexLabel [a] = [?];  IndexLabel [b] = [?];
+    Tensor<double> S([a, b], {CSR});
+    Tensor<double> x([a], {Dense});      Tensor<double> y([b], {Dense});
+    Tensor<double> A([m, a], {Dense});   Tensor<double> C([m, b], {Dense});
+    Tensor<double> D([a, b], {Dense});   Tensor<double> E([a, b], {CSR});   Tensor<double> F([a, b], {Dense});
+    S[a, b] = comet_read(0);
+    x[a] = 1.7;  y[b] = 0.0;  A[m, a] = 1.7;  C[m, b] = 0.0;  D[a, b] = 2.7;  F[a, b] = 0.0;
+    y[b] = x[a] * S[a, b];
+    C[m, b] = A[m, a] * S[a, b];
+    E[a, b] = S[a, b] .* D[a, b];
+    F[a, b] = D[a, b] .* S[a, b];
+    print(y);  print(C);  print(E);  print(F);
+}
+"""
+    out = _run(prog, ["test_rank2.mtx"], tmp_path, monkeypatch, golden_dir)
+    g = golden["eltwise_mult_csr_dense"]
+    want = (golden["vecmat_csr"]["printed"] + golden["densemat_csr"]["printed"] + _ints([5]) + _ints([-1]) +
+            _ints(g["pos"]) + _ints(g["crd"]) + g["printed_val"] + g["printed_dense"])
+    _check(out, want, tmp_path)
