@@ -337,7 +337,7 @@ def bench_spgemm(rt, orc, gen, args):
     alg_bytes = nnzA * (8 + ib) + (n + 1) * ib + nnzC * (8 + ib) + 8 * (n + 1)
     sym_ms = kt["spgemm_symbolic"]["avg_ms"] * kt["spgemm_symbolic"]["launches"] / args.steps
     num_ms = sum(kt[k]["avg_ms"] * kt[k]["launches"] for k in
-                 ("spgemm_numeric", "spgemm_numeric_dense", "spgemm_row_products") if k in kt) / args.steps
+                 ("spgemm_numeric", "spgemm_numeric_dense", "spgemm_row_products", "radix_sort_pairs") if k in kt) / args.steps
     # sum of all values is a size-independent invariant: sum(C) = sum_k colsum(A)[k] * rowsum(A)[k]
     rowsum = np.add.reduceat(val, pos[:-1][np.diff(pos) > 0])
     rs = np.zeros(n)

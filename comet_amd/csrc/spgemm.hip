@@ -127,6 +127,19 @@ __device__ inline double wave_sum_f64(double v)
 // back edge with the draw at its end (no `continue`): with a draw at the top and
 // a `continue` below it the compiler splits the loop per lane and parks lanes
 // 1..1023 in a barrier loop that never draws again, which hangs the workgroup.
+// What a ticket indexes is a list of the rows that have work, heaviest first
+// (RowList): empty rows and rows another kernel serves cost no ticket, and the
+// rows that take milliseconds start first instead of forming the tail.
+struct RowList {
+    const int32_t *rows;       // row - row_begin, by descending number of products
+    const int64_t *bounds;     // [0] rows with >= dense_threshold products, [1] rows with any product
+};
+__device__ inline void list_range(const RowList &l, int part, int64_t *first, int64_t *end)
+{
+    // part 0: the heavy rows, 1: the others that have products, 2: both
+    *first = part == 1 ? l.bounds[0] : 0;
+    *end = part == 0 ? l.bounds[0] : l.bounds[1];
+}
 __device__ inline int64_t draw_row(unsigned long long *ticket, int64_t first, int64_t *slot)
 {
     if (threadIdx.x == 0)
@@ -180,7 +193,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_symbolic_kernel(
     int64_t nrows, const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd,
     const int64_t *__restrict__ Bpos, const int32_t *__restrict__ Bcrd, const int64_t *__restrict__ Mpos,
     const int32_t *__restrict__ Mcrd, int logW, uint32_t *__restrict__ gbm, unsigned long long *ticket,
-    int64_t *__restrict__ rowcount)
+    RowList list, int64_t *__restrict__ rowcount)
 {
     __shared__ int64_t row_slot;
     __shared__ int wave_cnt[SG_WAVES];
@@ -196,8 +209,11 @@ __global__ __launch_bounds__(SG_T) void spgemm_symbolic_kernel(
             bm[w] = 0;
     }
     __syncthreads();
-    int64_t i = draw_row(ticket, 0, &row_slot);
-    while (i < nrows) {
+    int64_t t_first, t_end;
+    list_range(list, 2, &t_first, &t_end);
+    int64_t t = draw_row(ticket, t_first, &row_slot);
+    while (t < t_end) {
+        const int64_t i = list.rows[t];       // rows outside the list keep the zero the host put there
         const int64_t as = Apos[i], ae = Apos[i + 1];
         int64_t ms = 0, me = 1;
         if constexpr (MASKED) {
@@ -205,8 +221,6 @@ __global__ __launch_bounds__(SG_T) void spgemm_symbolic_kernel(
             me = Mpos[i + 1];
         }
         const bool work = as != ae && ms != me;
-        if (!work && threadIdx.x == 0)
-            rowcount[i] = 0;
         if (work) {
         if constexpr (MASKED) {
             for (int64_t t = ms + threadIdx.x; t < me; t += SG_T)
@@ -246,7 +260,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_symbolic_kernel(
                                     [&](int j, int64_t, double, int64_t, int64_t) { atomicAnd(&bm[ad.word(j)], 0u); });
         }
         }   // work
-        i = draw_row(ticket, 0, &row_slot);     // its barriers also close this row's bitmap clean-up
+        t = draw_row(ticket, t_first, &row_slot);     // its barriers also close this row's bitmap clean-up
     }
 }
 
@@ -266,8 +280,8 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
     const int32_t *__restrict__ Acrd, const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
     const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval, const int64_t *__restrict__ Mpos,
     const int32_t *__restrict__ Mcrd, int logW, uint32_t *__restrict__ gbm, uint32_t *__restrict__ gmask,
-    double *__restrict__ slabs, unsigned long long *ticket, const int64_t *__restrict__ rowprod,
-    int64_t dense_threshold, int reduce_op, int mult_op, const int64_t *__restrict__ Cpos,
+    double *__restrict__ slabs, unsigned long long *ticket, RowList list, int part,
+    int reduce_op, int mult_op, const int64_t *__restrict__ Cpos,
     int32_t *__restrict__ Ccrd, double *__restrict__ Cval)
 {
     __shared__ int64_t row_slot;
@@ -289,13 +303,14 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
     }
     __syncthreads();
     const int64_t out0 = Cpos[row_begin];
-    int64_t i = draw_row(ticket, row_begin, &row_slot);
-    while (i < row_end) {
+    int64_t t_first, t_end;
+    list_range(list, part, &t_first, &t_end);      // rows with many products are left to spgemm_numeric_dense_kernel
+    int64_t t = draw_row(ticket, t_first, &row_slot);
+    while (t < t_end) {
+        const int64_t i = row_begin + list.rows[t];
         const int64_t as = Apos[i], ae = Apos[i + 1];
         const int64_t ob = Cpos[i], oe = Cpos[i + 1];
-        // rows with many products are left to spgemm_numeric_dense_kernel
-        const bool mine_to_do = rowprod == nullptr || rowprod[i - row_begin] < dense_threshold;
-        if (as != ae && ob != oe && mine_to_do) {
+        if (as != ae && ob != oe) {
         if constexpr (MASKED) {
             for (int64_t t = Mpos[i] + threadIdx.x; t < Mpos[i + 1]; t += SG_T)
                 atomicOr(&mbm[ad.word(Mcrd[t])], ad.bit(Mcrd[t]));
@@ -382,7 +397,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
                 atomicAnd(&mbm[ad.word(Mcrd[t])], 0u);
         }
         }   // row with output
-        i = draw_row(ticket, row_begin, &row_slot);     // its barriers also close this row's clean-up
+        t = draw_row(ticket, t_first, &row_slot);     // its barriers also close this row's clean-up
     }
 }
 
@@ -451,7 +466,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
     int64_t row_begin, int64_t row_end, const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd,
     const double *__restrict__ Aval, const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval,
     const int64_t *__restrict__ blkptr, int nblk,
-    unsigned long long *ticket, const int64_t *__restrict__ rowprod, int64_t dense_threshold,
+    unsigned long long *ticket, RowList list,
     const int64_t *__restrict__ Cpos, int32_t *__restrict__ Ccrd, double *__restrict__ Cval)
 {
     __shared__ int64_t row_slot;
@@ -469,10 +484,13 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
         block_touched = 0;
     __syncthreads();
     const int64_t out0 = Cpos[row_begin];
-    int64_t i = draw_row(ticket, row_begin, &row_slot);
-    while (i < row_end) {
+    int64_t t_first, t_end;
+    list_range(list, 0, &t_first, &t_end);
+    int64_t t = draw_row(ticket, t_first, &row_slot);
+    while (t < t_end) {
+        const int64_t i = row_begin + list.rows[t];
         const int64_t as = Apos[i], ae = Apos[i + 1];
-        if (as != ae && rowprod[i - row_begin] >= dense_threshold) {
+        if (as != ae) {
             int64_t off = Cpos[i] - out0;
             for (int cb = 0; cb < nblk; ++cb) {
                 const int col0 = cb << SG_CB_LOG;
@@ -591,7 +609,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                 }   // block received products
             }
         }
-        i = draw_row(ticket, row_begin, &row_slot);
+        t = draw_row(ticket, t_first, &row_slot);
     }
 }
 
@@ -605,7 +623,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_masked_sum_kernel(
     int64_t nrows, const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd,
     const double *__restrict__ Aval, const int64_t *__restrict__ Bpos, const int32_t *__restrict__ Bcrd,
     const double *__restrict__ Bval, const int64_t *__restrict__ Mpos, const int32_t *__restrict__ Mcrd,
-    int logW, uint32_t *__restrict__ gbm, unsigned long long *ticket, double *__restrict__ rowsum)
+    int logW, uint32_t *__restrict__ gbm, unsigned long long *ticket, RowList list, double *__restrict__ rowsum)
 {
     __shared__ int64_t row_slot;
     __shared__ double wave_part[SG_WAVES];
@@ -621,13 +639,14 @@ __global__ __launch_bounds__(SG_T) void spgemm_masked_sum_kernel(
             bm[w] = 0;
     }
     __syncthreads();
-    int64_t i = draw_row(ticket, 0, &row_slot);
-    while (i < nrows) {
+    int64_t t_first, t_end;
+    list_range(list, 2, &t_first, &t_end);
+    int64_t tk = draw_row(ticket, t_first, &row_slot);
+    while (tk < t_end) {
+        const int64_t i = list.rows[tk];      // rows outside the list keep the zero the host put there
         const int64_t as = Apos[i], ae = Apos[i + 1];
         const int64_t ms = Mpos[i], me = Mpos[i + 1];
         const bool work = as != ae && ms != me;
-        if (!work && threadIdx.x == 0)
-            rowsum[i] = 0.0;
         if (work) {
         for (int64_t t = ms + threadIdx.x; t < me; t += SG_T)
             atomicOr(&bm[ad.word(Mcrd[t])], ad.bit(Mcrd[t]));
@@ -655,7 +674,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_masked_sum_kernel(
         for (int64_t t = ms + threadIdx.x; t < me; t += SG_T)
             atomicAnd(&bm[ad.word(Mcrd[t])], 0u);
         }   // work
-        i = draw_row(ticket, 0, &row_slot);     // its barriers also close this row's bitmap clean-up
+        tk = draw_row(ticket, t_first, &row_slot);     // its barriers also close this row's bitmap clean-up
     }
 }
 
@@ -725,7 +744,6 @@ struct SgScratch {
     Workspace gbm;        // global bitmaps (only when the bitmap does not fit LDS)
     Workspace gmask;      // global mask bitmaps (masked numeric)
     Workspace slabs;      // dense accumulators, zero between calls
-    Workspace rowprod;    // products per row of the current row range
 };
 static SgScratch g_sg;
 
@@ -781,11 +799,81 @@ static int check_product_shapes(const Csr *a, const Csr *b, const Csr *m, const 
     return COMET_HIP_OK;
 }
 
+// keys that order rows by descending products; rows without products sort to the very end
+__global__ void sg_row_keys(int64_t n, const int64_t *__restrict__ rowprod, uint64_t *__restrict__ keys,
+                            uint32_t *__restrict__ idx)
+{
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r < n) {
+        const int64_t p = rowprod[r];
+        keys[r] = p > 0 ? (uint64_t)((1ll << 62) - p) : ~0ull >> 1;
+        idx[r] = (uint32_t)r;
+    }
+}
+
+// bounds[0] = rows with >= threshold products, bounds[1] = rows with any, in the sorted key array
+__global__ void sg_row_bounds(int64_t n, const uint64_t *__restrict__ keys, int64_t threshold,
+                              int64_t *__restrict__ bounds)
+{
+    if (threadIdx.x > 1 || blockIdx.x > 0)
+        return;
+    // first key that is larger than the limit: keys ascend as products descend
+    const uint64_t limit = threadIdx.x == 0 ? (uint64_t)((1ll << 62) - threshold) : (uint64_t)((1ll << 62) - 1);
+    int64_t lo = 0, hi = n;
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (keys[mid] <= limit)
+            lo = mid + 1;
+        else
+            hi = mid;
+    }
+    bounds[threadIdx.x] = lo;
+}
+
+struct SgRowLists {
+    Workspace rowprod, keys_in, keys_out, idx_in, idx_out, bounds;
+};
+static SgRowLists g_rl;
+
+// Products per row of rows [rb, re) of A*B and the list of those rows by descending products.
+static int sg_row_list(const Csr *a, const Csr *b, int64_t rb, int64_t re, int64_t dense_threshold, RowList *out)
+{
+    const int64_t n = re - rb;
+    COMET_CHK(g_rl.rowprod.ensure(sizeof(int64_t) * (size_t)n, false));
+    COMET_CHK(g_rl.keys_in.ensure(8 * (size_t)n, false));
+    COMET_CHK(g_rl.keys_out.ensure(8 * (size_t)n, false));
+    COMET_CHK(g_rl.idx_in.ensure(4 * (size_t)n, false));
+    COMET_CHK(g_rl.idx_out.ensure(4 * (size_t)n, false));
+    COMET_CHK(g_rl.bounds.ensure(16, false));
+    int64_t *rowprod = (int64_t *)g_rl.rowprod.ptr;
+    {
+        KernelTimer t("spgemm_row_products");
+        spgemm_row_products<<<dim3((unsigned)ceil_div(n, 4)), dim3(256), 0, stream()>>>(rb, re, a->pos, a->crd, b->pos,
+                                                                                        rowprod);
+        sg_row_keys<<<dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, stream()>>>(
+            n, rowprod, (uint64_t *)g_rl.keys_in.ptr, (uint32_t *)g_rl.idx_in.ptr);
+    }
+    COMET_HIPCHK(hipGetLastError());
+    COMET_CHK(sort_pairs_u64_u32((const uint64_t *)g_rl.keys_in.ptr, (uint64_t *)g_rl.keys_out.ptr,
+                                 (const uint32_t *)g_rl.idx_in.ptr, (uint32_t *)g_rl.idx_out.ptr, n, 63));
+    sg_row_bounds<<<dim3(1), dim3(64), 0, stream()>>>(n, (const uint64_t *)g_rl.keys_out.ptr, dense_threshold,
+                                                      (int64_t *)g_rl.bounds.ptr);
+    COMET_HIPCHK(hipGetLastError());
+    out->rows = (const int32_t *)g_rl.idx_out.ptr;
+    out->bounds = (const int64_t *)g_rl.bounds.ptr;
+    return COMET_HIP_OK;
+}
+
+constexpr int64_t SG_NO_DENSE = 1ll << 61;     // a threshold no row reaches: every row stays on the slab path
+
 static int symbolic_counts(const Csr *a, const Csr *b, const Csr *m, int64_t *rowcount)
 {
     SgGeom g;
     COMET_CHK(sg_geometry(b->ncols, &g));
     COMET_CHK(sg_reset_ticket());
+    RowList list;
+    COMET_CHK(sg_row_list(a, b, 0, a->nrows, SG_NO_DENSE, &list));
+    COMET_HIPCHK(hipMemsetAsync(rowcount, 0, sizeof(int64_t) * (size_t)a->nrows, stream()));
     uint32_t *gbm = nullptr;
     if (!g.lds) {
         COMET_CHK(g_sg.gbm.ensure(sizeof(uint32_t) * g.bm_words * (size_t)g.groups, true));
@@ -798,7 +886,7 @@ static int symbolic_counts(const Csr *a, const Csr *b, const Csr *m, int64_t *ro
         KernelTimer t(M ? "spgemm_symbolic_masked" : "spgemm_symbolic");                                   \
         spgemm_symbolic_kernel<L, M><<<grid, block, g.lds_bytes, stream()>>>(                              \
             a->nrows, a->pos, a->crd, b->pos, b->crd, m ? m->pos : nullptr, m ? m->crd : nullptr, g.logW,  \
-            gbm, (unsigned long long *)g_sg.ticket.ptr, rowcount);                                                                        \
+            gbm, (unsigned long long *)g_sg.ticket.ptr, list, rowcount);                                   \
     } while (0)
     if (g.lds) {
         if (m) LAUNCH_SYM(true, true); else LAUNCH_SYM(true, false);
@@ -851,17 +939,11 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
     // rows with many products go to the LDS-accumulator kernel (unmasked products only)
     const int nblk = (int)ceil_div(b->ncols > 0 ? b->ncols : 1, SG_CB);
     const bool dense = !m && !semi && nblk <= SG_DENSE_MAX_BLOCKS;
-    const int64_t dense_threshold = SG_DENSE_PER_BLOCK * nblk;
-    int64_t *rowprod = nullptr;
-    if (dense) {
+    const int64_t dense_threshold = dense ? SG_DENSE_PER_BLOCK * nblk : SG_NO_DENSE;
+    if (dense)
         COMET_CHK(sg_plan_blocks(b));
-        COMET_CHK(g_sg.rowprod.ensure(sizeof(int64_t) * (size_t)(re - rb), false));
-        rowprod = (int64_t *)g_sg.rowprod.ptr;
-        KernelTimer t("spgemm_row_products");
-        spgemm_row_products<<<dim3((unsigned)ceil_div(re - rb, 4)), dim3(256), 0, stream()>>>(rb, re, a->pos, a->crd,
-                                                                                              b->pos, rowprod);
-        COMET_HIPCHK(hipGetLastError());
-    }
+    RowList list;
+    COMET_CHK(sg_row_list(a, b, rb, re, dense_threshold, &list));
     uint32_t *gbm = nullptr, *gmask = nullptr;
     if (!g.lds) {
         COMET_CHK(g_sg.gbm.ensure(sizeof(uint32_t) * g.bm_words * (size_t)g.groups, true));
@@ -880,8 +962,7 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
         spgemm_numeric_kernel<L, M, S><<<grid, block, g.lds_bytes, stream()>>>(                            \
             rb, re, b->ncols, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m ? m->pos : nullptr,        \
             m ? m->crd : nullptr, g.logW, gbm, gmask, (double *)g_sg.slabs.ptr,                            \
-            (unsigned long long *)g_sg.ticket.ptr, rowprod, dense_threshold, reduce_op, mult_op, Cpos,     \
-            Ccrd, Cval);                                                                                   \
+            (unsigned long long *)g_sg.ticket.ptr, list, 1, reduce_op, mult_op, Cpos, Ccrd, Cval);         \
     } while (0)
 #define LAUNCH_NUM_S(L, M)                                                                                 \
     do {                                                                                                   \
@@ -900,8 +981,9 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
         COMET_CHK(sg_allow_lds(spgemm_numeric_dense_kernel, SG_DENSE_LDS));
         KernelTimer t("spgemm_numeric_dense");
         spgemm_numeric_dense_kernel<<<dim3((unsigned)(num_cus() > 0 ? num_cus() : 256)), block, SG_DENSE_LDS,
-                                      stream()>>>(rb, re, a->pos, a->crd, a->val, b->crd, b->val, b->sg_blkptr, nblk, (unsigned long long *)g_sg.ticket.ptr, rowprod,
-                                                  dense_threshold, Cpos, Ccrd, Cval);
+                                      stream()>>>(rb, re, a->pos, a->crd, a->val, b->crd, b->val, b->sg_blkptr,
+                                                  nblk, (unsigned long long *)g_sg.ticket.ptr, list, Cpos, Ccrd,
+                                                  Cval);
         COMET_HIPCHK(hipGetLastError());
     }
     return COMET_HIP_OK;
@@ -1031,18 +1113,21 @@ extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, d
         gbm = (uint32_t *)g_sg.gbm.ptr;
     }
     double *rowsum = (double *)g_sg.rowcount.ptr;
+    RowList list;
+    COMET_CHK(sg_row_list(a, b, 0, a->nrows, SG_NO_DENSE, &list));
+    COMET_HIPCHK(hipMemsetAsync(rowsum, 0, sizeof(double) * (size_t)a->nrows, stream()));
     const dim3 grid((unsigned)g.groups), block(SG_T);
     if (g.lds) {
         COMET_CHK(sg_allow_lds(spgemm_masked_sum_kernel<true>, g.lds_bytes));
         KernelTimer t("spgemm_masked_sum");
         spgemm_masked_sum_kernel<true><<<grid, block, g.lds_bytes, stream()>>>(
             a->nrows, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m->pos, m->crd, g.logW, gbm,
-            (unsigned long long *)g_sg.ticket.ptr, rowsum);
+            (unsigned long long *)g_sg.ticket.ptr, list, rowsum);
     } else {
         KernelTimer t("spgemm_masked_sum");
         spgemm_masked_sum_kernel<false><<<grid, block, 0, stream()>>>(
             a->nrows, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m->pos, m->crd, g.logW, gbm,
-            (unsigned long long *)g_sg.ticket.ptr, rowsum);
+            (unsigned long long *)g_sg.ticket.ptr, list, rowsum);
     }
     COMET_HIPCHK(hipGetLastError());
     return reduce_sum_device(rowsum, a->nrows, out);
