@@ -134,32 +134,48 @@ int csr_alloc(Csr *c, int64_t nrows, int64_t ncols, int64_t nnz)
     return COMET_HIP_OK;
 }
 
-void csr_release(Csr *c)
+// Everything the kernels derived from the matrix and keep in its handle.
+static void csr_drop_plans(Csr *c)
 {
     if (c->light)
         csr_release(c->light);
     if (c->transposed)
         csr_release(c->transposed);
+    c->light = c->transposed = nullptr;
     (void)hipFree(c->heavy_seg);
     (void)hipFree(c->heavy_col);
     (void)hipFree(c->heavy_val);
     (void)hipFree(c->heavy_row);
     (void)hipFree(c->heavy_code);
+    c->heavy_seg = nullptr;
+    c->heavy_col = c->heavy_row = c->heavy_code = nullptr;
+    c->heavy_val = nullptr;
+    c->heavy_state = 0;
+    c->heavy_nnz = c->heavy_rows = 0;
+    (void)hipFree(c->spmm_chunk_row);
+    c->spmm_chunk_row = nullptr;
+    c->spmm_nchunks = 0;
+    (void)hipFree(c->sg_blkptr);
+    c->sg_blkptr = nullptr;
+    c->sg_nblk = 0;
+    (void)hipFree(c->spmv_bpos);
+    (void)hipFree(c->spmv_bcrd);
+    (void)hipFree(c->spmv_bval);
+    c->spmv_bpos = nullptr;
+    c->spmv_bcrd = nullptr;
+    c->spmv_bval = nullptr;
+    c->spmv_nb = 0;
+    c->spmv_base.clear();
+}
+
+void csr_release(Csr *c)
+{
+    csr_drop_plans(c);
     if (c->owns) {
         (void)hipFree(c->pos);
         (void)hipFree(c->crd);
         (void)hipFree(c->val);
     }
-    if (c->spmm_chunk_row)
-        (void)hipFree(c->spmm_chunk_row);
-    if (c->sg_blkptr)
-        (void)hipFree(c->sg_blkptr);
-    if (c->spmv_bpos)
-        (void)hipFree(c->spmv_bpos);
-    if (c->spmv_bcrd)
-        (void)hipFree(c->spmv_bcrd);
-    if (c->spmv_bval)
-        (void)hipFree(c->spmv_bval);
     delete c;
 }
 
@@ -729,6 +745,16 @@ int comet_hip_csr_download_i32(int64_t csr, int32_t *pos, int32_t *crd, double *
     if (val && c->nnz)
         COMET_HIPCHK(hipMemcpyAsync(val, c->val, sizeof(double) * (size_t)c->nnz, hipMemcpyDeviceToHost, s));
     COMET_HIPCHK(hipStreamSynchronize(s));
+    return COMET_HIP_OK;
+}
+
+int comet_hip_csr_invalidate(int64_t csr)
+{
+    Csr *c = csr_from_handle(csr);
+    if (!c)
+        return COMET_HIP_ERR_HANDLE;
+    COMET_HIPCHK(hipStreamSynchronize(stream()));
+    csr_drop_plans(c);
     return COMET_HIP_OK;
 }
 

@@ -72,6 +72,7 @@ SIGNATURES = {
     "comet_hip_csr_arrays": (_int, [_i64, _pi64, _pi64, _pi64]),
     "comet_hip_csr_download_i64": (_int, [_i64, _vp, _vp, _vp]),
     "comet_hip_csr_download_i32": (_int, [_i64, _vp, _vp, _vp]),
+    "comet_hip_csr_invalidate": (_int, [_i64]),
     "comet_hip_csr_destroy": (_int, [_i64]),
     "comet_hip_spmv_csr_f64": (_int, [_i64, _i64, _i64, _int]),
     "comet_hip_spmm_csr_f64": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
@@ -337,6 +338,10 @@ class CsrMatrix:
         fn = lib().comet_hip_csr_download_i64 if idt == np.int64 else lib().comet_hip_csr_download_i32
         _check(fn(self.handle, _vptr(pos), _vptr(crd) if nnz else None, _vptr(val) if nnz else None), "csr download")
         return pos, crd, val
+
+    def invalidate(self):
+        """Drop what the kernels cached about this matrix (needed after writing into wrapped arrays)."""
+        _check(lib().comet_hip_csr_invalidate(self.handle), "comet_hip_csr_invalidate")
 
     def free(self):
         if self.handle:

@@ -74,13 +74,17 @@ int64_t comet_hip_csr_upload_i64(int64_t nrows, int64_t ncols, const int64_t *po
 int64_t comet_hip_csr_upload_i32(int64_t nrows, int64_t ncols, const int32_t *pos,
                                  const int32_t *crd, const double *val);
 /* Wrap device arrays the caller already filled (pos int64, crd int32, val f64);
- * the handle does not own them. */
+ * the handle does not own them.  The kernels keep what they derive from a
+ * matrix in its handle (re-ordered copies, block pointers, the transpose), so
+ * after writing into wrapped arrays call comet_hip_csr_invalidate before the
+ * handle is used again. */
 int64_t comet_hip_csr_wrap(int64_t nrows, int64_t ncols, int64_t nnz,
                            int64_t pos_dptr, int64_t crd_dptr, int64_t val_dptr);
 int comet_hip_csr_dims(int64_t csr, int64_t *nrows, int64_t *ncols, int64_t *nnz);
 int comet_hip_csr_arrays(int64_t csr, int64_t *pos_dptr, int64_t *crd_dptr, int64_t *val_dptr);
 int comet_hip_csr_download_i64(int64_t csr, int64_t *pos, int64_t *crd, double *val);
 int comet_hip_csr_download_i32(int64_t csr, int32_t *pos, int32_t *crd, double *val);
+int comet_hip_csr_invalidate(int64_t csr);
 int comet_hip_csr_destroy(int64_t csr);
 
 /* ---- SpMV  y[i] (+)= sum_p val[p] * x[crd[p]] ------------------------------

@@ -847,3 +847,27 @@ def test_vecmat_densemat_vs_checker(n, m, M, density, seed):
     out = rt.eltwise_mult_dense(B, dD, rt.DeviceArray.from_numpy(keep)).to_numpy()
     keep[np.repeat(np.arange(n), np.diff(pos)), crd] = v
     assert np.array_equal(out, keep)
+
+
+def test_wrapped_arrays_changed_in_place_need_invalidate():
+    """A handle over caller-owned device arrays caches re-ordered copies; after the caller rewrites the values
+    comet_hip_csr_invalidate makes every kernel see them."""
+    pos, crd, val = gen.zipf_csr(n=40_000, mean=16.0, cap=4096, seed=11)      # large enough for every plan
+    n, nnz = 40_000, len(crd)
+    dpos = rt.DeviceArray.from_numpy(pos.astype(np.int64))
+    dcrd = rt.DeviceArray.from_numpy(crd.astype(np.int32))
+    dval = rt.DeviceArray.from_numpy(val)
+    L = rt.lib()
+    A = rt.CsrMatrix(rt._handle(L.comet_hip_csr_wrap(n, n, nnz, dpos.ptr, dcrd.ptr, dval.ptr), "wrap"))
+    B = gen.dense((n, 32), seed=12)
+    x = gen.dense(n, seed=13)
+    dB, dx = rt.DeviceArray.from_numpy(B), rt.DeviceArray.from_numpy(x)
+    first = rt.spmm(A, dB).to_numpy()
+    y1 = rt.spmv(A, dx).to_numpy()
+    z1 = rt.vecmat(dx, A).to_numpy()
+    val2 = -2.0 * val
+    rt._check(L.comet_hip_memcpy(dval.ptr, val2.ctypes.data, val2.nbytes, 0), "upload")
+    A.invalidate()
+    assert np.array_equal(rt.spmm(A, dB).to_numpy(), -2.0 * first)       # scaling by -2 is exact
+    assert np.array_equal(rt.spmv(A, dx).to_numpy(), -2.0 * y1)
+    assert np.array_equal(rt.vecmat(dx, A).to_numpy(), -2.0 * z1)
