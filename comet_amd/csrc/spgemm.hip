@@ -714,7 +714,9 @@ __global__ void eltwise_mult_kernel(int64_t nrows, const int64_t *__restrict__ A
         rowcount[i] = n;
 }
 
-// CSR .* Dense: the stored entries of A times the dense values under them.  TO_DENSE writes them into a dense
+// CSR (op) Dense, op = * for the plain elementwise product and any other COMET_OP_* for the monoid forms
+// A @(op) B of test/integration/semiring/eltwise_monoid*_COOxDense_oCOO.ta: the stored entries of A combined
+// with the dense values under them.  TO_DENSE writes them into a dense
 // output at their positions and leaves every other element as it was (the nest only visits the entries of
 // A, test/integration/ops/eltwise_mult_CSRxDense_oDense.ta); otherwise they become the values of a CSR with
 // A's structure (eltwise_mult_CSRxDense_oCSR.ta).
@@ -722,14 +724,14 @@ template <bool TO_DENSE>
 __global__ void eltwise_mult_dense_kernel(int64_t nrows, const int64_t *__restrict__ pos,
                                           const int32_t *__restrict__ crd, const double *__restrict__ val,
                                           const double *__restrict__ D, int64_t ldd, double *__restrict__ out,
-                                          int64_t ldo)
+                                          int64_t ldo, int op)
 {
     // one 16-lane group per row
     const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
     if (i >= nrows)
         return;
     for (int64_t p = pos[i] + (threadIdx.x & 15); p < pos[i + 1]; p += 16) {
-        const double v = val[p] * D[i * ldd + crd[p]];
+        const double v = semiring_mult(op, val[p], D[i * ldd + crd[p]]);
         if (TO_DENSE)
             out[i * ldo + crd[p]] = v;
         else
@@ -1200,15 +1202,15 @@ extern "C" int64_t comet_hip_eltwise_mult_csr(int64_t ah, int64_t bh)
     return csr_register(c);
 }
 
-extern "C" int64_t comet_hip_eltwise_mult_csr_dense_csr(int64_t ah, int64_t d_dptr, int64_t ldd)
+extern "C" int64_t comet_hip_eltwise_csr_dense_csr(int64_t ah, int64_t d_dptr, int64_t ldd, int op)
 {
     if (ensure_init() != COMET_HIP_OK)
         return 0;
     Csr *a = csr_from_handle(ah);
     if (!a)
         return 0;
-    if (ldd < a->ncols || (a->nnz > 0 && !d_dptr)) {
-        set_error(COMET_HIP_ERR_ARG, "bad dense operand passed to comet_hip_eltwise_mult_csr_dense_csr");
+    if (ldd < a->ncols || (a->nnz > 0 && !d_dptr) || op < 0 || op > COMET_OP_DIV) {
+        set_error(COMET_HIP_ERR_ARG, "bad dense operand or operator passed to comet_hip_eltwise_csr_dense_csr");
         return 0;
     }
     Csr *c = new Csr();
@@ -1223,7 +1225,7 @@ extern "C" int64_t comet_hip_eltwise_mult_csr_dense_csr(int64_t ah, int64_t d_dp
              hipSuccess;
         KernelTimer t("eltwise_mult_dense");
         eltwise_mult_dense_kernel<false><<<dim3((unsigned)ceil_div(a->nrows * 16, 256)), dim3(256), 0, stream()>>>(
-            a->nrows, a->pos, a->crd, a->val, (const double *)d_dptr, ldd, c->val, 0);
+            a->nrows, a->pos, a->crd, a->val, (const double *)d_dptr, ldd, c->val, 0, op);
     }
     if (!ok || hipGetLastError() != hipSuccess) {
         set_error(COMET_HIP_ERR_HIP, "CSR .* Dense failed");
@@ -1233,20 +1235,45 @@ extern "C" int64_t comet_hip_eltwise_mult_csr_dense_csr(int64_t ah, int64_t d_dp
     return csr_register(c);
 }
 
-extern "C" int comet_hip_eltwise_mult_csr_dense_dense(int64_t ah, int64_t d_dptr, int64_t ldd, int64_t c_dptr,
-                                                      int64_t ldc)
+extern "C" int comet_hip_eltwise_csr_dense_dense(int64_t ah, int64_t d_dptr, int64_t ldd, int64_t c_dptr,
+                                                 int64_t ldc, int op)
 {
     COMET_CHK(ensure_init());
     Csr *a = csr_from_handle(ah);
     if (!a)
         return COMET_HIP_ERR_HANDLE;
-    if (ldd < a->ncols || ldc < a->ncols || (a->nnz > 0 && (!d_dptr || !c_dptr)))
-        return set_error(COMET_HIP_ERR_ARG, "bad dense operand passed to comet_hip_eltwise_mult_csr_dense_dense");
+    if (ldd < a->ncols || ldc < a->ncols || (a->nnz > 0 && (!d_dptr || !c_dptr)) || op < 0 || op > COMET_OP_DIV)
+        return set_error(COMET_HIP_ERR_ARG, "bad dense operand or operator passed to comet_hip_eltwise_csr_dense_dense");
     if (a->nnz == 0)
         return COMET_HIP_OK;
     KernelTimer t("eltwise_mult_dense");
     eltwise_mult_dense_kernel<true><<<dim3((unsigned)ceil_div(a->nrows * 16, 256)), dim3(256), 0, stream()>>>(
-        a->nrows, a->pos, a->crd, a->val, (const double *)d_dptr, ldd, (double *)c_dptr, ldc);
+        a->nrows, a->pos, a->crd, a->val, (const double *)d_dptr, ldd, (double *)c_dptr, ldc, op);
+    COMET_HIPCHK(hipGetLastError());
+    return COMET_HIP_OK;
+}
+
+// Dense (op) Dense over n elements (test/integration/semiring/eltwise_monoid*_DensexDense_oDense.ta).
+__global__ void eltwise_dense_kernel(int64_t n, const double *__restrict__ a, const double *__restrict__ b,
+                                     double *__restrict__ c, int op)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step)
+        c[i] = semiring_mult(op, a[i], b[i]);
+}
+
+extern "C" int comet_hip_eltwise_dense_f64(int64_t n, int64_t a_dptr, int64_t b_dptr, int64_t c_dptr, int op)
+{
+    COMET_CHK(ensure_init());
+    if (n < 0 || (n > 0 && (!a_dptr || !b_dptr || !c_dptr)) || op < 0 || op > COMET_OP_DIV)
+        return set_error(COMET_HIP_ERR_ARG, "bad arguments to comet_hip_eltwise_dense_f64");
+    if (n == 0)
+        return COMET_HIP_OK;
+    KernelTimer t("eltwise_dense");
+    const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div(n, 256), (int64_t)num_cus() * 32);
+    eltwise_dense_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(n, (const double *)a_dptr, (const double *)b_dptr,
+                                                                  (double *)c_dptr, op);
     COMET_HIPCHK(hipGetLastError());
     return COMET_HIP_OK;
 }

@@ -83,8 +83,9 @@ SIGNATURES = {
     "comet_hip_spgemm_csr_semiring": (_i64, [_i64, _i64, _i64, _int, _int]),
     "comet_hip_vecmat_csr_f64": (_int, [_i64, _i64, _i64, _int]),
     "comet_hip_densemat_csr_f64": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
-    "comet_hip_eltwise_mult_csr_dense_csr": (_i64, [_i64, _i64, _i64]),
-    "comet_hip_eltwise_mult_csr_dense_dense": (_int, [_i64, _i64, _i64, _i64, _i64]),
+    "comet_hip_eltwise_csr_dense_csr": (_i64, [_i64, _i64, _i64, _int]),
+    "comet_hip_eltwise_csr_dense_dense": (_int, [_i64, _i64, _i64, _i64, _i64, _int]),
+    "comet_hip_eltwise_dense_f64": (_int, [_i64, _i64, _i64, _i64, _int]),
     "comet_hip_mtx_read_csr": (_i64, [C.c_char_p, _int]),
     "comet_hip_read_input_sizes_2D_f64": (None, [_i32, _i32, _i32, _i32, _i32, _int, _vp, _i32]),
     "comet_hip_read_input_2D_f64_i64": (None, [_i32, _i32, _i32, _i32, _i32] + [_int, _vp] * 9 + [_i32]),
@@ -483,16 +484,32 @@ def densemat(A, B, Cm=None, accumulate=None):
     return Cm
 
 
-def eltwise_mult_dense(A, D, out=None):
-    """A .* D for a sparse A and a dense D of the same shape: a CsrMatrix with A's structure, or, when a
-    dense `out` is given, written into it at A's stored positions."""
+def eltwise_csr_dense(A, D, out=None, op="times"):
+    """A (op) D elementwise for a sparse A and a dense D of the same shape (op: a MULT_OPS name; "times" is
+    the language's .*): a CsrMatrix with A's structure, or, when a dense `out` is given, written into it at
+    A's stored positions."""
     if tuple(D.shape) != tuple(A.shape):
         raise ValueError("operands differ in shape")
+    code = MULT_OPS[op]
     if out is None:
-        return CsrMatrix(_handle(lib().comet_hip_eltwise_mult_csr_dense_csr(A.handle, D.ptr, A.shape[1]),
-                                 "comet_hip_eltwise_mult_csr_dense_csr"))
-    _check(lib().comet_hip_eltwise_mult_csr_dense_dense(A.handle, D.ptr, A.shape[1], out.ptr, A.shape[1]),
-           "comet_hip_eltwise_mult_csr_dense_dense")
+        return CsrMatrix(_handle(lib().comet_hip_eltwise_csr_dense_csr(A.handle, D.ptr, A.shape[1], code),
+                                 "comet_hip_eltwise_csr_dense_csr"))
+    _check(lib().comet_hip_eltwise_csr_dense_dense(A.handle, D.ptr, A.shape[1], out.ptr, A.shape[1], code),
+           "comet_hip_eltwise_csr_dense_dense")
+    return out
+
+
+def eltwise_mult_dense(A, D, out=None):
+    return eltwise_csr_dense(A, D, out, "times")
+
+
+def eltwise_dense(A, B, out=None, op="times"):
+    """out = A (op) B over dense arrays of one shape."""
+    if tuple(A.shape) != tuple(B.shape):
+        raise ValueError("operands differ in shape")
+    if out is None:
+        out = DeviceArray(A.shape)
+    _check(lib().comet_hip_eltwise_dense_f64(A.size, A.ptr, B.ptr, out.ptr, MULT_OPS[op]), "comet_hip_eltwise_dense_f64")
     return out
 
 

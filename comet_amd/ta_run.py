@@ -17,6 +17,7 @@ include/comet_hip_rt.h.  Statements it understands (frontends/comet_dsl/include/
     C[a, c] = A[a, b] @(min,+) B[b, c];                               (SpGEMM over a semiring)
     C[i, k]<M, push> = A[i, j] * B[j, k];                             (masked SpGEMM)
     C[i, j] = A[i, j] .* B[i, j];    (CSR .* CSR, CSR .* Dense, Dense .* CSR)
+    C[i, j] = A[i, j] @(+) B[i, j];  (elementwise monoids +, -, *, min, max: Dense x Dense, sparse x Dense)
     B[j, i] = transpose(A[i, j], {j, i});                             (dense)
     var s = SUM(C[i, j]);  var t = getTime();  printElapsedTime(t0, t1);  print(C);  print(s);
 
@@ -152,27 +153,41 @@ class Program:
         c, a, b = self._tensor(cname), self._tensor(aname), self._tensor(bname)
         al, bl, cl = self._labels(alabels), self._labels(blabels), self._labels(clabels)
         semiring = None
-        if red is not None:
+        if red is not None and mul is not None:
             try:
                 semiring = (_SEMIRING_TOKENS[red.strip()], _SEMIRING_TOKENS[mul.strip()])
             except KeyError:
                 raise TaError(f"semiring @({red},{mul}) is not supported") from None
-        if op == ".*":
-            if not (al == bl == cl) or len(al) != 2:
-                raise TaError("elementwise .* is supported for matrices over the same indices")
-            if a.fmt == b.fmt == c.fmt == "CSR":
+        if op == ".*" or (red is not None and mul is None):
+            # `.*`, or the monoid form A @(op) B with a single operator
+            if op == ".*":
+                ew = "times"
+            else:
+                if red.strip() not in _SEMIRING_TOKENS:
+                    raise TaError(f"elementwise operator @({red}) is not supported")
+                ew = _SEMIRING_TOKENS[red.strip()]
+            if not (al == bl == cl):
+                raise TaError("elementwise operations need the same indices on every tensor")
+            if a.fmt == b.fmt == c.fmt == "Dense":
+                c.value = rt.eltwise_dense(self._dense(a), self._dense(b), op=ew)
+                return
+            if len(al) != 2:
+                raise TaError("sparse elementwise operations are supported for matrices")
+            if a.fmt == b.fmt == c.fmt == "CSR" and ew == "times":
                 c.value = rt.eltwise_mult(self._sparse(a), self._sparse(b))
                 return
-            sp_, de_ = (a, b) if a.fmt == "CSR" else (b, a)
-            if sp_.fmt == "CSR" and de_.fmt == "Dense" and c.fmt in ("CSR", "Dense"):
+            sp_, de_ = (a, b) if a.fmt != "Dense" else (b, a)
+            commutes = ew in ("times", "plus", "min", "max")
+            if sp_.fmt != "Dense" and de_.fmt == "Dense" and (sp_ is a or commutes) and c.fmt in (sp_.fmt, "Dense"):
                 S = self._sparse(sp_)
                 self._bind(al, S.shape)
-                if c.fmt == "CSR":
-                    c.value = rt.eltwise_mult_dense(S, self._dense(de_))
+                if c.fmt != "Dense":
+                    c.value = rt.eltwise_csr_dense(S, self._dense(de_), op=ew)
                 else:
-                    rt.eltwise_mult_dense(S, self._dense(de_), self._dense(c))
+                    rt.eltwise_csr_dense(S, self._dense(de_), self._dense(c), op=ew)
                 return
-            raise TaError("elementwise .* is supported for CSR .* CSR -> CSR and CSR .* Dense -> CSR or Dense")
+            raise TaError("elementwise operations are supported for Dense x Dense, CSR .* CSR -> CSR and "
+                          "sparse x Dense -> the sparse format or Dense")
         if a.fmt == "Dense" and b.fmt != "Dense" and c.fmt == "Dense":
             if semiring not in (None, ("plus", "times")) or mask:
                 raise TaError("semirings and masks are supported for sparse x sparse products")
@@ -264,7 +279,7 @@ class Program:
         (r"(\w+)\s*" + _IDX + r"\s*=\s*comet_read\(\s*(\d+)\s*(?:,\s*(\d+)\s*)?\)", _read),
         (r"(\w+)\s*" + _IDX + r"\s*=\s*([-+]?[0-9.]+(?:[eE][-+]?\d+)?)", _fill),
         (r"(\w+)\s*" + _IDX + r"\s*(?:<\s*(\w+)\s*,\s*(\w+)\s*>)?\s*=\s*(\w+)\s*" + _IDX +
-         r"\s*(\.\*|\*|@\(\s*([^,()]+),\s*([^,()]+)\))\s*(\w+)\s*" + _IDX, _product),
+         r"\s*(\.\*|\*|@\(\s*([^,()]+?)\s*(?:,\s*([^,()]+?)\s*)?\))\s*(\w+)\s*" + _IDX, _product),
         (r"(\w+)\s*" + _IDX + r"\s*=\s*transpose\(\s*(\w+)\s*" + _IDX + r"\s*,\s*\{([^}]*)\}\s*\)", _transpose),
         (r"var\s+(\w+)\s*=\s*SUM\(\s*(\w+)\s*" + _IDX + r"\s*\)", _sum),
         (r"var\s+(\w+)\s*=\s*getTime\(\s*\)", _get_time),

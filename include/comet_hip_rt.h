@@ -162,14 +162,21 @@ int64_t comet_hip_spgemm_csr_semiring(int64_t a, int64_t b, int64_t mask, int re
 int comet_hip_vecmat_csr_f64(int64_t csr, int64_t x_dptr, int64_t y_dptr, int accumulate);
 int comet_hip_densemat_csr_f64(int64_t csr, int64_t M, int64_t a_dptr, int64_t lda,
                                int64_t c_dptr, int64_t ldc, int accumulate);
-/* C = A .* D for A in CSR and D dense (row-major, leading dimension ldd), with
- * either operand order of the source program (the product commutes): as a new
- * CSR with A's structure (eltwise_mult_CSRxDense_oCSR.ta), or written into a
- * dense C at A's stored positions, every other element of C left as it is
- * (eltwise_mult_CSRxDense_oDense.ta, eltwise_mult_DensexCSR_oDense.ta). */
-int64_t comet_hip_eltwise_mult_csr_dense_csr(int64_t a, int64_t d_dptr, int64_t ldd);
-int comet_hip_eltwise_mult_csr_dense_dense(int64_t a, int64_t d_dptr, int64_t ldd,
-                                           int64_t c_dptr, int64_t ldc);
+/* C = A (op) D elementwise for A in CSR and D dense (row-major, leading dimension
+ * ldd); op is a COMET_OP_* code: COMET_OP_TIMES is the `.*` of the language,
+ * the others its monoid forms `A @(+) D`, `@(-)`, `@(min)`, ...
+ * (test/integration/semiring/eltwise_monoid*_COOxDense_oCOO.ta; lowering as
+ * "noop_<op>", frontends/comet_dsl/mlir/MLIRGen.cpp:960-990).  A's value is the
+ * left operand; for the source order D (op) A of a commutative op pass the same
+ * call.  Result: a new CSR with A's structure (eltwise_mult_CSRxDense_oCSR.ta),
+ * or written into a dense C at A's stored positions, every other element of C
+ * left as it is (eltwise_mult_CSRxDense_oDense.ta, eltwise_mult_DensexCSR_oDense.ta). */
+int64_t comet_hip_eltwise_csr_dense_csr(int64_t a, int64_t d_dptr, int64_t ldd, int op);
+int comet_hip_eltwise_csr_dense_dense(int64_t a, int64_t d_dptr, int64_t ldd,
+                                      int64_t c_dptr, int64_t ldc, int op);
+/* c[i] = a[i] (op) b[i] over n dense elements
+ * (eltwise_monoid{Plus,Minus,Min,Times}_DensexDense_oDense.ta). */
+int comet_hip_eltwise_dense_f64(int64_t n, int64_t a_dptr, int64_t b_dptr, int64_t c_dptr, int op);
 
 /* ---- input side: MatrixMarket files, read modes, the file-id protocol ---------
  * Read modes of comet_read(id, mode): lib/ExecutionEngine/SparseUtils.cpp:40-64.

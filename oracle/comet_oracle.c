@@ -119,18 +119,28 @@ void oracle_densemat_csr(idx_t M, idx_t nrows, idx_t ncols, const double *A,
 }
 
 /* ------------------------------------------------------------------------- */
-/* CSR .* Dense: out[p] = val[p] * D[i, crd[p]] over the stored entries of A   */
-/* (the "noop_times" compute of an elementwise statement assigns, it does not  */
+/* CSR (op) Dense: out[p] = op(val[p], D[i, crd[p]]) over the stored entries of */
+/* A; op as the mult codes of oracle_spgemm_numeric_semiring, 0 = times = `.*`  */
+/* (the "noop_<op>" compute of an elementwise statement assigns, it does not    */
 /* accumulate: lib/Conversion/IndexTreeToSCF/IndexTreeToSCF.cpp:346-353,       */
 /* 1249-1284; frontends/comet_dsl/mlir/MLIRGen.cpp:960-990).  The caller puts  */
 /* out[p] into a CSR with A's structure or into a dense C at (i, crd[p]).      */
 /* ------------------------------------------------------------------------- */
-void oracle_eltwise_mult_csr_dense(idx_t nrows, idx_t ncols, const idx_t *pos, const idx_t *crd,
-                                   const double *val, const double *D, double *out)
+static double semiring_mult(int op, double a, double b);
+
+void oracle_eltwise_csr_dense(idx_t nrows, idx_t ncols, const idx_t *pos, const idx_t *crd,
+                              const double *val, const double *D, int op, double *out)
 {
     for (idx_t i = 0; i < nrows; ++i)
         for (idx_t p = pos[i]; p < pos[i + 1]; ++p)
-            out[p] = val[p] * D[i * ncols + crd[p]];
+            out[p] = semiring_mult(op, val[p], D[i * ncols + crd[p]]);
+}
+
+/* Dense (op) Dense, element by element.                                       */
+void oracle_eltwise_dense(idx_t n, const double *a, const double *b, int op, double *out)
+{
+    for (idx_t i = 0; i < n; ++i)
+        out[i] = semiring_mult(op, a[i], b[i]);
 }
 
 /* ------------------------------------------------------------------------- */

@@ -57,8 +57,10 @@ def lib():
     L.oracle_vecmat_csr.restype = None
     L.oracle_densemat_csr.argtypes = [C.c_int64, C.c_int64, C.c_int64, f64p, i64p, i64p, f64p, f64p]
     L.oracle_densemat_csr.restype = None
-    L.oracle_eltwise_mult_csr_dense.argtypes = [C.c_int64, C.c_int64, i64p, i64p, f64p, f64p, f64p]
-    L.oracle_eltwise_mult_csr_dense.restype = None
+    L.oracle_eltwise_csr_dense.argtypes = [C.c_int64, C.c_int64, i64p, i64p, f64p, f64p, C.c_int, f64p]
+    L.oracle_eltwise_csr_dense.restype = None
+    L.oracle_eltwise_dense.argtypes = [C.c_int64, f64p, f64p, C.c_int, f64p]
+    L.oracle_eltwise_dense.restype = None
     L.oracle_spgemm_symbolic.argtypes = [C.c_int64, C.c_int64, C.c_int64, i64p, i64p, i64p, i64p, vp, vp, i64p]
     L.oracle_spgemm_symbolic.restype = C.c_int64
     L.oracle_spgemm_numeric.argtypes = [C.c_int64, C.c_int64, C.c_int64, i64p, i64p, f64p, i64p, i64p, f64p,
@@ -140,12 +142,23 @@ def densemat(A, pos, crd, val, ncols, C0=None):
     return Cm
 
 
-def eltwise_mult_dense(pos, crd, val, D):
-    """Values of A .* D at A's stored positions, in storage order."""
+def eltwise_csr_dense(pos, crd, val, D, op="times"):
+    """Values of A (op) D at A's stored positions, in storage order."""
     pos, crd, val, D = _i64(pos), _i64(crd), _f64(val), _f64(D)
     out = np.zeros(max(len(val), 1))
-    lib().oracle_eltwise_mult_csr_dense(len(pos) - 1, D.shape[1], pos, crd, val, D, out)
+    lib().oracle_eltwise_csr_dense(len(pos) - 1, D.shape[1], pos, crd, val, D, MULT_OPS[op], out)
     return out[:len(val)]
+
+
+def eltwise_mult_dense(pos, crd, val, D):
+    return eltwise_csr_dense(pos, crd, val, D, "times")
+
+
+def eltwise_dense(a, b, op="times"):
+    a, b = _f64(a), _f64(b)
+    out = np.zeros(a.shape)
+    lib().oracle_eltwise_dense(a.size, a, b, MULT_OPS[op], out)
+    return out
 
 
 def spgemm_symbolic(Apos, Acrd, Bpos, Bcrd, ncolsB, mask=None, rows=None):

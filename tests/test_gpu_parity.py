@@ -871,3 +871,27 @@ def test_wrapped_arrays_changed_in_place_need_invalidate():
     assert np.array_equal(rt.spmm(A, dB).to_numpy(), -2.0 * first)       # scaling by -2 is exact
     assert np.array_equal(rt.spmv(A, dx).to_numpy(), -2.0 * y1)
     assert np.array_equal(rt.vecmat(dx, A).to_numpy(), -2.0 * z1)
+
+
+def test_eltwise_monoid_golden_and_checker(golden, golden_dir):
+    for g in golden["eltwise_monoid"]["dense"]:
+        a, b = np.full(g["shape"], g["a"]), np.full(g["shape"], g["b"])
+        out = rt.eltwise_dense(rt.DeviceArray.from_numpy(a), rt.DeviceArray.from_numpy(b), op=g["op"])
+        assert orc.format_f64(out.to_numpy()) == g["printed"], g["source"]
+    for g in golden["eltwise_monoid"]["coo_dense"]:
+        A = rt.CsrMatrix.from_mtx(os.path.join(golden_dir, g["matrix"]))
+        D = rt.DeviceArray.from_numpy(np.full(A.shape, g["d_fill"]))
+        r, c, v = rt.eltwise_csr_dense(A, D, op=g["op"]).to_coo()
+        assert r.tolist() == g["a1crd"] and c.tolist() == g["a2crd"] and orc.format_f64(v) == g["printed_val"]
+    rng = np.random.default_rng(5)
+    pos, crd, val = _rand_csr(rng, 400, 300, 0.05)
+    A = rt.CsrMatrix.from_arrays((400, 300), pos, crd, val)
+    D = rng.uniform(0.5, 2.0, (400, 300))
+    x, y = rng.uniform(-1, 1, 100_003), rng.uniform(0.5, 2, 100_003)
+    for op in rt.MULT_OPS:
+        if op in ("*", "+", "-", "/"):
+            continue
+        got = rt.eltwise_csr_dense(A, rt.DeviceArray.from_numpy(D), op=op).to_arrays()[2]
+        assert np.array_equal(got, orc.eltwise_csr_dense(pos, crd, val, D, op)), op
+        got = rt.eltwise_dense(rt.DeviceArray.from_numpy(x), rt.DeviceArray.from_numpy(y), op=op).to_numpy()
+        assert np.array_equal(got, orc.eltwise_dense(x, y, op)), op

@@ -509,3 +509,15 @@ def test_eltwise_mult_csr_dense_golden(golden, golden_dir):
     dense = np.zeros((nr, nc))
     dense[np.repeat(np.arange(nr), np.diff(pos)), crd] = v
     assert orc.format_f64(dense) == g["printed_dense"]
+
+
+def test_eltwise_monoid_golden(golden, golden_dir):
+    for g in golden["eltwise_monoid"]["dense"]:
+        out = orc.eltwise_dense(np.full(g["shape"], g["a"]), np.full(g["shape"], g["b"]), g["op"])
+        assert orc.format_f64(out) == g["printed"], g["source"]
+    for g in golden["eltwise_monoid"]["coo_dense"]:
+        (nr, nc), pos, crd, val = _mtx(golden_dir, g["matrix"])
+        v = orc.eltwise_csr_dense(pos, crd, val, np.full((nr, nc), g["d_fill"]), g["op"])
+        a1pos, a1crd, _, a2crd, _ = orc.coo_layout(pos, crd, val)
+        assert a1pos.tolist() == g["a1pos"] and a1crd.tolist() == g["a1crd"] and a2crd.tolist() == g["a2crd"]
+        assert orc.format_f64(v) == g["printed_val"], g["source"]

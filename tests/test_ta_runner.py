@@ -181,3 +181,28 @@ def main() {
     want = (golden["vecmat_csr"]["printed"] + golden["densemat_csr"]["printed"] + _ints([5]) + _ints([-1]) +
             _ints(g["pos"]) + _ints(g["crd"]) + g["printed_val"] + g["printed_dense"])
     _check(out, want, tmp_path)
+
+
+def test_elementwise_monoid_programs(golden, golden_dir, tmp_path, monkeypatch):
+    tok = {"plus": "+", "minus": "-", "times": "*", "min": "min"}
+    for g in golden["eltwise_monoid"]["dense"]:
+        labels = "abcd"[:len(g["shape"])]
+        idx = ", ".join(labels)
+        decl = "".join(f"    IndexLabel [{l}] = [{n}];\n" for l, n in zip(labels, g["shape"]))
+        prog = ("def main() {\n" + decl +
+                "".join(f"    Tensor<double> {t}([{idx}], {{Dense}});\n" for t in "ABC") +
+                f"    A[{idx}] = {g['a']};\n    B[{idx}] = {g['b']};\n    C[{idx}] = 0.0;\n" +
+                f"    C[{idx}] = A[{idx}] @({tok[g['op']]}) B[{idx}];\n    print(C);\n}}\n")
+        _check(_run(prog, [], tmp_path, monkeypatch, golden_dir), g["printed"], tmp_path)
+    for g in golden["eltwise_monoid"]["coo_dense"]:
+        prog = _decl("COO") + f"""
+    Tensor<double> D([a, b], {{Dense}});
+    Tensor<double> E([a, b], {{COO}});
+    A[a, b] = comet_read(0);
+    D[a, b] = {g['d_fill']};
+    E[a, b] = A[a, b] @({tok[g['op']]}) D[a, b];
+    print(E);
+}}
+"""
+        out = _run(prog, [g["matrix"]], tmp_path, monkeypatch, golden_dir)
+        _check(out, _ints(g["a1pos"]) + _ints(g["a1crd"]) + _ints([-1]) + _ints(g["a2crd"]) + g["printed_val"], tmp_path)
