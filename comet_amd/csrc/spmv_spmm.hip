@@ -410,36 +410,57 @@ constexpr int SPMM_HCB = 32;                         // column blocks a wavefron
 // is cut into 32 column blocks; inside a block the entries of one row follow
 // each other, columns ascending, so a row is still summed in ascending column
 // order, and a run of entries of one row is added into one plain register: the
-// register file is indexed dynamically only where a run begins (entry bit 3).
+// register file is indexed dynamically only where a run begins.
+//
+// A lane owns two adjacent dense columns and a half-wavefront one row of B, so
+// one load instruction fetches two rows, 16 bytes per lane: a CU takes 8-byte
+// gathers out of the L2 at 23 bytes per clock however few rows are in play,
+// 16-byte ones at 42 (measured with a gather-only kernel on a table of 0.3 to
+// 4 MB per XCD).  The two halves take the even and the odd entries of the same
+// run - runs are padded to even length by the plan, the pad carries no value -
+// and their sums are added once, at the end.
+//
 // A wavefront holds 64 entries of its list at a time, one per lane, and hands
 // them out with readlane; the next 64 are fetched while these are used, and the
-// gathers of the next 16 entries are in flight while the current 16 are added.
-// Entry = column << (SPMM_HRB + 1) | first-of-run << SPMM_HRB | owned row.
-__device__ inline void heavy_issue(double (&b)[SPMM_U], int ents, int t0, int cnt, const double *__restrict__ B,
-                                   int64_t ldb, int64_t col)
+// gathers of the next 8 pairs are in flight while the current 8 are added.
+// Entry = column << (SPMM_HRB + 2) | real << (SPMM_HRB + 1) | first-of-run << SPMM_HRB | owned row.
+constexpr int SPMM_HP = 8;       // pairs of entries per batch of gathers
+
+__device__ inline void heavy_issue(double2 (&b)[SPMM_HP], int ents, int t0, int npairs, int half,
+                                   const double *__restrict__ B, int64_t ldb, int64_t col)
 {
 #pragma unroll
-    for (int u = 0; u < SPMM_U; ++u) {
-        const int t = t0 + u < cnt ? t0 + u : cnt - 1;      // past the end: reload the last one, never used
-        const int64_t j = (int64_t)((unsigned)__builtin_amdgcn_readlane(ents, t) >> (SPMM_HRB + 1));
-        b[u] = B[j * ldb + col];
+    for (int u = 0; u < SPMM_HP; ++u) {
+        const int t = t0 + u < npairs ? t0 + u : npairs - 1;     // past the end: reload the last one, never used
+        const unsigned mine = (unsigned)__shfl(ents, 2 * t + half, 64);       // each half its own entry
+        const int64_t j = (int64_t)(mine >> (SPMM_HRB + 2));
+        b[u] = *reinterpret_cast<const double2 *>(B + j * ldb + col);
     }
 }
 
-__device__ inline void heavy_add(double (&acc)[SPMM_HR], double &run, int &run_slot, const double (&b)[SPMM_U],
-                                 int ents, double vals, int t0, int cnt)
+__device__ inline void heavy_add(double (&accx)[SPMM_HR], double (&accy)[SPMM_HR], double2 &run, int &run_slot,
+                                 const double2 (&b)[SPMM_HP], int ents, double vals, int t0, int npairs, int half)
 {
 #pragma unroll
-    for (int u = 0; u < SPMM_U; ++u) {
-        if (t0 + u < cnt) {
-            const int ent = __builtin_amdgcn_readlane(ents, t0 + u);
-            if (ent & SPMM_HR) {
-                acc[run_slot] = run;
-                run_slot = ent & (SPMM_HR - 1);
-                run = acc[run_slot];
+    for (int u = 0; u < SPMM_HP; ++u) {
+        if (t0 + u < npairs) {
+            const int t = t0 + u;
+            const int e0 = __builtin_amdgcn_readlane(ents, 2 * t);
+            if (e0 & SPMM_HR) {                  // a run starts on an even entry
+                accx[run_slot] = run.x;
+                accy[run_slot] = run.y;
+                run_slot = e0 & (SPMM_HR - 1);
+                run.x = accx[run_slot];
+                run.y = accy[run_slot];
             }
-            const double prod = readlane_f64(vals, t0 + u) * b[u];
-            run = run + prod;
+            const int mine = __shfl(ents, 2 * t + half, 64);
+            const double v = __hiloint2double(__shfl(__double2hiint(vals), 2 * t + half, 64),
+                                              __shfl(__double2loint(vals), 2 * t + half, 64));
+            const double px = v * b[u].x, py = v * b[u].y;
+            if (mine & (2 * SPMM_HR)) {          // a pad carries no value
+                run.x = run.x + px;
+                run.y = run.y + py;
+            }
         }
     }
 }
@@ -449,22 +470,22 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
     const double *__restrict__ B, int64_t ldb, int64_t K, double *__restrict__ partial)
 {
     constexpr int G = SPMM_HG;
-    const int lane = threadIdx.x & 63;
+    const int lane = threadIdx.x & 63, half = lane >> 5, sub = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int x = blockIdx.x & 7, g = blockIdx.x >> 3;
-    int64_t col = (int64_t)blockIdx.y * 64 + lane;
+    int64_t col = (int64_t)blockIdx.y * 64 + 2 * sub;          // K is even: a lane's two columns exist or neither
     const bool active = col < K;
     if (!active)
-        col = K - 1;            // idle lanes gather a valid address and store nothing
-    double acc[SPMM_HR];
+        col = K - 2;            // idle lanes gather a valid address and store nothing
+    double accx[SPMM_HR], accy[SPMM_HR];      // two plain arrays: each is indexed through M0, a double2 array is not
 #pragma unroll
     for (int r = 0; r < SPMM_HR; ++r)
-        acc[r] = 0.0;
+        accx[r] = accy[r] = 0.0;
     const int64_t bin = ((int64_t)x * G + g) * SPMM_HW + wave;
-    const int64_t s = seg[bin], e = seg[bin + 1];
+    const int64_t s = seg[bin], e = seg[bin + 1];          // both even
     if (s < e) {
-        double bA[SPMM_U], bB[SPMM_U];
-        double run = 0.0;
+        double2 bA[SPMM_HP], bB[SPMM_HP];
+        double2 run = make_double2(0.0, 0.0);
         int run_slot = 0;
         int cnt = (int)(e - s < 64 ? e - s : 64);
         int c_ent = 0;
@@ -473,7 +494,7 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
             c_ent = __builtin_nontemporal_load(hent + s + lane);
             c_val = __builtin_nontemporal_load(hval + s + lane);
         }
-        heavy_issue(bA, c_ent, 0, cnt, B, ldb, col);
+        heavy_issue(bA, c_ent, 0, cnt >> 1, half, B, ldb, col);
         for (int64_t base = s; base < e; base += 64) {
             const int64_t left = e - base - 64;
             const int ncnt = (int)(left < 0 ? 0 : (left < 64 ? left : 64));
@@ -483,30 +504,36 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
                 n_ent = __builtin_nontemporal_load(hent + base + 64 + lane);
                 n_val = __builtin_nontemporal_load(hval + base + 64 + lane);
             }
-            static_assert(SPMM_U == 16, "the sweep is unrolled for four batches of 16 per 64 entries");
-            if (cnt > 16)
-                heavy_issue(bB, c_ent, 16, cnt, B, ldb, col);
-            heavy_add(acc, run, run_slot, bA, c_ent, c_val, 0, cnt);
-            if (cnt > 32)
-                heavy_issue(bA, c_ent, 32, cnt, B, ldb, col);
-            heavy_add(acc, run, run_slot, bB, c_ent, c_val, 16, cnt);
-            if (cnt > 48)
-                heavy_issue(bB, c_ent, 48, cnt, B, ldb, col);
-            heavy_add(acc, run, run_slot, bA, c_ent, c_val, 32, cnt);
+            const int np = cnt >> 1;
+            static_assert(SPMM_HP == 8, "the sweep is unrolled for four batches of 8 pairs per 64 entries");
+            if (np > 8)
+                heavy_issue(bB, c_ent, 8, np, half, B, ldb, col);
+            heavy_add(accx, accy, run, run_slot, bA, c_ent, c_val, 0, np, half);
+            if (np > 16)
+                heavy_issue(bA, c_ent, 16, np, half, B, ldb, col);
+            heavy_add(accx, accy, run, run_slot, bB, c_ent, c_val, 8, np, half);
+            if (np > 24)
+                heavy_issue(bB, c_ent, 24, np, half, B, ldb, col);
+            heavy_add(accx, accy, run, run_slot, bA, c_ent, c_val, 16, np, half);
             if (ncnt > 0)
-                heavy_issue(bA, n_ent, 0, ncnt, B, ldb, col);
-            heavy_add(acc, run, run_slot, bB, c_ent, c_val, 48, cnt);
+                heavy_issue(bA, n_ent, 0, ncnt >> 1, half, B, ldb, col);
+            heavy_add(accx, accy, run, run_slot, bB, c_ent, c_val, 24, np, half);
             c_ent = n_ent;
             c_val = n_val;
             cnt = ncnt;
         }
-        acc[run_slot] = run;
+        accx[run_slot] = run.x;
+        accy[run_slot] = run.y;
     }
-    if (active) {
-        double *out = partial + (((int64_t)x * G + g) * SPMM_HW + wave) * SPMM_HR * K;
+    // even entries + odd entries, then the lower half writes both columns
+    double *out = partial + (((int64_t)x * G + g) * SPMM_HW + wave) * SPMM_HR * K;
 #pragma unroll
-        for (int r = 0; r < SPMM_HR; ++r)
-            out[(int64_t)r * K + col] = acc[r];
+    for (int r = 0; r < SPMM_HR; ++r) {
+        const double ox = __shfl_down(accx[r], 32, 64), oy = __shfl_down(accy[r], 32, 64);
+        if (active && half == 0) {
+            out[(int64_t)r * K + col] = accx[r] + ox;
+            out[(int64_t)r * K + col + 1] = accy[r] + oy;
+        }
     }
 }
 
@@ -590,21 +617,56 @@ __global__ void heavy_make_keys(int64_t nheavy, const int32_t *__restrict__ hrow
     }
 }
 
-__global__ void heavy_fill(int64_t n, const uint64_t *__restrict__ keys, const uint32_t *__restrict__ idx,
-                           const double *__restrict__ val, int32_t *__restrict__ hent, double *__restrict__ hval)
+// first[e] = 1 where entry e of the ordered list opens a run (another row, column block or wavefront)
+__global__ void heavy_mark_runs(int64_t n, const uint64_t *__restrict__ keys, int64_t *__restrict__ first)
 {
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e < n) {
-        const uint64_t k = keys[e];
-        const bool first = e == 0 || (keys[e - 1] >> 28) != (k >> 28);     // another row, block or wavefront
-        hent[e] = (int32_t)(uint32_t)(((k & 0xfffffffull) << (SPMM_HRB + 1)) | (first ? (uint64_t)SPMM_HR : 0u) |
-                                      ((k >> 28) & (SPMM_HR - 1)));
-        hval[e] = val[idx[e]];
+    if (e < n)
+        first[e] = (e == 0 || (keys[e - 1] >> 28) != (keys[e] >> 28)) ? 1 : 0;
+}
+
+// start[r] = first entry of run r (runs[e] = runs opened before e); start[nruns] = n
+__global__ void heavy_run_starts(int64_t n, const int64_t *__restrict__ first, const int64_t *__restrict__ runs,
+                                 int64_t *__restrict__ start)
+{
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < n && first[e])
+        start[runs[e]] = e;
+    if (e == n)
+        start[runs[n]] = n;
+}
+
+__global__ void heavy_run_odd(int64_t nruns, const int64_t *__restrict__ start, int64_t *__restrict__ odd)
+{
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r < nruns)
+        odd[r] = (start[r + 1] - start[r]) & 1;
+}
+
+// Writes the list with every run padded to even length: entry e of run r lands at e + (pads in front of r).
+__global__ void heavy_fill(int64_t n, const uint64_t *__restrict__ keys, const uint32_t *__restrict__ idx,
+                           const double *__restrict__ val, const int64_t *__restrict__ first,
+                           const int64_t *__restrict__ runs, const int64_t *__restrict__ start,
+                           const int64_t *__restrict__ pads, int32_t *__restrict__ hent, double *__restrict__ hval)
+{
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n)
+        return;
+    const uint64_t k = keys[e];
+    const int64_t r = runs[e] + first[e] - 1;
+    const int64_t p = e + pads[r];
+    const uint32_t body = (uint32_t)(((k & 0xfffffffull) << (SPMM_HRB + 2)) | ((k >> 28) & (SPMM_HR - 1)));
+    hent[p] = (int32_t)(body | (2u * SPMM_HR) | (first[e] ? (uint32_t)SPMM_HR : 0u));
+    hval[p] = val[idx[e]];
+    if (e + 1 == start[r + 1] && ((start[r + 1] - start[r]) & 1)) {     // last entry of a run of odd length
+        hent[p + 1] = (int32_t)body;       // same column (a valid address), no value
+        hval[p + 1] = 0.0;
     }
 }
 
-// seg[b] = first list entry whose (XCD, wavefront) number is >= b
-__global__ void heavy_segments(int64_t n, const uint64_t *__restrict__ keys, int64_t *__restrict__ seg)
+// seg[b] = position in the padded list of the first entry whose (XCD, wavefront) number is >= b
+__global__ void heavy_segments(int64_t n, const uint64_t *__restrict__ keys, const int64_t *__restrict__ runs,
+                               const int64_t *__restrict__ pads, int64_t *__restrict__ seg)
 {
     const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (b > 8 * SPMM_HBINS)
@@ -617,7 +679,7 @@ __global__ void heavy_segments(int64_t n, const uint64_t *__restrict__ keys, int
         else
             hi = mid;
     }
-    seg[b] = lo;
+    seg[b] = lo + pads[runs[lo]];      // lo opens a run (or is n): runs[lo] is that run's number
 }
 
 __global__ void light_lengths(int64_t nrows, const int64_t *__restrict__ pos, const int32_t *__restrict__ rowcode,
@@ -698,6 +760,7 @@ static int spmm_heavy_plan(Csr *a)
     }
     int32_t *d_cnt = nullptr, *d_rowcode = nullptr;
     int64_t *d_hstart = nullptr, *d_len = nullptr;
+    int64_t *d_first = nullptr, *d_runs = nullptr, *d_start = nullptr, *d_odd = nullptr, *d_pads = nullptr;
     uint64_t *k_in = nullptr, *k_out = nullptr;
     uint32_t *i_in = nullptr, *i_out = nullptr;
     Csr *light = new Csr();
@@ -706,6 +769,11 @@ static int spmm_heavy_plan(Csr *a)
         (void)hipFree(d_rowcode);
         (void)hipFree(d_hstart);
         (void)hipFree(d_len);
+        (void)hipFree(d_first);
+        (void)hipFree(d_runs);
+        (void)hipFree(d_start);
+        (void)hipFree(d_odd);
+        (void)hipFree(d_pads);
         (void)hipFree(k_in);
         (void)hipFree(k_out);
         (void)hipFree(i_in);
@@ -739,8 +807,6 @@ static int spmm_heavy_plan(Csr *a)
     HEAVY_TRY(hipMalloc((void **)&i_in, 4 * (size_t)hnnz));
     HEAVY_TRY(hipMalloc((void **)&i_out, 4 * (size_t)hnnz));
     HEAVY_TRY(hipMalloc((void **)&a->heavy_seg, 8 * (size_t)(8 * SPMM_HBINS + 1)));
-    HEAVY_TRY(hipMalloc((void **)&a->heavy_col, 4 * (size_t)hnnz));
-    HEAVY_TRY(hipMalloc((void **)&a->heavy_val, 8 * (size_t)hnnz));
     HEAVY_TRY(hipMalloc((void **)&a->heavy_row, 4 * (size_t)H));
     HEAVY_TRY(hipMalloc((void **)&a->heavy_code, 4 * (size_t)(8 * H)));
     HEAVY_TRY(hipMemcpyAsync(a->heavy_row, hrow.data(), 4 * (size_t)H, hipMemcpyHostToDevice, stream()));
@@ -789,12 +855,37 @@ static int spmm_heavy_plan(Csr *a)
         cleanup(true);
         return COMET_HIP_ERR_HIP;
     }
+    // runs (entries of one row inside one column block of one wavefront's list) are padded to even length
+    HEAVY_TRY(hipMalloc((void **)&d_first, 8 * (size_t)hnnz));
+    HEAVY_TRY(hipMalloc((void **)&d_runs, 8 * (size_t)(hnnz + 1)));
+    HEAVY_TRY(hipMalloc((void **)&d_start, 8 * (size_t)(hnnz + 1)));
+    HEAVY_TRY(hipMalloc((void **)&d_odd, 8 * (size_t)hnnz));
+    HEAVY_TRY(hipMalloc((void **)&d_pads, 8 * (size_t)(hnnz + 1)));
+    const dim3 per_entry((unsigned)ceil_div(hnnz + 1, 256));
+    heavy_mark_runs<<<per_entry, dim3(256), 0, stream()>>>(hnnz, k_out, d_first);
+    if (exclusive_scan_i64(d_first, hnnz, d_runs) != COMET_HIP_OK) {
+        cleanup(true);
+        return COMET_HIP_ERR_HIP;
+    }
+    int64_t nruns = 0, npads = 0;
+    HEAVY_TRY(hipMemcpyAsync(&nruns, d_runs + hnnz, 8, hipMemcpyDeviceToHost, stream()));
+    HEAVY_TRY(hipStreamSynchronize(stream()));
+    heavy_run_starts<<<per_entry, dim3(256), 0, stream()>>>(hnnz, d_first, d_runs, d_start);
+    heavy_run_odd<<<dim3((unsigned)ceil_div(nruns, 256)), dim3(256), 0, stream()>>>(nruns, d_start, d_odd);
+    if (exclusive_scan_i64(d_odd, nruns, d_pads) != COMET_HIP_OK) {
+        cleanup(true);
+        return COMET_HIP_ERR_HIP;
+    }
+    HEAVY_TRY(hipMemcpyAsync(&npads, d_pads + nruns, 8, hipMemcpyDeviceToHost, stream()));
+    HEAVY_TRY(hipStreamSynchronize(stream()));
+    HEAVY_TRY(hipMalloc((void **)&a->heavy_col, 4 * (size_t)(hnnz + npads)));
+    HEAVY_TRY(hipMalloc((void **)&a->heavy_val, 8 * (size_t)(hnnz + npads)));
     {
         KernelTimer t("heavy_fill");
         heavy_fill<<<dim3((unsigned)ceil_div(hnnz, 256)), dim3(256), 0, stream()>>>(
-            hnnz, k_out, i_out, a->val, a->heavy_col, a->heavy_val);
+            hnnz, k_out, i_out, a->val, d_first, d_runs, d_start, d_pads, a->heavy_col, a->heavy_val);
         heavy_segments<<<dim3((unsigned)ceil_div(8 * SPMM_HBINS + 1, 256)), dim3(256), 0, stream()>>>(
-            hnnz, k_out, a->heavy_seg);
+            hnnz, k_out, d_runs, d_pads, a->heavy_seg);
     }
     // the rest of the matrix, long rows left empty
     light->nrows = n;
@@ -892,9 +983,12 @@ static int spmm_run(Csr *a, int64_t K, int64_t b_dptr, int64_t ldb, int64_t c_dp
     if (ceil_div(K, 64) > 65535)
         return set_error(COMET_HIP_ERR_SIZE, "K = %lld needs more than 65535 column tiles", (long long)K);
     // long rows: column sweep with the sums on chip; everything else: one wavefront per 256 nonzeros
-    if (K >= 16 && K <= 2048 && getenv("COMET_SPMM_NO_SWEEP") == nullptr)
+    // (the sweep loads B sixteen bytes at a time: two columns per lane, rows aligned to that)
+    const bool sweep_fits = K >= 16 && K <= 2048 && (K & 1) == 0 && (ldb & 1) == 0 && (b_dptr & 15) == 0 &&
+                            getenv("COMET_SPMM_NO_SWEEP") == nullptr;
+    if (sweep_fits)
         COMET_CHK(spmm_heavy_plan(a));
-    if (a->heavy_state != 2 || K < 16 || K > 2048 || getenv("COMET_SPMM_NO_SWEEP") != nullptr)
+    if (a->heavy_state != 2 || !sweep_fits)
         return spmm_chunks(a, K, B, ldb, C, ldc, accumulate);
     // the long rows are empty in `light`: cleared (or, accumulating, left alone) there, then added to below
     COMET_CHK(spmm_chunks(a->light, K, B, ldb, C, ldc, accumulate));
