@@ -426,6 +426,9 @@ constexpr int SPMM_HCB = 32;                         // column blocks a wavefron
 // Entry = column << (SPMM_HRB + 2) | real << (SPMM_HRB + 1) | first-of-run << SPMM_HRB | owned row.
 constexpr int SPMM_HP = 8;       // pairs of entries per batch of gathers
 
+// SMALL: B spans less than 4 GiB and has fewer than 2^24 rows of fewer than 2^24 bytes, so the byte offset of a
+// gather is one 24-bit multiply and one add in 32 bits on top of a scalar base, instead of a 64-bit multiply.
+template <bool SMALL>
 __device__ inline void heavy_issue(double2 (&b)[SPMM_HP], int ents, int t0, int npairs, int half,
                                    const double *__restrict__ B, int64_t ldb, int64_t col)
 {
@@ -433,8 +436,13 @@ __device__ inline void heavy_issue(double2 (&b)[SPMM_HP], int ents, int t0, int 
     for (int u = 0; u < SPMM_HP; ++u) {
         const int t = t0 + u < npairs ? t0 + u : npairs - 1;     // past the end: reload the last one, never used
         const unsigned mine = (unsigned)__shfl(ents, 2 * t + half, 64);       // each half its own entry
-        const int64_t j = (int64_t)(mine >> (SPMM_HRB + 2));
-        b[u] = *reinterpret_cast<const double2 *>(B + j * ldb + col);
+        if constexpr (SMALL) {
+            const unsigned off = __umul24(mine >> (SPMM_HRB + 2), (unsigned)ldb * 8u) + (unsigned)col * 8u;
+            b[u] = *reinterpret_cast<const double2 *>(reinterpret_cast<const char *>(B) + off);
+        } else {
+            const int64_t j = (int64_t)(mine >> (SPMM_HRB + 2));
+            b[u] = *reinterpret_cast<const double2 *>(B + j * ldb + col);
+        }
     }
 }
 
@@ -465,6 +473,7 @@ __device__ inline void heavy_add(double (&accx)[SPMM_HR], double (&accy)[SPMM_HR
     }
 }
 
+template <bool SMALL>
 __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
     const int64_t *__restrict__ seg, const int32_t *__restrict__ hent, const double *__restrict__ hval,
     const double *__restrict__ B, int64_t ldb, int64_t K, double *__restrict__ partial)
@@ -494,7 +503,7 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
             c_ent = __builtin_nontemporal_load(hent + s + lane);
             c_val = __builtin_nontemporal_load(hval + s + lane);
         }
-        heavy_issue(bA, c_ent, 0, cnt >> 1, half, B, ldb, col);
+        heavy_issue<SMALL>(bA, c_ent, 0, cnt >> 1, half, B, ldb, col);
         for (int64_t base = s; base < e; base += 64) {
             const int64_t left = e - base - 64;
             const int ncnt = (int)(left < 0 ? 0 : (left < 64 ? left : 64));
@@ -507,16 +516,16 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
             const int np = cnt >> 1;
             static_assert(SPMM_HP == 8, "the sweep is unrolled for four batches of 8 pairs per 64 entries");
             if (np > 8)
-                heavy_issue(bB, c_ent, 8, np, half, B, ldb, col);
+                heavy_issue<SMALL>(bB, c_ent, 8, np, half, B, ldb, col);
             heavy_add(accx, accy, run, run_slot, bA, c_ent, c_val, 0, np, half);
             if (np > 16)
-                heavy_issue(bA, c_ent, 16, np, half, B, ldb, col);
+                heavy_issue<SMALL>(bA, c_ent, 16, np, half, B, ldb, col);
             heavy_add(accx, accy, run, run_slot, bB, c_ent, c_val, 8, np, half);
             if (np > 24)
-                heavy_issue(bB, c_ent, 24, np, half, B, ldb, col);
+                heavy_issue<SMALL>(bB, c_ent, 24, np, half, B, ldb, col);
             heavy_add(accx, accy, run, run_slot, bA, c_ent, c_val, 16, np, half);
             if (ncnt > 0)
-                heavy_issue(bA, n_ent, 0, ncnt >> 1, half, B, ldb, col);
+                heavy_issue<SMALL>(bA, n_ent, 0, ncnt >> 1, half, B, ldb, col);
             heavy_add(accx, accy, run, run_slot, bB, c_ent, c_val, 24, np, half);
             c_ent = n_ent;
             c_val = n_val;
@@ -829,8 +838,8 @@ static int spmm_heavy_plan(Csr *a)
         std::sort(order.begin(), order.end());
         // (time the wavefront needs for its list so far, wavefront).  The four wavefronts of a SIMD do not
         // run at the same speed: the older one wins every arbitration, and the measured entry rates of
-        // wavefronts 0-3, 4-7, 8-11, 12-15 of a workgroup are as 1.21 : 1.06 : 0.91 : 0.81.
-        static const double pace[4] = {1.0 / 1.215, 1.0 / 1.059, 1.0 / 0.913, 1.0 / 0.812};
+        // wavefronts 0-3, 4-7, 8-11, 12-15 of a workgroup are as 1.12 : 1.05 : 0.96 : 0.87.
+        static const double pace[4] = {1.0 / 1.12, 1.0 / 1.05, 1.0 / 0.96, 1.0 / 0.87};
         std::priority_queue<std::pair<double, int32_t>, std::vector<std::pair<double, int32_t>>,
                             std::greater<std::pair<double, int32_t>>> bins;
         std::vector<int32_t> used(SPMM_HBINS, 0);
@@ -996,8 +1005,13 @@ static int spmm_run(Csr *a, int64_t K, int64_t b_dptr, int64_t ldb, int64_t c_dp
     const unsigned tiles = (unsigned)ceil_div(K, 64);
     {
         KernelTimer t("spmm_heavy_sweep");
-        spmm_heavy_sweep<<<dim3(8 * SPMM_HG, tiles), dim3(SPMM_HW * 64), 0, stream()>>>(
-            a->heavy_seg, a->heavy_col, a->heavy_val, B, ldb, K, (double *)g_heavy_partial.ptr);
+        const bool small_b = a->ncols < (1 << 24) && ldb * 8 < (1 << 24) && a->ncols * ldb * 8 < (1ll << 32);
+        if (small_b)
+            spmm_heavy_sweep<true><<<dim3(8 * SPMM_HG, tiles), dim3(SPMM_HW * 64), 0, stream()>>>(
+                a->heavy_seg, a->heavy_col, a->heavy_val, B, ldb, K, (double *)g_heavy_partial.ptr);
+        else
+            spmm_heavy_sweep<false><<<dim3(8 * SPMM_HG, tiles), dim3(SPMM_HW * 64), 0, stream()>>>(
+                a->heavy_seg, a->heavy_col, a->heavy_val, B, ldb, K, (double *)g_heavy_partial.ptr);
     }
     {
         KernelTimer t("spmm_heavy_combine");
