@@ -43,6 +43,13 @@ struct Workspace {
     void release();
 };
 
+// One entry of the lists the SpMM sweep reads (16 bytes, one load).
+struct HeavyEnt {
+    int32_t ent;        // column, flags and the owned row the value adds to (see spmm_heavy_sweep)
+    int32_t row;        // row of C the product is stored to, for a row with a single nonzero
+    double val;
+};
+
 struct Csr {
     int64_t nrows = 0, ncols = 0, nnz = 0;
     int64_t *pos = nullptr;
@@ -70,12 +77,16 @@ struct Csr {
     int heavy_state = 0;
     int64_t heavy_nnz = 0;
     int64_t *heavy_seg = nullptr;            // [8 * 512 + 1] list boundaries
-    int32_t *heavy_col = nullptr;            // column << 4 | first entry of a run << 3 | which of the wavefront's rows
-    double *heavy_val = nullptr;
+    HeavyEnt *heavy_ent = nullptr;           // the lists, runs padded to even length
     int64_t heavy_rows = 0;
     int32_t *heavy_row = nullptr;            // [heavy_rows] row ids of the long rows
     int32_t *heavy_code = nullptr;           // [8][heavy_rows] wavefront * 8 + slot that holds the row on each XCD
     Csr *light = nullptr;
+    // only in a `light` matrix: it lists some rows of the product only, row r of pos being row rowmap[r] of C
+    int32_t *rowmap = nullptr;
+    // rows of the original that store nothing (the product clears them when it does not accumulate)
+    int32_t *empty_rows = nullptr;
+    int64_t nempty = 0;
     // the transpose, built the first time a dense-times-sparse product needs it
     Csr *transposed = nullptr;
 };

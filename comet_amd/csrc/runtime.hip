@@ -142,14 +142,17 @@ static void csr_drop_plans(Csr *c)
     if (c->transposed)
         csr_release(c->transposed);
     c->light = c->transposed = nullptr;
+    (void)hipFree(c->rowmap);
+    (void)hipFree(c->empty_rows);
+    c->rowmap = c->empty_rows = nullptr;
+    c->nempty = 0;
     (void)hipFree(c->heavy_seg);
-    (void)hipFree(c->heavy_col);
-    (void)hipFree(c->heavy_val);
+    (void)hipFree(c->heavy_ent);
     (void)hipFree(c->heavy_row);
     (void)hipFree(c->heavy_code);
     c->heavy_seg = nullptr;
-    c->heavy_col = c->heavy_row = c->heavy_code = nullptr;
-    c->heavy_val = nullptr;
+    c->heavy_ent = nullptr;
+    c->heavy_row = c->heavy_code = nullptr;
     c->heavy_state = 0;
     c->heavy_nnz = c->heavy_rows = 0;
     (void)hipFree(c->spmm_chunk_row);

@@ -266,8 +266,10 @@ __global__ __launch_bounds__(SPMM_WAVES * 64) void spmm_csr_nnzsplit(
     const int64_t *__restrict__ pos, const int32_t *__restrict__ crd, const double *__restrict__ val,
     int64_t nnz, int64_t nrows, const int32_t *__restrict__ chunk_row, int64_t nchunks,
     const double *__restrict__ B, int64_t ldb, double *__restrict__ C, int64_t ldc, int64_t K,
-    double *__restrict__ carry)
+    double *__restrict__ carry, const int32_t *__restrict__ rowmap)
 {
+    // rowmap: the matrix lists only some rows of C (row r of pos is row rowmap[r] of C); nullptr: all of them
+    auto crow = [&](int64_t r) -> int64_t { return rowmap ? (int64_t)rowmap[r] : r; };
     const int lane = threadIdx.x & 63;
     const int64_t chunk =
         (int64_t)blockIdx.x * SPMM_WAVES + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -287,12 +289,12 @@ __global__ __launch_bounds__(SPMM_WAVES * 64) void spmm_csr_nnzsplit(
     // rows in front of the first stored nonzero are empty: chunk 0 clears them
     if (!ACC && chunk == 0 && active)
         for (int64_t z = 0; z < r; ++z)
-            C[z * ldc + col] = 0.0;
+            C[crow(z) * ldc + col] = 0.0;
 
     double acc = 0.0;
     // a row that goes on past this chunk leaves its C value to the fix-up kernel
     if (ACC && !head && rend <= e && active)
-        acc = C[r * ldc + col];
+        acc = C[crow(r) * ldc + col];
 
     for (int64_t base = s; base < e; base += 64) {
         const int cnt = (int)(e - base < 64 ? e - base : 64);
@@ -327,7 +329,7 @@ __global__ __launch_bounds__(SPMM_WAVES * 64) void spmm_csr_nnzsplit(
                             if (first_piece && head)
                                 carry0[lane] = acc;
                             else     // C is written once and not read again by this kernel
-                                __builtin_nontemporal_store(acc, C + r * ldc + col);
+                                __builtin_nontemporal_store(acc, C + crow(r) * ldc + col);
                         }
                         first_piece = false;
                         open = false;
@@ -339,7 +341,7 @@ __global__ __launch_bounds__(SPMM_WAVES * 64) void spmm_csr_nnzsplit(
                         acc = 0.0;
                         // a row that starts here and ends later keeps its C value for the fix-up instead
                         if (ACC && active && rend > p && rend <= e)
-                            acc = C[r * ldc + col];
+                            acc = C[crow(r) * ldc + col];
                     }
                 }
             }
@@ -358,7 +360,8 @@ __global__ __launch_bounds__(SPMM_WAVES * 64) void spmm_csr_nnzsplit(
 template <bool ACC>
 __global__ __launch_bounds__(SPMM_WAVES * 64) void spmm_csr_fixup(
     const int64_t *__restrict__ pos, int64_t nnz, const int32_t *__restrict__ chunk_row, int64_t nchunks,
-    double *__restrict__ C, int64_t ldc, int64_t K, const double *__restrict__ carry)
+    double *__restrict__ C, int64_t ldc, int64_t K, const double *__restrict__ carry,
+    const int32_t *__restrict__ rowmap)
 {
     const int lane = threadIdx.x & 63;
     const int64_t chunk =
@@ -377,11 +380,12 @@ __global__ __launch_bounds__(SPMM_WAVES * 64) void spmm_csr_fixup(
     const int64_t c0 = rs / SPMM_CH;
     const double *cb = carry + ((int64_t)blockIdx.y * nchunks * 2) * 64;
     double acc = cb[(c0 * 2 + 1) * 64 + lane];
+    const int64_t cr = rowmap ? (int64_t)rowmap[r] : r;
     if (ACC)
-        acc = C[r * ldc + col] + acc;
+        acc = C[cr * ldc + col] + acc;
     for (int64_t c = c0 + 1; c <= chunk; ++c)
         acc = acc + cb[(c * 2) * 64 + lane];
-    C[r * ldc + col] = acc;
+    C[cr * ldc + col] = acc;
 }
 
 // ============================================================================
@@ -399,7 +403,8 @@ constexpr int SPMM_HR = 1 << SPMM_HRB;               // rows a wavefront can own
 constexpr int SPMM_HCOLB = 28 - SPMM_HRB;            // bits of a list entry left for the column
 constexpr int SPMM_HG = 32;      // workgroups per XCD: one per CU, so that all of them sweep together
 constexpr int SPMM_HBINS = SPMM_HG * SPMM_HW;        // wavefronts (= row bins) per XCD
-constexpr int SPMM_HSLOTS = SPMM_HBINS * SPMM_HR;    // long rows the plan can hold
+constexpr int SPMM_HSLOTS = SPMM_HBINS * SPMM_HR;    // slots for partial sums: 16 wavefronts x 8 rows per workgroup
+constexpr int SPMM_HROWS = SPMM_HG * (SPMM_HW - 1) * SPMM_HR;    // long rows the plan can hold
 constexpr int SPMM_HEAVY_MIN_LEN = COMET_SPMM_HEAVY_MIN;              // a long row has at least this many nonzeros
 constexpr int SPMM_HCB = 32;                         // column blocks a wavefront's list is cut into
 
@@ -412,6 +417,14 @@ constexpr int SPMM_HCB = 32;                         // column blocks a wavefron
 // order, and a run of entries of one row is added into one plain register: the
 // register file is indexed dynamically only where a run begins.
 //
+// Rows with a single nonzero ride along: the last wavefront of every workgroup
+// owns no long rows; its list holds such rows, ordered by column, and it stores
+// each product straight to that row of C.  It moves through the columns with
+// the others, so its rows of B come out of the L2 window the long rows keep
+// warm instead of being fetched from HBM one row each.  (Stores inside the
+// lists of the long rows would stall them: loads and stores share one in-order
+// counter, so every wait for a gather behind a store waits for that store too.)
+//
 // A lane owns two adjacent dense columns and a half-wavefront one row of B, so
 // one load instruction fetches two rows, 16 bytes per lane: a CU takes 8-byte
 // gathers out of the L2 at 23 bytes per clock however few rows are in play,
@@ -423,8 +436,12 @@ constexpr int SPMM_HCB = 32;                         // column blocks a wavefron
 // A wavefront holds 64 entries of its list at a time, one per lane, and hands
 // them out with readlane; the next 64 are fetched while these are used, and the
 // gathers of the next 8 pairs are in flight while the current 8 are added.
-// Entry = column << (SPMM_HRB + 2) | real << (SPMM_HRB + 1) | first-of-run << SPMM_HRB | owned row.
+// Entry = column << SPMM_E_COL | real | first-of-run | owned row.
 constexpr int SPMM_HP = 8;       // pairs of entries per batch of gathers
+constexpr int SPMM_E_FIRST = SPMM_HR;          // the entry opens a run of one owned row
+constexpr int SPMM_E_REAL = 2 * SPMM_HR;       // not a pad
+constexpr int SPMM_E_COL = SPMM_HRB + 2;
+constexpr int SPMM_HWL = SPMM_HW - 1;          // wavefronts of a workgroup that own long rows
 
 // SMALL: B spans less than 4 GiB and has fewer than 2^24 rows of fewer than 2^24 bytes, so the byte offset of a
 // gather is one 24-bit multiply and one add in 32 bits on top of a scalar base, instead of a 64-bit multiply.
@@ -437,10 +454,10 @@ __device__ inline void heavy_issue(double2 (&b)[SPMM_HP], int ents, int t0, int 
         const int t = t0 + u < npairs ? t0 + u : npairs - 1;     // past the end: reload the last one, never used
         const unsigned mine = (unsigned)__shfl(ents, 2 * t + half, 64);       // each half its own entry
         if constexpr (SMALL) {
-            const unsigned off = __umul24(mine >> (SPMM_HRB + 2), (unsigned)ldb * 8u) + (unsigned)col * 8u;
+            const unsigned off = __umul24(mine >> SPMM_E_COL, (unsigned)ldb * 8u) + (unsigned)col * 8u;
             b[u] = *reinterpret_cast<const double2 *>(reinterpret_cast<const char *>(B) + off);
         } else {
-            const int64_t j = (int64_t)(mine >> (SPMM_HRB + 2));
+            const int64_t j = (int64_t)(mine >> SPMM_E_COL);
             b[u] = *reinterpret_cast<const double2 *>(B + j * ldb + col);
         }
     }
@@ -454,7 +471,7 @@ __device__ inline void heavy_add(double (&accx)[SPMM_HR], double (&accy)[SPMM_HR
         if (t0 + u < npairs) {
             const int t = t0 + u;
             const int e0 = __builtin_amdgcn_readlane(ents, 2 * t);
-            if (e0 & SPMM_HR) {                  // a run starts on an even entry
+            if (e0 & SPMM_E_FIRST) {             // a run starts on an even entry
                 accx[run_slot] = run.x;
                 accy[run_slot] = run.y;
                 run_slot = e0 & (SPMM_HR - 1);
@@ -465,7 +482,7 @@ __device__ inline void heavy_add(double (&accx)[SPMM_HR], double (&accy)[SPMM_HR
             const double v = __hiloint2double(__shfl(__double2hiint(vals), 2 * t + half, 64),
                                               __shfl(__double2loint(vals), 2 * t + half, 64));
             const double px = v * b[u].x, py = v * b[u].y;
-            if (mine & (2 * SPMM_HR)) {          // a pad carries no value
+            if (mine & SPMM_E_REAL) {            // a pad carries no value
                 run.x = run.x + px;
                 run.y = run.y + py;
             }
@@ -473,10 +490,97 @@ __device__ inline void heavy_add(double (&accx)[SPMM_HR], double (&accy)[SPMM_HR
     }
 }
 
-template <bool SMALL>
+typedef int spmm_v4i __attribute__((ext_vector_type(4)));
+typedef double spmm_v2d __attribute__((ext_vector_type(2)));
+
+// The list of rows with one nonzero: a stream of pairs of entries, one entry per half-wavefront; each is one
+// gather of B and one store to C.  Loads and stores share one in-order counter, so the loop is built to have
+// the same number of each on every path: 32 entries at a time go through a 64-entry ring in LDS that only
+// this wavefront touches (fetched one turn ahead, so no wait ever reaches back past a store), every lane always
+// stores - pads, idle lanes and the turns past the end of the list store to a dump row - and nothing is
+// branched around.  A wait for a batch of gathers then never includes the stores issued behind it.
+// NB = pairs per batch; KB = where the turn's 32 entries start in the ring.
+template <bool SMALL, bool ACC, int NB, int KB>
+__device__ inline void single_issue(double2 (&b)[NB], double2 (&c)[NB], const spmm_v4i *ring_half, int t,
+                                    const double *__restrict__ B, int64_t ldb, const double *__restrict__ C,
+                                    int64_t ldc, int64_t col)
+{
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+        const spmm_v4i q = ring_half[(KB + 2 * (t + u)) & 63];
+        const unsigned mine = (unsigned)q.x;
+        if constexpr (SMALL) {
+            const unsigned off = __umul24(mine >> SPMM_E_COL, (unsigned)ldb * 8u) + (unsigned)col * 8u;
+            b[u] = *reinterpret_cast<const double2 *>(reinterpret_cast<const char *>(B) + off);
+        } else {
+            const int64_t j = (int64_t)(mine >> SPMM_E_COL);
+            b[u] = *reinterpret_cast<const double2 *>(B + j * ldb + col);
+        }
+        if constexpr (ACC)
+            c[u] = *reinterpret_cast<const double2 *>(C + (int64_t)q.y * ldc + col);
+    }
+    __builtin_amdgcn_sched_barrier(0);       // the gathers stay in front of the stores of the other batch
+}
+
+template <bool ACC, int NB, int KB>
+__device__ inline void single_store(const double2 (&b)[NB], const double2 (&c)[NB], const spmm_v4i *ring_half, int t,
+                                    int64_t pair0, int64_t npairs, double *__restrict__ C, int64_t ldc, int64_t col,
+                                    bool active, double *__restrict__ dump)
+{
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+        const spmm_v4i q = ring_half[(KB + 2 * (t + u)) & 63];
+        const double v = __hiloint2double(q.w, q.z);
+        spmm_v2d o;
+        o.x = (ACC ? c[u].x : 0.0) + v * b[u].x;
+        o.y = (ACC ? c[u].y : 0.0) + v * b[u].y;
+        const bool ok = pair0 + t + u < npairs && active && (q.x & SPMM_E_REAL);
+        double *dst = ok ? C + (int64_t)q.y * ldc + col : dump;
+        __builtin_nontemporal_store(o, reinterpret_cast<spmm_v2d *>(dst));       // C is written once, not read again
+        if (u & 1)
+            __builtin_amdgcn_sched_barrier(0);       // two pairs at a time: keeps the entries read ahead few
+    }
+}
+
+template <bool SMALL, bool ACC>
+__device__ inline void single_rows(const spmm_v4i *__restrict__ list, int64_t n, int lane, int half,
+                                   const double *__restrict__ B, int64_t ldb, double *__restrict__ C, int64_t ldc,
+                                   int64_t col, bool active, spmm_v4i *ring, double *__restrict__ dump)
+{
+    constexpr int NB = ACC ? 4 : 8;
+    double2 b0[NB], b1[NB], c0[NB], c1[NB];
+    const int64_t npairs = n >> 1;           // the list has an even number of entries
+    const int l32 = lane & 31;
+    auto fetch = [&](int64_t turn) {         // the 32 entries of a turn, one per lane of each half
+        const int64_t i = turn * 32 + l32;
+        return __builtin_nontemporal_load(list + (i < n ? i : n - 1));
+    };
+    const spmm_v4i *ring_half = ring + half;
+    ring[l32] = fetch(0);
+    spmm_v4i next = fetch(1);
+    single_issue<SMALL, ACC, NB, 0>(b0, c0, ring_half, 0, B, ldb, C, ldc, col);
+    // a turn = 16 pairs: its entries, and those of the next turn for the gathers issued ahead, are in the ring
+    auto turn = [&](auto kb, int64_t k) {
+        constexpr int KB = decltype(kb)::value;
+        ring[((KB + 32) & 63) + l32] = next;            // turn k + 1, over the entries of turn k - 1
+        next = fetch(k + 2);
+        for (int t = 0; t < 16; t += 2 * NB) {
+            single_issue<SMALL, ACC, NB, KB>(b1, c1, ring_half, t + NB, B, ldb, C, ldc, col);
+            single_store<ACC, NB, KB>(b0, c0, ring_half, t, k * 16, npairs, C, ldc, col, active, dump);
+            single_issue<SMALL, ACC, NB, KB>(b0, c0, ring_half, t + 2 * NB, B, ldb, C, ldc, col);
+            single_store<ACC, NB, KB>(b1, c1, ring_half, t + NB, k * 16, npairs, C, ldc, col, active, dump);
+        }
+    };
+    for (int64_t k = 0; k * 16 < npairs; k += 2) {
+        turn(std::integral_constant<int, 0>(), k);
+        turn(std::integral_constant<int, 32>(), k + 1);
+    }
+}
+
+template <bool SMALL, bool ACC>
 __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
-    const int64_t *__restrict__ seg, const int32_t *__restrict__ hent, const double *__restrict__ hval,
-    const double *__restrict__ B, int64_t ldb, int64_t K, double *__restrict__ partial)
+    const int64_t *__restrict__ seg, const HeavyEnt *__restrict__ hent, const double *__restrict__ B, int64_t ldb,
+    int64_t K, double *__restrict__ partial, double *__restrict__ C, int64_t ldc)
 {
     constexpr int G = SPMM_HG;
     const int lane = threadIdx.x & 63, half = lane >> 5, sub = lane & 31;
@@ -486,12 +590,20 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
     const bool active = col < K;
     if (!active)
         col = K - 2;            // idle lanes gather a valid address and store nothing
+    const int64_t bin = ((int64_t)x * G + g) * SPMM_HW + wave;
+    const int64_t s = seg[bin], e = seg[bin + 1];          // both even
+    const spmm_v4i *list = reinterpret_cast<const spmm_v4i *>(hent);
+    if (wave == SPMM_HWL) {                   // the wavefront of the rows with one nonzero
+        __shared__ spmm_v4i single_ring[64];
+        if (s < e)             // this wavefront's slots of `partial` hold no row: the dump
+            single_rows<SMALL, ACC>(list + s, e - s, lane, half, B, ldb, C, ldc, col, active, single_ring,
+                                    partial + bin * SPMM_HR * K + col);
+        return;
+    }
     double accx[SPMM_HR], accy[SPMM_HR];      // two plain arrays: each is indexed through M0, a double2 array is not
 #pragma unroll
     for (int r = 0; r < SPMM_HR; ++r)
         accx[r] = accy[r] = 0.0;
-    const int64_t bin = ((int64_t)x * G + g) * SPMM_HW + wave;
-    const int64_t s = seg[bin], e = seg[bin + 1];          // both even
     if (s < e) {
         double2 bA[SPMM_HP], bB[SPMM_HP];
         double2 run = make_double2(0.0, 0.0);
@@ -500,8 +612,9 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
         int c_ent = 0;
         double c_val = 0.0;
         if (lane < cnt) {
-            c_ent = __builtin_nontemporal_load(hent + s + lane);
-            c_val = __builtin_nontemporal_load(hval + s + lane);
+            const spmm_v4i q = __builtin_nontemporal_load(list + s + lane);
+            c_ent = q.x;
+            c_val = __hiloint2double(q.w, q.z);
         }
         heavy_issue<SMALL>(bA, c_ent, 0, cnt >> 1, half, B, ldb, col);
         for (int64_t base = s; base < e; base += 64) {
@@ -510,8 +623,9 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
             int n_ent = 0;
             double n_val = 0.0;
             if (lane < ncnt) {
-                n_ent = __builtin_nontemporal_load(hent + base + 64 + lane);
-                n_val = __builtin_nontemporal_load(hval + base + 64 + lane);
+                const spmm_v4i q = __builtin_nontemporal_load(list + base + 64 + lane);
+                n_ent = q.x;
+                n_val = __hiloint2double(q.w, q.z);
             }
             const int np = cnt >> 1;
             static_assert(SPMM_HP == 8, "the sweep is unrolled for four batches of 8 pairs per 64 entries");
@@ -544,6 +658,16 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
             out[(int64_t)r * K + col + 1] = accy[r] + oy;
         }
     }
+}
+
+// C[rows[i]][0..K) = 0
+__global__ void zero_listed_rows_f64(double *__restrict__ C, const int32_t *__restrict__ rows, int64_t nlisted,
+                                     int64_t K, int64_t ldc)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t total = nlisted * K, step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < total; i += step)
+        C[(int64_t)rows[i / K] * ldc + (i % K)] = 0.0;
 }
 
 __global__ void fill_rows_f64(double *__restrict__ C, int64_t nrows, int64_t K, int64_t ldc, double v)
@@ -620,10 +744,27 @@ __global__ void heavy_make_keys(int64_t nheavy, const int32_t *__restrict__ hrow
         const uint64_t x = c / (uint64_t)xcols;
         const uint64_t cb = (c - x * (uint64_t)xcols) * SPMM_HCB / (uint64_t)xcols;   // column block inside the range
         const uint64_t code = (uint64_t)hcode[x * nheavy + h];       // wavefront * SPMM_HR + slot on that XCD
-        keys[o + t] = ((((x * SPMM_HBINS + (code >> SPMM_HRB)) * SPMM_HCB + cb) * SPMM_HR + (code & (SPMM_HR - 1)))
-                       << 28) | c;
+        keys[o + t] = ((((x * SPMM_HBINS + (code >> SPMM_HRB)) * SPMM_HCB + cb) * (2 * SPMM_HR) +
+                        (code & (SPMM_HR - 1))) << 28) | c;
         idx[o + t] = (uint32_t)(ps + t);
     }
+}
+
+// The rows with one nonzero, dealt round-robin to the last wavefronts of the workgroups of the XCD that sweeps
+// their column; these wavefronts own no long rows, so their lists are simply ordered by column.
+__global__ void single_make_keys(int64_t nsingle, const int32_t *__restrict__ srow, const int64_t *__restrict__ pos,
+                                 const int32_t *__restrict__ crd, int64_t xcols, uint64_t *__restrict__ keys,
+                                 uint32_t *__restrict__ idx)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= nsingle)
+        return;
+    const uint64_t c = (uint64_t)(uint32_t)crd[pos[srow[i]]];
+    const uint64_t x = c / (uint64_t)xcols;
+    const uint64_t cb = (c - x * (uint64_t)xcols) * SPMM_HCB / (uint64_t)xcols;
+    const uint64_t bin = (uint64_t)(i % SPMM_HG) * SPMM_HW + SPMM_HWL;
+    keys[i] = ((((x * SPMM_HBINS + bin) * SPMM_HCB + cb) * (2 * SPMM_HR) + SPMM_HR) << 28) | c;
+    idx[i] = (uint32_t)i;
 }
 
 // first[e] = 1 where entry e of the ordered list opens a run (another row, column block or wavefront)
@@ -653,10 +794,12 @@ __global__ void heavy_run_odd(int64_t nruns, const int64_t *__restrict__ start, 
 }
 
 // Writes the list with every run padded to even length: entry e of run r lands at e + (pads in front of r).
+// idx is a position in val for a long row's entry, and a position in srow for a row with one nonzero.
 __global__ void heavy_fill(int64_t n, const uint64_t *__restrict__ keys, const uint32_t *__restrict__ idx,
-                           const double *__restrict__ val, const int64_t *__restrict__ first,
+                           const double *__restrict__ val, const int64_t *__restrict__ pos,
+                           const int32_t *__restrict__ srow, const int64_t *__restrict__ first,
                            const int64_t *__restrict__ runs, const int64_t *__restrict__ start,
-                           const int64_t *__restrict__ pads, int32_t *__restrict__ hent, double *__restrict__ hval)
+                           const int64_t *__restrict__ pads, HeavyEnt *__restrict__ hent)
 {
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= n)
@@ -664,12 +807,24 @@ __global__ void heavy_fill(int64_t n, const uint64_t *__restrict__ keys, const u
     const uint64_t k = keys[e];
     const int64_t r = runs[e] + first[e] - 1;
     const int64_t p = e + pads[r];
-    const uint32_t body = (uint32_t)(((k & 0xfffffffull) << (SPMM_HRB + 2)) | ((k >> 28) & (SPMM_HR - 1)));
-    hent[p] = (int32_t)(body | (2u * SPMM_HR) | (first[e] ? (uint32_t)SPMM_HR : 0u));
-    hval[p] = val[idx[e]];
+    const bool direct = ((k >> 28) & SPMM_HR) != 0;
+    const uint32_t col = (uint32_t)(k & 0xfffffffull) << SPMM_E_COL;
+    HeavyEnt out;
+    if (direct) {
+        out.ent = (int32_t)(col | SPMM_E_REAL);
+        out.row = srow[idx[e]];
+        out.val = val[pos[out.row]];
+    } else {
+        out.ent = (int32_t)(col | SPMM_E_REAL | (first[e] ? (uint32_t)SPMM_E_FIRST : 0u) |
+                            (uint32_t)((k >> 28) & (SPMM_HR - 1)));
+        out.row = 0;
+        out.val = val[idx[e]];
+    }
+    hent[p] = out;
     if (e + 1 == start[r + 1] && ((start[r + 1] - start[r]) & 1)) {     // last entry of a run of odd length
-        hent[p + 1] = (int32_t)body;       // same column (a valid address), no value
-        hval[p + 1] = 0.0;
+        out.ent &= ~(SPMM_E_REAL | SPMM_E_FIRST);      // same column (a valid address), no value
+        out.val = 0.0;
+        hent[p + 1] = out;
     }
 }
 
@@ -683,7 +838,7 @@ __global__ void heavy_segments(int64_t n, const uint64_t *__restrict__ keys, con
     int64_t lo = 0, hi = n;
     while (lo < hi) {
         const int64_t mid = (lo + hi) >> 1;
-        if ((int64_t)(keys[mid] >> 28) / (SPMM_HCB * SPMM_HR) < b)
+        if ((int64_t)(keys[mid] >> 28) / (SPMM_HCB * 2 * SPMM_HR) < b)
             lo = mid + 1;
         else
             hi = mid;
@@ -691,31 +846,32 @@ __global__ void heavy_segments(int64_t n, const uint64_t *__restrict__ keys, con
     seg[b] = lo + pads[runs[lo]];      // lo opens a run (or is n): runs[lo] is that run's number
 }
 
-__global__ void light_lengths(int64_t nrows, const int64_t *__restrict__ pos, const int32_t *__restrict__ rowcode,
+__global__ void light_lengths(int64_t nlight, const int32_t *__restrict__ rowmap, const int64_t *__restrict__ pos,
                               int64_t *__restrict__ len)
 {
     const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (r < nrows)
-        len[r] = rowcode[r] >= 0 ? 0 : pos[r + 1] - pos[r];
+    if (r < nlight)
+        len[r] = pos[rowmap[r] + 1] - pos[rowmap[r]];
 }
 
-__global__ void light_copy(int64_t nrows, const int64_t *__restrict__ pos, const int32_t *__restrict__ crd,
-                           const double *__restrict__ val, const int64_t *__restrict__ lpos,
-                           int32_t *__restrict__ lcrd, double *__restrict__ lval)
+__global__ void light_copy(int64_t nlight, const int32_t *__restrict__ rowmap, const int64_t *__restrict__ pos,
+                           const int32_t *__restrict__ crd, const double *__restrict__ val,
+                           const int64_t *__restrict__ lpos, int32_t *__restrict__ lcrd, double *__restrict__ lval)
 {
     // one 16-lane group per row: the rows copied here are short
     const int64_t r = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
     const int sub = threadIdx.x & 15;
-    if (r >= nrows)
+    if (r >= nlight)
         return;
-    const int64_t n = lpos[r + 1] - lpos[r], src = pos[r], dst = lpos[r];
+    const int64_t n = lpos[r + 1] - lpos[r], src = pos[rowmap[r]], dst = lpos[r];
     for (int64_t t = sub; t < n; t += 16) {
         lcrd[dst + t] = crd[src + t];
         lval[dst + t] = val[src + t];
     }
 }
 
-// C[row] += the eight per-XCD sums of a long row, in XCD (= column) order
+// C[row] (+)= the eight per-XCD sums of a long row, in XCD (= column) order
+template <bool ACC>
 __global__ __launch_bounds__(256) void spmm_heavy_combine(int64_t nheavy, const int32_t *__restrict__ hrow,
                                                           const int32_t *__restrict__ hcode,
                                                           const double *__restrict__ partial,
@@ -727,7 +883,7 @@ __global__ __launch_bounds__(256) void spmm_heavy_combine(int64_t nheavy, const 
     if (h >= nheavy || col >= K)
         return;
     const int64_t row = hrow[h];
-    double acc = C[row * ldc + col];
+    double acc = ACC ? C[row * ldc + col] : 0.0;
     for (int x = 0; x < 8; ++x)
         acc = acc + partial[((int64_t)x * SPMM_HSLOTS + hcode[x * nheavy + h]) * K + col];
     C[row * ldc + col] = acc;
@@ -752,22 +908,33 @@ static int spmm_heavy_plan(Csr *a)
         if (pos[(size_t)r + 1] - pos[(size_t)r] >= SPMM_HEAVY_MIN_LEN)
             cand.emplace_back(-(pos[(size_t)r + 1] - pos[(size_t)r]), (int32_t)r);
     std::sort(cand.begin(), cand.end());
-    if ((int64_t)cand.size() > SPMM_HSLOTS)
-        cand.resize(SPMM_HSLOTS);
+    if ((int64_t)cand.size() > SPMM_HROWS)
+        cand.resize(SPMM_HROWS);
     const int64_t H = (int64_t)cand.size();
     int64_t hnnz = 0;
     for (auto &c : cand)
         hnnz -= c.first;
     if (H == 0 || hnnz * 4 < a->nnz)
         return COMET_HIP_OK;        // the long rows hold too little of the matrix to pay for a second kernel
-    std::vector<int32_t> hrow((size_t)H), hcode((size_t)(8 * H)), rowcode((size_t)n, -1), cnt((size_t)(8 * H));
+    std::vector<int32_t> hrow((size_t)H), hcode((size_t)(8 * H)), cnt((size_t)(8 * H));
     std::vector<int64_t> hstart((size_t)H + 1, 0);
+    std::vector<char> is_long((size_t)n, 0);
     for (int64_t k = 0; k < H; ++k) {
         hrow[(size_t)k] = cand[(size_t)k].second;
-        rowcode[(size_t)hrow[(size_t)k]] = 0;
+        is_long[(size_t)hrow[(size_t)k]] = 1;
         hstart[(size_t)k + 1] = hstart[(size_t)k] - cand[(size_t)k].first;
     }
-    int32_t *d_cnt = nullptr, *d_rowcode = nullptr;
+    // the other rows: one nonzero -> an entry of the sweep's lists; none -> cleared; the rest -> `light`
+    std::vector<int32_t> srow, erow, lrow;
+    for (int64_t r = 0; r < n; ++r) {
+        const int64_t len = pos[(size_t)r + 1] - pos[(size_t)r];
+        if (is_long[(size_t)r])
+            continue;
+        (len == 0 ? erow : len == 1 ? srow : lrow).push_back((int32_t)r);
+    }
+    const int64_t S = (int64_t)srow.size(), E = (int64_t)erow.size(), L = (int64_t)lrow.size();
+    const int64_t nent = hnnz + S;          // entries of the lists before padding
+    int32_t *d_cnt = nullptr, *d_srow = nullptr;
     int64_t *d_hstart = nullptr, *d_len = nullptr;
     int64_t *d_first = nullptr, *d_runs = nullptr, *d_start = nullptr, *d_odd = nullptr, *d_pads = nullptr;
     uint64_t *k_in = nullptr, *k_out = nullptr;
@@ -775,7 +942,7 @@ static int spmm_heavy_plan(Csr *a)
     Csr *light = new Csr();
     auto cleanup = [&](bool failed) {
         (void)hipFree(d_cnt);
-        (void)hipFree(d_rowcode);
+        (void)hipFree(d_srow);
         (void)hipFree(d_hstart);
         (void)hipFree(d_len);
         (void)hipFree(d_first);
@@ -789,13 +956,14 @@ static int spmm_heavy_plan(Csr *a)
         (void)hipFree(i_out);
         if (failed) {
             (void)hipFree(a->heavy_seg);
-            (void)hipFree(a->heavy_col);
-            (void)hipFree(a->heavy_val);
+            (void)hipFree(a->heavy_ent);
             (void)hipFree(a->heavy_row);
             (void)hipFree(a->heavy_code);
+            (void)hipFree(a->empty_rows);
             a->heavy_seg = nullptr;
-            a->heavy_col = a->heavy_row = a->heavy_code = nullptr;
-            a->heavy_val = nullptr;
+            a->heavy_ent = nullptr;
+            a->heavy_row = a->heavy_code = a->empty_rows = nullptr;
+            a->nempty = 0;
             light->owns = true;
             csr_release(light);
         }
@@ -807,20 +975,27 @@ static int spmm_heavy_plan(Csr *a)
             return set_error(COMET_HIP_ERR_HIP, "%s failed while planning the long rows", #call);             \
         }                                                                                                     \
     } while (0)
+    auto at_least_one = [](int64_t v) { return (size_t)(v > 0 ? v : 1); };
     HEAVY_TRY(hipMalloc((void **)&d_cnt, 4 * (size_t)(8 * H)));
-    HEAVY_TRY(hipMalloc((void **)&d_rowcode, 4 * (size_t)n));
+    HEAVY_TRY(hipMalloc((void **)&d_srow, 4 * at_least_one(S)));
     HEAVY_TRY(hipMalloc((void **)&d_hstart, 8 * (size_t)(H + 1)));
-    HEAVY_TRY(hipMalloc((void **)&d_len, 8 * (size_t)n));
-    HEAVY_TRY(hipMalloc((void **)&k_in, 8 * (size_t)hnnz));
-    HEAVY_TRY(hipMalloc((void **)&k_out, 8 * (size_t)hnnz));
-    HEAVY_TRY(hipMalloc((void **)&i_in, 4 * (size_t)hnnz));
-    HEAVY_TRY(hipMalloc((void **)&i_out, 4 * (size_t)hnnz));
+    HEAVY_TRY(hipMalloc((void **)&d_len, 8 * at_least_one(L)));
+    HEAVY_TRY(hipMalloc((void **)&k_in, 8 * (size_t)nent));
+    HEAVY_TRY(hipMalloc((void **)&k_out, 8 * (size_t)nent));
+    HEAVY_TRY(hipMalloc((void **)&i_in, 4 * (size_t)nent));
+    HEAVY_TRY(hipMalloc((void **)&i_out, 4 * (size_t)nent));
     HEAVY_TRY(hipMalloc((void **)&a->heavy_seg, 8 * (size_t)(8 * SPMM_HBINS + 1)));
     HEAVY_TRY(hipMalloc((void **)&a->heavy_row, 4 * (size_t)H));
     HEAVY_TRY(hipMalloc((void **)&a->heavy_code, 4 * (size_t)(8 * H)));
+    HEAVY_TRY(hipMalloc((void **)&a->empty_rows, 4 * at_least_one(E)));
+    HEAVY_TRY(hipMalloc((void **)&light->rowmap, 4 * at_least_one(L)));
     HEAVY_TRY(hipMemcpyAsync(a->heavy_row, hrow.data(), 4 * (size_t)H, hipMemcpyHostToDevice, stream()));
-
-    HEAVY_TRY(hipMemcpyAsync(d_rowcode, rowcode.data(), 4 * (size_t)n, hipMemcpyHostToDevice, stream()));
+    if (S > 0)
+        HEAVY_TRY(hipMemcpyAsync(d_srow, srow.data(), 4 * (size_t)S, hipMemcpyHostToDevice, stream()));
+    if (E > 0)
+        HEAVY_TRY(hipMemcpyAsync(a->empty_rows, erow.data(), 4 * (size_t)E, hipMemcpyHostToDevice, stream()));
+    if (L > 0)
+        HEAVY_TRY(hipMemcpyAsync(light->rowmap, lrow.data(), 4 * (size_t)L, hipMemcpyHostToDevice, stream()));
     HEAVY_TRY(hipMemcpyAsync(d_hstart, hstart.data(), 8 * (size_t)(H + 1), hipMemcpyHostToDevice, stream()));
     const int64_t xcols = ceil_div(a->ncols, 8);
     // Every XCD gets its own assignment of rows to wavefronts, by what the row holds in that XCD's column
@@ -844,7 +1019,8 @@ static int spmm_heavy_plan(Csr *a)
                             std::greater<std::pair<double, int32_t>>> bins;
         std::vector<int32_t> used(SPMM_HBINS, 0);
         for (int32_t b = 0; b < SPMM_HBINS; ++b)
-            bins.push({0.0, b});
+            if (b % SPMM_HW != SPMM_HWL)        // the last wavefront of a workgroup takes the rows with one nonzero
+                bins.push({0.0, b});
         for (auto &o : order) {
             auto top = bins.top();
             bins.pop();
@@ -859,27 +1035,30 @@ static int spmm_heavy_plan(Csr *a)
         KernelTimer t("heavy_make_keys");
         heavy_make_keys<<<dim3((unsigned)H), dim3(256), 0, stream()>>>(H, a->heavy_row, a->heavy_code, d_hstart,
                                                                        a->pos, a->crd, xcols, k_in, i_in);
+        if (S > 0)
+            single_make_keys<<<dim3((unsigned)ceil_div(S, 256)), dim3(256), 0, stream()>>>(
+                S, d_srow, a->pos, a->crd, xcols, k_in + hnnz, i_in + hnnz);
     }
-    if (sort_pairs_u64_u32(k_in, k_out, i_in, i_out, hnnz, 28 + SPMM_HRB + 5 + 12) != COMET_HIP_OK) {
+    if (sort_pairs_u64_u32(k_in, k_out, i_in, i_out, nent, 28 + (SPMM_HRB + 1) + 5 + 12) != COMET_HIP_OK) {
         cleanup(true);
         return COMET_HIP_ERR_HIP;
     }
     // runs (entries of one row inside one column block of one wavefront's list) are padded to even length
-    HEAVY_TRY(hipMalloc((void **)&d_first, 8 * (size_t)hnnz));
-    HEAVY_TRY(hipMalloc((void **)&d_runs, 8 * (size_t)(hnnz + 1)));
-    HEAVY_TRY(hipMalloc((void **)&d_start, 8 * (size_t)(hnnz + 1)));
-    HEAVY_TRY(hipMalloc((void **)&d_odd, 8 * (size_t)hnnz));
-    HEAVY_TRY(hipMalloc((void **)&d_pads, 8 * (size_t)(hnnz + 1)));
-    const dim3 per_entry((unsigned)ceil_div(hnnz + 1, 256));
-    heavy_mark_runs<<<per_entry, dim3(256), 0, stream()>>>(hnnz, k_out, d_first);
-    if (exclusive_scan_i64(d_first, hnnz, d_runs) != COMET_HIP_OK) {
+    HEAVY_TRY(hipMalloc((void **)&d_first, 8 * (size_t)nent));
+    HEAVY_TRY(hipMalloc((void **)&d_runs, 8 * (size_t)(nent + 1)));
+    HEAVY_TRY(hipMalloc((void **)&d_start, 8 * (size_t)(nent + 1)));
+    HEAVY_TRY(hipMalloc((void **)&d_odd, 8 * (size_t)nent));
+    HEAVY_TRY(hipMalloc((void **)&d_pads, 8 * (size_t)(nent + 1)));
+    const dim3 per_entry((unsigned)ceil_div(nent + 1, 256));
+    heavy_mark_runs<<<per_entry, dim3(256), 0, stream()>>>(nent, k_out, d_first);
+    if (exclusive_scan_i64(d_first, nent, d_runs) != COMET_HIP_OK) {
         cleanup(true);
         return COMET_HIP_ERR_HIP;
     }
     int64_t nruns = 0, npads = 0;
-    HEAVY_TRY(hipMemcpyAsync(&nruns, d_runs + hnnz, 8, hipMemcpyDeviceToHost, stream()));
+    HEAVY_TRY(hipMemcpyAsync(&nruns, d_runs + nent, 8, hipMemcpyDeviceToHost, stream()));
     HEAVY_TRY(hipStreamSynchronize(stream()));
-    heavy_run_starts<<<per_entry, dim3(256), 0, stream()>>>(hnnz, d_first, d_runs, d_start);
+    heavy_run_starts<<<per_entry, dim3(256), 0, stream()>>>(nent, d_first, d_runs, d_start);
     heavy_run_odd<<<dim3((unsigned)ceil_div(nruns, 256)), dim3(256), 0, stream()>>>(nruns, d_start, d_odd);
     if (exclusive_scan_i64(d_odd, nruns, d_pads) != COMET_HIP_OK) {
         cleanup(true);
@@ -887,32 +1066,33 @@ static int spmm_heavy_plan(Csr *a)
     }
     HEAVY_TRY(hipMemcpyAsync(&npads, d_pads + nruns, 8, hipMemcpyDeviceToHost, stream()));
     HEAVY_TRY(hipStreamSynchronize(stream()));
-    HEAVY_TRY(hipMalloc((void **)&a->heavy_col, 4 * (size_t)(hnnz + npads)));
-    HEAVY_TRY(hipMalloc((void **)&a->heavy_val, 8 * (size_t)(hnnz + npads)));
+    HEAVY_TRY(hipMalloc((void **)&a->heavy_ent, sizeof(HeavyEnt) * (size_t)(nent + npads)));
     {
         KernelTimer t("heavy_fill");
-        heavy_fill<<<dim3((unsigned)ceil_div(hnnz, 256)), dim3(256), 0, stream()>>>(
-            hnnz, k_out, i_out, a->val, d_first, d_runs, d_start, d_pads, a->heavy_col, a->heavy_val);
+        heavy_fill<<<dim3((unsigned)ceil_div(nent, 256)), dim3(256), 0, stream()>>>(
+            nent, k_out, i_out, a->val, a->pos, d_srow, d_first, d_runs, d_start, d_pads, a->heavy_ent);
         heavy_segments<<<dim3((unsigned)ceil_div(8 * SPMM_HBINS + 1, 256)), dim3(256), 0, stream()>>>(
-            hnnz, k_out, d_runs, d_pads, a->heavy_seg);
+            nent, k_out, d_runs, d_pads, a->heavy_seg);
     }
-    // the rest of the matrix, long rows left empty
-    light->nrows = n;
+    // the rows of two and more nonzeros that are not long, as a matrix of their own
+    light->nrows = L;
     light->ncols = a->ncols;
-    light->nnz = a->nnz - hnnz;
+    light->nnz = a->nnz - hnnz - S;
     light->owns = true;
-    HEAVY_TRY(hipMalloc((void **)&light->pos, 8 * (size_t)(n + 1)));
-    HEAVY_TRY(hipMalloc((void **)&light->crd, 4 * (size_t)(light->nnz > 0 ? light->nnz : 1)));
-    HEAVY_TRY(hipMalloc((void **)&light->val, 8 * (size_t)(light->nnz > 0 ? light->nnz : 1)));
-    light_lengths<<<dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, stream()>>>(n, a->pos, d_rowcode, d_len);
-    if (exclusive_scan_i64(d_len, n, light->pos) != COMET_HIP_OK) {
-        cleanup(true);
-        return COMET_HIP_ERR_HIP;
-    }
-    {
+    HEAVY_TRY(hipMalloc((void **)&light->pos, 8 * (size_t)(L + 1)));
+    HEAVY_TRY(hipMalloc((void **)&light->crd, 4 * at_least_one(light->nnz)));
+    HEAVY_TRY(hipMalloc((void **)&light->val, 8 * at_least_one(light->nnz)));
+    if (L > 0) {
+        light_lengths<<<dim3((unsigned)ceil_div(L, 256)), dim3(256), 0, stream()>>>(L, light->rowmap, a->pos, d_len);
+        if (exclusive_scan_i64(d_len, L, light->pos) != COMET_HIP_OK) {
+            cleanup(true);
+            return COMET_HIP_ERR_HIP;
+        }
         KernelTimer t("light_copy");
-        light_copy<<<dim3((unsigned)ceil_div(n * 16, 256)), dim3(256), 0, stream()>>>(n, a->pos, a->crd, a->val,
-                                                                                      light->pos, light->crd, light->val);
+        light_copy<<<dim3((unsigned)ceil_div(L * 16, 256)), dim3(256), 0, stream()>>>(
+            L, light->rowmap, a->pos, a->crd, a->val, light->pos, light->crd, light->val);
+    } else {
+        HEAVY_TRY(hipMemsetAsync(light->pos, 0, 8, stream()));
     }
     HEAVY_TRY(hipGetLastError());
     HEAVY_TRY(hipStreamSynchronize(stream()));
@@ -922,6 +1102,7 @@ static int spmm_heavy_plan(Csr *a)
     a->light = light;
     a->heavy_nnz = hnnz;
     a->heavy_rows = H;
+    a->nempty = E;
     a->heavy_state = 2;
     return COMET_HIP_OK;
 }
@@ -992,31 +1173,51 @@ static int spmm_run(Csr *a, int64_t K, int64_t b_dptr, int64_t ldb, int64_t c_dp
     if (ceil_div(K, 64) > 65535)
         return set_error(COMET_HIP_ERR_SIZE, "K = %lld needs more than 65535 column tiles", (long long)K);
     // long rows: column sweep with the sums on chip; everything else: one wavefront per 256 nonzeros
-    // (the sweep loads B sixteen bytes at a time: two columns per lane, rows aligned to that)
+    // (the sweep loads B and stores C sixteen bytes at a time: two columns per lane, rows aligned to that)
     const bool sweep_fits = K >= 16 && K <= 2048 && (K & 1) == 0 && (ldb & 1) == 0 && (b_dptr & 15) == 0 &&
-                            getenv("COMET_SPMM_NO_SWEEP") == nullptr;
+                            (ldc & 1) == 0 && (c_dptr & 15) == 0 && getenv("COMET_SPMM_NO_SWEEP") == nullptr;
     if (sweep_fits)
         COMET_CHK(spmm_heavy_plan(a));
     if (a->heavy_state != 2 || !sweep_fits)
         return spmm_chunks(a, K, B, ldb, C, ldc, accumulate);
-    // the long rows are empty in `light`: cleared (or, accumulating, left alone) there, then added to below
-    COMET_CHK(spmm_chunks(a->light, K, B, ldb, C, ldc, accumulate));
-    COMET_CHK(g_heavy_partial.ensure(sizeof(double) * 8 * (size_t)SPMM_HSLOTS * (size_t)K, false));
+    // rows of two and more nonzeros that are not long: one wavefront per 256 nonzeros
+    if (a->light->nnz > 0)
+        COMET_CHK(spmm_chunks(a->light, K, B, ldb, C, ldc, accumulate));
     const unsigned tiles = (unsigned)ceil_div(K, 64);
+    if (!accumulate && a->nempty > 0) {
+        KernelTimer t("zero_listed_rows_f64");
+        const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div(a->nempty * K, 256), 65536);
+        zero_listed_rows_f64<<<dim3(blocks), dim3(256), 0, stream()>>>(C, a->empty_rows, a->nempty, K, ldc);
+    }
+    // long rows (sums on chip, left in `partial`) and rows of one nonzero (stored to C)
+    COMET_CHK(g_heavy_partial.ensure(sizeof(double) * 8 * (size_t)SPMM_HSLOTS * (size_t)K, false));
+    double *partial = (double *)g_heavy_partial.ptr;
     {
         KernelTimer t("spmm_heavy_sweep");
         const bool small_b = a->ncols < (1 << 24) && ldb * 8 < (1 << 24) && a->ncols * ldb * 8 < (1ll << 32);
-        if (small_b)
-            spmm_heavy_sweep<true><<<dim3(8 * SPMM_HG, tiles), dim3(SPMM_HW * 64), 0, stream()>>>(
-                a->heavy_seg, a->heavy_col, a->heavy_val, B, ldb, K, (double *)g_heavy_partial.ptr);
+        const dim3 grid(8 * SPMM_HG, tiles), block(SPMM_HW * 64);
+        if (small_b && accumulate)
+            spmm_heavy_sweep<true, true><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K, partial,
+                                                                       C, ldc);
+        else if (small_b)
+            spmm_heavy_sweep<true, false><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K, partial,
+                                                                        C, ldc);
+        else if (accumulate)
+            spmm_heavy_sweep<false, true><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K, partial,
+                                                                        C, ldc);
         else
-            spmm_heavy_sweep<false><<<dim3(8 * SPMM_HG, tiles), dim3(SPMM_HW * 64), 0, stream()>>>(
-                a->heavy_seg, a->heavy_col, a->heavy_val, B, ldb, K, (double *)g_heavy_partial.ptr);
+            spmm_heavy_sweep<false, false><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K,
+                                                                         partial, C, ldc);
     }
     {
         KernelTimer t("spmm_heavy_combine");
-        spmm_heavy_combine<<<dim3((unsigned)ceil_div(a->heavy_rows, 4), tiles), dim3(256), 0, stream()>>>(
-            a->heavy_rows, a->heavy_row, a->heavy_code, (const double *)g_heavy_partial.ptr, C, ldc, K);
+        const dim3 grid((unsigned)ceil_div(a->heavy_rows, 4), tiles);
+        if (accumulate)
+            spmm_heavy_combine<true><<<grid, dim3(256), 0, stream()>>>(a->heavy_rows, a->heavy_row, a->heavy_code,
+                                                                       partial, C, ldc, K);
+        else
+            spmm_heavy_combine<false><<<grid, dim3(256), 0, stream()>>>(a->heavy_rows, a->heavy_row, a->heavy_code,
+                                                                        partial, C, ldc, K);
     }
     COMET_HIPCHK(hipGetLastError());
     return COMET_HIP_OK;
@@ -1046,20 +1247,20 @@ static int spmm_chunks(Csr *a, int64_t K, const double *B, int64_t ldb, double *
         if (accumulate)
             spmm_csr_nnzsplit<true><<<grid, block, 0, stream()>>>(a->pos, a->crd, a->val, a->nnz, a->nrows,
                                                                   a->spmm_chunk_row, nchunks, (const double *)b_dptr,
-                                                                  ldb, C, ldc, K, carry);
+                                                                  ldb, C, ldc, K, carry, a->rowmap);
         else
             spmm_csr_nnzsplit<false><<<grid, block, 0, stream()>>>(a->pos, a->crd, a->val, a->nnz, a->nrows,
                                                                    a->spmm_chunk_row, nchunks, (const double *)b_dptr,
-                                                                   ldb, C, ldc, K, carry);
+                                                                   ldb, C, ldc, K, carry, a->rowmap);
     }
     {
         KernelTimer t("spmm_csr_fixup");
         if (accumulate)
             spmm_csr_fixup<true><<<grid, block, 0, stream()>>>(a->pos, a->nnz, a->spmm_chunk_row, nchunks, C, ldc, K,
-                                                               carry);
+                                                               carry, a->rowmap);
         else
             spmm_csr_fixup<false><<<grid, block, 0, stream()>>>(a->pos, a->nnz, a->spmm_chunk_row, nchunks, C, ldc, K,
-                                                                carry);
+                                                                carry, a->rowmap);
     }
     COMET_HIPCHK(hipGetLastError());
     return COMET_HIP_OK;

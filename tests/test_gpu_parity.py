@@ -158,10 +158,10 @@ def test_spmm_golden(golden, golden_dir):
 
 def _long_rows(pos, K):
     """The rows the library hands to the column sweep (its rule restated): at least 128 nonzeros, at most
-    the 4096 longest (ties: lower row first), and only if they hold a quarter of a matrix of >= 2^19 nonzeros."""
+    the 3840 longest (ties: lower row first), and only if they hold a quarter of a matrix of >= 2^19 nonzeros."""
     lens = np.diff(pos)
     rows = np.flatnonzero(lens >= 128)
-    rows = rows[np.argsort(-lens[rows], kind="stable")][:4096]
+    rows = rows[np.argsort(-lens[rows], kind="stable")][:3840]
     if not (16 <= K <= 2048) or pos[-1] < (1 << 19) or 4 * lens[rows].sum() < pos[-1]:
         return rows[:0]
     return rows
@@ -169,12 +169,16 @@ def _long_rows(pos, K):
 
 def _bit_exact_rows(pos, K):
     """Rows summed in the checker's order: those that lie inside one 256-nonzero chunk of the matrix the
-    chunk kernel sees (the matrix without the rows the sweep takes), and empty rows."""
+    chunk kernel sees (with long rows: the rows of two and more nonzeros that are not long, packed), and the
+    rows of at most one nonzero."""
     lens = np.diff(pos)
     light = lens.copy()
-    light[_long_rows(pos, K)] = 0
+    long_rows = _long_rows(pos, K)
+    if len(long_rows):
+        light[long_rows] = 0
+        light[lens == 1] = 0        # these ride on the sweep: one product each
     lpos = np.concatenate([[0], np.cumsum(light)])
-    return (lens == 0) | ((light > 0) & (lpos[:-1] // 256 == (lpos[1:] - 1) // 256))
+    return (lens <= 1) | ((light > 0) & (lpos[:-1] // 256 == (lpos[1:] - 1) // 256))
 
 
 def _spmm_check(pos, crd, val, B, C0=None):
@@ -764,7 +768,7 @@ def _sweep_check(pos, crd, val, B, C0=None, ld_pad=0):
                                                      int(C0 is not None)), "spmm")
     rep = _kernels_of(run)
     swept = K % 2 == 0 and ld_pad % 2 == 0       # the sweep loads pairs of columns: even K and leading dimensions
-    assert ("spmm_heavy_sweep" in rep) == swept and "spmm_csr_nnzsplit" in rep, sorted(rep)
+    assert ("spmm_heavy_sweep" in rep) == swept, sorted(rep)
     out = dC.to_numpy()
     assert np.all(out[:, K:] == 123.0)             # the padding of C is not touched
     got = out[:, :K]
@@ -792,7 +796,7 @@ def test_spmm_long_rows_sweep(K, acc, pad):
 
 
 def test_spmm_more_long_rows_than_the_sweep_holds():
-    """5000 rows of 300 nonzeros: the 4096 longest (ties: lowest row ids) sweep, the others stay on the
+    """5000 rows of 300 nonzeros: the 3840 longest (ties: lowest row ids) sweep, the others stay on the
     chunk kernel; an empty row and a short row sit between them."""
     rng = np.random.default_rng(31)
     n, m = 5002, 3000
@@ -800,7 +804,25 @@ def test_spmm_more_long_rows_than_the_sweep_holds():
     pos = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
     crd = np.concatenate([np.sort(rng.choice(m, l, replace=False)) for l in lens]).astype(np.int64)
     val = rng.uniform(-1, 1, len(crd))
-    assert _sweep_check(pos, crd, val, gen.dense((m, 64), seed=2)) == 4096
+    assert _sweep_check(pos, crd, val, gen.dense((m, 64), seed=2)) == 3840
+
+
+@pytest.mark.parametrize("acc", [False, True])
+def test_spmm_sweep_with_only_single_and_empty_rows_besides(acc):
+    """2100 rows of 260 nonzeros, and around them rows of one nonzero and empty rows only: nothing is left
+    for the chunk kernel; the single products are stored (or added to C) by the sweep, bit-exact."""
+    rng = np.random.default_rng(41)
+    n, m, K = 9000, 5000, 32
+    lens = np.where(np.arange(n) % 3 == 0, 1, 0); lens[rng.choice(n, 2100, replace=False)] = 260
+    pos = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    assert pos[-1] >= 1 << 19
+    crd = np.concatenate([np.sort(rng.choice(m, l, replace=False)) for l in lens if l]).astype(np.int64)
+    val = rng.uniform(-1, 1, len(crd))
+    C0 = gen.dense((n, K), seed=5) if acc else None
+    assert _sweep_check(pos, crd, val, gen.dense((m, K), seed=4), C0) == 2100
+    A = rt.CsrMatrix.from_arrays((n, m), pos, crd, val)
+    rep = _kernels_of(lambda: rt.spmm(A, rt.DeviceArray.from_numpy(gen.dense((m, K), seed=4))))
+    assert "spmm_csr_nnzsplit" not in rep and "spmm_heavy_sweep" in rep, sorted(rep)
 
 
 # ----------------------------------------------------------------- dense operand on the left, CSR .* Dense
