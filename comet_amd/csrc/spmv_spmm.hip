@@ -1355,3 +1355,81 @@ extern "C" int comet_hip_densemat_csr_f64(int64_t csr, int64_t M, int64_t a_dptr
     COMET_CHK(spmm_run(t, M, (int64_t)at, M, (int64_t)ct, M, accumulate));
     return transpose2d(ct, M, b->ncols, M, (double *)c_dptr, ldc);
 }
+
+// ============================================================================
+// SDDMM: A = B .* (C x D), B and A sparse with one structure, C and D dense.
+// The reference computes this as T = C x D followed by B .* T, and with
+// --opt-fusion keeps only the entries of T that B samples
+// (lib/Dialect/IndexTree/Transforms/KernelFusion.cpp:1049-1220; the test is
+// test/integration/kernels/sddmm.ta).  Either way a stored entry (i, j) gets
+// val * sum_k C[i,k] * D[k,j], the sum unfused and in ascending k.
+// One lane per stored entry; its row is found by bisection in pos.  D is
+// transposed first, so that a lane walks along a row of K contiguous values
+// instead of striding through D.
+// ============================================================================
+__global__ __launch_bounds__(256) void sddmm_kernel(int64_t nrows, int64_t nnz, const int64_t *__restrict__ pos,
+                                                    const int32_t *__restrict__ crd,
+                                                    const double *__restrict__ val, const double *__restrict__ C,
+                                                    int64_t ldc, const double *__restrict__ Dt, int64_t K,
+                                                    double *__restrict__ out)
+{
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= nnz)
+        return;
+    int64_t lo = 0, hi = nrows - 1;          // the row r with pos[r] <= p < pos[r + 1]
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (pos[mid + 1] <= p)
+            lo = mid + 1;
+        else
+            hi = mid;
+    }
+    const double *c = C + lo * ldc, *d = Dt + (int64_t)crd[p] * K;
+    double t = 0.0;
+    for (int64_t k = 0; k < K; ++k)
+        t = t + c[k] * d[k];
+    out[p] = val[p] * t;
+}
+
+static Workspace g_sddmm_dt;
+
+extern "C" int64_t comet_hip_sddmm_csr_f64(int64_t bh, int64_t K, int64_t c_dptr, int64_t ldc, int64_t d_dptr,
+                                           int64_t ldd)
+{
+    if (ensure_init() != COMET_HIP_OK)
+        return 0;
+    Csr *b = csr_from_handle(bh);
+    if (!b)
+        return 0;
+    if (K < 0 || ldc < K || ldd < b->ncols || (b->nnz > 0 && K > 0 && (!c_dptr || !d_dptr))) {
+        set_error(COMET_HIP_ERR_ARG, "bad dense operands passed to comet_hip_sddmm_csr_f64 (K %lld, ldc %lld, ldd %lld)",
+                  (long long)K, (long long)ldc, (long long)ldd);
+        return 0;
+    }
+    Csr *a = new Csr();
+    if (csr_alloc(a, b->nrows, b->ncols, b->nnz) != COMET_HIP_OK) {
+        delete a;
+        return 0;
+    }
+    bool ok = hipMemcpyAsync(a->pos, b->pos, sizeof(int64_t) * (size_t)(b->nrows + 1), hipMemcpyDeviceToDevice,
+                             stream()) == hipSuccess;
+    if (ok && b->nnz > 0) {
+        ok = hipMemcpyAsync(a->crd, b->crd, sizeof(int32_t) * (size_t)b->nnz, hipMemcpyDeviceToDevice, stream()) ==
+             hipSuccess;
+        if (ok && K > 0)
+            ok = g_sddmm_dt.ensure(sizeof(double) * (size_t)b->ncols * (size_t)K, false) == COMET_HIP_OK &&
+                 transpose2d((const double *)d_dptr, ldd, K, b->ncols, (double *)g_sddmm_dt.ptr, K) == COMET_HIP_OK;
+        if (ok) {
+            KernelTimer t("sddmm_kernel");
+            sddmm_kernel<<<dim3((unsigned)ceil_div(b->nnz, 256)), dim3(256), 0, stream()>>>(
+                b->nrows, b->nnz, b->pos, b->crd, b->val, (const double *)c_dptr, ldc,
+                (const double *)g_sddmm_dt.ptr, K, a->val);
+        }
+    }
+    if (!ok || hipGetLastError() != hipSuccess) {
+        set_error(COMET_HIP_ERR_HIP, "SDDMM failed");
+        csr_release(a);
+        return 0;
+    }
+    return csr_register(a);
+}

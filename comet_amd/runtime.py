@@ -84,6 +84,7 @@ SIGNATURES = {
     "comet_hip_vecmat_csr_f64": (_int, [_i64, _i64, _i64, _int]),
     "comet_hip_densemat_csr_f64": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
     "comet_hip_eltwise_csr_dense_csr": (_i64, [_i64, _i64, _i64, _int]),
+    "comet_hip_sddmm_csr_f64": (_i64, [_i64, _i64, _i64, _i64, _i64, _i64]),
     "comet_hip_eltwise_csr_dense_dense": (_int, [_i64, _i64, _i64, _i64, _i64, _int]),
     "comet_hip_eltwise_dense_f64": (_int, [_i64, _i64, _i64, _i64, _int]),
     "comet_hip_mtx_read_csr": (_i64, [C.c_char_p, _int]),
@@ -497,6 +498,18 @@ def eltwise_csr_dense(A, D, out=None, op="times"):
     _check(lib().comet_hip_eltwise_csr_dense_dense(A.handle, D.ptr, A.shape[1], out.ptr, A.shape[1], code),
            "comet_hip_eltwise_csr_dense_dense")
     return out
+
+
+def sddmm(B, Cm, D):
+    """B .* (Cm @ D) for a sparse B (nrows x ncols), dense Cm (nrows x K) and D (K x ncols): a CsrMatrix with
+    B's structure; the dense product is never formed."""
+    nrows, ncols = B.shape
+    if len(Cm.shape) != 2 or len(D.shape) != 2 or Cm.shape[0] != nrows or D.shape[1] != ncols or \
+            Cm.shape[1] != D.shape[0]:
+        raise ValueError("SDDMM needs B (n x m), C (n x K) and D (K x m)")
+    K = Cm.shape[1]
+    return CsrMatrix(_handle(lib().comet_hip_sddmm_csr_f64(B.handle, K, Cm.ptr, K, D.ptr, ncols),
+                             "comet_hip_sddmm_csr_f64"))
 
 
 def eltwise_mult_dense(A, D, out=None):

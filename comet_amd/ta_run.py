@@ -19,6 +19,9 @@ include/comet_hip_rt.h.  Statements it understands (frontends/comet_dsl/include/
     C[i, j] = A[i, j] .* B[i, j];    (CSR .* CSR, CSR .* Dense, Dense .* CSR)
     C[i, j] = A[i, j] @(+) B[i, j];  (elementwise monoids +, -, *, min, max: Dense x Dense, sparse x Dense)
     B[j, i] = transpose(A[i, j], {j, i});                             (dense)
+    A[i, l] = B[i, j] * C[j, k] * D[k, l];                            (chains, evaluated left to right)
+    C[k, i] = A[k, j] * transpose(B[i, j], {j, i});                   (transposed dense operands)
+    T[i, j] = C[i, k] * D[k, j];  A[i, j] = B[i, j] .* T[i, j];       (SDDMM: T is never formed, as with --opt-fusion)
     var s = SUM(C[i, j]);  var t = getTime();  printElapsedTime(t0, t1);  print(C);  print(s);
 
 Anything else raises TaError naming the statement.  Like the generated code, `C = A * B` adds into what C
@@ -60,6 +63,8 @@ class _Tensor:
     def __init__(self, name, labels, fmt):
         self.name, self.labels, self.fmt = name, labels, fmt
         self.value = None        # DeviceArray (Dense) or CsrMatrix (every sparse format)
+        self.zero = True         # Dense: holds zeros only (never written, or filled with 0.0)
+        self.pending = None      # Dense: (C, D) of a product C x D that has not been formed yet
 
 
 class Program:
@@ -99,9 +104,18 @@ class Program:
                 raise TaError(f"index {l} has size {self.extent[l]} but the tensor has {n}")
 
     def _dense(self, t):
+        if t.pending is not None:           # someone needs all of it after all
+            cm, d = t.pending
+            t.pending = None
+            t.value = rt.dgemm(self._dense(cm), self._dense(d))
+            t.zero = False
         if t.value is None:       # declared, never filled: the reference allocates without initialising
             t.value = rt.DeviceArray(self._shape(t.labels), zero=True)
         return t.value
+
+    def _written(self, t):
+        t.zero = False
+        t.pending = None
 
     def _sparse(self, t):
         if t.value is None:
@@ -126,10 +140,11 @@ class Program:
                 return handler(self, *m.groups())
         raise TaError(f"statement not supported by this runner: {s}")
 
-    def _index_label(self, name, size):
-        self.extent[name] = None if size == "?" else int(size)
-        if name not in self.order:
-            self.order.append(name)
+    def _index_label(self, names, size):
+        for name in (n.strip() for n in names.split(",")):
+            self.extent[name] = None if size == "?" else int(size)
+            if name not in self.order:
+                self.order.append(name)
 
     def _declare(self, name, labels, fmt):
         if fmt not in _FORMATS:
@@ -148,6 +163,67 @@ class Program:
         if t.fmt != "Dense":
             raise TaError("only dense tensors can be filled with a constant")
         t.value = rt.DeviceArray.from_numpy(np.full(self._shape(t.labels), float(value)))
+        t.zero = float(value) == 0.0
+        t.pending = None
+
+    _OPERAND = re.compile(r"\s*(?:transpose\(\s*(\w+)\s*\[([^\]]*)\]\s*,\s*\{([^}]*)\}\s*\)|(\w+)\s*\[([^\]]*)\])\s*")
+    _OPERATOR = re.compile(r"(\.\*|\*|@\(\s*([^,()]+?)\s*(?:,\s*([^,()]+?)\s*)?\))")
+
+    def _temp(self, labels, fmt):
+        t = _Tensor(f"%t{len(self.tensors)}", labels, fmt)
+        self.tensors[t.name] = t
+        return t
+
+    def _assign(self, cname, clabels, mask, mode, rhs):
+        """C[...] = operand (operator operand)*: transposed operands become dense temporaries, a chain is
+        evaluated left to right through temporaries (frontends/comet_dsl/mlir/MLIRGen.cpp builds the same
+        left-leaning tree), and the last operation writes C."""
+        operands, operators, at = [], [], 0
+        while True:
+            m = self._OPERAND.match(rhs, at)
+            if not m:
+                raise TaError(f"cannot read the expression: {rhs}")
+            if m.group(1):          # transpose(A[..], {..})
+                a = self._tensor(m.group(1))
+                al, order = self._labels(m.group(2)), self._labels(m.group(3))
+                if a.fmt != "Dense" or sorted(al) != sorted(order):
+                    raise TaError("transpose inside an expression is supported for dense tensors")
+                t = self._temp(order, "Dense")
+                t.value = rt.transpose(self._dense(a), [al.index(l) for l in order])
+                t.zero = False
+                operands.append((t.name, ", ".join(order)))
+            else:
+                operands.append((m.group(4), m.group(5)))
+            at = m.end()
+            if at == len(rhs):
+                break
+            m = self._OPERATOR.match(rhs, at)
+            if not m:
+                raise TaError(f"cannot read the expression: {rhs}")
+            operators.append(m.groups())
+            at = m.end()
+        if len(operands) < 2:
+            raise TaError(f"statement not supported by this runner: {cname}[{clabels}] = {rhs}")
+        cl = self._labels(clabels)
+        while len(operands) > 2:
+            (an, als), (bn, bls) = operands[0], operands[1]
+            a, b = self._tensor(an), self._tensor(bn)
+            al, bl = self._labels(als), self._labels(bls)
+            later = set(cl)
+            for _, ls in operands[2:]:
+                later.update(self._labels(ls))
+            op = operators[0]
+            if op[0] == "*" or (op[1] is not None and op[2] is not None):
+                tl = [l for l in al if l not in bl or l in later] + [l for l in bl if l not in al]
+            else:
+                tl = al
+            fmt = "Dense" if "Dense" in (a.fmt, b.fmt) else "CSR"
+            t = self._temp(tl, fmt)
+            self._product(t.name, ", ".join(tl), None, None, an, als, *op, bn, bls)
+            operands[:2] = [(t.name, ", ".join(tl))]
+            operators.pop(0)
+        (an, als), (bn, bls) = operands
+        self._product(cname, clabels, mask, mode, an, als, *operators[0], bn, bls)
 
     def _product(self, cname, clabels, mask, _mode, aname, alabels, op, red, mul, bname, blabels):
         c, a, b = self._tensor(cname), self._tensor(aname), self._tensor(bname)
@@ -170,6 +246,7 @@ class Program:
                 raise TaError("elementwise operations need the same indices on every tensor")
             if a.fmt == b.fmt == c.fmt == "Dense":
                 c.value = rt.eltwise_dense(self._dense(a), self._dense(b), op=ew)
+                self._written(c)
                 return
             if len(al) != 2:
                 raise TaError("sparse elementwise operations are supported for matrices")
@@ -181,6 +258,12 @@ class Program:
             if sp_.fmt != "Dense" and de_.fmt == "Dense" and (sp_ is a or commutes) and c.fmt in (sp_.fmt, "Dense"):
                 S = self._sparse(sp_)
                 self._bind(al, S.shape)
+                if de_.pending is not None and ew == "times" and c.fmt != "Dense":
+                    cm, d = de_.pending          # B .* (C x D): only the sampled entries are computed
+                    c.value = rt.sddmm(S, self._dense(cm), self._dense(d))
+                    return
+                if c.fmt == "Dense":
+                    self._written(c)
                 if c.fmt != "Dense":
                     c.value = rt.eltwise_csr_dense(S, self._dense(de_), op=ew)
                 else:
@@ -193,6 +276,7 @@ class Program:
                 raise TaError("semirings and masks are supported for sparse x sparse products")
             Bm = self._sparse(b)
             self._bind(bl, Bm.shape)
+            self._written(c)
             if len(bl) == 2 and al == [bl[0]] and cl == [bl[1]]:
                 rt.vecmat(self._dense(a), Bm, self._dense(c), accumulate=True)
             elif len(bl) == 2 and len(al) == 2 and al[1] == bl[0] and cl == [al[0], bl[1]]:
@@ -205,6 +289,7 @@ class Program:
                 raise TaError("semirings and masks are supported for sparse x sparse products")
             A = self._sparse(a)
             self._bind(al, A.shape)
+            self._written(c)
             if len(al) == 2 and bl == [al[1]] and cl == [al[0]]:
                 rt.spmv(A, self._dense(b), self._dense(c), accumulate=True)
             elif len(al) == 2 and len(bl) == 2 and bl[0] == al[1] and cl == [al[0], bl[1]]:
@@ -222,6 +307,15 @@ class Program:
         if a.fmt == b.fmt == c.fmt == "Dense":
             if semiring not in (None, ("plus", "times")) or mask:
                 raise TaError("dense contractions are plus-times and unmasked")
+            if (len(al) == len(bl) == 2 and al[1] == bl[0] and cl == [al[0], bl[1]] and c.zero
+                    and c.pending is None and a is not c and b is not c):
+                # a matrix product into zeros: left unformed until something reads it; `S .* T` with a sparse S
+                # then computes the sampled entries only (the reference's --opt-fusion does this to SDDMM)
+                c.pending = (a, b)
+                c.value = None
+                return
+            self._dense(c)
+            self._written(c)
             # one character per label, numbered as the front end does: by first appearance in A, B, C
             names = {}
             for l in al + bl + cl:
@@ -239,6 +333,7 @@ class Program:
         if self._labels(order) != bl or sorted(al) != sorted(bl):
             raise TaError("the index list of transpose must be the output's")
         b.value = rt.transpose(self._dense(a), [al.index(l) for l in bl])
+        self._written(b)
 
     def _sum(self, var, name, _labels):
         t = self._tensor(name)
@@ -274,13 +369,12 @@ class Program:
 
     _IDX = r"\[([^\]]*)\]"
     _RULES = [
-        (r"IndexLabel\s*\[\s*(\w+)\s*\]\s*=\s*\[\s*(\?|\d+)\s*\]", _index_label),
+        (r"IndexLabel\s*\[\s*(\w+(?:\s*,\s*\w+)*)\s*\]\s*=\s*\[\s*(\?|\d+)\s*\]", _index_label),
         (r"Tensor\s*<\s*double\s*>\s*(\w+)\s*\(\s*\[([^\]]*)\]\s*,\s*\{?\s*(\w+)\s*\}?\s*\)", _declare),
         (r"(\w+)\s*" + _IDX + r"\s*=\s*comet_read\(\s*(\d+)\s*(?:,\s*(\d+)\s*)?\)", _read),
         (r"(\w+)\s*" + _IDX + r"\s*=\s*([-+]?[0-9.]+(?:[eE][-+]?\d+)?)", _fill),
-        (r"(\w+)\s*" + _IDX + r"\s*(?:<\s*(\w+)\s*,\s*(\w+)\s*>)?\s*=\s*(\w+)\s*" + _IDX +
-         r"\s*(\.\*|\*|@\(\s*([^,()]+?)\s*(?:,\s*([^,()]+?)\s*)?\))\s*(\w+)\s*" + _IDX, _product),
         (r"(\w+)\s*" + _IDX + r"\s*=\s*transpose\(\s*(\w+)\s*" + _IDX + r"\s*,\s*\{([^}]*)\}\s*\)", _transpose),
+        (r"(\w+)\s*" + _IDX + r"\s*(?:<\s*(\w+)\s*,\s*(\w+)\s*>)?\s*=\s*(.+)", _assign),
         (r"var\s+(\w+)\s*=\s*SUM\(\s*(\w+)\s*" + _IDX + r"\s*\)", _sum),
         (r"var\s+(\w+)\s*=\s*getTime\(\s*\)", _get_time),
         (r"printElapsedTime\(\s*(\w+)\s*,\s*(\w+)\s*\)", _elapsed),

@@ -178,6 +178,14 @@ int comet_hip_eltwise_csr_dense_dense(int64_t a, int64_t d_dptr, int64_t ldd,
  * (eltwise_monoid{Plus,Minus,Min,Times}_DensexDense_oDense.ta). */
 int comet_hip_eltwise_dense_f64(int64_t n, int64_t a_dptr, int64_t b_dptr, int64_t c_dptr, int op);
 
+/* Sampled dense-dense matrix product, A = B .* (C x D): B is CSR (nrows x ncols), C is nrows x K (leading
+ * dimension ldc), D is K x ncols (ldd), all fp64 on the device.  Returns a new CSR handle with B's structure
+ * and val[p] * sum_k C[i,k] * D[k,j] for the stored entry p = (i, j), the sum unfused and in ascending k, as
+ * the reference's loops compute it whether T = C x D is materialised or fused away (--opt-fusion,
+ * lib/Dialect/IndexTree/Transforms/KernelFusion.cpp:1049-1220; test/integration/kernels/sddmm.ta:27-28).
+ * The dense product is never formed.  0 on failure. */
+int64_t comet_hip_sddmm_csr_f64(int64_t b, int64_t K, int64_t c_dptr, int64_t ldc, int64_t d_dptr, int64_t ldd);
+
 /* ---- input side: MatrixMarket files, read modes, the file-id protocol ---------
  * Read modes of comet_read(id, mode): lib/ExecutionEngine/SparseUtils.cpp:40-64.
  * Storage format codes per dimension: include/comet/ExecutionEngine/

@@ -136,6 +136,25 @@ void oracle_eltwise_csr_dense(idx_t nrows, idx_t ncols, const idx_t *pos, const 
             out[p] = semiring_mult(op, val[p], D[i * ncols + crd[p]]);
 }
 
+/* Sampled dense-dense product A = B .* (C x D) at B's stored entries:          */
+/* T[i,j] = sum_k C[i,k] * D[k,j] (test/integration/kernels/sddmm.ta:27, loop    */
+/* order i, k, j from the index order of C[i,k] * D[k,j], so ascending k for     */
+/* every (i, j); unfused), then B[i,j] * T[i,j] (:28).  C is nrows x K, D is     */
+/* K x ncols, both row-major and dense.                                          */
+void oracle_sddmm_csr(idx_t nrows, idx_t ncols, const idx_t *pos, const idx_t *crd, const double *val,
+                      idx_t K, const double *C, const double *D, double *out)
+{
+    for (idx_t i = 0; i < nrows; ++i)
+        for (idx_t p = pos[i]; p < pos[i + 1]; ++p) {
+            double t = 0.0;
+            for (idx_t k = 0; k < K; ++k) {
+                double prod = C[i * K + k] * D[k * ncols + crd[p]];
+                t = t + prod;
+            }
+            out[p] = val[p] * t;
+        }
+}
+
 /* Dense (op) Dense, element by element.                                       */
 void oracle_eltwise_dense(idx_t n, const double *a, const double *b, int op, double *out)
 {

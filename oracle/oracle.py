@@ -59,6 +59,8 @@ def lib():
     L.oracle_densemat_csr.restype = None
     L.oracle_eltwise_csr_dense.argtypes = [C.c_int64, C.c_int64, i64p, i64p, f64p, f64p, C.c_int, f64p]
     L.oracle_eltwise_csr_dense.restype = None
+    L.oracle_sddmm_csr.argtypes = [C.c_int64, C.c_int64, i64p, i64p, f64p, C.c_int64, f64p, f64p, f64p]
+    L.oracle_sddmm_csr.restype = None
     L.oracle_eltwise_dense.argtypes = [C.c_int64, f64p, f64p, C.c_int, f64p]
     L.oracle_eltwise_dense.restype = None
     L.oracle_spgemm_symbolic.argtypes = [C.c_int64, C.c_int64, C.c_int64, i64p, i64p, i64p, i64p, vp, vp, i64p]
@@ -147,6 +149,14 @@ def eltwise_csr_dense(pos, crd, val, D, op="times"):
     pos, crd, val, D = _i64(pos), _i64(crd), _f64(val), _f64(D)
     out = np.zeros(max(len(val), 1))
     lib().oracle_eltwise_csr_dense(len(pos) - 1, D.shape[1], pos, crd, val, D, MULT_OPS[op], out)
+    return out[:len(val)]
+
+
+def sddmm(pos, crd, val, C, D):
+    """Values of B .* (C @ D) at B's stored positions; C is nrows x K, D is K x ncols."""
+    pos, crd, val, C, D = _i64(pos), _i64(crd), _f64(val), _f64(C), _f64(D)
+    out = np.zeros(max(len(val), 1))
+    lib().oracle_sddmm_csr(len(pos) - 1, D.shape[1], pos, crd, val, C.shape[1], C, D, out)
     return out[:len(val)]
 
 

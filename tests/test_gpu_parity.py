@@ -920,3 +920,40 @@ def test_eltwise_monoid_golden_and_checker(golden, golden_dir):
         assert np.array_equal(got, orc.eltwise_csr_dense(pos, crd, val, D, op)), op
         got = rt.eltwise_dense(rt.DeviceArray.from_numpy(x), rt.DeviceArray.from_numpy(y), op=op).to_numpy()
         assert np.array_equal(got, orc.eltwise_dense(x, y, op)), op
+
+
+# ----------------------------------------------------------------- SDDMM
+def test_sddmm_golden(golden, golden_dir):
+    g = golden["kernels_and_compound"]["sddmm"]
+    B = rt.CsrMatrix.from_mtx(os.path.join(golden_dir, g["matrix"]))
+    nr, nc = B.shape
+    A = rt.sddmm(B, rt.DeviceArray.from_numpy(np.full((nr, g["K"]), g["c_fill"])),
+                 rt.DeviceArray.from_numpy(np.full((g["K"], nc), g["d_fill"])))
+    p, c, v = A.to_arrays()
+    printed = orc.format_i64([nr]) + orc.format_i64([-1]) + orc.format_i64(p) + orc.format_i64(c) + orc.format_f64(v)
+    assert printed == g["printed"]
+
+
+@pytest.mark.parametrize("n,m,K,density,seed", [(300, 200, 7, 0.05, 0), (2000, 1500, 64, 0.02, 1), (50, 3000, 33, 0.2, 2),
+                                                (100, 100, 0, 0.1, 3), (513, 257, 1, 0.3, 4)])
+def test_sddmm_vs_checker(n, m, K, density, seed):
+    """Same additions in the same order as the checker: bit-exact; rows without entries in between."""
+    rng = np.random.default_rng(seed)
+    pos, crd, val = _rand_csr(rng, n, m, density)
+    B = rt.CsrMatrix.from_arrays((n, m), pos, crd, val)
+    Cm, D = rng.uniform(-1, 1, (n, K)), rng.uniform(-1, 1, (K, m))
+    A = rt.sddmm(B, rt.DeviceArray.from_numpy(Cm), rt.DeviceArray.from_numpy(D))
+    p, c, v = A.to_arrays()
+    assert np.array_equal(p, pos) and np.array_equal(c, crd)
+    assert np.array_equal(v, orc.sddmm(pos, crd, val, Cm, D))
+
+
+def test_sddmm_empty_and_errors():
+    B = rt.CsrMatrix.from_arrays((4, 5), np.zeros(5, dtype=np.int64), np.zeros(0, dtype=np.int64), np.zeros(0))
+    A = rt.sddmm(B, rt.DeviceArray((4, 3), zero=True), rt.DeviceArray((3, 5), zero=True))
+    assert A.to_arrays()[0].tolist() == [0] * 5 and A.nnz == 0
+    with pytest.raises(ValueError):
+        rt.sddmm(B, rt.DeviceArray((4, 3), zero=True), rt.DeviceArray((2, 5), zero=True))
+    L = rt.lib()
+    assert L.comet_hip_sddmm_csr_f64(B.handle, 3, 0, 2, 0, 5) == 0          # ldc < K
+    assert b"sddmm" in L.comet_hip_last_error()

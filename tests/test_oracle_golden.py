@@ -521,3 +521,25 @@ def test_eltwise_monoid_golden(golden, golden_dir):
         a1pos, a1crd, _, a2crd, _ = orc.coo_layout(pos, crd, val)
         assert a1pos.tolist() == g["a1pos"] and a1crd.tolist() == g["a1crd"] and a2crd.tolist() == g["a2crd"]
         assert orc.format_f64(v) == g["printed_val"], g["source"]
+
+
+def test_sddmm_golden_and_brute_force(golden, golden_dir):
+    """kernels/sddmm.ta: B .* (C x D) at B's entries; then an independent restatement on random data (T formed
+    as a sum of outer products in ascending k, which adds in the same order) and scipy within rounding."""
+    g = golden["kernels_and_compound"]["sddmm"]
+    (nr, nc), pos, crd, val = _mtx(golden_dir, g["matrix"])
+    v = orc.sddmm(pos, crd, val, np.full((nr, g["K"]), g["c_fill"]), np.full((g["K"], nc), g["d_fill"]))
+    printed = orc.format_i64([nr]) + orc.format_i64([-1]) + orc.format_i64(pos) + orc.format_i64(crd) + orc.format_f64(v)
+    assert printed == g["printed"]
+    rng = np.random.default_rng(5)
+    A = sp.random(40, 30, 0.15, random_state=3, format="csr"); A.sort_indices()
+    Cm, D = rng.uniform(-1, 1, (40, 9)), rng.uniform(-1, 1, (9, 30))
+    got = orc.sddmm(A.indptr, A.indices, A.data, Cm, D)
+    T = np.zeros((40, 30))
+    for k in range(9):
+        T = T + np.outer(Cm[:, k], D[k, :])
+    rows = np.repeat(np.arange(40), np.diff(A.indptr))
+    assert np.array_equal(got, A.data * T[rows, A.indices])
+    assert np.allclose(got, A.data * (Cm @ D)[rows, A.indices], rtol=1e-13, atol=1e-15)
+    # a dropped term, a transposed operand or B's value left out would all show here
+    assert np.array_equal(orc.sddmm(A.indptr, A.indices, A.data, Cm[:, :0], D[:0, :]), A.data * 0.0)

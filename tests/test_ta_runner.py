@@ -206,3 +206,113 @@ def test_elementwise_monoid_programs(golden, golden_dir, tmp_path, monkeypatch):
 """
         out = _run(prog, [g["matrix"]], tmp_path, monkeypatch, golden_dir)
         _check(out, _ints(g["a1pos"]) + _ints(g["a1crd"]) + _ints([-1]) + _ints(g["a2crd"]) + g["printed_val"], tmp_path)
+
+
+# ------------------------------------------------------ kernels/ and compound_exps/ of the reference's tests
+def _kc_programs(g):
+    """name -> (program, input files); sizes and fills come from the golden entry."""
+    lab = lambda **kw: "".join(f"    IndexLabel [{k}] = [{v}];\n" for k, v in kw.items())
+    ten = lambda *decls: "".join(f"    Tensor<double> {n}([{', '.join(ls)}], {{{f}}});\n" for n, ls, f in decls)
+    body = lambda text: "def main() {\n" + text + "}\n"
+    P = {}
+    e = g["sddmm"]
+    P["sddmm"] = (body(lab(i="?", j="?", k=e["K"]) +
+                       ten(("B", "ij", "CSR"), ("C", "ik", "Dense"), ("D", "kj", "Dense"), ("A", "ij", "CSR"),
+                           ("T", "ij", "Dense")) +
+                       f"    B[i, j] = comet_read(0);\n    C[i, k] = {e['c_fill']};\n    D[k, j] = {e['d_fill']};\n"
+                       "    T[i, j] = 0.0;\n    T[i, j] = C[i, k] * D[k, j];\n    A[i, j] = B[i, j] .* T[i, j];\n"
+                       "    print(A);\n"), [e["matrix"]])
+    e = g["gnn"]
+    P["gnn"] = (body(lab(i="?", k="?", j=e["J"], h=e["H"]) +
+                     ten(("B", "ik", "CSR"), ("C", "kh", "Dense"), ("D", "hj", "Dense"), ("A", "ij", "Dense"),
+                         ("T", "ih", "Dense")) +
+                     f"    B[i, k] = comet_read(0);\n    C[k, h] = {e['c_fill']};\n    D[h, j] = {e['d_fill']};\n"
+                     "    A[i, j] = 0.0;\n    T[i, h] = 0.0;\n    T[i, h] = B[i, k] * C[k, h];\n"
+                     "    A[i, j] = T[i, h] * D[h, j];\n    print(A);\n"), [e["matrix"]])
+    e = g["gram_matrix"]
+    P["gram_matrix"] = (body(f"    IndexLabel [i, k] = [{e['I']}];\n" + lab(j=e["J"]) +
+                             ten(("A", "ij", "Dense"), ("B", "ii", "Dense")) +
+                             f"    A[i, j] = {e['a_fill']};\n    B[i, k] = 0.0;\n"
+                             "    B[i, k] = A[i, j] * transpose(A[k, j], {j, k});\n    print(B);\n"), [])
+    e = g["csr_dense_chain"]
+    P["csr_dense_chain"] = (body(lab(i="?", j="?", k=e["K"], l=e["L"]) +
+                                 ten(("B", "ij", "CSR"), ("A", "il", "Dense"), ("C", "jk", "Dense"),
+                                     ("D", "kl", "Dense")) +
+                                 f"    B[i, j] = comet_read(0);\n    A[i, l] = 0.0;\n    C[j, k] = {e['c_fill']};\n"
+                                 f"    D[k, l] = {e['d_fill']};\n    A[i, l] = B[i, j] * C[j, k] * D[k, l];\n"
+                                 "    print(A);\n"), [e["matrix"]])
+    e = g["csr_mult_dtranspose"]
+    P["csr_mult_dtranspose"] = (body(lab(i=e["I"], j="?", k="?") +
+                                     "    Tensor<double> A([k, j], CSR);\n    Tensor<double> B([i, j], Dense);\n"
+                                     "    Tensor<double> C([k, i], Dense);\n"
+                                     f"    A[k, j] = comet_read(0);\n    B[i, j] = {e['b_fill']};\n    C[k, i] = 0.0;\n"
+                                     "    C[k, i] = A[k, j] * transpose(B[i, j], {j, i});\n    print(C);\n"),
+                                [e["matrix"]])
+    e = g["dtranspose_eltwise_csr"]
+    P["dtranspose_eltwise_csr"] = (body(lab(i="?", j="?") +
+                                        ten(("B", "ji", "CSR"), ("C", "ji", "CSR"), ("A", "ij", "Dense")) +
+                                        f"    B[j, i] = comet_read(0);\n    A[i, j] = {e['a_fill']};\n"
+                                        "    C[j, i] = transpose(A[i, j], {j, i}) .* B[j, i];\n    print(C);\n"),
+                                   [e["matrix"]])
+    e = g["dtranspose_mult_csr"]
+    P["dtranspose_mult_csr"] = (body(lab(i="?", j=e["J"], k="?") +
+                                     ten(("B", "ik", "CSR"), ("A", "ij", "Dense"), ("C", "jk", "Dense")) +
+                                     f"    B[i, k] = comet_read(0);\n    A[i, j] = {e['a_fill']};\n    C[j, k] = 0.0;\n"
+                                     "    C[j, k] = transpose(A[i, j], {j, i}) * B[i, k];\n    print(C);\n"),
+                                [e["matrix"]])
+    e = g["dense_chain"]
+    si, sj, sk, sl = e["sizes"]
+    P["dense_chain"] = (body(lab(i=si, j=sj, k=sk, l=sl) +
+                             ten(("A", "ij", "Dense"), ("B", "jk", "Dense"), ("C", "kl", "Dense"), ("D", "il", "Dense")) +
+                             f"    A[i, j] = {e['fills'][0]};\n    B[j, k] = {e['fills'][1]};\n"
+                             f"    C[k, l] = {e['fills'][2]};\n    D[i, l] = 0.0;\n"
+                             "    D[i, l] = A[i, j] * B[j, k] * C[k, l];\n    print(D);\n"), [])
+    e = g["dense_eltwise_dtranspose"]
+    for name, expr in (("dense_eltwise_dtranspose", "B[j, i] .* transpose(A[i, j], {j, i})"),
+                       ("dtranspose_eltwise_dense", "transpose(A[i, j], {j, i}) .* B[j, i]")):
+        P[name] = (body(lab(i=e["N"], j=e["N"]) + ten(("A", "ij", "Dense"), ("B", "ji", "Dense"), ("C", "ji", "Dense")) +
+                        f"    A[i, j] = {e['a_fill']};\n    B[j, i] = {e['b_fill']};\n    C[j, i] = 0.0;\n"
+                        f"    C[j, i] = {expr};\n    print(C);\n"), [])
+    e = g["dense_mult_dtranspose"]
+    P["dense_mult_dtranspose"] = (body(lab(i=e["N"], j=e["N"], k=e["N"]) +
+                                       ten(("B", "ij", "Dense"), ("A", "kj", "Dense"), ("C", "ki", "Dense")) +
+                                       f"    B[i, j] = {e['b_fill']};\n    A[k, j] = {e['a_fill']};\n    C[k, i] = 0.0;\n"
+                                       "    C[k, i] = A[k, j] * transpose(B[i, j], {j, i});\n    print(C);\n"), [])
+    e = g["dtranspose_mult_dense"]
+    P["dtranspose_mult_dense"] = (body(lab(i=e["N"], j=e["N"], k=e["N"]) +
+                                       ten(("A", "ij", "Dense"), ("B", "ik", "Dense"), ("C", "jk", "Dense")) +
+                                       f"    A[i, j] = {e['a_fill']};\n    B[i, k] = {e['b_fill']};\n    C[j, k] = 0.0;\n"
+                                       "    C[j, k] = transpose(A[i, j], {j, i}) * B[i, k];\n    print(C);\n"), [])
+    e = g["dense_transpose_4d"]
+    si, sj, sk, sl = e["sizes"]
+    P["dense_transpose_4d"] = (body(lab(i=si, j=sj, k=sk, l=sl) +
+                                    ten(("A", "ijkl", "Dense"), ("B", "ikjl", "Dense")) +
+                                    f"    A[i, j, k, l] = {e['fill']};\n"
+                                    "    B[i, k, j, l] = transpose(A[i, j, k, l], {i, k, j, l});\n    print(B);\n"), [])
+    return P
+
+
+_KC_NAMES = ["sddmm", "gnn", "gram_matrix", "csr_dense_chain", "csr_mult_dtranspose", "dtranspose_eltwise_csr",
+             "dtranspose_mult_csr", "dense_chain", "dense_eltwise_dtranspose", "dtranspose_eltwise_dense",
+             "dense_mult_dtranspose", "dtranspose_mult_dense", "dense_transpose_4d"]
+
+
+@pytest.mark.parametrize("name", _KC_NAMES)
+def test_kernel_and_compound_expression_programs(golden, golden_dir, tmp_path, monkeypatch, name):
+    g = golden["kernels_and_compound"]
+    prog, files = _kc_programs(g)[name]
+    out = _run(prog, files, tmp_path, monkeypatch, golden_dir)
+    _check(out, g["dense_eltwise_dtranspose" if name == "dtranspose_eltwise_dense" else name]["printed"], tmp_path)
+
+
+def test_sddmm_program_never_forms_the_dense_product(golden, golden_dir, tmp_path, monkeypatch):
+    """T = C x D followed by B .* T runs as one SDDMM launch; no GEMM and no dense elementwise kernel."""
+    from comet_amd import runtime as rt
+    g = golden["kernels_and_compound"]
+    prog, files = _kc_programs(g)["sddmm"]
+    rt.init(0)
+    rt.profile_reset(); rt.profile_enable(True)
+    _run(prog, files, tmp_path, monkeypatch, golden_dir)
+    rep = rt.profile_report()
+    rt.profile_enable(False)
+    assert "sddmm_kernel" in rep and not any("gemm" in k or "eltwise" in k for k in rep), sorted(rep)
