@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the index-tree kernel path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload spmm|spmv|ttgt|tricount|spgemm|coo2csr]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload spmm|spmv|sddmm|ttgt|tricount|spgemm|coo2csr]
 
 A step is one pass of the kernel over one batch of seeded synthetic input that is already
 resident in HBM.  The default workload is the one the headline metric is quoted on: CSR SpMM,
@@ -140,6 +140,49 @@ def bench_spmm(rt, orc, gen, args):
                      "traffic": SPMM_TRAFFIC_BYTES if (n, K) == (500_000, 64) else None,
                      "kernel": dom, "kernel_avg_ms": dom_ms, "algorithmic_bytes": int(alg_bytes),
                      "gather_inclusive_bytes": int(nnz * 8 * K + nnz * (8 + ib) + 8 * n * K)},
+        "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
+    }
+
+
+def bench_sddmm(rt, orc, gen, args):
+    """A = B .* (C x D) on the SpMM matrix: B 500,000^2 CSR, C n x 64, D 64 x n."""
+    n, K = args.n or 500_000, 64
+    pos, crd, val = gen.zipf_csr(n=n, mean=16.0, cap=4096, seed=2)
+    nnz = len(crd)
+    Cm, D = gen.dense((n, K), seed=5), gen.dense((K, n), seed=6)
+    B = rt.CsrMatrix.from_arrays((n, n), pos, crd, val)
+    dC, dD = rt.DeviceArray.from_numpy(Cm), rt.DeviceArray.from_numpy(D)
+    vals = rt.DeviceArray(nnz)               # A shares B's structure: the step writes its values
+    step = lambda: rt.sddmm(B, dC, dD, out_values=vals)
+    step()
+    wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
+    kt = kernel_times(rt, step, args.steps)
+    rows = np.arange(0, n, max(1, n // 2000))            # the checker on a sample of rows
+    lo, hi = pos[rows], pos[rows + 1]
+    sel = np.concatenate([np.arange(a, b) for a, b in zip(lo, hi)])
+    spos = np.concatenate([[0], np.cumsum(hi - lo)])
+    parity_ok = bool(np.array_equal(vals.to_numpy()[sel],
+                                    orc.sddmm(spos, crd[sel], val[sel], Cm[rows], D)))
+    flops = 2.0 * nnz * K + nnz
+    ib = 4
+    alg_bytes = nnz * (8 + ib) + (n + 1) * ib + 8 * n * K * 2 + nnz * 8      # B, C and D once, A's values once
+    dom = "sddmm_kernel"
+    dom_ms = kt[dom]["avg_ms"]
+    cpu = None
+    if not args.no_cpu:
+        res = np.zeros(nnz)
+        t, reps = cpu_time(lambda: orc.lib().oracle_sddmm_csr(n, n, pos, crd, val, K, Cm, D, res), budget_s=20.0)
+        cpu = {"value": flops / t / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
+               "sample": f"the full workload, best of {reps} runs, {t * 1e3:.0f} ms each (single thread)"}
+    return {
+        "metric": "SDDMM GFLOP/s (+ achieved HBM GB/s as % of roofline) on 1 MI355X",
+        "value": flops / (dev_ms * 1e-3) / 1e9, "unit": "GFLOP/s", "ms_per_step": dev_ms, "dtype": "f64",
+        "config": {"workload": "sddmm_csr_zipf", "rows": n, "cols": n, "nnz": int(nnz), "inner": K, "seed": 2,
+                   "index_bytes": ib},
+        "roofline": {"bound": "hbm", "achieved": alg_bytes / (dev_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": alg_bytes / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": dom + " (+ transpose of D: the whole step is timed)",
+                     "kernel_avg_ms": dom_ms, "algorithmic_bytes": int(alg_bytes)},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
     }
 
@@ -460,7 +503,7 @@ def bench_coo2csr(rt, orc, gen, args):
     }
 
 
-WORKLOADS = {"copy": bench_copy, "spmm": bench_spmm, "spmv": bench_spmv, "ttgt": bench_ttgt, "tricount": bench_tricount,
+WORKLOADS = {"copy": bench_copy, "spmm": bench_spmm, "spmv": bench_spmv, "sddmm": bench_sddmm, "ttgt": bench_ttgt, "tricount": bench_tricount,
              "spgemm": bench_spgemm, "coo2csr": bench_coo2csr}
 
 

@@ -87,6 +87,8 @@ struct Csr {
     // rows of the original that store nothing (the product clears them when it does not accumulate)
     int32_t *empty_rows = nullptr;
     int64_t nempty = 0;
+    // entry_row[p] = the row that holds stored entry p (built on first use by csr_entry_rows)
+    int32_t *entry_row = nullptr;
     // the transpose, built the first time a dense-times-sparse product needs it
     Csr *transposed = nullptr;
 };
@@ -95,6 +97,7 @@ Csr *csr_from_handle(int64_t h);           // nullptr (and error set) if unknown
 int64_t csr_register(Csr *c);              // takes ownership of the struct
 int csr_alloc(Csr *c, int64_t nrows, int64_t ncols, int64_t nnz);   // allocates pos/crd/val, owns = true
 void csr_release(Csr *c);                  // frees the arrays it owns, its plans and the struct
+int csr_entry_rows(Csr *a, const int32_t **rows);      // the row of every stored entry, kept in the handle
 Csr *csr_transposed_copy(const Csr *a);    // new unregistered struct holding the transpose (nullptr on failure)
 
 // Records an event pair around a kernel launch when profiling is on.

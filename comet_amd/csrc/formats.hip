@@ -221,6 +221,22 @@ __global__ void csr_expand_rows(int64_t nrows, int64_t nnz, const int64_t *__res
     rowid[e] = (int32_t)lo;
 }
 
+// Kernels that give one lane to an entry read its row here instead of searching pos.
+int csr_entry_rows(Csr *a, const int32_t **rows)
+{
+    if (!a->entry_row && a->nnz > 0) {
+        if (a->nrows >= (1ll << 31))
+            return set_error(COMET_HIP_ERR_SIZE, "row ids of %lld rows do not fit 32 bits", (long long)a->nrows);
+        COMET_HIPCHK(hipMalloc((void **)&a->entry_row, sizeof(int32_t) * (size_t)a->nnz));
+        KernelTimer t("csr_expand_rows");
+        csr_expand_rows<<<dim3((unsigned)ceil_div(a->nnz, 256)), dim3(256), 0, stream()>>>(a->nrows, a->nnz, a->pos,
+                                                                                           a->entry_row);
+        COMET_HIPCHK(hipGetLastError());
+    }
+    *rows = a->entry_row;
+    return COMET_HIP_OK;
+}
+
 __global__ void widen_i32(int64_t n, const int32_t *__restrict__ in, int64_t *__restrict__ out)
 {
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;

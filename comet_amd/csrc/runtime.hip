@@ -142,6 +142,8 @@ static void csr_drop_plans(Csr *c)
     if (c->transposed)
         csr_release(c->transposed);
     c->light = c->transposed = nullptr;
+    (void)hipFree(c->entry_row);
+    c->entry_row = nullptr;
     (void)hipFree(c->rowmap);
     (void)hipFree(c->empty_rows);
     c->rowmap = c->empty_rows = nullptr;

@@ -1363,35 +1363,101 @@ extern "C" int comet_hip_densemat_csr_f64(int64_t csr, int64_t M, int64_t a_dptr
 // (lib/Dialect/IndexTree/Transforms/KernelFusion.cpp:1049-1220; the test is
 // test/integration/kernels/sddmm.ta).  Either way a stored entry (i, j) gets
 // val * sum_k C[i,k] * D[k,j], the sum unfused and in ascending k.
-// One lane per stored entry; its row is found by bisection in pos.  D is
-// transposed first, so that a lane walks along a row of K contiguous values
-// instead of striding through D.
+// A wavefront takes 32 consecutive stored entries.  Entry by entry it loads the
+// row of C and the (transposed) row of D with the lanes along k - two coalesced
+// loads - and leaves the 64 products in LDS; then lane e walks along the
+// products of entry e and adds them in ascending k.  D is transposed first, so
+// that its "row" for a column j is contiguous; the row of every entry comes
+// from a list kept in B's handle (searching pos per entry cost 80 % of the time).
 // ============================================================================
-__global__ __launch_bounds__(256) void sddmm_kernel(int64_t nrows, int64_t nnz, const int64_t *__restrict__ pos,
-                                                    const int32_t *__restrict__ crd,
-                                                    const double *__restrict__ val, const double *__restrict__ C,
-                                                    int64_t ldc, const double *__restrict__ Dt, int64_t K,
-                                                    double *__restrict__ out)
+#ifndef COMET_SDDMM_E
+#define COMET_SDDMM_E 16
+#endif
+constexpr int SDDMM_E = COMET_SDDMM_E;          // entries per wavefront tile
+constexpr int SDDMM_W = 4;           // wavefronts per workgroup
+constexpr int SDDMM_LD = 65;         // tile row length in doubles: 64 products + 1, so a column walk hits all banks
+
+__global__ __launch_bounds__(SDDMM_W * 64) void sddmm_kernel(int64_t nnz, const int32_t *__restrict__ entry_row,
+                                                             const int32_t *__restrict__ crd,
+                                                             const double *__restrict__ val,
+                                                             const double *__restrict__ C, int64_t ldc,
+                                                             const double *__restrict__ Dt, int64_t K,
+                                                             double *__restrict__ out)
 {
-    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (p >= nnz)
+    __shared__ double tiles[SDDMM_W][SDDMM_E * SDDMM_LD];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    double *tile = tiles[wave];
+    const int64_t base = ((int64_t)blockIdx.x * SDDMM_W + wave) * SDDMM_E;
+    if (base >= nnz)
         return;
-    int64_t lo = 0, hi = nrows - 1;          // the row r with pos[r] <= p < pos[r + 1]
-    while (lo < hi) {
-        const int64_t mid = (lo + hi) >> 1;
-        if (pos[mid + 1] <= p)
-            lo = mid + 1;
-        else
-            hi = mid;
-    }
-    const double *c = C + lo * ldc, *d = Dt + (int64_t)crd[p] * K;
+    const int cnt = (int)(nnz - base < SDDMM_E ? nnz - base : SDDMM_E);
+    const int64_t p = base + (lane < cnt ? lane : cnt - 1);        // lane e < cnt owns entry base + e
+    const int my_col = crd[p], my_row = entry_row[p];
     double t = 0.0;
-    for (int64_t k = 0; k < K; ++k)
-        t = t + c[k] * d[k];
-    out[p] = val[p] * t;
+    for (int64_t kc = 0; kc < K; kc += 64) {
+        const int kn = (int)(K - kc < 64 ? K - kc : 64);
+        const int64_t k = kc + (lane < kn ? lane : 0);
+        double c[SDDMM_E], d[SDDMM_E];
+#pragma unroll
+        for (int e = 0; e < SDDMM_E; ++e) {          // past the end of a short tile: its last entry again
+            const int ec = e < cnt ? e : cnt - 1;
+            const int64_t j = __builtin_amdgcn_readlane(my_col, ec);
+            const int64_t r = __builtin_amdgcn_readlane(my_row, ec);
+            c[e] = C[r * ldc + k];
+            d[e] = Dt[j * K + k];
+        }
+#pragma unroll
+        for (int e = 0; e < SDDMM_E; ++e)
+            tile[e * SDDMM_LD + lane] = c[e] * d[e];
+        if (lane < cnt) {
+            if (kn == 64) {
+#pragma unroll 16
+                for (int q = 0; q < 64; ++q)
+                    t = t + tile[lane * SDDMM_LD + q];
+            } else {
+                for (int q = 0; q < kn; ++q)
+                    t = t + tile[lane * SDDMM_LD + q];
+            }
+        }
+    }
+    if (lane < cnt)
+        out[p] = val[p] * t;
 }
 
 static Workspace g_sddmm_dt;
+
+static int sddmm_values(Csr *b, int64_t K, int64_t c_dptr, int64_t ldc, int64_t d_dptr, int64_t ldd, double *out)
+{
+    if (K < 0 || ldc < K || ldd < b->ncols || (b->nnz > 0 && (!out || (K > 0 && (!c_dptr || !d_dptr)))))
+        return set_error(COMET_HIP_ERR_ARG, "bad operands passed to the sddmm entry point (K %lld, ldc %lld, ldd %lld)",
+                         (long long)K, (long long)ldc, (long long)ldd);
+    if (b->nnz == 0)
+        return COMET_HIP_OK;
+    if (K > 0) {
+        COMET_CHK(g_sddmm_dt.ensure(sizeof(double) * (size_t)b->ncols * (size_t)K, false));
+        COMET_CHK(transpose2d((const double *)d_dptr, ldd, K, b->ncols, (double *)g_sddmm_dt.ptr, K));
+    }
+    const int32_t *rows = nullptr;
+    COMET_CHK(csr_entry_rows(b, &rows));
+    {
+        KernelTimer t("sddmm_kernel");
+        sddmm_kernel<<<dim3((unsigned)ceil_div(b->nnz, SDDMM_W * SDDMM_E)), dim3(SDDMM_W * 64), 0, stream()>>>(
+            b->nnz, rows, b->crd, b->val, (const double *)c_dptr, ldc, (const double *)g_sddmm_dt.ptr, K, out);
+    }
+    COMET_HIPCHK(hipGetLastError());
+    return COMET_HIP_OK;
+}
+
+extern "C" int comet_hip_sddmm_csr_values_f64(int64_t bh, int64_t K, int64_t c_dptr, int64_t ldc, int64_t d_dptr,
+                                              int64_t ldd, int64_t out_val_dptr)
+{
+    COMET_CHK(ensure_init());
+    Csr *b = csr_from_handle(bh);
+    if (!b)
+        return COMET_HIP_ERR_HANDLE;
+    return sddmm_values(b, K, c_dptr, ldc, d_dptr, ldd, (double *)out_val_dptr);
+}
 
 extern "C" int64_t comet_hip_sddmm_csr_f64(int64_t bh, int64_t K, int64_t c_dptr, int64_t ldc, int64_t d_dptr,
                                            int64_t ldd)
@@ -1401,11 +1467,6 @@ extern "C" int64_t comet_hip_sddmm_csr_f64(int64_t bh, int64_t K, int64_t c_dptr
     Csr *b = csr_from_handle(bh);
     if (!b)
         return 0;
-    if (K < 0 || ldc < K || ldd < b->ncols || (b->nnz > 0 && K > 0 && (!c_dptr || !d_dptr))) {
-        set_error(COMET_HIP_ERR_ARG, "bad dense operands passed to comet_hip_sddmm_csr_f64 (K %lld, ldc %lld, ldd %lld)",
-                  (long long)K, (long long)ldc, (long long)ldd);
-        return 0;
-    }
     Csr *a = new Csr();
     if (csr_alloc(a, b->nrows, b->ncols, b->nnz) != COMET_HIP_OK) {
         delete a;
@@ -1413,21 +1474,12 @@ extern "C" int64_t comet_hip_sddmm_csr_f64(int64_t bh, int64_t K, int64_t c_dptr
     }
     bool ok = hipMemcpyAsync(a->pos, b->pos, sizeof(int64_t) * (size_t)(b->nrows + 1), hipMemcpyDeviceToDevice,
                              stream()) == hipSuccess;
-    if (ok && b->nnz > 0) {
+    if (ok && b->nnz > 0)
         ok = hipMemcpyAsync(a->crd, b->crd, sizeof(int32_t) * (size_t)b->nnz, hipMemcpyDeviceToDevice, stream()) ==
              hipSuccess;
-        if (ok && K > 0)
-            ok = g_sddmm_dt.ensure(sizeof(double) * (size_t)b->ncols * (size_t)K, false) == COMET_HIP_OK &&
-                 transpose2d((const double *)d_dptr, ldd, K, b->ncols, (double *)g_sddmm_dt.ptr, K) == COMET_HIP_OK;
-        if (ok) {
-            KernelTimer t("sddmm_kernel");
-            sddmm_kernel<<<dim3((unsigned)ceil_div(b->nnz, 256)), dim3(256), 0, stream()>>>(
-                b->nrows, b->nnz, b->pos, b->crd, b->val, (const double *)c_dptr, ldc,
-                (const double *)g_sddmm_dt.ptr, K, a->val);
-        }
-    }
-    if (!ok || hipGetLastError() != hipSuccess) {
-        set_error(COMET_HIP_ERR_HIP, "SDDMM failed");
+    if (!ok)
+        set_error(COMET_HIP_ERR_HIP, "copying the structure of the sampled matrix failed");
+    if (!ok || sddmm_values(b, K, c_dptr, ldc, d_dptr, ldd, a->val) != COMET_HIP_OK) {
         csr_release(a);
         return 0;
     }

@@ -85,6 +85,7 @@ SIGNATURES = {
     "comet_hip_densemat_csr_f64": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
     "comet_hip_eltwise_csr_dense_csr": (_i64, [_i64, _i64, _i64, _int]),
     "comet_hip_sddmm_csr_f64": (_i64, [_i64, _i64, _i64, _i64, _i64, _i64]),
+    "comet_hip_sddmm_csr_values_f64": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _i64]),
     "comet_hip_eltwise_csr_dense_dense": (_int, [_i64, _i64, _i64, _i64, _i64, _int]),
     "comet_hip_eltwise_dense_f64": (_int, [_i64, _i64, _i64, _i64, _int]),
     "comet_hip_mtx_read_csr": (_i64, [C.c_char_p, _int]),
@@ -500,14 +501,21 @@ def eltwise_csr_dense(A, D, out=None, op="times"):
     return out
 
 
-def sddmm(B, Cm, D):
+def sddmm(B, Cm, D, out_values=None):
     """B .* (Cm @ D) for a sparse B (nrows x ncols), dense Cm (nrows x K) and D (K x ncols): a CsrMatrix with
-    B's structure; the dense product is never formed."""
+    B's structure, or, when a DeviceArray `out_values` of nnz(B) doubles is given, just the values written
+    there; the dense product is never formed."""
     nrows, ncols = B.shape
     if len(Cm.shape) != 2 or len(D.shape) != 2 or Cm.shape[0] != nrows or D.shape[1] != ncols or \
             Cm.shape[1] != D.shape[0]:
         raise ValueError("SDDMM needs B (n x m), C (n x K) and D (K x m)")
     K = Cm.shape[1]
+    if out_values is not None:
+        if out_values.size < B.nnz:
+            raise ValueError("out_values is shorter than the number of stored entries")
+        _check(lib().comet_hip_sddmm_csr_values_f64(B.handle, K, Cm.ptr, K, D.ptr, ncols, out_values.ptr),
+               "comet_hip_sddmm_csr_values_f64")
+        return out_values
     return CsrMatrix(_handle(lib().comet_hip_sddmm_csr_f64(B.handle, K, Cm.ptr, K, D.ptr, ncols),
                              "comet_hip_sddmm_csr_f64"))
 

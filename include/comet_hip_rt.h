@@ -185,6 +185,11 @@ int comet_hip_eltwise_dense_f64(int64_t n, int64_t a_dptr, int64_t b_dptr, int64
  * lib/Dialect/IndexTree/Transforms/KernelFusion.cpp:1049-1220; test/integration/kernels/sddmm.ta:27-28).
  * The dense product is never formed.  0 on failure. */
 int64_t comet_hip_sddmm_csr_f64(int64_t b, int64_t K, int64_t c_dptr, int64_t ldc, int64_t d_dptr, int64_t ldd);
+/* The same values written to a device array of nnz(B) doubles the caller owns (A shares B's pos and crd, which
+ * is how the lowered code holds the output of an elementwise operation: SparseTensorConversionPass.cpp:1281-1333
+ * gives every sparse tensor its own value array).  Nothing is allocated for the result. */
+int comet_hip_sddmm_csr_values_f64(int64_t b, int64_t K, int64_t c_dptr, int64_t ldc, int64_t d_dptr,
+                                   int64_t ldd, int64_t out_val_dptr);
 
 /* ---- input side: MatrixMarket files, read modes, the file-id protocol ---------
  * Read modes of comet_read(id, mode): lib/ExecutionEngine/SparseUtils.cpp:40-64.

@@ -957,3 +957,15 @@ def test_sddmm_empty_and_errors():
     L = rt.lib()
     assert L.comet_hip_sddmm_csr_f64(B.handle, 3, 0, 2, 0, 5) == 0          # ldc < K
     assert b"sddmm" in L.comet_hip_last_error()
+
+
+def test_sddmm_values_into_a_caller_array():
+    rng = np.random.default_rng(9)
+    pos, crd, val = _rand_csr(rng, 700, 400, 0.03)
+    B = rt.CsrMatrix.from_arrays((700, 400), pos, crd, val)
+    Cm, D = rng.uniform(-1, 1, (700, 20)), rng.uniform(-1, 1, (20, 400))
+    out = rt.DeviceArray.from_numpy(np.full(len(val) + 3, 7.0))
+    rt.sddmm(B, rt.DeviceArray.from_numpy(Cm), rt.DeviceArray.from_numpy(D), out_values=out)
+    got = out.to_numpy()
+    assert np.array_equal(got[:len(val)], orc.sddmm(pos, crd, val, Cm, D)) and np.all(got[len(val):] == 7.0)
+    assert rt.lib().comet_hip_sddmm_csr_values_f64(B.handle, 20, 0, 20, 0, 400, out.ptr) != 0      # null operands
