@@ -521,8 +521,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on exactly one GPU (every kernel is single-device; see DESIGN.md "
-                 "for how the path would shard); rerun with --gpus 1")
+        sys.exit("bench.py: this build runs on exactly one GPU (every kernel is single-device and no figure at "
+                 "several GPUs is produced); rerun with --gpus 1")
     from comet_amd import gen, runtime as rt
     from oracle import oracle as orc
     rt.init(0)
