@@ -18,6 +18,8 @@ include/comet_hip_rt.h.  Statements it understands (frontends/comet_dsl/include/
     C[i, k]<M, push> = A[i, j] * B[j, k];                             (masked SpGEMM)
     C[i, j] = A[i, j] .* B[i, j];    (CSR .* CSR, CSR .* Dense, Dense .* CSR)
     C[i, j] = A[i, j] @(+) B[i, j];  (elementwise monoids +, -, *, min, max: Dense x Dense, sparse x Dense)
+    C[i, j] = A[i, j] + B[i, j];     C[i, j] = A[i, j] - B[i, j];     (dense)
+    var n = SUM(L[i, k] * L[k, j] .* L[i, j]);                        (SUM of an expression)
     B[j, i] = transpose(A[i, j], {j, i});                             (dense)
     A[i, l] = B[i, j] * C[j, k] * D[k, l];                            (chains, evaluated left to right)
     C[k, i] = A[k, j] * transpose(B[i, j], {j, i});                   (transposed dense operands)
@@ -167,7 +169,7 @@ class Program:
         t.pending = None
 
     _OPERAND = re.compile(r"\s*(?:transpose\(\s*(\w+)\s*\[([^\]]*)\]\s*,\s*\{([^}]*)\}\s*\)|(\w+)\s*\[([^\]]*)\])\s*")
-    _OPERATOR = re.compile(r"(\.\*|\*|@\(\s*([^,()]+?)\s*(?:,\s*([^,()]+?)\s*)?\))")
+    _OPERATOR = re.compile(r"(\.\*|\*|\+|-|@\(\s*([^,()]+?)\s*(?:,\s*([^,()]+?)\s*)?\))")
 
     def _temp(self, labels, fmt):
         t = _Tensor(f"%t{len(self.tensors)}", labels, fmt)
@@ -234,10 +236,10 @@ class Program:
                 semiring = (_SEMIRING_TOKENS[red.strip()], _SEMIRING_TOKENS[mul.strip()])
             except KeyError:
                 raise TaError(f"semiring @({red},{mul}) is not supported") from None
-        if op == ".*" or (red is not None and mul is None):
-            # `.*`, or the monoid form A @(op) B with a single operator
-            if op == ".*":
-                ew = "times"
+        if op in (".*", "+", "-") or (red is not None and mul is None):
+            # `.*`, `+`, `-`, or the monoid form A @(op) B with a single operator
+            if op in (".*", "+", "-"):
+                ew = {".*": "times", "+": "plus", "-": "minus"}[op]
             else:
                 if red.strip() not in _SEMIRING_TOKENS:
                     raise TaError(f"elementwise operator @({red}) is not supported")
@@ -339,6 +341,19 @@ class Program:
         t = self._tensor(name)
         self.scalars[var] = rt.reduce_sum(self._dense(t)) if t.fmt == "Dense" else rt.sum_values(self._sparse(t))
 
+    def _sum_of(self, var, expr):
+        """var s = SUM(A[i,k] * B[k,j] .* C[i,j]): the expression goes into a temporary that takes the indices
+        and the format of its last operand (kernels/triangleCount_SandiaLL.ta:32), then its values are added."""
+        last = None
+        for m in self._OPERAND.finditer(expr):
+            last = m
+        if last is None or last.group(4) is None:
+            raise TaError(f"cannot read the expression: {expr}")
+        labels = self._labels(last.group(5))
+        t = self._temp(labels, self._tensor(last.group(4)).fmt)
+        self._assign(t.name, ", ".join(labels), None, None, expr)
+        self._sum(var, t.name, None)
+
     def _get_time(self, var):
         rt.sync()
         self.scalars[var] = time.perf_counter()
@@ -376,9 +391,10 @@ class Program:
         (r"(\w+)\s*" + _IDX + r"\s*=\s*transpose\(\s*(\w+)\s*" + _IDX + r"\s*,\s*\{([^}]*)\}\s*\)", _transpose),
         (r"(\w+)\s*" + _IDX + r"\s*(?:<\s*(\w+)\s*,\s*(\w+)\s*>)?\s*=\s*(.+)", _assign),
         (r"var\s+(\w+)\s*=\s*SUM\(\s*(\w+)\s*" + _IDX + r"\s*\)", _sum),
+        (r"var\s+(\w+)\s*=\s*SUM\(\s*(.+)\)", _sum_of),
         (r"var\s+(\w+)\s*=\s*getTime\(\s*\)", _get_time),
         (r"printElapsedTime\(\s*(\w+)\s*,\s*(\w+)\s*\)", _elapsed),
-        (r"print\(\s*(\w+)\s*\)", _print),
+        (r"print\(\s*(\w+)\s*(?:\[[^\]]*\]\s*)?\)", _print),
     ]
 
 

@@ -316,3 +316,75 @@ def test_sddmm_program_never_forms_the_dense_product(golden, golden_dir, tmp_pat
     rep = rt.profile_report()
     rt.profile_enable(False)
     assert "sddmm_kernel" in rep and not any("gemm" in k or "eltwise" in k for k in rep), sorted(rep)
+
+
+# ------------------------------------------------------ further dense and SUM programs of the reference's tests
+def _ds_programs(g):
+    lab = lambda **kw: "".join(f"    IndexLabel [{k}] = [{v}];\n" for k, v in kw.items())
+    ten = lambda *decls: "".join(f"    Tensor<double> {n}([{', '.join(ls)}], {{{f}}});\n" for n, ls, f in decls)
+    body = lambda text: "def main() {\n" + text + "}\n"
+    P = {}
+    for name, op in (("eltwise_add_dense", "+"), ("eltwise_subtract_dense", "-")):
+        e = g[name]
+        P[name] = (body(lab(i=e["N"], j=e["N"]) + ten(("A", "ij", "Dense"), ("B", "ij", "Dense"), ("C", "ij", "Dense")) +
+                        f"    A[i, j] = {e['a']};\n    B[i, j] = {e['b']};\n    C[i, j] = 0.0;\n"
+                        f"    C[i, j] = A[i, j] {op} B[i, j];\n    print(C);\n"), [])
+    e = g["eltwise_mult_dense_4d"]
+    P["eltwise_mult_dense_4d"] = (body(lab(a=e["N"], b=e["N"], c=e["N"], d=e["N"]) +
+                                       ten(("A", "abcd", "Dense"), ("B", "abcd", "Dense"), ("C", "abcd", "Dense")) +
+                                       f"    A[a, b, c, d] = {e['a']};\n    B[a, b, c, d] = {e['b']};\n"
+                                       "    C[a, b, c, d] = 0.0;\n    C[a, b, c, d] = A[a, b, c, d] .* B[a, b, c, d];\n"
+                                       "    print(C);\n"), [])
+    e = g["dense_matvec"]
+    P["dense_matvec"] = (body(lab(i=e["I"], j=e["J"]) + ten(("A", "ij", "Dense"), ("B", "j", "Dense"), ("C", "i", "Dense")) +
+                              f"    A[i, j] = {e['a']};\n    B[j] = {e['b']};\n    C[i] = 0.0;\n"
+                              "    C[i] = A[i, j] * B[j];\n    print(C);\n"), [])
+    e = g["dense_matmul"]
+    P["dense_matmul"] = (body(lab(i=e["I"], j=e["J"], k=e["K"]) +
+                              ten(("A", "ij", "Dense"), ("B", "jk", "Dense"), ("C", "ik", "Dense")) +
+                              f"    A[i, j] = {e['a']};\n    B[j, k] = {e['b']};\n    C[i, k] = 0.0;\n"
+                              "    C[i, k] = A[i, j] * B[j, k];\n    print(C);\n"), [])
+    e = g["ccsd_t1_3"]
+    P["ccsd_t1_3"] = (body(f"    IndexLabel [i, c] = [{e['IC']}];\n" + lab(a=e["A"]) +
+                           ten(("f", "ca", "Dense"), ("t1", "ic", "Dense"), ("i0", "ia", "Dense")) +
+                           f"    f[c, a] = {e['f']};\n    t1[i, c] = {e['t1']};\n    i0[i, a] = 0.0;\n"
+                           "    i0[i, a] = f[c, a] * t1[i, c];\n    print(i0);\n"), [])
+    e = g["ccsd_t1_11"]
+    P["ccsd_t1_11"] = (body(f"    IndexLabel [i, j, m, n] = [{e['N']}];\n    IndexLabel [a, b, c, d] = [{e['N']}];\n" +
+                            ten(("i0", "ia", "Dense"), ("t1", "ia", "Dense"), ("t2", "ijab", "Dense"),
+                                ("v", "abij", "Dense")) +
+                            f"    i0[i, a] = 0.0;\n    t1[i, a] = {e['t1']};\n    t2[i, j, a, b] = {e['t2']};\n"
+                            f"    v[i, a, j, b] = {e['v']};\n"
+                            "    i0[i, a] = v[c, d, m, n] * t2[i, n, a, d] * t1[m, c];\n    print(i0[i, a]);\n"), [])
+    e = g["tricount_unmasked"]
+    P["tricount_unmasked"] = (body(lab(i="?", j="?", k="?") + ten(("L1", "ij", "CSR")) +
+                                   f"    L1[i, j] = comet_read(0, {e['read_mode']});\n"
+                                   "    var ntri = SUM(L1[i, k] * L1[k, j] .* L1[i, j]);\n    print(ntri);\n"),
+                              [e["matrix"]])
+    for name, idx in (("sum_dense_matrix", "ij"), ("sum_dense_tensor", "ijk")):
+        e = g[name]
+        ls = ", ".join(idx)
+        P[name] = (body(lab(**{l: n for l, n in zip(idx, e["shape"])}) + ten(("A", idx, "Dense")) +
+                        f"    A[{ls}] = {e['fill']};\n    var a = SUM(A[{ls}]);\n    print(a);\n"), [])
+    e = g["sum_coo"]
+    P["sum_coo"] = (body(lab(i="?", j="?") + ten(("A", "ij", "COO")) +
+                         "    A[i, j] = comet_read(0);\n    var a = SUM(A[i, j]);\n    print(a);\n"), [e["matrix"]])
+    e = g["transpose_dense_tensor"]
+    P["transpose_dense_tensor"] = (body(lab(i=e["N"], j=e["N"], k=e["N"]) +
+                                        ten(("A", "ijk", "Dense"), ("B", "kij", "Dense")) +
+                                        f"    A[i, j, k] = {e['fill']};\n"
+                                        "    B[k, i, j] = transpose(A[i, j, k], {k, i, j});\n    print(B);\n"), [])
+    return P
+
+
+_DS_NAMES = ["eltwise_add_dense", "eltwise_subtract_dense", "eltwise_mult_dense_4d", "dense_matvec", "dense_matmul",
+             "ccsd_t1_3", "ccsd_t1_11", "tricount_unmasked", "sum_dense_matrix", "sum_dense_tensor", "sum_coo",
+             "transpose_dense_tensor"]
+
+
+@pytest.mark.parametrize("name", _DS_NAMES)
+def test_dense_and_sum_programs(golden, golden_dir, tmp_path, monkeypatch, name):
+    g = golden["dense_and_sum_programs"]
+    prog, files = _ds_programs(g)[name]
+    out = _run(prog, files, tmp_path, monkeypatch, golden_dir)
+    _check(out, g[name]["printed"], tmp_path)
