@@ -434,8 +434,14 @@ constexpr int SPMM_HCB = 32;                         // column blocks a wavefron
 // and their sums are added once, at the end.
 //
 // A wavefront holds 64 entries of its list at a time, one per lane, and hands
-// them out with readlane; the next 64 are fetched while these are used, and the
-// gathers of the next 8 pairs are in flight while the current 8 are added.
+// them out with readlane; the next 64 are fetched while these are used.  The
+// gathers go out in batches of 8 pairs (16 rows of B) and the batch is added
+// before the next one is issued: a second batch in flight while the first is
+// added made the sweep slower (0.205 against 0.193 ms for the long rows alone,
+// 0.227 ms when the waits were made exact so that both batches really stayed in
+// flight; batches of 4 or 16 pairs: 0.25 ms) - with sixteen wavefronts per CU
+// the memory path is kept busy by the other wavefronts, and more requests
+// queued per wavefront only lengthen the queues.
 // Entry = column << SPMM_E_COL | real | first-of-run | owned row.
 constexpr int SPMM_HP = 8;       // pairs of entries per batch of gathers
 constexpr int SPMM_E_FIRST = SPMM_HR;          // the entry opens a run of one owned row
@@ -605,7 +611,7 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
     for (int r = 0; r < SPMM_HR; ++r)
         accx[r] = accy[r] = 0.0;
     if (s < e) {
-        double2 bA[SPMM_HP], bB[SPMM_HP];
+        double2 b[SPMM_HP];
         double2 run = make_double2(0.0, 0.0);
         int run_slot = 0;
         int cnt = (int)(e - s < 64 ? e - s : 64);
@@ -616,7 +622,7 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
             c_ent = q.x;
             c_val = __hiloint2double(q.w, q.z);
         }
-        heavy_issue<SMALL>(bA, c_ent, 0, cnt >> 1, half, B, ldb, col);
+        heavy_issue<SMALL>(b, c_ent, 0, cnt >> 1, half, B, ldb, col);
         for (int64_t base = s; base < e; base += 64) {
             const int64_t left = e - base - 64;
             const int ncnt = (int)(left < 0 ? 0 : (left < 64 ? left : 64));
@@ -628,19 +634,15 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
                 n_val = __hiloint2double(q.w, q.z);
             }
             const int np = cnt >> 1;
-            static_assert(SPMM_HP == 8, "the sweep is unrolled for four batches of 8 pairs per 64 entries");
-            if (np > 8)
-                heavy_issue<SMALL>(bB, c_ent, 8, np, half, B, ldb, col);
-            heavy_add(accx, accy, run, run_slot, bA, c_ent, c_val, 0, np, half);
-            if (np > 16)
-                heavy_issue<SMALL>(bA, c_ent, 16, np, half, B, ldb, col);
-            heavy_add(accx, accy, run, run_slot, bB, c_ent, c_val, 8, np, half);
-            if (np > 24)
-                heavy_issue<SMALL>(bB, c_ent, 24, np, half, B, ldb, col);
-            heavy_add(accx, accy, run, run_slot, bA, c_ent, c_val, 16, np, half);
-            if (ncnt > 0)
-                heavy_issue<SMALL>(bA, n_ent, 0, ncnt >> 1, half, B, ldb, col);
-            heavy_add(accx, accy, run, run_slot, bB, c_ent, c_val, 24, np, half);
+            heavy_add(accx, accy, run, run_slot, b, c_ent, c_val, 0, np, half);
+#pragma unroll
+            for (int t0 = SPMM_HP; t0 < 32; t0 += SPMM_HP)
+                if (np > t0) {
+                    heavy_issue<SMALL>(b, c_ent, t0, np, half, B, ldb, col);
+                    heavy_add(accx, accy, run, run_slot, b, c_ent, c_val, t0, np, half);
+                }
+            if (ncnt > 0)         // the first batch of the next 64 entries: in flight over the loop's back edge
+                heavy_issue<SMALL>(b, n_ent, 0, ncnt >> 1, half, B, ldb, col);
             c_ent = n_ent;
             c_val = n_val;
             cnt = ncnt;
