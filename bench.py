@@ -26,7 +26,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP64_MFMA_PEAK_TFLOPS = 78.6  # MI355X dense fp64 matrix, published
 # HBM bytes per SpMM product (all of its kernels) on the default workload, from rocprofv3 --pmc FETCH_SIZE (x 2.000)
 # and WRITE_SIZE (x 1.000), factors from a 1 GiB copy kernel; see profiles/spmm_kernels__spmm_zipf_500k_k64.txt
-SPMM_TRAFFIC_BYTES = int((481_573 * 2.000 + 276_201 * 1.000) * 1024)
+SPMM_TRAFFIC_BYTES = int((436_260 * 2.000 + 272_815 * 1.000) * 1024)
 
 
 _T0 = time.perf_counter()
