@@ -31,6 +31,7 @@ __device__ inline double readlane_f64(double v, int lane)
 // products: all lanes compute val*x[crd] with coalesced loads of crd/val,
 // then each lane adds the slice of the pass that belongs to its row, in
 // order.  HBM traffic is the compulsory one (crd, val, pos once; x gathered).
+// A slice of 128 products and more is added by the whole workgroup instead.
 // ============================================================================
 #ifndef COMET_SPMV_T
 #define COMET_SPMV_T 256
@@ -41,6 +42,14 @@ __device__ inline double readlane_f64(double v, int lane)
 constexpr int SPMV_T = COMET_SPMV_T;         // rows (= lanes) per workgroup
 constexpr int SPMV_PASS = COMET_SPMV_PASS;   // products staged in LDS per pass
 
+constexpr int SPMV_LONG = 128;               // a row's share of a pass from which the workgroup adds it together
+
+__device__ inline int64_t uniform_i64(int64_t v)
+{
+    return ((int64_t)__builtin_amdgcn_readfirstlane((int)(v >> 32)) << 32) |
+           (uint32_t)__builtin_amdgcn_readfirstlane((int)(v & 0xffffffff));
+}
+
 template <bool ACC>
 __global__ __launch_bounds__(SPMV_T) void spmv_csr_stream(const int64_t *__restrict__ pos,
                                                           const int32_t *__restrict__ crd,
@@ -49,24 +58,65 @@ __global__ __launch_bounds__(SPMV_T) void spmv_csr_stream(const int64_t *__restr
                                                           double *__restrict__ y, int64_t nrows)
 {
     __shared__ double prod[SPMV_PASS];
+    __shared__ double part[SPMV_T / 64];
+    __shared__ int64_t long_lo[SPMV_PASS / SPMV_LONG + 1], long_hi[SPMV_PASS / SPMV_LONG + 1];
+    __shared__ int long_owner[SPMV_PASS / SPMV_LONG + 1], nlong;
     const int tid = threadIdx.x;
     const int64_t r0 = (int64_t)blockIdx.x * SPMV_T;
     const int64_t r = r0 + tid;
     const int64_t rlast = r0 + SPMV_T < nrows ? r0 + SPMV_T : nrows;
     const int64_t ps = pos[r < nrows ? r : nrows];
     const int64_t pe = pos[r + 1 < nrows ? r + 1 : nrows];
-    const int64_t bs = pos[r0], be = pos[rlast];
+    const int64_t bs = uniform_i64(pos[r0]), be = uniform_i64(pos[rlast]);
     double acc = 0.0;
     if (ACC && r < nrows)
         acc = y[r];
     for (int64_t cs = bs; cs < be; cs += SPMV_PASS) {
         const int64_t ce = cs + SPMV_PASS < be ? cs + SPMV_PASS : be;
+        // a pass with fewer products than SPMV_LONG holds no long share: it skips the bookkeeping and its barriers
+        const bool may_be_long = ce - cs >= SPMV_LONG;
+        if (may_be_long && tid == 0)
+            nlong = 0;
         for (int64_t i = cs + tid; i < ce; i += SPMV_T)
             prod[i - cs] = val[i] * x[crd[i]];
         __syncthreads();
         const int64_t lo = ps > cs ? ps : cs, hi = pe < ce ? pe : ce;
-        for (int64_t p = lo; p < hi; ++p)
-            acc = acc + prod[p - cs];
+        if (hi - lo < SPMV_LONG) {           // the usual case: the lane adds its row's share in order
+            for (int64_t p = lo; p < hi; ++p)
+                acc = acc + prod[p - cs];
+        } else {                             // at most SPMV_PASS / SPMV_LONG lanes per pass come here
+            const int slot = atomicAdd(&nlong, 1);
+            long_owner[slot] = tid;
+            long_lo[slot] = lo;
+            long_hi[slot] = hi;
+        }
+        if (may_be_long) {
+            // Shares of SPMV_LONG products and more are added by the whole workgroup: lane t takes products
+            // t, t + 256, ..., the partial sums are added along each wavefront and then across wavefronts.
+            // A fixed order, though not the row's own: such a row agrees with the sequential sum to rounding,
+            // not to the bit.  The shares are of different rows, so the order in which they are taken is free.
+            __syncthreads();
+            const int n = __builtin_amdgcn_readfirstlane(nlong);
+            for (int k = 0; k < n; ++k) {
+                const int owner = __builtin_amdgcn_readfirstlane(long_owner[k]);
+                const int64_t l = uniform_i64(long_lo[k]), h = uniform_i64(long_hi[k]);
+                double s = 0.0;
+                for (int64_t p = l + tid; p < h; p += SPMV_T)
+                    s = s + prod[p - cs];
+                for (int d = 32; d > 0; d >>= 1)
+                    s = s + __shfl_down(s, d, 64);
+                if ((tid & 63) == 0)
+                    part[tid >> 6] = s;
+                __syncthreads();
+                if (tid == owner) {
+                    double t = part[0];
+                    for (int w = 1; w < SPMV_T / 64; ++w)
+                        t = t + part[w];
+                    acc = acc + t;
+                }
+                __syncthreads();
+            }
+        }
         __syncthreads();
     }
     if (r < nrows)

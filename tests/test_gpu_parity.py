@@ -127,6 +127,30 @@ def test_spmv_column_blocked_plan_is_bit_exact():
     assert np.array_equal(rt.spmv(A, dx).to_numpy(), orc.spmv(pos, crd, val, x))      # plan reused
 
 
+@pytest.mark.parametrize("acc", [False, True])
+def test_spmv_long_rows(acc):
+    """Rows of 127 nonzeros and fewer are summed by one lane in the checker's order (bit-exact); longer ones,
+    here up to 60,000 nonzeros and crossing many LDS passes, by the whole workgroup (fixed order, to rounding)."""
+    rng = np.random.default_rng(17)
+    m = 70_000
+    lens = rng.integers(0, 12, 3000)
+    for at, l in ((3, 127), (4, 128), (5, 129), (700, 2048), (701, 2049), (1500, 5000), (2999, 60_000), (2000, 300)):
+        lens[at] = l
+    pos = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    crd = np.concatenate([np.sort(rng.choice(m, l, replace=False)) for l in lens if l]).astype(np.int64)
+    val, x, y0 = rng.uniform(-1, 1, len(crd)), rng.uniform(-1, 1, m), rng.uniform(-1, 1, len(lens))
+    A = rt.CsrMatrix.from_arrays((len(lens), m), pos, crd, val)
+    y = rt.DeviceArray.from_numpy(y0) if acc else None
+    got = rt.spmv(A, rt.DeviceArray.from_numpy(x), y).to_numpy()
+    want = orc.spmv(pos, crd, val, x, y0 if acc else None)
+    short = lens < 128
+    assert np.array_equal(got[short], want[short])
+    bound = orc.spmv(pos, crd, np.abs(val), np.abs(x), np.abs(y0) if acc else None)
+    assert np.all(np.abs(got - want) <= RTOL * bound)
+    assert np.array_equal(rt.spmv(A, rt.DeviceArray.from_numpy(x), rt.DeviceArray.from_numpy(y0) if acc else None)
+                          .to_numpy(), got)                          # the same bits every time
+
+
 def test_spmv_edge_cases():
     # empty matrix rows, one very long row (longer than an LDS pass), trailing empty rows
     n, m = 600, 9000
@@ -139,7 +163,10 @@ def test_spmv_edge_cases():
     x = rng.uniform(-1, 1, m)
     A = rt.CsrMatrix.from_arrays((n, m), pos, crd, val)
     got = rt.spmv(A, rt.DeviceArray.from_numpy(x)).to_numpy()
-    assert np.array_equal(got, orc.spmv(pos, crd, val, x))
+    want = orc.spmv(pos, crd, val, x)
+    short = np.diff(pos) < 128           # longer rows are added by the whole workgroup, in another fixed order
+    assert np.array_equal(got[short], want[short])
+    assert np.all(np.abs(got - want) <= RTOL * orc.spmv(pos, crd, np.abs(val), np.abs(x)))
     Z = rt.CsrMatrix.from_arrays((3, 3), np.zeros(4, dtype=np.int64), np.zeros(0, dtype=np.int64), np.zeros(0))
     y = rt.spmv(Z, rt.DeviceArray.from_numpy(np.ones(3)), rt.DeviceArray.from_numpy(np.array([1.0, 2.0, 3.0])))
     assert y.to_numpy().tolist() == [1.0, 2.0, 3.0]
