@@ -27,6 +27,10 @@ FP64_MFMA_PEAK_TFLOPS = 78.6  # MI355X dense fp64 matrix, published
 # HBM bytes per SpMM product (all of its kernels) on the default workload, from rocprofv3 --pmc FETCH_SIZE (x 2.000)
 # and WRITE_SIZE (x 1.000), factors from a 1 GiB copy kernel; see profiles/spmm_kernels__spmm_zipf_500k_k64.txt
 SPMM_TRAFFIC_BYTES = int((436_260 * 2.000 + 272_815 * 1.000) * 1024)
+# the same two counters for the other workloads at their default sizes (per step; profiles/*.txt hold the tables)
+SPMV_TRAFFIC_BYTES = int((124_163 * 2.000 + 31_250 * 1.000) * 1024)            # four column-block passes
+SDDMM_TRAFFIC_BYTES = int((2_288_233 * 2.000 + 312_341 * 1.000) * 1024)        # kernel + transpose of D
+TRICOUNT_TRAFFIC_BYTES = int((20_131_202 * 2.000 + 37_655 * 1.000) * 1024)     # spgemm_masked_sum_kernel
 
 
 _T0 = time.perf_counter()
@@ -180,7 +184,8 @@ def bench_sddmm(rt, orc, gen, args):
         "config": {"workload": "sddmm_csr_zipf", "rows": n, "cols": n, "nnz": int(nnz), "inner": K, "seed": 2,
                    "index_bytes": ib},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (dev_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": alg_bytes / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "unit": "GB/s", "frac": alg_bytes / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": SDDMM_TRAFFIC_BYTES if (n, K) == (500_000, 64) else None,
                      "kernel": dom + " (+ transpose of D: the whole step is timed)",
                      "kernel_avg_ms": dom_ms, "algorithmic_bytes": int(alg_bytes)},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
@@ -220,7 +225,8 @@ def bench_spmv(rt, orc, gen, args):
         "config": {"workload": "spmv_csr_poisson", "rows": n, "cols": n, "nnz": int(nnz), "seed": 1, "index_bytes": ib,
                    "column_block_passes": passes},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": alg_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "unit": "GB/s", "frac": alg_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": SPMV_TRAFFIC_BYTES if n == 1_000_000 else None,
                      "kernel": dom, "kernel_avg_ms": dom_ms, "launches_per_step": passes,
                      "algorithmic_bytes": int(alg_bytes)},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
@@ -320,7 +326,8 @@ def bench_tricount(rt, orc, gen, args):
         "config": {"workload": "tricount_rmat", "scale": scale, "edge_factor": 16, "nnz_L": int(nnzL),
                    "products": nprod, "triangles": out["count"], "seed": 20},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": alg_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel": dom,
+                     "frac": alg_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": TRICOUNT_TRAFFIC_BYTES if scale == 20 else None, "kernel": dom,
                      "kernel_avg_ms": dom_ms, "algorithmic_bytes": int(alg_bytes)},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity,
     }
