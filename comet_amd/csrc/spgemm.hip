@@ -412,7 +412,9 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
 // ---------------------------------------------------------------------------
 constexpr int SG_CB_LOG = 14;
 constexpr int SG_CB = 1 << SG_CB_LOG;                                 // columns per block
-constexpr size_t SG_DENSE_LDS = (size_t)SG_CB * 8 + (size_t)SG_CB / 8;  // accumulators + bitmap
+constexpr int SG_EMIT = 8192;                                         // entries written out per turn of the emit
+constexpr size_t SG_DENSE_LDS = (size_t)SG_CB * 8 + (size_t)SG_CB / 8 + (size_t)SG_EMIT * 2;  // accumulators, bitmap,
+                                                                      // list of the columns being written out
 
 // products[i - row_begin] = sum over k in A_i of nnz(B_k); one wavefront per row
 __global__ __launch_bounds__(256) void spgemm_row_products(int64_t row_begin, int64_t row_end,
@@ -474,6 +476,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
     __shared__ int block_touched;
     double *acc = reinterpret_cast<double *>(sg_dyn_lds);
     uint32_t *bm = sg_dyn_lds + SG_CB * 2;
+    uint16_t *emit_col = reinterpret_cast<uint16_t *>(bm + SG_CB / 32);
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     for (int j = threadIdx.x; j < SG_CB; j += SG_T)
@@ -584,21 +587,32 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                 if (lane == 63)
                     wave_tot[wave] = inc;
                 __syncthreads();
-                int64_t o = off + (inc - mine);
+                int first = inc - mine;          // position of this lane's first column among the block's
                 int total = 0;
                 for (int w = 0; w < SG_WAVES; ++w) {
                     if (w < wave)
-                        o += wave_tot[w];
+                        first += wave_tot[w];
                     total += wave_tot[w];
                 }
+                total = __builtin_amdgcn_readfirstlane(total);
+                // The owner of a bitmap word knows where its columns go, but writing them from there would
+                // scatter every store over 64 cache lines.  So the columns are listed in LDS, SG_EMIT at a
+                // time, and then every lane writes the entry at its own place in the list: coalesced stores.
                 const int jbase = (int)threadIdx.x << 5;
-                while (word) {
-                    const int b = __ffs(word) - 1;
-                    word &= word - 1;
-                    Ccrd[o] = col0 + jbase + b;
-                    Cval[o] = acc[jbase + b];
-                    acc[jbase + b] = 0.0;
-                    ++o;
+                for (int c0 = 0; c0 < total; c0 += SG_EMIT) {
+                    int at = first;
+                    for (uint32_t w = word; w; w &= w - 1, ++at)
+                        if (at >= c0 && at < c0 + SG_EMIT)
+                            emit_col[at - c0] = (uint16_t)(jbase + __ffs(w) - 1);
+                    __syncthreads();
+                    const int n = total - c0 < SG_EMIT ? total - c0 : SG_EMIT;
+                    for (int q = threadIdx.x; q < n; q += SG_T) {
+                        const int j = emit_col[q];
+                        Ccrd[off + c0 + q] = col0 + j;
+                        Cval[off + c0 + q] = acc[j];
+                        acc[j] = 0.0;
+                    }
+                    __syncthreads();
                 }
                 if (threadIdx.x < SG_CB / 32)
                     bm[threadIdx.x] = 0;
