@@ -178,3 +178,113 @@ extern "C" double _mlir_ciface_comet_hip_tricount_f64_i64(int64_t ncols, comet_m
     (void)comet_hip_csr_destroy(l);
     return out;
 }
+
+// ---------------------------------------------------------------------------
+// The small host utilities every lowered program calls besides the kernels, so
+// that this library can be the only -shared-libs entry of a run: printing of
+// memrefs in the runtime's text form, the index sort, wall-clock time.
+// An unranked memref arrives as (rank, pointer to StridedMemRefType<T, rank>):
+// {T *allocated; T *aligned; int64 offset; int64 sizes[rank]; int64 strides[rank]}.
+// ---------------------------------------------------------------------------
+#include <sys/time.h>
+
+#include <algorithm>
+
+namespace {
+
+template <typename T>
+struct Unranked {
+    T *data;
+    int64_t offset;
+    const int64_t *sizes, *strides;
+    int64_t rank;
+    Unranked(int64_t r, void *desc) : rank(r)
+    {
+        char *p = static_cast<char *>(desc);
+        data = *reinterpret_cast<T **>(p + sizeof(T *));                 // the aligned pointer
+        offset = *reinterpret_cast<int64_t *>(p + 2 * sizeof(T *));
+        sizes = reinterpret_cast<const int64_t *>(p + 2 * sizeof(T *) + sizeof(int64_t));
+        strides = sizes + r;
+    }
+};
+
+void print_one(double v) { printf("%g,", v); }      // an ostream's default form: six significant digits
+void print_one(float v) { printf("%g,", (double)v); }
+void print_one(int64_t v) { printf("%lld,", (long long)v); }
+void print_one(int32_t v) { printf("%d,", v); }
+
+template <typename T>
+void print_dims(const T *base, int64_t dims_left, int64_t offset, const int64_t *sizes, const int64_t *strides)
+{
+    if (dims_left == 0) {
+        print_one(base[offset]);
+        return;
+    }
+    for (int64_t i = 0; i < sizes[0]; ++i)
+        print_dims(base, dims_left - 1, offset + i * strides[0], sizes + 1, strides + 1);
+}
+
+// include/comet/ExecutionEngine/RunnerUtils.h:232-266: nothing for an empty first dimension, else "data = ",
+// a line break, every element followed by a comma in row-major order of the strided view, a line break
+template <typename T>
+void print_memref(int64_t rank, void *desc)
+{
+    if (!desc || rank < 0)
+        return;
+    Unranked<T> m(rank, desc);
+    if (rank > 0 && m.sizes[0] <= 0)
+        return;
+    printf("data = \n");
+    print_dims(m.data, rank, m.offset, m.sizes, m.strides);
+    printf("\n");
+    fflush(stdout);
+}
+
+template <typename T>
+void sort_range(int64_t rank, void *desc, int64_t first, int64_t last)
+{
+    if (!desc || last <= first)
+        return;
+    Unranked<T> m(rank, desc);
+    std::sort(m.data + m.offset + first, m.data + m.offset + last);
+}
+
+}  // namespace
+
+// lib/ExecutionEngine/StatUtils.cpp:109-137
+extern "C" void comet_print_memref_f64(int64_t rank, void *ptr) { print_memref<double>(rank, ptr); }
+extern "C" void comet_print_memref_f32(int64_t rank, void *ptr) { print_memref<float>(rank, ptr); }
+extern "C" void comet_print_memref_i64(int64_t rank, void *ptr) { print_memref<int64_t>(rank, ptr); }
+extern "C" void comet_print_memref_i32(int64_t rank, void *ptr) { print_memref<int32_t>(rank, ptr); }
+extern "C" void comet_print_memref_index(int64_t rank, void *ptr) { print_memref<int64_t>(rank, ptr); }
+
+// lib/ExecutionEngine/SparseUtils.cpp:2610-2626: ascending sort of elements [first, last) of a 1-D memref
+extern "C" void comet_sort_index(int64_t rank, void *ptr, int64_t first, int64_t last)
+{
+    sort_range<int64_t>(rank, ptr, first, last);
+}
+extern "C" void comet_sort64(int64_t rank, void *ptr, int64_t first, int64_t last)
+{
+    sort_range<int64_t>(rank, ptr, first, last);
+}
+extern "C" void comet_sort32(int64_t rank, void *ptr, int64_t first, int64_t last)
+{
+    sort_range<int32_t>(rank, ptr, first, last);
+}
+
+// lib/ExecutionEngine/StatUtils.cpp:42-59.  Kernels here are asynchronous: the device is drained first, so that
+// the interval between two calls covers the work launched between them.
+extern "C" double getTime()
+{
+    if (is_initialised())
+        (void)comet_hip_sync();
+    struct timeval tp;
+    if (gettimeofday(&tp, nullptr) != 0)
+        fprintf(stderr, "Error returning time from gettimeofday\n");
+    return (double)tp.tv_sec + (double)tp.tv_usec * 1.0e-6;
+}
+
+extern "C" void printElapsedTime(double stime, double etime)
+{
+    fprintf(stdout, "ELAPSED_TIME = %lf\n", etime - stime);
+}

@@ -15,6 +15,7 @@ namespace comet {
 // library is ordered on it.
 hipStream_t stream();
 int ensure_init();
+bool is_initialised();     // has any call brought the device up yet
 int set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int num_cus();
 

@@ -64,6 +64,8 @@ static int do_init(int device)
     return COMET_HIP_OK;
 }
 
+bool is_initialised() { return g_inited; }
+
 int ensure_init()
 {
     std::lock_guard<std::mutex> lk(g_mu);

@@ -86,6 +86,16 @@ SIGNATURES = {
     "comet_hip_eltwise_csr_dense_csr": (_i64, [_i64, _i64, _i64, _int]),
     "comet_hip_sddmm_csr_f64": (_i64, [_i64, _i64, _i64, _i64, _i64, _i64]),
     "comet_hip_sddmm_csr_values_f64": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _i64]),
+    "comet_print_memref_f64": (None, [_i64, C.c_void_p]),
+    "comet_print_memref_f32": (None, [_i64, C.c_void_p]),
+    "comet_print_memref_i64": (None, [_i64, C.c_void_p]),
+    "comet_print_memref_i32": (None, [_i64, C.c_void_p]),
+    "comet_print_memref_index": (None, [_i64, C.c_void_p]),
+    "comet_sort_index": (None, [_i64, C.c_void_p, _i64, _i64]),
+    "comet_sort64": (None, [_i64, C.c_void_p, _i64, _i64]),
+    "comet_sort32": (None, [_i64, C.c_void_p, _i64, _i64]),
+    "getTime": (C.c_double, []),
+    "printElapsedTime": (None, [C.c_double, C.c_double]),
     "comet_hip_eltwise_csr_dense_dense": (_int, [_i64, _i64, _i64, _i64, _i64, _int]),
     "comet_hip_eltwise_dense_f64": (_int, [_i64, _i64, _i64, _i64, _int]),
     "comet_hip_mtx_read_csr": (_i64, [C.c_char_p, _int]),

@@ -356,6 +356,23 @@ void _mlir_ciface_comet_hip_spgemm_csr_fill_f64_i64(comet_memref_1d *Cpos, comet
 double _mlir_ciface_comet_hip_tricount_f64_i64(int64_t ncols, comet_memref_1d *pos, comet_memref_1d *crd,
                                                comet_memref_1d *val);
 
+/* ---- host utilities of the reference's runtime ----------------------------
+ * The names and argument lists lowered programs already call
+ * (lib/ExecutionEngine/StatUtils.cpp:42-59,109-137, SparseUtils.cpp:2610-2626), so that this library can
+ * stand alone behind -shared-libs.  An unranked memref is (rank, pointer to StridedMemRefType<T, rank>).
+ * Printing follows include/comet/ExecutionEngine/RunnerUtils.h:232-266 ("data = ", line break, every element
+ * and a comma, line break; nothing for an empty tensor).  getTime drains the device first. */
+void comet_print_memref_f64(int64_t rank, void *desc);
+void comet_print_memref_f32(int64_t rank, void *desc);
+void comet_print_memref_i64(int64_t rank, void *desc);
+void comet_print_memref_i32(int64_t rank, void *desc);
+void comet_print_memref_index(int64_t rank, void *desc);
+void comet_sort_index(int64_t rank, void *desc, int64_t first, int64_t last);
+void comet_sort64(int64_t rank, void *desc, int64_t first, int64_t last);
+void comet_sort32(int64_t rank, void *desc, int64_t first, int64_t last);
+double getTime(void);
+void printElapsedTime(double stime, double etime);
+
 #ifdef __cplusplus
 }
 #endif

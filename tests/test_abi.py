@@ -17,7 +17,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def _declared_symbols():
     text = open(os.path.join(ROOT, "include", "comet_hip_rt.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    names = re.findall(r"\b((?:comet_hip_|_mlir_ciface_comet_hip_|Hip)[A-Za-z0-9_]+)\s*\(", text)
+    names = re.findall(r"\b((?:comet_hip_|_mlir_ciface_comet_hip_|Hip|comet_print_memref_|comet_sort)[A-Za-z0-9_]+|"
+                       r"getTime|printElapsedTime)\s*\(", text)
     return sorted(set(names))
 
 
@@ -92,3 +93,56 @@ def test_ttgt_plan_rejects_non_gemm_expressions():
         rt.ttgt_plan("ab", "ab", "ab", {"a": 2, "b": 2})        # element-wise: label in A, B and C
     with pytest.raises(rt.CometHipError):
         rt.ttgt_plan("ab", "bc", "ac", {"a": 2, "b": 2, "c": 2}, which=99)
+
+
+def test_host_utilities_print_sort_and_time(tmp_path):
+    """comet_print_memref_*, comet_sort_* and the timers keep the reference's argument lists and text form
+    (include/comet/ExecutionEngine/RunnerUtils.h:232-266, lib/ExecutionEngine/StatUtils.cpp:42-59); they need
+    no GPU.  Run in a child process so that the C library's stdout can be captured."""
+    import subprocess, sys, textwrap
+    code = textwrap.dedent("""
+        import ctypes as C, numpy as np
+        from comet_amd import runtime as rt
+        L = rt.lib()
+        def desc(a, shape=None, strides=None, offset=0):
+            shape = list(a.shape if shape is None else shape)
+            strides = list((np.array(a.strides) // a.itemsize) if strides is None else strides)
+            n = len(shape)
+            class D(C.Structure):
+                _fields_ = [("alloc", C.c_void_p), ("aligned", C.c_void_p), ("offset", C.c_int64),
+                            ("sizes", C.c_int64 * n), ("strides", C.c_int64 * n)]
+            d = D(a.ctypes.data, a.ctypes.data, offset, (C.c_int64 * n)(*shape), (C.c_int64 * n)(*strides))
+            return n, d
+        keep = []
+        def call(fn, a, *extra, **kw):
+            n, d = desc(a, **kw); keep.append((a, d))
+            fn(n, C.byref(d), *extra)
+        call(L.comet_print_memref_f64, np.array([[4.08, 7.65], [0.1 + 0.2, 1e-7], [123456789.0, -0.0]]))
+        call(L.comet_print_memref_i64, np.array([0, 2, 4, 5], dtype=np.int64))
+        call(L.comet_print_memref_index, np.array([7], dtype=np.int64))
+        call(L.comet_print_memref_i32, np.array([[1, -2], [3, 4]], dtype=np.int32))
+        call(L.comet_print_memref_f32, np.array([1.5, 2.25], dtype=np.float32))
+        call(L.comet_print_memref_f64, np.zeros((0, 3)))                      # empty: prints nothing
+        base = np.arange(12, dtype=np.float64)
+        call(L.comet_print_memref_f64, base, shape=[2, 3], strides=[1, 4], offset=1)      # a strided view
+        v = np.array([9, 3, 7, 1, 8, 2], dtype=np.int64)
+        call(L.comet_sort_index, v, 1, 5)
+        call(L.comet_print_memref_i64, v)
+        w = np.array([5, 4, 3, 2, 1], dtype=np.int32)
+        call(L.comet_sort32, w, 0, 5)
+        call(L.comet_print_memref_i32, w)
+        t0 = L.getTime(); t1 = L.getTime()
+        assert 0.0 <= t1 - t0 < 5.0 and t0 > 1.0e9
+        L.printElapsedTime(1.0, 3.5)
+    """)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    assert r.returncode == 0, r.stderr
+    assert r.stdout == ("data = \n4.08,7.65,0.3,1e-07,1.23457e+08,-0,\n"
+                        "data = \n0,2,4,5,\n"
+                        "data = \n7,\n"
+                        "data = \n1,-2,3,4,\n"
+                        "data = \n1.5,2.25,\n"
+                        "data = \n1,5,9,2,6,10,\n"
+                        "data = \n9,1,3,7,8,2,\n"
+                        "data = \n1,2,3,4,5,\n"
+                        "ELAPSED_TIME = 2.500000\n")
