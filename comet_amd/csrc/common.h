@@ -14,6 +14,11 @@ namespace comet {
 // One process-wide stream at default priority; every kernel and copy of the
 // library is ordered on it.
 hipStream_t stream();
+// A second stream for a kernel that may run beside the one on stream(): aux_fork makes it wait for what
+// stream() holds so far, aux_join makes stream() wait for it.  Both streams have the default priority.
+hipStream_t aux_stream();
+int aux_fork();
+int aux_join();
 int ensure_init();
 bool is_initialised();     // has any call brought the device up yet
 int set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
@@ -104,8 +109,10 @@ Csr *csr_transposed_copy(const Csr *a);    // new unregistered struct holding th
 // Records an event pair around a kernel launch when profiling is on.
 struct KernelTimer {
     explicit KernelTimer(const char *name);
+    KernelTimer(const char *name, hipStream_t on);      // for a launch on aux_stream()
     ~KernelTimer();
     int slot;
+    hipStream_t on;
 };
 
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }

@@ -20,10 +20,27 @@ static bool g_inited = false;
 static int g_device = 0;
 static int g_num_cus = 0;
 static hipStream_t g_stream = nullptr;
+static hipStream_t g_aux = nullptr;
+static hipEvent_t g_fork = nullptr, g_join = nullptr;
 static thread_local std::string g_last_error;
 static std::unordered_set<Csr *> g_live;
 
 hipStream_t stream() { return g_stream; }
+hipStream_t aux_stream() { return g_aux; }
+
+int aux_fork()
+{
+    COMET_HIPCHK(hipEventRecord(g_fork, g_stream));
+    COMET_HIPCHK(hipStreamWaitEvent(g_aux, g_fork, 0));
+    return COMET_HIP_OK;
+}
+
+int aux_join()
+{
+    COMET_HIPCHK(hipEventRecord(g_join, g_aux));
+    COMET_HIPCHK(hipStreamWaitEvent(g_stream, g_join, 0));
+    return COMET_HIP_OK;
+}
 int num_cus() { return g_num_cus; }
 
 int set_error(int code, const char *fmt, ...)
@@ -59,6 +76,9 @@ static int do_init(int device)
                          device, prop.gcnArchName);
     g_num_cus = prop.multiProcessorCount;
     COMET_HIPCHK(hipStreamCreate(&g_stream));
+    COMET_HIPCHK(hipStreamCreate(&g_aux));
+    COMET_HIPCHK(hipEventCreateWithFlags(&g_fork, hipEventDisableTiming));
+    COMET_HIPCHK(hipEventCreateWithFlags(&g_join, hipEventDisableTiming));
     g_device = device;
     g_inited = true;
     return COMET_HIP_OK;
@@ -212,6 +232,7 @@ static void drain_pending()
     if (g_pending.empty())
         return;
     (void)hipStreamSynchronize(g_stream);
+    (void)hipStreamSynchronize(g_aux);
     for (auto &p : g_pending) {
         float ms = 0.f;
         if (hipEventElapsedTime(&ms, p.a, p.b) == hipSuccess) {
@@ -225,7 +246,9 @@ static void drain_pending()
     g_pending.clear();
 }
 
-KernelTimer::KernelTimer(const char *name) : slot(-1)
+KernelTimer::KernelTimer(const char *name) : KernelTimer(name, g_stream) {}
+
+KernelTimer::KernelTimer(const char *name, hipStream_t s) : slot(-1), on(s)
 {
     if (!g_prof_on)
         return;
@@ -235,7 +258,7 @@ KernelTimer::KernelTimer(const char *name) : slot(-1)
     p.name = name;
     p.a = take_event();
     p.b = take_event();
-    (void)hipEventRecord(p.a, g_stream);
+    (void)hipEventRecord(p.a, on);
     g_pending.push_back(p);
     slot = (int)g_pending.size() - 1;
 }
@@ -243,7 +266,7 @@ KernelTimer::KernelTimer(const char *name) : slot(-1)
 KernelTimer::~KernelTimer()
 {
     if (slot >= 0)
-        (void)hipEventRecord(g_pending[slot].b, g_stream);
+        (void)hipEventRecord(g_pending[slot].b, on);
 }
 
 // ------------------------------------------------------------------ kernels
@@ -485,8 +508,13 @@ int comet_hip_finalize(void)
     g_live.clear();
     for (Workspace *w : g_workspaces)
         w->release();
+    (void)hipStreamSynchronize(g_aux);
+    (void)hipEventDestroy(g_fork);
+    (void)hipEventDestroy(g_join);
+    (void)hipStreamDestroy(g_aux);
     (void)hipStreamDestroy(g_stream);
-    g_stream = nullptr;
+    g_stream = g_aux = nullptr;
+    g_fork = g_join = nullptr;
     g_inited = false;
     return COMET_HIP_OK;
 }

@@ -152,6 +152,25 @@ __device__ inline int64_t draw_row(unsigned long long *ticket, int64_t first, in
     return ((int64_t)hi << 32) | (uint32_t)lo;
 }
 
+// Two kernels that share one list, one taking rows from its front and one from its back until they meet: the
+// ticket word holds both counts (front in the low half, back in the high half), so the value an atomic add
+// returns tells the claimant how many rows were taken from either end before it, and a claim is good while
+// their sum is below n.  Every row is claimed once, and the meeting point settles where both kernels finish.
+__device__ inline int64_t draw_front(unsigned long long *ticket, int64_t n, int64_t *slot)
+{
+    if (threadIdx.x == 0) {
+        const unsigned long long old = atomicAdd(ticket, 1ull);
+        const int64_t f = (int64_t)(old & 0xffffffffull), b = (int64_t)(old >> 32);
+        *slot = f + b < n ? f : n;
+    }
+    __syncthreads();
+    const int64_t r = *slot;
+    __syncthreads();
+    const int lo = __builtin_amdgcn_readfirstlane((int)(r & 0xffffffff));
+    const int hi = __builtin_amdgcn_readfirstlane((int)(r >> 32));
+    return ((int64_t)hi << 32) | (uint32_t)lo;
+}
+
 // Semiring operators of C = A @(reduce, mult) B.  The codes are the C ABI's.
 enum { SR_PLUS = 0, SR_MIN = 1, SR_MAX = 2, SR_ANY = 3 };
 __device__ inline double semiring_mult(int op, double a, double b)
@@ -639,6 +658,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_masked_sum_kernel(
     const double *__restrict__ Bval, const int64_t *__restrict__ Mpos, const int32_t *__restrict__ Mcrd,
     int logW, uint32_t *__restrict__ gbm, unsigned long long *ticket, RowList list, double *__restrict__ rowsum)
 {
+    // takes the rows with work from the heavy end of the list; spgemm_masked_sum_small_kernel comes from the other
     __shared__ int64_t row_slot;
     __shared__ double wave_part[SG_WAVES];
     uint32_t *bm;
@@ -655,7 +675,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_masked_sum_kernel(
     __syncthreads();
     int64_t t_first, t_end;
     list_range(list, 2, &t_first, &t_end);
-    int64_t tk = draw_row(ticket, t_first, &row_slot);
+    int64_t tk = draw_front(ticket, t_end, &row_slot);
     while (tk < t_end) {
         const int64_t i = list.rows[tk];      // rows outside the list keep the zero the host put there
         const int64_t as = Apos[i], ae = Apos[i + 1];
@@ -688,7 +708,140 @@ __global__ __launch_bounds__(SG_T) void spgemm_masked_sum_kernel(
         for (int64_t t = ms + threadIdx.x; t < me; t += SG_T)
             atomicAnd(&bm[ad.word(Mcrd[t])], 0u);
         }   // work
-        tk = draw_row(ticket, t_first, &row_slot);     // its barriers also close this row's bitmap clean-up
+        tk = draw_front(ticket, t_end, &row_slot);     // its barriers also close this row's bitmap clean-up
+    }
+}
+
+// ---------------------------------------------------------------------------
+// The same sum for rows with few products: one wavefront per row, no workgroup
+// barrier anywhere.  A row of a thousand products spends more time on the
+// ticket, bitmap and reduction barriers of the kernel above than on its
+// products.  Here the mask row goes into a small hash table in LDS that belongs
+// to the wavefront; the neighbours of the row are taken one at a time and the
+// lanes walk along that neighbour's row of B, probing the table.  A mask row too
+// long for the table is searched by bisection in memory instead.
+// ---------------------------------------------------------------------------
+constexpr int SM_WAVES = 4;                    // wavefronts per workgroup
+constexpr int SM_SLOTS = 256;                  // hash slots per wavefront (1 KB: four such workgroups fit a CU beside
+                                               // one workgroup of the kernel above and its 132 KB bitmap)
+constexpr int SM_MASK_MAX = 96;                // longest mask row that goes into the table
+
+__device__ inline int sm_hash(int j) { return (int)(((uint32_t)j * 2654435761u) >> 24) & (SM_SLOTS - 1); }
+
+__global__ __launch_bounds__(SM_WAVES * 64) void spgemm_masked_sum_small_kernel(
+    const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd, const double *__restrict__ Aval,
+    const int64_t *__restrict__ Bpos, const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval,
+    const int64_t *__restrict__ Mpos, const int32_t *__restrict__ Mcrd, unsigned long long *ticket, RowList list,
+    double *__restrict__ rowsum)
+{
+    __shared__ int table[SM_WAVES][SM_SLOTS];
+    const int lane = threadIdx.x & 63;
+    int *tab = table[threadIdx.x >> 6];
+    for (int s = lane; s < SM_SLOTS; s += 64)
+        tab[s] = -1;
+    int64_t t_first, t_end;
+    list_range(list, 2, &t_first, &t_end);
+    for (;;) {
+        // a row from the light end of the list (see draw_front)
+        unsigned long long drawn = 0;
+        if (lane == 0)
+            drawn = atomicAdd(ticket, 1ull << 32);
+        const int64_t f = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(drawn & 0xffffffffu));
+        const int64_t b = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(drawn >> 32));
+        if (f + b >= t_end)
+            break;
+        const int64_t tk = t_end - 1 - b;
+        const int64_t i = list.rows[tk];
+        const int64_t as = Apos[i], ae = Apos[i + 1], ms = Mpos[i], me = Mpos[i + 1];
+        if (as == ae || ms == me)
+            continue;               // rowsum[i] keeps the zero the host put there
+        const bool hashed = me - ms <= SM_MASK_MAX;
+        if (hashed)
+            for (int64_t t = ms + lane; t < me; t += 64) {
+                const int j = Mcrd[t];
+                int h = sm_hash(j);
+                while (atomicCAS(&tab[h], -1, j) != -1)
+                    h = (h + 1) & (SM_SLOTS - 1);
+            }
+        double part = 0.0;
+        for (int64_t p0 = as; p0 < ae; p0 += 64) {
+            // up to 64 neighbours at a time: lane l holds neighbour p0 + l, its value and its row of B
+            const int cnt = (int)(ae - p0 < 64 ? ae - p0 : 64);
+            int64_t bs = 0, be = 0;
+            double a = 0.0;
+            if (lane < cnt) {
+                const int k = Acrd[p0 + lane];
+                bs = Bpos[k];
+                be = Bpos[k + 1];
+                a = Aval[p0 + lane];
+            }
+            auto probe = [&](int j, int64_t q, double al) {
+                bool hit = false;
+                if (hashed) {
+                    int h = sm_hash(j);
+                    for (int v = tab[h]; v != -1; v = tab[h]) {
+                        if (v == j) {
+                            hit = true;
+                            break;
+                        }
+                        h = (h + 1) & (SM_SLOTS - 1);
+                    }
+                } else {
+                    int64_t lo = ms, hi = me;
+                    while (lo < hi) {
+                        const int64_t mid = (lo + hi) >> 1;
+                        if (Mcrd[mid] < j)
+                            lo = mid + 1;
+                        else
+                            hi = mid;
+                    }
+                    hit = lo < me && Mcrd[lo] == j;
+                }
+                if (hit)
+                    part += al * Bval[q];
+            };
+            // rows of B with 64 entries and more take the whole wavefront, one at a time; shorter ones (a row
+            // of the lower triangle holds 15 entries on average) go to the four 16-lane quarters, four at a time.
+            // (Laying all products of the row end to end, lane x taking product x after a bisection over the
+            // running totals, fills every lane and was slower: 11.0 against 10.0 ms - the kernel is bound by
+            // instructions per product, not by idle lanes.)
+            unsigned long long big = __ballot(be - bs >= 64);
+            unsigned long long todo = __ballot(bs < be && be - bs < 64);
+            while (big) {
+                const int l = __builtin_ctzll(big);
+                big &= big - 1;
+                const int64_t s = readlane_i64(bs, l), e = readlane_i64(be, l);
+                const double al = readlane_d(a, l);
+                for (int64_t q = s + lane; q < e; q += 64)
+                    probe(Bcrd[q], q, al);
+            }
+            const int quarter = lane >> 4, sub = lane & 15;
+            while (todo) {
+                int pick = -1;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int l = todo ? __builtin_ctzll(todo) : -1;
+                    todo = todo ? (todo & (todo - 1)) : 0;
+                    pick = quarter == g ? l : pick;
+                }
+                const int src = pick < 0 ? lane : pick;
+                const int64_t s = ((int64_t)__shfl((int)(bs >> 32), src, 64) << 32) |
+                                  (uint32_t)__shfl((int)(bs & 0xffffffff), src, 64);
+                const int64_t e = ((int64_t)__shfl((int)(be >> 32), src, 64) << 32) |
+                                  (uint32_t)__shfl((int)(be & 0xffffffff), src, 64);
+                const double al = __hiloint2double(__shfl(__double2hiint(a), src, 64),
+                                                   __shfl(__double2loint(a), src, 64));
+                if (pick >= 0)
+                    for (int64_t q = s + sub; q < e; q += 16)
+                        probe(Bcrd[q], q, al);
+            }
+        }
+        part = wave_sum_f64(part);
+        if (lane == 0)
+            rowsum[i] = part;
+        if (hashed)
+            for (int s = lane; s < SM_SLOTS; s += 64)
+                tab[s] = -1;
     }
 }
 
@@ -1133,6 +1286,15 @@ extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, d
     COMET_CHK(sg_row_list(a, b, 0, a->nrows, SG_NO_DENSE, &list));
     COMET_HIPCHK(hipMemsetAsync(rowsum, 0, sizeof(double) * (size_t)a->nrows, stream()));
     const dim3 grid((unsigned)g.groups), block(SG_T);
+    // Two kernels side by side, the second on the auxiliary stream: a workgroup per row from the heavy end of
+    // the list, a wavefront per row from the light end, until they meet.  A row of a thousand products costs
+    // the first kernel more in barriers than in products; a row of a million would keep one wavefront of the
+    // second busy for a millisecond.  Triangle count of the scale-20 R-MAT graph: 29.2 ms with the first
+    // kernel alone, 22.1 ms one after the other with a fixed split at 65536 products, 17.6 ms side by side with
+    // the best fixed split (49152 products), 18.9 ms with the two ends meeting by themselves (the difference is
+    // the last wavefront-rows near the meeting point; looking at the ticket word before drawing from it, to keep
+    // the wavefronts away from those rows, or drawing 16 rows at a time, costs more on that one word than it saves).
+    COMET_CHK(aux_fork());
     if (g.lds) {
         COMET_CHK(sg_allow_lds(spgemm_masked_sum_kernel<true>, g.lds_bytes));
         KernelTimer t("spgemm_masked_sum");
@@ -1145,7 +1307,14 @@ extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, d
             a->nrows, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m->pos, m->crd, g.logW, gbm,
             (unsigned long long *)g_sg.ticket.ptr, list, rowsum);
     }
+    {   // eight workgroups of four wavefronts per CU: four fit beside the kernel above, the rest follow it
+        KernelTimer t("spgemm_masked_sum_small", aux_stream());
+        spgemm_masked_sum_small_kernel<<<dim3((unsigned)(num_cus() * 8)), dim3(SM_WAVES * 64), 0, aux_stream()>>>(
+            a->pos, a->crd, a->val, b->pos, b->crd, b->val, m->pos, m->crd,
+            (unsigned long long *)g_sg.ticket.ptr, list, rowsum);
+    }
     COMET_HIPCHK(hipGetLastError());
+    COMET_CHK(aux_join());
     return reduce_sum_device(rowsum, a->nrows, out);
 }
 
