@@ -725,6 +725,7 @@ constexpr int SM_WAVES = 4;                    // wavefronts per workgroup
 constexpr int SM_SLOTS = 256;                  // hash slots per wavefront (1 KB: four such workgroups fit a CU beside
                                                // one workgroup of the kernel above and its 132 KB bitmap)
 constexpr int SM_MASK_MAX = 96;                // longest mask row that goes into the table
+constexpr int SM_BATCH = 16;                   // rows a wavefront claims at a time in the lighter half of the list
 
 __device__ inline int sm_hash(int j) { return (int)(((uint32_t)j * 2654435761u) >> 24) & (SM_SLOTS - 1); }
 
@@ -741,16 +742,28 @@ __global__ __launch_bounds__(SM_WAVES * 64) void spgemm_masked_sum_small_kernel(
         tab[s] = -1;
     int64_t t_first, t_end;
     list_range(list, 2, &t_first, &t_end);
+    int take = SM_BATCH;
+    int64_t mine_next = 0, mine_end = 0;     // the rows t_end - 1 - b, b in [mine_next, mine_end), are this wavefront's
     for (;;) {
-        // a row from the light end of the list (see draw_front)
-        unsigned long long drawn = 0;
-        if (lane == 0)
-            drawn = atomicAdd(ticket, 1ull << 32);
-        const int64_t f = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(drawn & 0xffffffffu));
-        const int64_t b = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(drawn >> 32));
-        if (f + b >= t_end)
-            break;
-        const int64_t tk = t_end - 1 - b;
+        if (mine_next == mine_end) {
+            // rows from the light end of the list (see draw_front): SM_BATCH at a time in the lighter half of the
+            // list - rows of a few thousand products at most, and 600,000 draws on one word are what the L2 does
+            // in the time the whole count takes - a quarter of that in the next quarter, then one by one: a
+            // batch of rows near the meeting point would keep one wavefront for long
+            unsigned long long drawn = 0;
+            if (lane == 0)
+                drawn = atomicAdd(ticket, (unsigned long long)take << 32);
+            const int64_t f = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(drawn & 0xffffffffu));
+            const int64_t b = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(drawn >> 32));
+            if (f + b >= t_end)
+                break;
+            mine_next = b;
+            mine_end = b + take < t_end - f ? b + take : t_end - f;     // what the front had not reached
+            const int64_t taken = b + take;
+            take = taken < t_end / 2 ? SM_BATCH : taken < t_end - t_end / 4 ? SM_BATCH / 4 : 1;
+        }
+        const int64_t tk = t_end - 1 - mine_next;
+        ++mine_next;
         const int64_t i = list.rows[tk];
         const int64_t as = Apos[i], ae = Apos[i + 1], ms = Mpos[i], me = Mpos[i + 1];
         if (as == ae || ms == me)
