@@ -483,6 +483,95 @@ __global__ void spgemm_block_pointers(int64_t nrows, const int64_t *__restrict__
     }
 }
 
+// Adds the products of one slice per lane (entries [lo, hi) of a row of B, all inside the column block that
+// starts at col0, times a) to the block's accumulators and bitmap in LDS.  Returns whether this wavefront
+// added anything.
+__device__ __forceinline__ int dense_add_slices(int64_t lo, int64_t hi, double a, int col0, int lane,
+                                                const int32_t *__restrict__ Bcrd,
+                                                const double *__restrict__ Bval, double *acc, uint32_t *bm)
+{
+    // Long slices take the whole wavefront, one at a time; short ones (a slice of one block often holds a
+    // dozen entries) are handed to the four 16-lane quarters, eight at a time.  A wavefront runs its loads
+    // one after the other (there is room for one workgroup per CU, so nobody else hides the latency):
+    // every turn below therefore issues all of its loads, up to four of each array per lane, before the
+    // first LDS operation waits for one.  Lanes beyond the end of a slice load entry 0 again and add nothing.
+    unsigned long long big = __ballot(hi - lo >= 32);
+    unsigned long long todo = __ballot(lo < hi && hi - lo < 32);
+    const int touched = (big | todo) != 0;
+    while (big) {
+        const int t = __builtin_ctzll(big);
+        big &= big - 1;
+        const int64_t s = readlane_i64(lo, t), e = readlane_i64(hi, t);
+        const double at = readlane_d(a, t);
+        for (int64_t q = s + lane; q < e; q += 256) {
+            const bool p1 = q + 64 < e, p2 = q + 128 < e, p3 = q + 192 < e;
+            const int64_t q1 = p1 ? q + 64 : 0, q2 = p2 ? q + 128 : 0, q3 = p3 ? q + 192 : 0;
+            const int j0 = Bcrd[q] - col0, j1 = Bcrd[q1] - col0, j2 = Bcrd[q2] - col0, j3 = Bcrd[q3] - col0;
+            const double v0 = Bval[q], v1 = Bval[q1], v2 = Bval[q2], v3 = Bval[q3];
+            atomicOr(&bm[j0 >> 5], 1u << (j0 & 31));
+            __hip_atomic_fetch_add(&acc[j0], at * v0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (p1) {
+                atomicOr(&bm[j1 >> 5], 1u << (j1 & 31));
+                __hip_atomic_fetch_add(&acc[j1], at * v1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+            if (p2) {
+                atomicOr(&bm[j2 >> 5], 1u << (j2 & 31));
+                __hip_atomic_fetch_add(&acc[j2], at * v2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+            if (p3) {
+                atomicOr(&bm[j3 >> 5], 1u << (j3 & 31));
+                __hip_atomic_fetch_add(&acc[j3], at * v3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        }
+    }
+    const int quarter = lane >> 4, sub = lane & 15;
+    while (todo) {
+        int pick[2] = {-1, -1};
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int t = todo ? __builtin_ctzll(todo) : -1;
+                todo = todo ? (todo & (todo - 1)) : 0;
+                pick[u] = quarter == g ? t : pick[u];
+            }
+        }
+        int64_t q[4];
+        bool ok[4];
+        double at[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int src = pick[u] < 0 ? lane : pick[u];
+            const int64_t s = ((int64_t)__shfl((int)(lo >> 32), src, 64) << 32) |
+                              (uint32_t)__shfl((int)(lo & 0xffffffff), src, 64);
+            const int64_t e = ((int64_t)__shfl((int)(hi >> 32), src, 64) << 32) |
+                              (uint32_t)__shfl((int)(hi & 0xffffffff), src, 64);
+            at[u] = __hiloint2double(__shfl(__double2hiint(a), src, 64), __shfl(__double2loint(a), src, 64));
+            ok[2 * u] = pick[u] >= 0 && s + sub < e;             // a short slice has fewer than 32 entries:
+            ok[2 * u + 1] = pick[u] >= 0 && s + sub + 16 < e;    // two per lane cover it
+            q[2 * u] = ok[2 * u] ? s + sub : 0;
+            q[2 * u + 1] = ok[2 * u + 1] ? s + sub + 16 : 0;
+        }
+        int j[4];
+        double v[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+            j[x] = Bcrd[q[x]] - col0;
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+            v[x] = Bval[q[x]];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            if (ok[x]) {
+                atomicOr(&bm[j[x] >> 5], 1u << (j[x] & 31));
+                __hip_atomic_fetch_add(&acc[j[x]], at[x >> 1] * v[x], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        }
+    }
+    return touched;
+}
+
 __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
     int64_t row_begin, int64_t row_end, const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd,
     const double *__restrict__ Aval, const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval,
@@ -514,10 +603,34 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
         const int64_t as = Apos[i], ae = Apos[i + 1];
         if (as != ae) {
             int64_t off = Cpos[i] - out0;
+            // A row of at most one entry of A per lane (nearly all rows) keeps its entries in registers over
+            // the blocks: the end of a slice in one block is its start in the next, so a block costs one
+            // pointer load per lane, and that load is issued a block ahead.
+            const int held = __builtin_amdgcn_readfirstlane((int)(ae - as <= SG_T));
+            int64_t h_lo = 0, h_hi = 0;
+            double h_a = 0.0;
+            const int64_t *h_bp = nullptr;
+            if (held) {
+                const int64_t p = as + wave + (int64_t)lane * SG_WAVES;
+                if (p < ae) {
+                    h_bp = blkptr + (int64_t)Acrd[p] * (nblk + 1);
+                    h_lo = h_bp[0];
+                    h_hi = h_bp[1];
+                    h_a = Aval[p];
+                }
+            }
             for (int cb = 0; cb < nblk; ++cb) {
                 const int col0 = cb << SG_CB_LOG;
                 int touched = 0;     // did this wavefront add anything to the block
-                for (int64_t base = as + wave; base < ae; base += (int64_t)SG_WAVES * 64) {
+                if (held) {
+                    int64_t next = h_hi;
+                    if (h_bp && cb + 1 < nblk)
+                        next = h_bp[cb + 2];
+                    touched = dense_add_slices(h_lo, h_hi, h_a, col0, lane, Bcrd, Bval, acc, bm);
+                    h_lo = h_hi;
+                    h_hi = next;
+                }
+                for (int64_t base = as + wave; !held && base < ae; base += (int64_t)SG_WAVES * 64) {
                     const int64_t left = (ae - base + SG_WAVES - 1) / SG_WAVES;
                     const int cnt = (int)(left < 64 ? left : 64);
                     int64_t lo = 0, hi = 0;
@@ -529,62 +642,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                         hi = bp[1];
                         a = Aval[p];
                     }
-                    // long slices take the whole wavefront, one at a time; short ones (a slice of one block
-                    // often holds a dozen entries) are handed to the four 16-lane quarters, four at a time
-                    unsigned long long big = __ballot(hi - lo >= 32);
-                    unsigned long long todo = __ballot(lo < hi && hi - lo < 32);
-                    touched |= (big | todo) != 0;
-                    while (big) {
-                        const int t = __builtin_ctzll(big);
-                        big &= big - 1;
-                        const int64_t s = readlane_i64(lo, t), e = readlane_i64(hi, t);
-                        const double at = readlane_d(a, t);
-                        int64_t q = s + lane;
-                        for (; q + 192 < e; q += 256) {      // four loads in flight per lane
-                            const int j0 = Bcrd[q] - col0, j1 = Bcrd[q + 64] - col0;
-                            const int j2 = Bcrd[q + 128] - col0, j3 = Bcrd[q + 192] - col0;
-                            const double v0 = Bval[q], v1 = Bval[q + 64], v2 = Bval[q + 128], v3 = Bval[q + 192];
-                            atomicOr(&bm[j0 >> 5], 1u << (j0 & 31));
-                            atomicOr(&bm[j1 >> 5], 1u << (j1 & 31));
-                            atomicOr(&bm[j2 >> 5], 1u << (j2 & 31));
-                            atomicOr(&bm[j3 >> 5], 1u << (j3 & 31));
-                            __hip_atomic_fetch_add(&acc[j0], at * v0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                            __hip_atomic_fetch_add(&acc[j1], at * v1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                            __hip_atomic_fetch_add(&acc[j2], at * v2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                            __hip_atomic_fetch_add(&acc[j3], at * v3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                        }
-                        for (; q < e; q += 64) {
-                            const int j = Bcrd[q] - col0;
-                            atomicOr(&bm[j >> 5], 1u << (j & 31));
-                            __hip_atomic_fetch_add(&acc[j], at * Bval[q], __ATOMIC_RELAXED,
-                                                   __HIP_MEMORY_SCOPE_WORKGROUP);
-                        }
-                    }
-                    const int quarter = lane >> 4, sub = lane & 15;
-                    while (todo) {
-                        int pick = -1;
-#pragma unroll
-                        for (int g = 0; g < 4; ++g) {
-                            const int t = todo ? __builtin_ctzll(todo) : -1;
-                            todo = todo ? (todo & (todo - 1)) : 0;
-                            pick = quarter == g ? t : pick;
-                        }
-                        const int src = pick < 0 ? lane : pick;
-                        const int64_t s = ((int64_t)__shfl((int)(lo >> 32), src, 64) << 32) |
-                                          (uint32_t)__shfl((int)(lo & 0xffffffff), src, 64);
-                        const int64_t e = ((int64_t)__shfl((int)(hi >> 32), src, 64) << 32) |
-                                          (uint32_t)__shfl((int)(hi & 0xffffffff), src, 64);
-                        const double at = __hiloint2double(__shfl(__double2hiint(a), src, 64),
-                                                           __shfl(__double2loint(a), src, 64));
-                        if (pick >= 0) {
-                            for (int64_t q = s + sub; q < e; q += 16) {
-                                const int j = Bcrd[q] - col0;
-                                atomicOr(&bm[j >> 5], 1u << (j & 31));
-                                __hip_atomic_fetch_add(&acc[j], at * Bval[q], __ATOMIC_RELAXED,
-                                                       __HIP_MEMORY_SCOPE_WORKGROUP);
-                            }
-                        }
-                    }
+                    touched |= dense_add_slices(lo, hi, a, col0, lane, Bcrd, Bval, acc, bm);
                 }
                 // one barrier tells everybody whether the block received anything (an LDS flag that the
                 // emitting path resets); the value is made scalar so that the branch on it is uniform,
