@@ -140,13 +140,42 @@ __device__ inline void list_range(const RowList &l, int part, int64_t *first, in
     *first = part == 1 ? l.bounds[0] : 0;
     *end = part == 0 ? l.bounds[0] : l.bounds[1];
 }
+// A workgroup barrier that orders LDS traffic only.  __syncthreads() also makes every wavefront wait until its
+// global stores have been acknowledged, a microsecond that a kernel whose stores nobody reads back (the rows
+// of C going out) need not spend at every barrier.
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+// Inclusive prefix sum over the 64 lanes of a wavefront through the cross-lane data path of the vector ALU
+// (shifts within a row of 16 lanes, then the last lane of a row broadcast to the rows after it): no LDS round
+// trips, unlike a shuffle.  A lane whose source lies outside its row, or whose row is masked, adds 0.
+__device__ __forceinline__ int wave_inclusive_scan(int v)
+{
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);    // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);    // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);    // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);    // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);    // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);    // row_bcast:31 into rows 2 and 3
+    return v;
+}
+template <bool LDS_ONLY = false>
 __device__ inline int64_t draw_row(unsigned long long *ticket, int64_t first, int64_t *slot)
 {
     if (threadIdx.x == 0)
         *slot = first + (int64_t)atomicAdd(ticket, 1ull);
-    __syncthreads();
+    if (LDS_ONLY)
+        lds_barrier();
+    else
+        __syncthreads();
     const int64_t r = *slot;
-    __syncthreads();
+    if (LDS_ONLY)
+        lds_barrier();
+    else
+        __syncthreads();
     const int lo = __builtin_amdgcn_readfirstlane((int)(r & 0xffffffff));
     const int hi = __builtin_amdgcn_readfirstlane((int)(r >> 32));
     return ((int64_t)hi << 32) | (uint32_t)lo;
@@ -486,86 +515,91 @@ __global__ void spgemm_block_pointers(int64_t nrows, const int64_t *__restrict__
 // Adds the products of one slice per lane (entries [lo, hi) of a row of B, all inside the column block that
 // starts at col0, times a) to the block's accumulators and bitmap in LDS.  Returns whether this wavefront
 // added anything.
+constexpr int SG_SHORT = 32;                      // slices shorter than this are taken by 16 lanes, the others by 64
+constexpr int SG_SHORT_LOADS = SG_SHORT / 16;     // entries of a short slice per lane
+constexpr int SG_LONG_LOADS = 4;                  // entries of a long slice per lane and turn
+
 __device__ __forceinline__ int dense_add_slices(int64_t lo, int64_t hi, double a, int col0, int lane,
                                                 const int32_t *__restrict__ Bcrd,
                                                 const double *__restrict__ Bval, double *acc, uint32_t *bm)
 {
     // Long slices take the whole wavefront, one at a time; short ones (a slice of one block often holds a
-    // dozen entries) are handed to the four 16-lane quarters, eight at a time.  A wavefront runs its loads
-    // one after the other (there is room for one workgroup per CU, so nobody else hides the latency):
-    // every turn below therefore issues all of its loads, up to four of each array per lane, before the
-    // first LDS operation waits for one.  Lanes beyond the end of a slice load entry 0 again and add nothing.
-    unsigned long long big = __ballot(hi - lo >= 32);
-    unsigned long long todo = __ballot(lo < hi && hi - lo < 32);
+    // dozen entries) are handed to the four 16-lane quarters, four at a time.  A wavefront runs its turns
+    // one after the other (there is room for one workgroup per CU, so nobody else hides the latency), and
+    // a turn costs about one trip to memory: so every turn issues all of its loads before the first LDS
+    // operation waits for one, and a load that no lane needs is skipped.  Measured on A*A of an R-MAT
+    // graph of scale 20: two loads per lane and turn of a long slice instead of four, +18 % time in this
+    // kernel, eight +2 %; two long slices or eight short ones per turn, +2..8 %; slices of up to 4 or 8
+    // entries left to their own lane (64 slices per turn, but every lane a cache line of its own), +4..6 %;
+    // the 16-lane path up to 64 or 128 entries, +1..5 %.
+    unsigned long long big = __ballot(hi - lo >= SG_SHORT);
+    unsigned long long todo = __ballot(lo < hi && hi - lo < SG_SHORT);
     const int touched = (big | todo) != 0;
-    while (big) {
+    while (big) {               // one long slice per turn, up to SG_LONG_LOADS entries of it per lane
         const int t = __builtin_ctzll(big);
         big &= big - 1;
-        const int64_t s = readlane_i64(lo, t), e = readlane_i64(hi, t);
+        const int64_t s = readlane_i64(lo, t), len = readlane_i64(hi, t) - s;
         const double at = readlane_d(a, t);
-        for (int64_t q = s + lane; q < e; q += 256) {
-            const bool p1 = q + 64 < e, p2 = q + 128 < e, p3 = q + 192 < e;
-            const int64_t q1 = p1 ? q + 64 : 0, q2 = p2 ? q + 128 : 0, q3 = p3 ? q + 192 : 0;
-            const int j0 = Bcrd[q] - col0, j1 = Bcrd[q1] - col0, j2 = Bcrd[q2] - col0, j3 = Bcrd[q3] - col0;
-            const double v0 = Bval[q], v1 = Bval[q1], v2 = Bval[q2], v3 = Bval[q3];
-            atomicOr(&bm[j0 >> 5], 1u << (j0 & 31));
-            __hip_atomic_fetch_add(&acc[j0], at * v0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            if (p1) {
-                atomicOr(&bm[j1 >> 5], 1u << (j1 & 31));
-                __hip_atomic_fetch_add(&acc[j1], at * v1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        for (int64_t o = lane; o < len; o += 64 * SG_LONG_LOADS) {
+            int64_t q[SG_LONG_LOADS];
+            bool ok[SG_LONG_LOADS];
+#pragma unroll
+            for (int x = 0; x < SG_LONG_LOADS; ++x) {
+                ok[x] = o + 64 * x < len;
+                q[x] = ok[x] ? s + o + 64 * x : 0;
             }
-            if (p2) {
-                atomicOr(&bm[j2 >> 5], 1u << (j2 & 31));
-                __hip_atomic_fetch_add(&acc[j2], at * v2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            }
-            if (p3) {
-                atomicOr(&bm[j3 >> 5], 1u << (j3 & 31));
-                __hip_atomic_fetch_add(&acc[j3], at * v3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            int j[SG_LONG_LOADS];
+            double v[SG_LONG_LOADS];
+#pragma unroll
+            for (int x = 0; x < SG_LONG_LOADS; ++x)
+                j[x] = (ok[x] ? Bcrd[q[x]] : 0) - col0;
+#pragma unroll
+            for (int x = 0; x < SG_LONG_LOADS; ++x)
+                v[x] = (ok[x] ? Bval[q[x]] : 0.0);
+#pragma unroll
+            for (int x = 0; x < SG_LONG_LOADS; ++x) {
+                if (ok[x]) {
+                    atomicOr(&bm[j[x] >> 5], 1u << (j[x] & 31));
+                    __hip_atomic_fetch_add(&acc[j[x]], at * v[x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
             }
         }
     }
     const int quarter = lane >> 4, sub = lane & 15;
-    while (todo) {
-        int pick[2] = {-1, -1};
+    while (todo) {              // four short slices per turn, one to a quarter, SG_SHORT_LOADS entries per lane
+        int pick = -1;
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int t = todo ? __builtin_ctzll(todo) : -1;
-                todo = todo ? (todo & (todo - 1)) : 0;
-                pick[u] = quarter == g ? t : pick[u];
-            }
+        for (int g = 0; g < 4; ++g) {
+            const int t = todo ? __builtin_ctzll(todo) : -1;
+            todo = todo ? (todo & (todo - 1)) : 0;
+            pick = quarter == g ? t : pick;
         }
-        int64_t q[4];
-        bool ok[4];
-        double at[2];
+        const int src = pick < 0 ? lane : pick;
+        const int64_t s = ((int64_t)__shfl((int)(lo >> 32), src, 64) << 32) |
+                          (uint32_t)__shfl((int)(lo & 0xffffffff), src, 64);
+        const int64_t e = ((int64_t)__shfl((int)(hi >> 32), src, 64) << 32) |
+                          (uint32_t)__shfl((int)(hi & 0xffffffff), src, 64);
+        const double at = __hiloint2double(__shfl(__double2hiint(a), src, 64), __shfl(__double2loint(a), src, 64));
+        int64_t q[SG_SHORT_LOADS];
+        bool ok[SG_SHORT_LOADS];
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int src = pick[u] < 0 ? lane : pick[u];
-            const int64_t s = ((int64_t)__shfl((int)(lo >> 32), src, 64) << 32) |
-                              (uint32_t)__shfl((int)(lo & 0xffffffff), src, 64);
-            const int64_t e = ((int64_t)__shfl((int)(hi >> 32), src, 64) << 32) |
-                              (uint32_t)__shfl((int)(hi & 0xffffffff), src, 64);
-            at[u] = __hiloint2double(__shfl(__double2hiint(a), src, 64), __shfl(__double2loint(a), src, 64));
-            ok[2 * u] = pick[u] >= 0 && s + sub < e;             // a short slice has fewer than 32 entries:
-            ok[2 * u + 1] = pick[u] >= 0 && s + sub + 16 < e;    // two per lane cover it
-            q[2 * u] = ok[2 * u] ? s + sub : 0;
-            q[2 * u + 1] = ok[2 * u + 1] ? s + sub + 16 : 0;
+        for (int x = 0; x < SG_SHORT_LOADS; ++x) {
+            ok[x] = pick >= 0 && s + sub + 16 * x < e;
+            q[x] = ok[x] ? s + sub + 16 * x : 0;
         }
-        int j[4];
-        double v[4];
+        int j[SG_SHORT_LOADS];
+        double v[SG_SHORT_LOADS];
 #pragma unroll
-        for (int x = 0; x < 4; ++x)
-            j[x] = Bcrd[q[x]] - col0;
+        for (int x = 0; x < SG_SHORT_LOADS; ++x)
+            j[x] = (ok[x] ? Bcrd[q[x]] : 0) - col0;
 #pragma unroll
-        for (int x = 0; x < 4; ++x)
-            v[x] = Bval[q[x]];
+        for (int x = 0; x < SG_SHORT_LOADS; ++x)
+            v[x] = (ok[x] ? Bval[q[x]] : 0.0);
 #pragma unroll
-        for (int x = 0; x < 4; ++x) {
+        for (int x = 0; x < SG_SHORT_LOADS; ++x) {
             if (ok[x]) {
                 atomicOr(&bm[j[x] >> 5], 1u << (j[x] & 31));
-                __hip_atomic_fetch_add(&acc[j[x]], at[x >> 1] * v[x], __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(&acc[j[x]], at * v[x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
         }
     }
@@ -593,11 +627,11 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
         bm[threadIdx.x] = 0;
     if (threadIdx.x == 0)
         block_touched = 0;
-    __syncthreads();
+    lds_barrier();
     const int64_t out0 = Cpos[row_begin];
     int64_t t_first, t_end;
     list_range(list, 0, &t_first, &t_end);
-    int64_t t = draw_row(ticket, t_first, &row_slot);
+    int64_t t = draw_row<true>(ticket, t_first, &row_slot);
     while (t < t_end) {
         const int64_t i = row_begin + list.rows[t];
         const int64_t as = Apos[i], ae = Apos[i + 1];
@@ -626,7 +660,8 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                     int64_t next = h_hi;
                     if (h_bp && cb + 1 < nblk)
                         next = h_bp[cb + 2];
-                    touched = dense_add_slices(h_lo, h_hi, h_a, col0, lane, Bcrd, Bval, acc, bm);
+                    touched = dense_add_slices(h_lo, h_hi, h_a, col0, lane, Bcrd, Bval, acc, bm
+                                               );
                     h_lo = h_hi;
                     h_hi = next;
                 }
@@ -642,46 +677,52 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                         hi = bp[1];
                         a = Aval[p];
                     }
-                    touched |= dense_add_slices(lo, hi, a, col0, lane, Bcrd, Bval, acc, bm);
+                    touched |= dense_add_slices(lo, hi, a, col0, lane, Bcrd, Bval, acc, bm
+                                                );
                 }
                 // one barrier tells everybody whether the block received anything (an LDS flag that the
                 // emitting path resets); the value is made scalar so that the branch on it is uniform,
                 // because the block body below holds barriers
                 if (touched && lane == 0)
                     block_touched = 1;
-                __syncthreads();
+                lds_barrier();
                 const int any = __builtin_amdgcn_readfirstlane(block_touched);
                 if (any) {
-                // emit this block: lane t < 512 owns bitmap word t, i.e. 32 consecutive columns
-                uint32_t word = threadIdx.x < SG_CB / 32 ? bm[threadIdx.x] : 0u;
-                const int mine = __popc(word);
-                int inc = mine;
-                for (int d = 1; d < 64; d <<= 1) {
-                    const int o = __shfl_up(inc, d, 64);
-                    if (lane >= d)
-                        inc += o;
-                }
+                // Emit this block.  Thread t owns the columns [8t, 8t + 8) and [8192 + 8t, 8192 + 8t + 8): one
+                // byte from each half of the bitmap, so that the dense low columns of a half (the columns of a
+                // power-law graph thin out with the number of set bits of the id) are spread over all the
+                // wavefronts.  The counts of the two bytes are scanned together, packed into one word.
+                static_assert(SG_T * 16 == SG_CB && SG_WAVES <= 64, "one byte of each half of the bitmap per thread");
+                const uint8_t *bm8 = reinterpret_cast<const uint8_t *>(bm);
+                const uint32_t bits_a = bm8[threadIdx.x], bits_b = bm8[SG_CB / 16 + threadIdx.x];
+                const int mine = __popc(bits_a) | (__popc(bits_b) << 16);
+                const int inc = wave_inclusive_scan(mine);
                 if (lane == 63)
                     wave_tot[wave] = inc;
-                __syncthreads();
-                int first = inc - mine;          // position of this lane's first column among the block's
-                int total = 0;
-                for (int w = 0; w < SG_WAVES; ++w) {
-                    if (w < wave)
-                        first += wave_tot[w];
-                    total += wave_tot[w];
-                }
-                total = __builtin_amdgcn_readfirstlane(total);
-                // The owner of a bitmap word knows where its columns go, but writing them from there would
-                // scatter every store over 64 cache lines.  So the columns are listed in LDS, SG_EMIT at a
-                // time, and then every lane writes the entry at its own place in the list: coalesced stores.
-                const int jbase = (int)threadIdx.x << 5;
+                lds_barrier();
+                const int tots = wave_inclusive_scan(lane < SG_WAVES ? wave_tot[lane] : 0);
+                const int all = __builtin_amdgcn_readlane(tots, SG_WAVES - 1);
+                const int before = (wave ? __builtin_amdgcn_readlane(tots, wave - 1) : 0) + inc - mine;
+                const int total_a = all & 0xffff, total = total_a + (all >> 16);
+                const int first_a = before & 0xffff, first_b = total_a + (before >> 16);
+                if (threadIdx.x < SG_CB / 32)      // everybody has read its bytes: the bitmap is clean for the
+                    bm[threadIdx.x] = 0;           // next block, which nobody enters before the barrier below
+                if (threadIdx.x == 0)
+                    block_touched = 0;
+                // The owner of a byte knows where its columns go, but writing them from there would scatter
+                // every store over 64 cache lines.  So the columns are listed in LDS, SG_EMIT at a time, and
+                // then every lane writes the entry at its own place in the list: coalesced stores.
+                const int jbase = (int)threadIdx.x << 3;
                 for (int c0 = 0; c0 < total; c0 += SG_EMIT) {
-                    int at = first;
-                    for (uint32_t w = word; w; w &= w - 1, ++at)
-                        if (at >= c0 && at < c0 + SG_EMIT)
-                            emit_col[at - c0] = (uint16_t)(jbase + __ffs(w) - 1);
-                    __syncthreads();
+                    int at = first_a - c0;
+                    for (uint32_t w = bits_a; w; w &= w - 1, ++at)
+                        if (at >= 0 && at < SG_EMIT)
+                            emit_col[at] = (uint16_t)(jbase + __ffs(w) - 1);
+                    at = first_b - c0;
+                    for (uint32_t w = bits_b; w; w &= w - 1, ++at)
+                        if (at >= 0 && at < SG_EMIT)
+                            emit_col[at] = (uint16_t)(SG_CB / 2 + jbase + __ffs(w) - 1);
+                    lds_barrier();
                     const int n = total - c0 < SG_EMIT ? total - c0 : SG_EMIT;
                     for (int q = threadIdx.x; q < n; q += SG_T) {
                         const int j = emit_col[q];
@@ -689,18 +730,13 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                         Cval[off + c0 + q] = acc[j];
                         acc[j] = 0.0;
                     }
-                    __syncthreads();
+                    lds_barrier();
                 }
-                if (threadIdx.x < SG_CB / 32)
-                    bm[threadIdx.x] = 0;
-                if (threadIdx.x == 0)
-                    block_touched = 0;
                 off += total;
-                __syncthreads();
                 }   // block received products
             }
         }
-        t = draw_row(ticket, t_first, &row_slot);
+        t = draw_row<true>(ticket, t_first, &row_slot);
     }
 }
 
