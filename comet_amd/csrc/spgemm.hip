@@ -63,8 +63,12 @@ struct BmAddr {
 // one at a time (entry p goes to wavefront p mod 16), because in a sorted row
 // the neighbours with long rows sit next to each other and would otherwise all
 // land on one wavefront.  A wavefront fetches 64 of its entries at once (one per
-// lane), then walks them one by one with all lanes striding over B_k, four
-// loads in flight per lane.
+// lane).  Rows of B with at least FEP_SHORT entries are then walked one by one
+// with all lanes striding over B_k; shorter ones go to the four 16-lane quarters,
+// four rows at a time.  A wavefront runs these turns one after the other and a
+// turn costs about one trip to memory, so each turn issues all of its loads (up
+// to four per lane; a load no lane needs is skipped) before the visitor runs.
+constexpr int FEP_SHORT = 32, FEP_SHORT_LOADS = FEP_SHORT / 16, FEP_LONG_LOADS = 4;
 template <bool VALUES, typename F>
 __device__ inline void for_each_product(int64_t as, int64_t ae, const int32_t *__restrict__ Acrd,
                                         const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
@@ -72,6 +76,7 @@ __device__ inline void for_each_product(int64_t as, int64_t ae, const int32_t *_
 {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int quarter = lane >> 4, sub = lane & 15;
     for (int64_t base = as + wave; base < ae; base += (int64_t)SG_WAVES * 64) {
         const int64_t left = (ae - base + SG_WAVES - 1) / SG_WAVES;     // my entries from here on
         const int cnt = (int)(left < 64 ? left : 64);
@@ -85,20 +90,85 @@ __device__ inline void for_each_product(int64_t as, int64_t ae, const int32_t *_
             if (VALUES)
                 a = Aval[p];
         }
-        for (int t = 0; t < cnt; ++t) {
-            const int64_t s = readlane_i64(bs, t), e = readlane_i64(be, t);
+        unsigned long long big = __ballot(be - bs >= FEP_SHORT);
+        unsigned long long todo = __ballot(bs < be && be - bs < FEP_SHORT);
+        while (big) {
+            const int t = __builtin_ctzll(big);
+            big &= big - 1;
+            const int64_t s = readlane_i64(bs, t), len = readlane_i64(be, t) - s;
             const double at = VALUES ? readlane_d(a, t) : 0.0;
             const int64_t p = base + (int64_t)t * SG_WAVES;
-            int64_t q = s + lane;
-            for (; q + 192 < e; q += 256) {
-                const int j0 = Bcrd[q], j1 = Bcrd[q + 64], j2 = Bcrd[q + 128], j3 = Bcrd[q + 192];
-                f(j0, q, at, p, s);
-                f(j1, q + 64, at, p, s);
-                f(j2, q + 128, at, p, s);
-                f(j3, q + 192, at, p, s);
+            int64_t o = lane;
+            if (len >= 64 * FEP_LONG_LOADS) {
+                // Turns in which every lane has all its entries: straight-line code, so that the visitors'
+                // LDS operations are issued together as well, and the loads of the next turn are in flight
+                // while the visitor works on this one.
+                int j[FEP_LONG_LOADS];
+#pragma unroll
+                for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                    j[x] = Bcrd[s + o + 64 * x];
+                for (int64_t full = 64 * FEP_LONG_LOADS; full + 64 * FEP_LONG_LOADS <= len;
+                     full += 64 * FEP_LONG_LOADS) {
+                    int jn[FEP_LONG_LOADS];
+#pragma unroll
+                    for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                        jn[x] = Bcrd[s + o + 64 * (FEP_LONG_LOADS + x)];
+#pragma unroll
+                    for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                        f(j[x], s + o + 64 * x, at, p, s);
+#pragma unroll
+                    for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                        j[x] = jn[x];
+                    o += 64 * FEP_LONG_LOADS;
+                }
+#pragma unroll
+                for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                    f(j[x], s + o + 64 * x, at, p, s);
+                o += 64 * FEP_LONG_LOADS;
             }
-            for (; q < e; q += 64)
-                f(Bcrd[q], q, at, p, s);
+            if (o < len) {          // the rest of the row: fewer than 64 * FEP_LONG_LOADS entries
+                bool ok[FEP_LONG_LOADS];
+                int j[FEP_LONG_LOADS];
+#pragma unroll
+                for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                    ok[x] = o + 64 * x < len;
+#pragma unroll
+                for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                    j[x] = ok[x] ? Bcrd[s + o + 64 * x] : 0;
+#pragma unroll
+                for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                    if (ok[x])
+                        f(j[x], s + o + 64 * x, at, p, s);
+            }
+        }
+        while (todo) {
+            int pick = -1;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int t = todo ? __builtin_ctzll(todo) : -1;
+                todo = todo ? (todo & (todo - 1)) : 0;
+                pick = quarter == g ? t : pick;
+            }
+            const int src = pick < 0 ? lane : pick;
+            const int64_t s = ((int64_t)__shfl((int)(bs >> 32), src, 64) << 32) |
+                              (uint32_t)__shfl((int)(bs & 0xffffffff), src, 64);
+            const int64_t e = ((int64_t)__shfl((int)(be >> 32), src, 64) << 32) |
+                              (uint32_t)__shfl((int)(be & 0xffffffff), src, 64);
+            const double at =
+                VALUES ? __hiloint2double(__shfl(__double2hiint(a), src, 64), __shfl(__double2loint(a), src, 64)) : 0.0;
+            const int64_t p = base + (int64_t)src * SG_WAVES;
+            bool ok[FEP_SHORT_LOADS];
+            int j[FEP_SHORT_LOADS];
+#pragma unroll
+            for (int x = 0; x < FEP_SHORT_LOADS; ++x)
+                ok[x] = pick >= 0 && s + sub + 16 * x < e;
+#pragma unroll
+            for (int x = 0; x < FEP_SHORT_LOADS; ++x)
+                j[x] = ok[x] ? Bcrd[s + sub + 16 * x] : 0;
+#pragma unroll
+            for (int x = 0; x < FEP_SHORT_LOADS; ++x)
+                if (ok[x])
+                    f(j[x], s + sub + 16 * x, at, p, s);
         }
     }
 }
