@@ -610,7 +610,47 @@ __device__ __forceinline__ int dense_add_slices(int64_t lo, int64_t hi, double a
         big &= big - 1;
         const int64_t s = readlane_i64(lo, t), len = readlane_i64(hi, t) - s;
         const double at = readlane_d(a, t);
-        for (int64_t o = lane; o < len; o += 64 * SG_LONG_LOADS) {
+        int64_t o = lane;
+        if (len >= 64 * SG_LONG_LOADS) {
+            // turns in which every lane has all its entries run without predicates, and the loads of the next
+            // such turn are in flight while this one's products go into LDS
+            int j[SG_LONG_LOADS];
+            double v[SG_LONG_LOADS];
+#pragma unroll
+            for (int x = 0; x < SG_LONG_LOADS; ++x)
+                j[x] = Bcrd[s + o + 64 * x] - col0;
+#pragma unroll
+            for (int x = 0; x < SG_LONG_LOADS; ++x)
+                v[x] = Bval[s + o + 64 * x];
+            for (int64_t full = 64 * SG_LONG_LOADS; full + 64 * SG_LONG_LOADS <= len; full += 64 * SG_LONG_LOADS) {
+                int jn[SG_LONG_LOADS];
+                double vn[SG_LONG_LOADS];
+#pragma unroll
+                for (int x = 0; x < SG_LONG_LOADS; ++x)
+                    jn[x] = Bcrd[s + o + 64 * (SG_LONG_LOADS + x)] - col0;
+#pragma unroll
+                for (int x = 0; x < SG_LONG_LOADS; ++x)
+                    vn[x] = Bval[s + o + 64 * (SG_LONG_LOADS + x)];
+#pragma unroll
+                for (int x = 0; x < SG_LONG_LOADS; ++x) {
+                    atomicOr(&bm[j[x] >> 5], 1u << (j[x] & 31));
+                    __hip_atomic_fetch_add(&acc[j[x]], at * v[x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+#pragma unroll
+                for (int x = 0; x < SG_LONG_LOADS; ++x) {
+                    j[x] = jn[x];
+                    v[x] = vn[x];
+                }
+                o += 64 * SG_LONG_LOADS;
+            }
+#pragma unroll
+            for (int x = 0; x < SG_LONG_LOADS; ++x) {
+                atomicOr(&bm[j[x] >> 5], 1u << (j[x] & 31));
+                __hip_atomic_fetch_add(&acc[j[x]], at * v[x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+            o += 64 * SG_LONG_LOADS;
+        }
+        if (o < len) {
             int64_t q[SG_LONG_LOADS];
             bool ok[SG_LONG_LOADS];
 #pragma unroll
