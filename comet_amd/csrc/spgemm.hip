@@ -530,8 +530,9 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
 // ---------------------------------------------------------------------------
 constexpr int SG_CB_LOG = 14;
 constexpr int SG_CB = 1 << SG_CB_LOG;                                 // columns per block
+typedef uint16_t emit_t;                                              // a column of the block being written out
 constexpr int SG_EMIT = 8192;                                         // entries written out per turn of the emit
-constexpr size_t SG_DENSE_LDS = (size_t)SG_CB * 8 + (size_t)SG_CB / 8 + (size_t)SG_EMIT * 2;  // accumulators, bitmap,
+constexpr size_t SG_DENSE_LDS = (size_t)SG_CB * 8 + (size_t)SG_CB / 8 + (size_t)SG_EMIT * sizeof(emit_t);  // accumulators, bitmap,
                                                                       // list of the columns being written out
 
 // products[i - row_begin] = sum over k in A_i of nnz(B_k); one wavefront per row
@@ -728,7 +729,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
     __shared__ int block_touched;
     double *acc = reinterpret_cast<double *>(sg_dyn_lds);
     uint32_t *bm = sg_dyn_lds + SG_CB * 2;
-    uint16_t *emit_col = reinterpret_cast<uint16_t *>(bm + SG_CB / 32);
+    emit_t *emit_col = reinterpret_cast<emit_t *>(bm + SG_CB / 32);
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     for (int j = threadIdx.x; j < SG_CB; j += SG_T)
@@ -823,15 +824,31 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                 // every store over 64 cache lines.  So the columns are listed in LDS, SG_EMIT at a time, and
                 // then every lane writes the entry at its own place in the list: coalesced stores.
                 const int jbase = (int)threadIdx.x << 3;
+                if (total <= SG_EMIT) {         // the usual case: the whole block fits the list
+                    int at = first_a;
+                    for (uint32_t w = bits_a; w; w &= w - 1, ++at)
+                        emit_col[at] = (emit_t)(jbase + __ffs(w) - 1);
+                    at = first_b;
+                    for (uint32_t w = bits_b; w; w &= w - 1, ++at)
+                        emit_col[at] = (emit_t)(SG_CB / 2 + jbase + __ffs(w) - 1);
+                    lds_barrier();
+                    for (int q = threadIdx.x; q < total; q += SG_T) {
+                        const int j = emit_col[q];
+                        Ccrd[off + q] = col0 + j;
+                        Cval[off + q] = acc[j];
+                        acc[j] = 0.0;
+                    }
+                    lds_barrier();
+                } else {
                 for (int c0 = 0; c0 < total; c0 += SG_EMIT) {
                     int at = first_a - c0;
                     for (uint32_t w = bits_a; w; w &= w - 1, ++at)
                         if (at >= 0 && at < SG_EMIT)
-                            emit_col[at] = (uint16_t)(jbase + __ffs(w) - 1);
+                            emit_col[at] = (emit_t)(jbase + __ffs(w) - 1);
                     at = first_b - c0;
                     for (uint32_t w = bits_b; w; w &= w - 1, ++at)
                         if (at >= 0 && at < SG_EMIT)
-                            emit_col[at] = (uint16_t)(SG_CB / 2 + jbase + __ffs(w) - 1);
+                            emit_col[at] = (emit_t)(SG_CB / 2 + jbase + __ffs(w) - 1);
                     lds_barrier();
                     const int n = total - c0 < SG_EMIT ? total - c0 : SG_EMIT;
                     for (int q = threadIdx.x; q < n; q += SG_T) {
@@ -841,6 +858,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                         acc[j] = 0.0;
                     }
                     lds_barrier();
+                }
                 }
                 off += total;
                 }   // block received products
