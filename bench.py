@@ -389,7 +389,7 @@ def bench_spgemm(rt, orc, gen, args):
     alg_bytes = nnzA * (8 + ib) + (n + 1) * ib + nnzC * (8 + ib) + 8 * (n + 1)
     sym_ms = kt["spgemm_symbolic"]["avg_ms"] * kt["spgemm_symbolic"]["launches"] / args.steps
     num_ms = sum(kt[k]["avg_ms"] * kt[k]["launches"] for k in
-                 ("spgemm_numeric", "spgemm_numeric_dense", "spgemm_row_products", "radix_sort_pairs") if k in kt) / args.steps
+                 ("spgemm_numeric", "spgemm_numeric_dense", "spgemm_numeric_span", "spgemm_row_products", "radix_sort_pairs") if k in kt) / args.steps
     # sum of all values is a size-independent invariant: sum(C) = sum_k colsum(A)[k] * rowsum(A)[k]
     rowsum = np.add.reduceat(val, pos[:-1][np.diff(pos) > 0])
     rs = np.zeros(n)
@@ -440,7 +440,7 @@ def bench_spgemm(rt, orc, gen, args):
                    "seed": 20},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / ((sym_ms + num_ms) * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": alg_bytes / ((sym_ms + num_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": None, "kernel": "spgemm_symbolic + spgemm_numeric + spgemm_numeric_dense",
+                     "traffic": None, "kernel": "spgemm_symbolic + spgemm_numeric + spgemm_numeric_dense + spgemm_numeric_span",
                      "kernel_avg_ms": sym_ms + num_ms,
                      "symbolic_ms": sym_ms, "numeric_ms": num_ms, "algorithmic_bytes": int(alg_bytes)},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity,

@@ -202,13 +202,15 @@ __device__ inline double wave_sum_f64(double v)
 // rows that take milliseconds start first instead of forming the tail.
 struct RowList {
     const int32_t *rows;       // row - row_begin, by descending number of products
-    const int64_t *bounds;     // [0] rows with >= dense_threshold products, [1] rows with any product
+    const int64_t *bounds;     // [0] rows with >= dense_threshold products, [1] rows with any product,
+                               // [2] rows with >= wide_threshold products (a prefix of [0])
 };
 __device__ inline void list_range(const RowList &l, int part, int64_t *first, int64_t *end)
 {
-    // part 0: the heavy rows, 1: the others that have products, 2: both
-    *first = part == 1 ? l.bounds[0] : 0;
-    *end = part == 0 ? l.bounds[0] : l.bounds[1];
+    // part 0: the heavy rows, 1: the others that have products, 2: both, 3: the widest of the heavy rows,
+    // 4: the heavy rows that are not among the widest
+    *first = part == 1 ? l.bounds[0] : part == 4 ? l.bounds[2] : 0;
+    *end = part == 0 || part == 4 ? l.bounds[0] : part == 3 ? l.bounds[2] : l.bounds[1];
 }
 // A workgroup barrier that orders LDS traffic only.  __syncthreads() also makes every wavefront wait until its
 // global stores have been acknowledged, a microsecond that a kernel whose stores nobody reads back (the rows
@@ -583,16 +585,32 @@ __global__ void spgemm_block_pointers(int64_t nrows, const int64_t *__restrict__
     }
 }
 
-// Adds the products of one slice per lane (entries [lo, hi) of a row of B, all inside the column block that
-// starts at col0, times a) to the block's accumulators and bitmap in LDS.  Returns whether this wavefront
-// added anything.
+// One barrier tells every wavefront of the workgroup whether any of them had work in this visit.  The answer is
+// made scalar, so that a branch on it is uniform (the branches taken on it hold barriers).  Three flags take
+// turns: a wavefront may be a whole visit ahead of the slowest one, which is still to read this visit's flag
+// when the fast one raises the next; the flag of the visit after that is cleared here, before the barrier,
+// when everybody has long read its last use (they all came through the previous visit's barrier since).
+__device__ __forceinline__ int visit_flag(int *flags, int visit, int touched, int lane)
+{
+    if (threadIdx.x == 0)
+        flags[visit == 2 ? 0 : visit + 1] = 0;
+    if (touched && lane == 0)
+        flags[visit] = 1;
+    lds_barrier();
+    return __builtin_amdgcn_readfirstlane(flags[visit]);
+}
+
+// Visits the products of one slice per lane: f(j, x) for the entries [lo, hi) of a row of B (the part of it inside
+// the column block or blocks being swept), j the column and x = a times the entry's value (0 without VALUES,
+// when the value array is not read).  Returns whether this wavefront had anything to visit.
 constexpr int SG_SHORT = 32;                      // slices shorter than this are taken by 16 lanes, the others by 64
 constexpr int SG_SHORT_LOADS = SG_SHORT / 16;     // entries of a short slice per lane
 constexpr int SG_LONG_LOADS = 4;                  // entries of a long slice per lane and turn
 
-__device__ __forceinline__ int dense_add_slices(int64_t lo, int64_t hi, double a, int col0, int lane,
-                                                const int32_t *__restrict__ Bcrd,
-                                                const double *__restrict__ Bval, double *acc, uint32_t *bm)
+template <bool VALUES, typename F>
+__device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double a, int lane,
+                                                  const int32_t *__restrict__ Bcrd,
+                                                  const double *__restrict__ Bval, F f)
 {
     // Long slices take the whole wavefront, one at a time; short ones (a slice of one block often holds a
     // dozen entries) are handed to the four 16-lane quarters, four at a time.  A wavefront runs its turns
@@ -619,23 +637,22 @@ __device__ __forceinline__ int dense_add_slices(int64_t lo, int64_t hi, double a
             double v[SG_LONG_LOADS];
 #pragma unroll
             for (int x = 0; x < SG_LONG_LOADS; ++x)
-                j[x] = Bcrd[s + o + 64 * x] - col0;
+                j[x] = Bcrd[s + o + 64 * x];
 #pragma unroll
             for (int x = 0; x < SG_LONG_LOADS; ++x)
-                v[x] = Bval[s + o + 64 * x];
+                v[x] = VALUES ? Bval[s + o + 64 * x] : 0.0;
             for (int64_t full = 64 * SG_LONG_LOADS; full + 64 * SG_LONG_LOADS <= len; full += 64 * SG_LONG_LOADS) {
                 int jn[SG_LONG_LOADS];
                 double vn[SG_LONG_LOADS];
 #pragma unroll
                 for (int x = 0; x < SG_LONG_LOADS; ++x)
-                    jn[x] = Bcrd[s + o + 64 * (SG_LONG_LOADS + x)] - col0;
+                    jn[x] = Bcrd[s + o + 64 * (SG_LONG_LOADS + x)];
 #pragma unroll
                 for (int x = 0; x < SG_LONG_LOADS; ++x)
-                    vn[x] = Bval[s + o + 64 * (SG_LONG_LOADS + x)];
+                    vn[x] = VALUES ? Bval[s + o + 64 * (SG_LONG_LOADS + x)] : 0.0;
 #pragma unroll
                 for (int x = 0; x < SG_LONG_LOADS; ++x) {
-                    atomicOr(&bm[j[x] >> 5], 1u << (j[x] & 31));
-                    __hip_atomic_fetch_add(&acc[j[x]], at * v[x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    f(j[x], at * v[x]);
                 }
 #pragma unroll
                 for (int x = 0; x < SG_LONG_LOADS; ++x) {
@@ -646,8 +663,7 @@ __device__ __forceinline__ int dense_add_slices(int64_t lo, int64_t hi, double a
             }
 #pragma unroll
             for (int x = 0; x < SG_LONG_LOADS; ++x) {
-                atomicOr(&bm[j[x] >> 5], 1u << (j[x] & 31));
-                __hip_atomic_fetch_add(&acc[j[x]], at * v[x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                f(j[x], at * v[x]);
             }
             o += 64 * SG_LONG_LOADS;
         }
@@ -663,15 +679,14 @@ __device__ __forceinline__ int dense_add_slices(int64_t lo, int64_t hi, double a
             double v[SG_LONG_LOADS];
 #pragma unroll
             for (int x = 0; x < SG_LONG_LOADS; ++x)
-                j[x] = (ok[x] ? Bcrd[q[x]] : 0) - col0;
+                j[x] = (ok[x] ? Bcrd[q[x]] : 0);
 #pragma unroll
             for (int x = 0; x < SG_LONG_LOADS; ++x)
-                v[x] = (ok[x] ? Bval[q[x]] : 0.0);
+                v[x] = (VALUES && ok[x] ? Bval[q[x]] : 0.0);
 #pragma unroll
             for (int x = 0; x < SG_LONG_LOADS; ++x) {
                 if (ok[x]) {
-                    atomicOr(&bm[j[x] >> 5], 1u << (j[x] & 31));
-                    __hip_atomic_fetch_add(&acc[j[x]], at * v[x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    f(j[x], at * v[x]);
                 }
             }
         }
@@ -702,15 +717,14 @@ __device__ __forceinline__ int dense_add_slices(int64_t lo, int64_t hi, double a
         double v[SG_SHORT_LOADS];
 #pragma unroll
         for (int x = 0; x < SG_SHORT_LOADS; ++x)
-            j[x] = (ok[x] ? Bcrd[q[x]] : 0) - col0;
+            j[x] = (ok[x] ? Bcrd[q[x]] : 0);
 #pragma unroll
         for (int x = 0; x < SG_SHORT_LOADS; ++x)
-            v[x] = (ok[x] ? Bval[q[x]] : 0.0);
+            v[x] = (VALUES && ok[x] ? Bval[q[x]] : 0.0);
 #pragma unroll
         for (int x = 0; x < SG_SHORT_LOADS; ++x) {
             if (ok[x]) {
-                atomicOr(&bm[j[x] >> 5], 1u << (j[x] & 31));
-                __hip_atomic_fetch_add(&acc[j[x]], at * v[x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                f(j[x], at * v[x]);
             }
         }
     }
@@ -726,7 +740,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
 {
     __shared__ int64_t row_slot;
     __shared__ int wave_tot[SG_WAVES];
-    __shared__ int block_touched;
+    __shared__ int block_touched[3];            // see visit_flag
     double *acc = reinterpret_cast<double *>(sg_dyn_lds);
     uint32_t *bm = sg_dyn_lds + SG_CB * 2;
     emit_t *emit_col = reinterpret_cast<emit_t *>(bm + SG_CB / 32);
@@ -736,12 +750,13 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
         acc[j] = 0.0;
     if (threadIdx.x < SG_CB / 32)
         bm[threadIdx.x] = 0;
-    if (threadIdx.x == 0)
-        block_touched = 0;
+    if (threadIdx.x < 3)
+        block_touched[threadIdx.x] = 0;
     lds_barrier();
+    int visit = 0;
     const int64_t out0 = Cpos[row_begin];
     int64_t t_first, t_end;
-    list_range(list, 0, &t_first, &t_end);
+    list_range(list, 3, &t_first, &t_end);     // the other heavy rows go to spgemm_numeric_span_kernel
     int64_t t = draw_row<true>(ticket, t_first, &row_slot);
     while (t < t_end) {
         const int64_t i = row_begin + list.rows[t];
@@ -767,12 +782,16 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
             for (int cb = 0; cb < nblk; ++cb) {
                 const int col0 = cb << SG_CB_LOG;
                 int touched = 0;     // did this wavefront add anything to the block
+                const auto add = [&](int j, double x) {
+                    j -= col0;
+                    atomicOr(&bm[j >> 5], 1u << (j & 31));
+                    __hip_atomic_fetch_add(&acc[j], x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                };
                 if (held) {
                     int64_t next = h_hi;
                     if (h_bp && cb + 1 < nblk)
                         next = h_bp[cb + 2];
-                    touched = dense_add_slices(h_lo, h_hi, h_a, col0, lane, Bcrd, Bval, acc, bm
-                                               );
+                    touched = for_each_in_slices<true>(h_lo, h_hi, h_a, lane, Bcrd, Bval, add);
                     h_lo = h_hi;
                     h_hi = next;
                 }
@@ -788,16 +807,10 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                         hi = bp[1];
                         a = Aval[p];
                     }
-                    touched |= dense_add_slices(lo, hi, a, col0, lane, Bcrd, Bval, acc, bm
-                                                );
+                    touched |= for_each_in_slices<true>(lo, hi, a, lane, Bcrd, Bval, add);
                 }
-                // one barrier tells everybody whether the block received anything (an LDS flag that the
-                // emitting path resets); the value is made scalar so that the branch on it is uniform,
-                // because the block body below holds barriers
-                if (touched && lane == 0)
-                    block_touched = 1;
-                lds_barrier();
-                const int any = __builtin_amdgcn_readfirstlane(block_touched);
+                const int any = visit_flag(block_touched, visit, touched, lane);
+                visit = visit == 2 ? 0 : visit + 1;
                 if (any) {
                 // Emit this block.  Thread t owns the columns [8t, 8t + 8) and [8192 + 8t, 8192 + 8t + 8): one
                 // byte from each half of the bitmap, so that the dense low columns of a half (the columns of a
@@ -818,8 +831,6 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                 const int first_a = before & 0xffff, first_b = total_a + (before >> 16);
                 if (threadIdx.x < SG_CB / 32)      // everybody has read its bytes: the bitmap is clean for the
                     bm[threadIdx.x] = 0;           // next block, which nobody enters before the barrier below
-                if (threadIdx.x == 0)
-                    block_touched = 0;
                 // The owner of a byte knows where its columns go, but writing them from there would scatter
                 // every store over 64 cache lines.  So the columns are listed in LDS, SG_EMIT at a time, and
                 // then every lane writes the entry at its own place in the list: coalesced stores.
@@ -862,6 +873,181 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                 }
                 off += total;
                 }   // block received products
+            }
+        }
+        t = draw_row<true>(ticket, t_first, &row_slot);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Heavy rows that are not wide: a row with 10^4..10^5 products is the union of a few long rows of B with hardly
+// a column in common, so each of its 64 column blocks receives a few hundred products and a block visit of the
+// kernel above costs more in barriers and write-out than in products.  Here a visit spans up to SP_BLOCKS column
+// blocks and keeps the values compact: a first pass over the products sets the span's bitmap in LDS, a prefix
+// sum over the bitmap gives every column its rank, and a second pass adds each product at the rank of its column
+// (two LDS reads and one fp64 LDS atomic).  The values then leave in rank order, which is column order, and the
+// columns come from the bitmap.  The compact array holds SP_CAP = 16384 entries; a span that holds more is cut
+// at the last block boundary that fits (one block always does), so the kernel is right for any row and merely
+// slow for wide ones.
+// ---------------------------------------------------------------------------
+constexpr int SP_BLOCKS = 8;                              // column blocks per visit at most
+constexpr int SP_BLOCK_WORDS = SG_CB / 32;                // bitmap words of one block
+constexpr int SP_WORDS = SP_BLOCKS * SP_BLOCK_WORDS;      // bitmap words of a span
+constexpr int SP_WPT = SP_WORDS / SG_T;                   // consecutive bitmap words per thread
+constexpr int SP_CAP = SG_CB;                             // entries of C per visit at most
+constexpr size_t SG_SPAN_LDS = (size_t)SP_CAP * 8 + (size_t)SP_WORDS * 4 + (size_t)SP_WORDS * 2;   // values, bitmap, ranks
+static_assert(SP_WORDS % SG_T == 0 && SP_BLOCK_WORDS % SP_WPT == 0 && SP_CAP >= SG_CB && SP_CAP <= 65535,
+              "a thread's words lie in one block, one block fits the value array, ranks fit 16 bits");
+
+__global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
+    int64_t row_begin, int64_t row_end, const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd,
+    const double *__restrict__ Aval, const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval,
+    const int64_t *__restrict__ blkptr, int nblk,
+    unsigned long long *ticket, RowList list,
+    const int64_t *__restrict__ Cpos, int32_t *__restrict__ Ccrd, double *__restrict__ Cval)
+{
+    __shared__ int64_t row_slot;
+    __shared__ int wave_tot[SG_WAVES];
+    __shared__ int blk_pre[SP_BLOCKS + 1];      // entries of the span before each of its blocks, and in all
+    __shared__ int span_touched[3];             // see visit_flag below
+    double *val = reinterpret_cast<double *>(sg_dyn_lds);
+    uint32_t *bm = sg_dyn_lds + SP_CAP * 2;
+    uint16_t *pre = reinterpret_cast<uint16_t *>(bm + SP_WORDS);
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    for (int j = threadIdx.x; j < SP_CAP; j += SG_T)
+        val[j] = 0.0;
+    for (int w = threadIdx.x; w < SP_WORDS; w += SG_T)
+        bm[w] = 0;
+    if (threadIdx.x < 3)
+        span_touched[threadIdx.x] = 0;
+    lds_barrier();
+    int visit = 0;
+    const int64_t out0 = Cpos[row_begin];
+    int64_t t_first, t_end;
+    list_range(list, 4, &t_first, &t_end);
+    int64_t t = draw_row<true>(ticket, t_first, &row_slot);
+    while (t < t_end) {
+        const int64_t i = row_begin + list.rows[t];
+        const int64_t as = Apos[i], ae = Apos[i + 1];
+        if (as != ae) {
+            int64_t off = Cpos[i] - out0;
+            // A row of at most one entry of A per lane (nearly all rows) keeps the entry, the place of its block
+            // pointers and the slice of the span in registers; the end of the next span is loaded a visit ahead.
+            const int held = __builtin_amdgcn_readfirstlane((int)(ae - as <= SG_T));
+            double h_a = 0.0;
+            const int64_t *h_bp = nullptr;
+            int64_t h_lo = 0, h_hi = 0;
+            if (held) {
+                const int64_t p = as + wave + (int64_t)lane * SG_WAVES;
+                if (p < ae) {
+                    h_bp = blkptr + (int64_t)Acrd[p] * (nblk + 1);
+                    h_a = Aval[p];
+                    h_lo = h_bp[0];
+                    h_hi = h_bp[nblk < SP_BLOCKS ? nblk : SP_BLOCKS];
+                }
+            }
+            // f over the products of the row whose columns lie in the blocks [cbf, cbt); a held row's slice of these
+            // blocks is [held_lo, held_hi)
+            const auto walk = [&](int cbf, int cbt, int64_t held_lo, int64_t held_hi, auto values, auto f) -> int {
+                constexpr bool VALUES = decltype(values)::value;
+                int touched = 0;
+                if (held)
+                    touched = for_each_in_slices<VALUES>(held_lo, held_hi, h_a, lane, Bcrd, Bval, f);
+                for (int64_t base = as + wave; !held && base < ae; base += (int64_t)SG_WAVES * 64) {
+                    const int64_t left = (ae - base + SG_WAVES - 1) / SG_WAVES;
+                    const int cnt = (int)(left < 64 ? left : 64);
+                    int64_t lo = 0, hi = 0;
+                    double a = 0.0;
+                    if (lane < cnt) {
+                        const int64_t p = base + (int64_t)lane * SG_WAVES;
+                        const int64_t *bp = blkptr + (int64_t)Acrd[p] * (nblk + 1);
+                        lo = bp[cbf];
+                        hi = bp[cbt];
+                        a = Aval[p];
+                    }
+                    touched |= for_each_in_slices<VALUES>(lo, hi, a, lane, Bcrd, Bval, f);
+                }
+                return touched;
+            };
+            int cb = 0;
+            while (cb < nblk) {
+                const int nbv = nblk - cb < SP_BLOCKS ? nblk - cb : SP_BLOCKS;
+                const int col0 = cb << SG_CB_LOG;
+                int64_t h_next = h_hi;      // where the span after this one ends
+                if (h_bp && cb + nbv < nblk)
+                    h_next = h_bp[cb + nbv + SP_BLOCKS < nblk ? cb + nbv + SP_BLOCKS : nblk];
+                const int touched = walk(cb, cb + nbv, h_lo, h_hi, std::false_type{}, [&](int j, double) {
+                    j -= col0;
+                    atomicOr(&bm[j >> 5], 1u << (j & 31));
+                });
+                const int any = visit_flag(span_touched, visit, touched, lane);
+                visit = visit == 2 ? 0 : visit + 1;
+                int nb = nbv;
+                if (any) {
+                    // ranks: thread t owns the words [SP_WPT * t, SP_WPT * (t + 1))
+                    uint32_t w[SP_WPT];
+                    int mine = 0;
+#pragma unroll
+                    for (int k = 0; k < SP_WPT; ++k) {
+                        w[k] = bm[threadIdx.x * SP_WPT + k];
+                        mine += __popc(w[k]);
+                    }
+                    const int inc = wave_inclusive_scan(mine);
+                    if (lane == 63)
+                        wave_tot[wave] = inc;
+                    lds_barrier();
+                    const int tots = wave_inclusive_scan(lane < SG_WAVES ? wave_tot[lane] : 0);
+                    const int all = __builtin_amdgcn_readlane(tots, SG_WAVES - 1);
+                    const int before = (wave ? __builtin_amdgcn_readlane(tots, wave - 1) : 0) + inc - mine;
+                    int run = before;
+#pragma unroll
+                    for (int k = 0; k < SP_WPT; ++k) {
+                        pre[threadIdx.x * SP_WPT + k] = (uint16_t)(run < 65535 ? run : 65535);    // exact below the cut
+                        run += __popc(w[k]);
+                    }
+                    if (threadIdx.x % (SP_BLOCK_WORDS / SP_WPT) == 0)
+                        blk_pre[threadIdx.x / (SP_BLOCK_WORDS / SP_WPT)] = before;
+                    if (threadIdx.x == SG_T - 1)
+                        blk_pre[SP_BLOCKS] = all;
+                    lds_barrier();
+                    // the cut: as many blocks as fit the value array (blocks the span does not have are empty)
+                    nb = 1;
+                    for (int b = 2; b <= nbv; ++b)
+                        nb = __builtin_amdgcn_readfirstlane(blk_pre[b]) <= SP_CAP ? b : nb;
+                    const int total = __builtin_amdgcn_readfirstlane(blk_pre[nb]);
+                    if (nb < nbv) {              // cut: this visit ends, and the next span starts, at block cb + nb
+                        if (h_bp) {
+                            h_hi = h_bp[cb + nb];
+                            h_next = h_bp[cb + nb + SP_BLOCKS < nblk ? cb + nb + SP_BLOCKS : nblk];
+                        }
+                    }
+                    walk(cb, cb + nb, h_lo, h_hi, std::true_type{}, [&](int j, double x) {
+                        j -= col0;
+                        const uint32_t below = bm[j >> 5] & ((1u << (j & 31)) - 1u);
+                        const int r = pre[j >> 5] + __popc(below);
+                        __hip_atomic_fetch_add(&val[r], x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    });
+                    lds_barrier();
+                    for (int q = threadIdx.x; q < total; q += SG_T) {
+                        Cval[off + q] = val[q];
+                        val[q] = 0.0;
+                    }
+                    int64_t at = off + before;
+#pragma unroll
+                    for (int k = 0; k < SP_WPT; ++k) {
+                        const int wi = threadIdx.x * SP_WPT + k;
+                        if (wi < nb * SP_BLOCK_WORDS)
+                            for (uint32_t bits = w[k]; bits; bits &= bits - 1)
+                                Ccrd[at++] = col0 + wi * 32 + __ffs(bits) - 1;
+                        bm[wi] = 0;             // also the words beyond the cut: the next visit sets them again
+                    }
+                    off += total;
+                    lds_barrier();
+                }
+                cb += nb;
+                h_lo = h_hi;
+                h_hi = h_next;
             }
         }
         t = draw_row<true>(ticket, t_first, &row_slot);
@@ -1215,14 +1401,16 @@ __global__ void sg_row_keys(int64_t n, const int64_t *__restrict__ rowprod, uint
     }
 }
 
-// bounds[0] = rows with >= threshold products, bounds[1] = rows with any, in the sorted key array
-__global__ void sg_row_bounds(int64_t n, const uint64_t *__restrict__ keys, int64_t threshold,
+// bounds[0] = rows with >= threshold products, bounds[1] = rows with any, bounds[2] = rows with >= wide products,
+// in the sorted key array
+__global__ void sg_row_bounds(int64_t n, const uint64_t *__restrict__ keys, int64_t threshold, int64_t wide,
                               int64_t *__restrict__ bounds)
 {
-    if (threadIdx.x > 1 || blockIdx.x > 0)
+    if (threadIdx.x > 2 || blockIdx.x > 0)
         return;
     // first key that is larger than the limit: keys ascend as products descend
-    const uint64_t limit = threadIdx.x == 0 ? (uint64_t)((1ll << 62) - threshold) : (uint64_t)((1ll << 62) - 1);
+    const uint64_t limit = threadIdx.x == 1 ? (uint64_t)((1ll << 62) - 1)
+                                            : (uint64_t)((1ll << 62) - (threadIdx.x == 0 ? threshold : wide));
     int64_t lo = 0, hi = n;
     while (lo < hi) {
         const int64_t mid = (lo + hi) >> 1;
@@ -1240,7 +1428,8 @@ struct SgRowLists {
 static SgRowLists g_rl;
 
 // Products per row of rows [rb, re) of A*B and the list of those rows by descending products.
-static int sg_row_list(const Csr *a, const Csr *b, int64_t rb, int64_t re, int64_t dense_threshold, RowList *out)
+static int sg_row_list(const Csr *a, const Csr *b, int64_t rb, int64_t re, int64_t dense_threshold,
+                       int64_t wide_threshold, RowList *out)
 {
     const int64_t n = re - rb;
     COMET_CHK(g_rl.rowprod.ensure(sizeof(int64_t) * (size_t)n, false));
@@ -1248,7 +1437,7 @@ static int sg_row_list(const Csr *a, const Csr *b, int64_t rb, int64_t re, int64
     COMET_CHK(g_rl.keys_out.ensure(8 * (size_t)n, false));
     COMET_CHK(g_rl.idx_in.ensure(4 * (size_t)n, false));
     COMET_CHK(g_rl.idx_out.ensure(4 * (size_t)n, false));
-    COMET_CHK(g_rl.bounds.ensure(16, false));
+    COMET_CHK(g_rl.bounds.ensure(24, false));
     int64_t *rowprod = (int64_t *)g_rl.rowprod.ptr;
     {
         KernelTimer t("spgemm_row_products");
@@ -1261,7 +1450,7 @@ static int sg_row_list(const Csr *a, const Csr *b, int64_t rb, int64_t re, int64
     COMET_CHK(sort_pairs_u64_u32((const uint64_t *)g_rl.keys_in.ptr, (uint64_t *)g_rl.keys_out.ptr,
                                  (const uint32_t *)g_rl.idx_in.ptr, (uint32_t *)g_rl.idx_out.ptr, n, 63));
     sg_row_bounds<<<dim3(1), dim3(64), 0, stream()>>>(n, (const uint64_t *)g_rl.keys_out.ptr, dense_threshold,
-                                                      (int64_t *)g_rl.bounds.ptr);
+                                                      wide_threshold, (int64_t *)g_rl.bounds.ptr);
     COMET_HIPCHK(hipGetLastError());
     out->rows = (const int32_t *)g_rl.idx_out.ptr;
     out->bounds = (const int64_t *)g_rl.bounds.ptr;
@@ -1276,7 +1465,7 @@ static int symbolic_counts(const Csr *a, const Csr *b, const Csr *m, int64_t *ro
     COMET_CHK(sg_geometry(b->ncols, &g));
     COMET_CHK(sg_reset_ticket());
     RowList list;
-    COMET_CHK(sg_row_list(a, b, 0, a->nrows, SG_NO_DENSE, &list));
+    COMET_CHK(sg_row_list(a, b, 0, a->nrows, SG_NO_DENSE, SG_NO_DENSE, &list));
     COMET_HIPCHK(hipMemsetAsync(rowcount, 0, sizeof(int64_t) * (size_t)a->nrows, stream()));
     uint32_t *gbm = nullptr;
     if (!g.lds) {
@@ -1307,6 +1496,18 @@ constexpr int SG_DENSE_MAX_BLOCKS = 64;        // the dense path serves matrices
 #define COMET_SG_DENSE_PER_BLOCK 128
 #endif
 constexpr int64_t SG_DENSE_PER_BLOCK = COMET_SG_DENSE_PER_BLOCK;   // products per column block from which a block sweep pays
+
+// Heavy rows with at least this many products per column block of the matrix stay with the block kernel, the
+// others go to the span kernel (measured on A*A of an R-MAT graph of scale 20, 64 blocks, ms per product:
+// 512 per block 583, 1024 572, 2048 559, 4096 557, 8192 570, every heavy row to the span kernel 604, none 613).
+// COMET_HIP_SPGEMM_WIDE, a number of products per row, overrides the rule: either kernel is right for any row,
+// so the tests use it to send the same rows through both.
+constexpr int64_t SG_WIDE_PER_BLOCK = 4096;
+static int64_t sg_wide_threshold(int nblk)
+{
+    const char *e = getenv("COMET_HIP_SPGEMM_WIDE");
+    return e && *e ? atoll(e) : SG_WIDE_PER_BLOCK * nblk;
+}
 
 // Per-row block pointers of the right-hand operand, built once per matrix.
 static int sg_plan_blocks(Csr *b)
@@ -1347,7 +1548,8 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
     if (dense)
         COMET_CHK(sg_plan_blocks(b));
     RowList list;
-    COMET_CHK(sg_row_list(a, b, rb, re, dense_threshold, &list));
+    const int64_t wide = sg_wide_threshold(nblk) > dense_threshold ? sg_wide_threshold(nblk) : dense_threshold;
+    COMET_CHK(sg_row_list(a, b, rb, re, dense_threshold, dense ? wide : SG_NO_DENSE, &list));
     uint32_t *gbm = nullptr, *gmask = nullptr;
     if (!g.lds) {
         COMET_CHK(g_sg.gbm.ensure(sizeof(uint32_t) * g.bm_words * (size_t)g.groups, true));
@@ -1388,6 +1590,15 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
                                       stream()>>>(rb, re, a->pos, a->crd, a->val, b->crd, b->val, b->sg_blkptr,
                                                   nblk, (unsigned long long *)g_sg.ticket.ptr, list, Cpos, Ccrd,
                                                   Cval);
+        COMET_HIPCHK(hipGetLastError());
+    }
+    if (dense) {
+        COMET_CHK(sg_reset_ticket());
+        COMET_CHK(sg_allow_lds(spgemm_numeric_span_kernel, SG_SPAN_LDS));
+        KernelTimer t("spgemm_numeric_span");
+        spgemm_numeric_span_kernel<<<dim3((unsigned)(num_cus() > 0 ? num_cus() : 256)), block, SG_SPAN_LDS,
+                                     stream()>>>(rb, re, a->pos, a->crd, a->val, b->crd, b->val, b->sg_blkptr, nblk,
+                                                 (unsigned long long *)g_sg.ticket.ptr, list, Cpos, Ccrd, Cval);
         COMET_HIPCHK(hipGetLastError());
     }
     return COMET_HIP_OK;
@@ -1518,7 +1729,7 @@ extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, d
     }
     double *rowsum = (double *)g_sg.rowcount.ptr;
     RowList list;
-    COMET_CHK(sg_row_list(a, b, 0, a->nrows, SG_NO_DENSE, &list));
+    COMET_CHK(sg_row_list(a, b, 0, a->nrows, SG_NO_DENSE, SG_NO_DENSE, &list));
     COMET_HIPCHK(hipMemsetAsync(rowsum, 0, sizeof(double) * (size_t)a->nrows, stream()));
     const dim3 grid((unsigned)g.groups), block(SG_T);
     // Two kernels side by side, the second on the auxiliary stream: a workgroup per row from the heavy end of

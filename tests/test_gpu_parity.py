@@ -426,6 +426,46 @@ def test_spgemm_row_blocks_equal_whole():
         assert np.all(np.abs(v - wv[hp[rb]:hp[re]]) <= RTOL * np.abs(wv[hp[rb]:hp[re]]))
 
 
+def _rows_of_lengths(rng, lengths, ncols, pick=None, signed=True):
+    """CSR with the given row lengths; columns drawn without repetition from `pick` (default: all columns)."""
+    pos = np.zeros(len(lengths) + 1, dtype=np.int64)
+    np.cumsum(lengths, out=pos[1:])
+    pool = np.arange(ncols) if pick is None else np.asarray(pick)
+    crd = np.concatenate([np.sort(rng.choice(pool, l, replace=False)) for l in lengths] + [np.zeros(0, dtype=np.int64)])
+    val = rng.uniform(-1, 1, len(crd)) if signed else rng.uniform(0.1, 1, len(crd))
+    return pos, crd.astype(np.int64), val
+
+
+@pytest.mark.parametrize("m,long_len,wide", [(200_000, 2000, None), (40_000, 1200, None), (40_000, 1200, 1 << 40),
+                                             (200_000, 2000, 1 << 40), (200_000, 2000, 0)])
+def test_spgemm_rows_of_every_class(m, long_len, wide, monkeypatch):
+    # Rows of B: 200 long ones and 200 of 10 entries.  Rows of A pick among them so that the product has rows
+    # for each numeric kernel: no products, a few (values kept in a slab), thousands spread thinly over the
+    # column blocks (several blocks per visit, values compact) and many per block (one block per visit).
+    # `wide` moves the border between the last two: with 1 << 40 every heavy row takes the several-block
+    # kernel, and with 40,000 columns the thick rows then exceed the compact array, so their visits are cut
+    # short at a block boundary; with 0 every heavy row takes one block per visit.
+    if wide is not None:
+        monkeypatch.setenv("COMET_HIP_SPGEMM_WIDE", str(wide))
+    rng = np.random.default_rng(17)
+    k = 400
+    b = _rows_of_lengths(rng, [long_len] * 200 + [10] * 200, m)
+    long_rows, short_rows = np.arange(200), np.arange(200, 400)
+    lengths, picks = [], []
+    for n_long, n_short in [(0, 0), (0, 5), (1, 0), (3, 2), (10, 0), (25, 40), (40, 0), (120, 3), (200, 200), (0, 200),
+                            (2, 0), (60, 0), (0, 1), (7, 7)] * 3:
+        lengths.append(n_long + n_short)
+        picks.append(np.sort(np.concatenate([rng.choice(long_rows, n_long, replace=False),
+                                             rng.choice(short_rows, n_short, replace=False)])))
+    apos = np.zeros(len(lengths) + 1, dtype=np.int64)
+    np.cumsum(lengths, out=apos[1:])
+    acrd = np.concatenate(picks).astype(np.int64)
+    a = (apos, acrd, rng.uniform(-1, 1, len(acrd)))
+    first = _spgemm_check(a, b, m)
+    second = _spgemm_check(a, b, m)          # the kernels leave their LDS and slabs clean
+    assert np.array_equal(first[1], second[1])
+
+
 def test_spgemm_empty_and_repeatable():
     Z = rt.CsrMatrix.from_arrays((3, 3), np.zeros(4, dtype=np.int64), np.zeros(0, dtype=np.int64), np.zeros(0))
     p, c, v = rt.spgemm(Z, Z).to_arrays()
