@@ -353,11 +353,20 @@ __global__ __launch_bounds__(SG_T) void spgemm_symbolic_kernel(
             if constexpr (MASKED) {
                 const uint32_t old = atomicAnd(&bm[ad.word(j)], ~b);
                 count += (old & b) ? 1 : 0;
-            } else {
+            } else if constexpr (BM_LDS) {
+                atomicOr(&bm[ad.word(j)], b);       // nothing comes back, so the walk never waits for LDS:
+            } else {                                // the bits are counted when the bitmap is cleared
                 const uint32_t old = atomicOr(&bm[ad.word(j)], b);
                 count += (old & b) ? 0 : 1;
             }
         });
+        if constexpr (BM_LDS && !MASKED) {
+            __syncthreads();
+            for (int w = threadIdx.x; w < nwords; w += SG_T) {
+                count += __popc(bm[w]);
+                bm[w] = 0;
+            }
+        }
         count = wave_sum_i32(count);
         if ((threadIdx.x & 63) == 0)
             wave_cnt[threadIdx.x >> 6] = count;
@@ -372,10 +381,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_symbolic_kernel(
         if constexpr (MASKED) {
             for (int64_t t = Mpos[i] + threadIdx.x; t < Mpos[i + 1]; t += SG_T)
                 atomicAnd(&bm[ad.word(Mcrd[t])], 0u);
-        } else if constexpr (BM_LDS) {
-            for (int w = threadIdx.x; w < nwords; w += SG_T)
-                bm[w] = 0;
-        } else {
+        } else if constexpr (!BM_LDS) {
             for_each_product<false>(as, ae, Acrd, nullptr, Bpos, Bcrd,
                                     [&](int j, int64_t, double, int64_t, int64_t) { atomicAnd(&bm[ad.word(j)], 0u); });
         }
