@@ -609,9 +609,38 @@ __device__ __forceinline__ int visit_flag(int *flags, int visit, int touched, in
 // Visits the products of one slice per lane: f(j, x) for the entries [lo, hi) of a row of B (the part of it inside
 // the column block or blocks being swept), j the column and x = a times the entry's value (0 without VALUES,
 // when the value array is not read).  Returns whether this wavefront had anything to visit.
+
 constexpr int SG_SHORT = 32;                      // slices shorter than this are taken by 16 lanes, the others by 64
 constexpr int SG_SHORT_LOADS = SG_SHORT / 16;     // entries of a short slice per lane
 constexpr int SG_LONG_LOADS = 4;                  // entries of a long slice per lane and turn
+
+// One turn of a wavefront over a slice that starts at entry s of B and has len entries: lane l visits the
+// entries o + 64 x < len, x < SG_LONG_LOADS (o = l for the first turn of a slice).  All loads are issued before
+// the first visit, and a load that no lane needs is skipped.
+template <bool VALUES, typename F>
+__device__ __forceinline__ void turn_of_slice(int64_t s, int64_t o, int64_t len, double at,
+                                              const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval, F f)
+{
+    int64_t q[SG_LONG_LOADS];
+    bool ok[SG_LONG_LOADS];
+#pragma unroll
+    for (int x = 0; x < SG_LONG_LOADS; ++x) {
+        ok[x] = o + 64 * x < len;
+        q[x] = ok[x] ? s + o + 64 * x : 0;
+    }
+    int j[SG_LONG_LOADS];
+    double v[SG_LONG_LOADS];
+#pragma unroll
+    for (int x = 0; x < SG_LONG_LOADS; ++x)
+        j[x] = ok[x] ? Bcrd[q[x]] : 0;
+#pragma unroll
+    for (int x = 0; x < SG_LONG_LOADS; ++x)
+        v[x] = VALUES && ok[x] ? Bval[q[x]] : 0.0;
+#pragma unroll
+    for (int x = 0; x < SG_LONG_LOADS; ++x)
+        if (ok[x])
+            f(j[x], at * v[x]);
+}
 
 template <bool VALUES, typename F>
 __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double a, int lane,
@@ -673,29 +702,8 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
             }
             o += 64 * SG_LONG_LOADS;
         }
-        if (o < len) {
-            int64_t q[SG_LONG_LOADS];
-            bool ok[SG_LONG_LOADS];
-#pragma unroll
-            for (int x = 0; x < SG_LONG_LOADS; ++x) {
-                ok[x] = o + 64 * x < len;
-                q[x] = ok[x] ? s + o + 64 * x : 0;
-            }
-            int j[SG_LONG_LOADS];
-            double v[SG_LONG_LOADS];
-#pragma unroll
-            for (int x = 0; x < SG_LONG_LOADS; ++x)
-                j[x] = (ok[x] ? Bcrd[q[x]] : 0);
-#pragma unroll
-            for (int x = 0; x < SG_LONG_LOADS; ++x)
-                v[x] = (VALUES && ok[x] ? Bval[q[x]] : 0.0);
-#pragma unroll
-            for (int x = 0; x < SG_LONG_LOADS; ++x) {
-                if (ok[x]) {
-                    f(j[x], at * v[x]);
-                }
-            }
-        }
+        if (o < len)
+            turn_of_slice<VALUES>(s, o, len, at, Bcrd, Bval, f);
     }
     const int quarter = lane >> 4, sub = lane & 15;
     while (todo) {              // four short slices per turn, one to a quarter, SG_SHORT_LOADS entries per lane
@@ -901,6 +909,7 @@ constexpr int SP_BLOCK_WORDS = SG_CB / 32;                // bitmap words of one
 constexpr int SP_WORDS = SP_BLOCKS * SP_BLOCK_WORDS;      // bitmap words of a span
 constexpr int SP_WPT = SP_WORDS / SG_T;                   // consecutive bitmap words per thread
 constexpr int SP_CAP = SG_CB;                             // entries of C per visit at most
+constexpr int SP_CHUNK = 64 * SG_LONG_LOADS;              // entries of a slice that a wavefront takes in one turn
 constexpr size_t SG_SPAN_LDS = (size_t)SP_CAP * 8 + (size_t)SP_WORDS * 4 + (size_t)SP_WORDS * 2;   // values, bitmap, ranks
 static_assert(SP_WORDS % SG_T == 0 && SP_BLOCK_WORDS % SP_WPT == 0 && SP_CAP >= SG_CB && SP_CAP <= 65535,
               "a thread's words lie in one block, one block fits the value array, ranks fit 16 bits");
@@ -940,12 +949,16 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
             int64_t off = Cpos[i] - out0;
             // A row of at most one entry of A per lane (nearly all rows) keeps the entry, the place of its block
             // pointers and the slice of the span in registers; the end of the next span is loaded a visit ahead.
+            // A row of at most 64 entries of A (the usual heavy row that is not wide has 5..140) is held whole by
+            // every wavefront, entry l in lane l, and its slices are dealt to the wavefronts in chunks of
+            // SP_CHUNK entries: with an entry per wavefront, 5 entries would leave 11 wavefronts idle.
             const int held = __builtin_amdgcn_readfirstlane((int)(ae - as <= SG_T));
+            const int small = __builtin_amdgcn_readfirstlane((int)(ae - as <= 64));
             double h_a = 0.0;
             const int64_t *h_bp = nullptr;
             int64_t h_lo = 0, h_hi = 0;
             if (held) {
-                const int64_t p = as + wave + (int64_t)lane * SG_WAVES;
+                const int64_t p = small ? as + lane : as + wave + (int64_t)lane * SG_WAVES;
                 if (p < ae) {
                     h_bp = blkptr + (int64_t)Acrd[p] * (nblk + 1);
                     h_a = Aval[p];
@@ -958,7 +971,20 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
             const auto walk = [&](int cbf, int cbt, int64_t held_lo, int64_t held_hi, auto values, auto f) -> int {
                 constexpr bool VALUES = decltype(values)::value;
                 int touched = 0;
-                if (held)
+                if (small) {
+                    const int mine = (int)((held_hi - held_lo + SP_CHUNK - 1) / SP_CHUNK);
+                    const int upto = wave_inclusive_scan(mine);             // chunks of the entries 0..lane
+                    const int chunks = __builtin_amdgcn_readlane(upto, 63);
+                    touched = chunks > 0;
+                    for (int g = wave; g < chunks; g += SG_WAVES) {
+                        const int e = __builtin_ctzll(__ballot(upto > g));   // the entry that chunk g belongs to
+                        const int c = g - (__builtin_amdgcn_readlane(upto, e) - __builtin_amdgcn_readlane(mine, e));
+                        const int64_t s = readlane_i64(held_lo, e) + (int64_t)c * SP_CHUNK;
+                        const int64_t left = readlane_i64(held_hi, e) - s;
+                        turn_of_slice<VALUES>(s, lane, left < SP_CHUNK ? left : SP_CHUNK, readlane_d(h_a, e), Bcrd,
+                                              Bval, f);
+                    }
+                } else if (held)
                     touched = for_each_in_slices<VALUES>(held_lo, held_hi, h_a, lane, Bcrd, Bval, f);
                 for (int64_t base = as + wave; !held && base < ae; base += (int64_t)SG_WAVES * 64) {
                     const int64_t left = (ae - base + SG_WAVES - 1) / SG_WAVES;
@@ -1498,10 +1524,10 @@ static int symbolic_counts(const Csr *a, const Csr *b, const Csr *m, int64_t *ro
 }
 
 constexpr int SG_DENSE_MAX_BLOCKS = 64;        // the dense path serves matrices of up to 2^20 columns
-#ifndef COMET_SG_DENSE_PER_BLOCK
-#define COMET_SG_DENSE_PER_BLOCK 128
-#endif
-constexpr int64_t SG_DENSE_PER_BLOCK = COMET_SG_DENSE_PER_BLOCK;   // products per column block from which a block sweep pays
+// Rows with at least this many products per column block of the matrix keep their values in LDS (the span or
+// the block kernel); the others add into a slab in HBM through L2 atomics.  Measured as above, ms per product
+// with the span kernel in place: 128 per block 555, 64: 533, 32: 519, 16: 514, 8: 513.5, 4: 513, 1: 515.
+constexpr int64_t SG_DENSE_PER_BLOCK = 8;
 
 // Heavy rows with at least this many products per column block of the matrix stay with the block kernel, the
 // others go to the span kernel (measured on A*A of an R-MAT graph of scale 20, 64 blocks, ms per product:
