@@ -337,8 +337,8 @@ def bench_tricount(rt, orc, gen, args):
 
 def bench_spgemm(rt, orc, gen, args):
     """C = A*A on the symmetrised R-MAT graph.  The symbolic phase runs over all rows; the numeric
-    phase runs in row blocks sized to a fixed output budget, each block is checksummed and dropped
-    (at scale 20 the whole of C is larger than HBM)."""
+    phase runs in row blocks sized to a fixed output budget and each block is dropped (at scale 20 the
+    whole of C is larger than HBM); one extra, untimed pass sums the values of every block for the check."""
     scale = args.scale or 20
     n = 1 << scale
     log(f"generating R-MAT scale {scale}")
@@ -351,7 +351,10 @@ def bench_spgemm(rt, orc, gen, args):
     budget = int(args.budget_gb * (1 << 30)) // 12          # entries per block
     state = {}
 
-    def step():
+    def step(check=False):
+        # the whole product: symbolic over all rows, numeric block by block into the same buffers.  With `check`
+        # every block is also summed before it is dropped; that pass is the bench's own and stays out of the
+        # timed steps (it reads each block once more: 47 ms at scale 20).
         dpos, nnzC = rt.spgemm_symbolic(A, A)
         log(f"symbolic done: nnz(C) = {nnzC}")
         hpos = dpos.to_numpy()
@@ -368,13 +371,17 @@ def bench_spgemm(rt, orc, gen, args):
             re = int(np.searchsorted(hpos, hpos[rb] + cap, side="right")) - 1
             re = min(max(re, rb + 1), n)
             rt.spgemm_numeric(A, A, dpos, rb, re, dcrd, dval)
-            vsum += rt.reduce_sum(dval, int(hpos[re] - hpos[rb]))
+            if check:
+                vsum += rt.reduce_sum(dval, int(hpos[re] - hpos[rb]))
             log(f"numeric rows [{rb},{re}): {int(hpos[re] - hpos[rb])} entries")
             rb = re
             blocks += 1
-        state.update(nnzC=int(nnzC), blocks=blocks, vsum=vsum, hpos=hpos, dpos=dpos)
+        state.update(nnzC=int(nnzC), blocks=blocks, hpos=hpos, dpos=dpos)
+        if check:
+            state["vsum"] = vsum
 
     # every step is seconds long: per-kernel event timing stays on during the timed steps
+    step(check=True)
     for _ in range(args.warmup):
         step()
     rt.profile_reset()
