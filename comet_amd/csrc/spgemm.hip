@@ -1265,8 +1265,16 @@ __global__ __launch_bounds__(SM_WAVES * 64) void spgemm_masked_sum_small_kernel(
                 big &= big - 1;
                 const int64_t s = readlane_i64(bs, l), e = readlane_i64(be, l);
                 const double al = readlane_d(a, l);
-                for (int64_t q = s + lane; q < e; q += 64)
-                    probe(Bcrd[q], q, al);
+                for (int64_t q = s + lane; q < e; q += 256) {      // all loads of a turn first, then the probes
+                    int j[4];
+#pragma unroll
+                    for (int x = 0; x < 4; ++x)
+                        j[x] = q + 64 * x < e ? Bcrd[q + 64 * x] : 0;
+#pragma unroll
+                    for (int x = 0; x < 4; ++x)
+                        if (q + 64 * x < e)
+                            probe(j[x], q + 64 * x, al);
+                }
             }
             const int quarter = lane >> 4, sub = lane & 15;
             while (todo) {
@@ -1284,9 +1292,14 @@ __global__ __launch_bounds__(SM_WAVES * 64) void spgemm_masked_sum_small_kernel(
                                   (uint32_t)__shfl((int)(be & 0xffffffff), src, 64);
                 const double al = __hiloint2double(__shfl(__double2hiint(a), src, 64),
                                                    __shfl(__double2loint(a), src, 64));
-                if (pick >= 0)
-                    for (int64_t q = s + sub; q < e; q += 16)
-                        probe(Bcrd[q], q, al);
+                int j[4];                   // a row here has fewer than 64 entries: four per lane cover it
+#pragma unroll
+                for (int x = 0; x < 4; ++x)
+                    j[x] = pick >= 0 && s + sub + 16 * x < e ? Bcrd[s + sub + 16 * x] : 0;
+#pragma unroll
+                for (int x = 0; x < 4; ++x)
+                    if (pick >= 0 && s + sub + 16 * x < e)
+                        probe(j[x], s + sub + 16 * x, al);
             }
         }
         part = wave_sum_f64(part);
