@@ -945,7 +945,18 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
     while (t < t_end) {
         const int64_t i = row_begin + list.rows[t];
         const int64_t as = Apos[i], ae = Apos[i + 1];
-        if (as != ae) {
+        if (ae - as == 1) {
+            // one entry of A: the row of C is that row of B times the entry (0 + a * b, as an accumulator that
+            // starts at zero gives it).  70,000 rows of the R-MAT product at scale 20 are like that, each the
+            // copy of a hub's row.
+            const int64_t *bp = blkptr + (int64_t)Acrd[as] * (nblk + 1);
+            const int64_t bs = bp[0], len = bp[nblk] - bs, off = Cpos[i] - out0;
+            const double a = Aval[as];
+            for (int64_t q = threadIdx.x; q < len; q += SG_T) {
+                Ccrd[off + q] = Bcrd[bs + q];
+                Cval[off + q] = 0.0 + a * Bval[bs + q];
+            }
+        } else if (as != ae) {
             int64_t off = Cpos[i] - out0;
             // A row of at most one entry of A per lane (nearly all rows) keeps the entry, the place of its block
             // pointers and the slice of the span in registers; the end of the next span is loaded a visit ahead.
