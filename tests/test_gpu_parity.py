@@ -466,6 +466,18 @@ def test_spgemm_rows_of_every_class(m, long_len, wide, monkeypatch):
     assert np.array_equal(first[1], second[1])
 
 
+@pytest.mark.parametrize("wide", [1 << 40, 0])
+def test_spgemm_rows_with_more_entries_than_lanes(wide, monkeypatch):
+    # more than 1024 entries in a row of A: the LDS kernels then fetch the row's entries again at every visit
+    # instead of holding one per lane; `wide` sends the rows through either kernel
+    monkeypatch.setenv("COMET_HIP_SPGEMM_WIDE", str(wide))
+    rng = np.random.default_rng(23)
+    k, m = 3000, 40_000
+    b = _rows_of_lengths(rng, rng.integers(0, 17, k), m)
+    a = _rows_of_lengths(rng, [2500, 1100, 30, 0, 1025, 3000], k)
+    _spgemm_check(a, b, m)
+
+
 def test_spgemm_empty_and_repeatable():
     Z = rt.CsrMatrix.from_arrays((3, 3), np.zeros(4, dtype=np.int64), np.zeros(0, dtype=np.int64), np.zeros(0))
     p, c, v = rt.spgemm(Z, Z).to_arrays()
