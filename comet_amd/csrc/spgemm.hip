@@ -13,9 +13,14 @@
 // covers 2^20 columns), so counting is a popcount, "sort the touched columns"
 // (the reference's comet_sort call) is reading the bitmap in order, and the
 // mark array / mark value bookkeeping disappears.  Values accumulate with
-// workgroup-scope fp64 atomics into a dense per-workgroup slab in HBM that the
-// extraction step reads back and re-zeroes with an atomic exchange, so every
-// access to the slab is performed at the L2 and no stale L1 line can be seen.
+// fp64 atomics, in one of three places chosen by the number of products of the
+// row: a dense per-workgroup slab in HBM (few products, every masked product and
+// every semiring other than plus-times; the extraction step reads it back and
+// re-zeroes it with an atomic exchange, so every access to the slab is performed
+// at the L2 and no stale L1 line can be seen), a compact array in LDS indexed by
+// the rank of the column among the row's columns (spgemm_numeric_span_kernel),
+// or LDS accumulators for one block of 16384 columns at a time
+// (spgemm_numeric_dense_kernel, the widest rows).
 // The order in which the products of one (i,j) are added is therefore not the
 // reference's ascending-k order: values agree to rounding, structure exactly.
 #include "common.h"
