@@ -31,6 +31,7 @@ SPMM_TRAFFIC_BYTES = int((436_260 * 2.000 + 272_815 * 1.000) * 1024)
 SPMV_TRAFFIC_BYTES = int((124_163 * 2.000 + 31_250 * 1.000) * 1024)            # four column-block passes
 SDDMM_TRAFFIC_BYTES = int((2_288_233 * 2.000 + 312_341 * 1.000) * 1024)        # kernel + transpose of D
 TRICOUNT_TRAFFIC_BYTES = int((20_166_583 * 2.000 + 37_909 * 1.000) * 1024)     # both masked-sum kernels
+SPGEMM_TRAFFIC_BYTES = int((566_358_591 * 2.000 + 281_840_080 * 1.000) * 1024)  # symbolic + the numeric kernels of 6 blocks
 
 
 _T0 = time.perf_counter()
@@ -447,7 +448,8 @@ def bench_spgemm(rt, orc, gen, args):
                    "seed": 20},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / ((sym_ms + num_ms) * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": alg_bytes / ((sym_ms + num_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": None, "kernel": "spgemm_symbolic + spgemm_numeric + spgemm_numeric_dense + spgemm_numeric_span",
+                     "traffic": SPGEMM_TRAFFIC_BYTES if (scale, args.budget_gb) == (20, 48.0) else None,
+                     "kernel": "spgemm_symbolic + spgemm_numeric + spgemm_numeric_dense + spgemm_numeric_span",
                      "kernel_avg_ms": sym_ms + num_ms,
                      "symbolic_ms": sym_ms, "numeric_ms": num_ms, "algorithmic_bytes": int(alg_bytes)},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity,
