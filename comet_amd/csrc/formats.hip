@@ -145,12 +145,21 @@ static int parse_mtx(const char *path, HostCoo *out)
 // compacted in order, and row r's pointer is the position of the first kept
 // entry whose row is >= r.
 // ---------------------------------------------------------------------------
+// key = row << col_bits | col: no more bits than the matrix needs, because the radix sort's time goes with the
+// number of key bits.  A tuple outside the matrix raises *bad (its key could not be told from another tuple's).
 __global__ void coo_make_keys(int64_t n, const int32_t *__restrict__ row, const int32_t *__restrict__ col,
-                              uint64_t *__restrict__ keys, uint32_t *__restrict__ idx)
+                              int64_t nrows, int64_t ncols, int col_bits, uint64_t *__restrict__ keys,
+                              uint32_t *__restrict__ idx, int *__restrict__ bad)
 {
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e < n) {
-        keys[e] = ((uint64_t)(uint32_t)row[e] << 32) | (uint32_t)col[e];
+        const int64_t r = row[e], c = col[e];
+        if (r < 0 || r >= nrows || c < 0 || c >= ncols) {
+            atomicOr(bad, 1);
+            keys[e] = 0;
+        } else {
+            keys[e] = ((uint64_t)r << col_bits) | (uint64_t)c;
+        }
         idx[e] = (uint32_t)e;
     }
 }
@@ -166,22 +175,24 @@ __device__ inline bool keep_entry(int mode, uint32_t r, uint32_t c)
     }
 }
 
-__global__ void coo_flag(int64_t n, const uint64_t *__restrict__ keys, int mode, int64_t *__restrict__ flag)
+__global__ void coo_flag(int64_t n, const uint64_t *__restrict__ keys, int col_bits, int mode,
+                         int64_t *__restrict__ flag)
 {
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e < n)
-        flag[e] = keep_entry(mode, (uint32_t)(keys[e] >> 32), (uint32_t)keys[e]) ? 1 : 0;
+        flag[e] = keep_entry(mode, (uint32_t)(keys[e] >> col_bits), (uint32_t)(keys[e] & ((1ull << col_bits) - 1))) ? 1 : 0;
 }
 
-__global__ void coo_compact(int64_t n, const uint64_t *__restrict__ keys, const uint32_t *__restrict__ idx,
+__global__ void coo_compact(int64_t n, const uint64_t *__restrict__ keys, int col_bits,
+                            const uint32_t *__restrict__ idx,
                             const int64_t *__restrict__ off, const double *__restrict__ val_in,
                             int32_t *__restrict__ crow, int32_t *__restrict__ crd, double *__restrict__ val)
 {
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e < n && off[e + 1] != off[e]) {
         const int64_t o = off[e];
-        crow[o] = (int32_t)(keys[e] >> 32);
-        crd[o] = (int32_t)(uint32_t)keys[e];
+        crow[o] = (int32_t)(keys[e] >> col_bits);
+        crd[o] = (int32_t)(keys[e] & ((1ull << col_bits) - 1));
         val[o] = val_in[idx[e]];
     }
 }
@@ -339,33 +350,49 @@ static Csr *coo_device_to_csr_struct(int64_t nrows, int64_t ncols, int64_t n, co
     }
     // temporaries live in grow-only buffers kept for the life of the process: a conversion of a few million
     // tuples takes less time than the allocations would
-    static CachedBuf keys_in, keys_out, idx_in, idx_out, flag, off, crow;
+    static CachedBuf keys_in, keys_out, idx_in, idx_out, flag, off, crow, bad;
     int64_t kept = 0;
+    int row_bits = 1, col_bits = 1;
+    while (row_bits < 31 && (1ll << row_bits) < nrows)
+        ++row_bits;
+    while (col_bits < 31 && (1ll << col_bits) < ncols)
+        ++col_bits;
     if (n > 0) {
         if (keys_in.alloc(8 * (size_t)n) || keys_out.alloc(8 * (size_t)n) || idx_in.alloc(4 * (size_t)n) ||
-            idx_out.alloc(4 * (size_t)n) || flag.alloc(8 * (size_t)n) || off.alloc(8 * (size_t)(n + 1)))
+            idx_out.alloc(4 * (size_t)n) || flag.alloc(8 * (size_t)n) || off.alloc(8 * (size_t)(n + 1)) ||
+            bad.alloc(sizeof(int)))
             return fail();
+        if (hipMemsetAsync(bad.p, 0, sizeof(int), stream()) != hipSuccess) {
+            set_error(COMET_HIP_ERR_HIP, "clearing the range flag failed");
+            return fail();
+        }
         {
             KernelTimer t("coo_make_keys");
-            coo_make_keys<<<grid_for(n), dim3(256), 0, stream()>>>(n, row, col, keys_in.as<uint64_t>(),
-                                                                  idx_in.as<uint32_t>());
+            coo_make_keys<<<grid_for(n), dim3(256), 0, stream()>>>(n, row, col, nrows, ncols, col_bits,
+                                                                  keys_in.as<uint64_t>(), idx_in.as<uint32_t>(),
+                                                                  bad.as<int>());
         }
-        int row_bits = 1;
-        while (row_bits < 31 && (1ll << row_bits) < nrows)
-            ++row_bits;
         if (sort_pairs_u64_u32(keys_in.as<uint64_t>(), keys_out.as<uint64_t>(), idx_in.as<uint32_t>(),
-                               idx_out.as<uint32_t>(), n, 32 + row_bits) != COMET_HIP_OK)
+                               idx_out.as<uint32_t>(), n, col_bits + row_bits) != COMET_HIP_OK)
             return fail();
         {
             KernelTimer t("coo_flag");
-            coo_flag<<<grid_for(n), dim3(256), 0, stream()>>>(n, keys_out.as<uint64_t>(), mode, flag.as<int64_t>());
+            coo_flag<<<grid_for(n), dim3(256), 0, stream()>>>(n, keys_out.as<uint64_t>(), col_bits, mode,
+                                                             flag.as<int64_t>());
         }
         if (exclusive_scan_i64(flag.as<int64_t>(), n, off.as<int64_t>()) != COMET_HIP_OK)
             return fail();
+        int any_bad = 0;
         if (hipMemcpyAsync(&kept, off.as<int64_t>() + n, sizeof(int64_t), hipMemcpyDeviceToHost, stream()) !=
                 hipSuccess ||
+            hipMemcpyAsync(&any_bad, bad.p, sizeof(int), hipMemcpyDeviceToHost, stream()) != hipSuccess ||
             hipStreamSynchronize(stream()) != hipSuccess) {
             set_error(COMET_HIP_ERR_HIP, "reading the entry count failed");
+            return fail();
+        }
+        if (any_bad) {
+            set_error(COMET_HIP_ERR_ARG, "a tuple lies outside the %lld x %lld matrix", (long long)nrows,
+                      (long long)ncols);
             return fail();
         }
     }
@@ -378,7 +405,8 @@ static Csr *coo_device_to_csr_struct(int64_t nrows, int64_t ncols, int64_t n, co
     }
     if (n > 0) {
         KernelTimer t("coo_compact");
-        coo_compact<<<grid_for(n), dim3(256), 0, stream()>>>(n, keys_out.as<uint64_t>(), idx_out.as<uint32_t>(),
+        coo_compact<<<grid_for(n), dim3(256), 0, stream()>>>(n, keys_out.as<uint64_t>(), col_bits,
+                                                            idx_out.as<uint32_t>(),
                                                             off.as<int64_t>(), val, crow.as<int32_t>(), c->crd,
                                                             c->val);
     }

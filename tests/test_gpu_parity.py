@@ -818,6 +818,15 @@ def test_reader_rejects_bad_input(tmp_path):
     row = np.array([0, 5], dtype=np.int64)
     h = L.comet_hip_csr_from_coo_i64(3, 3, 2, row.ctypes.data, row.ctypes.data, np.zeros(2).ctypes.data, 1)
     assert h == 0 and b"outside" in L.comet_hip_last_error()
+    # tuples that are already on the device are checked there
+    drow = rt.DeviceArray.from_numpy(np.array([0, 2, 1], dtype=np.int32))
+    dcol = rt.DeviceArray.from_numpy(np.array([1, 3, 0], dtype=np.int32))
+    dval = rt.DeviceArray.from_numpy(np.ones(3))
+    h = L.comet_hip_csr_from_coo_device(3, 3, 3, drow.ptr, dcol.ptr, dval.ptr, 1)
+    assert h == 0 and b"outside" in L.comet_hip_last_error()
+    dcol = rt.DeviceArray.from_numpy(np.array([1, 2, 0], dtype=np.int32))
+    M = rt.CsrMatrix.from_coo_device((3, 3), drow, dcol, dval)
+    assert M.to_arrays()[0].tolist() == [0, 1, 2, 3] and M.to_arrays()[1].tolist() == [1, 0, 2]
 
 
 # ----------------------------------------------------------------- SpMM: long rows through the column sweep
