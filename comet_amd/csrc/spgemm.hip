@@ -1087,21 +1087,28 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
                         __hip_atomic_fetch_add(&val[r], x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                     });
                     lds_barrier();
-                    for (int q = threadIdx.x; q < total; q += SG_T) {
+                    for (int q = threadIdx.x; q < total; q += SG_T)
                         store_streaming(&Cval[off + q], val[q]);
-                        val[q] = 0.0;
-                    }
-                    int64_t at = off + before;
+                    lds_barrier();
+                    // the values are out: their array now takes the list of the columns, so that these leave
+                    // through coalesced stores too (from their owners they would scatter, four bytes per lane)
+                    uint32_t *cols = reinterpret_cast<uint32_t *>(val);
+                    int at = before;
 #pragma unroll
                     for (int k = 0; k < SP_WPT; ++k) {
                         const int wi = threadIdx.x * SP_WPT + k;
                         if (wi < nb * SP_BLOCK_WORDS)
                             for (uint32_t bits = w[k]; bits; bits &= bits - 1)
-                                Ccrd[at++] = col0 + wi * 32 + __ffs(bits) - 1;
+                                cols[at++] = (uint32_t)(wi * 32 + __ffs(bits) - 1);
                         bm[wi] = 0;             // also the words beyond the cut: the next visit sets them again
                     }
-                    off += total;
                     lds_barrier();
+                    for (int q = threadIdx.x; q < total; q += SG_T)
+                        store_streaming(&Ccrd[off + q], col0 + (int)cols[q]);
+                    lds_barrier();
+                    for (int q = threadIdx.x; q < total; q += SG_T)
+                        val[q] = 0.0;           // nobody adds into it before the next visit's three barriers
+                    off += total;
                 }
                 cb += nb;
                 h_lo = h_hi;
