@@ -20,6 +20,8 @@ hipStream_t aux_stream();
 int aux_fork();
 int aux_join();
 int ensure_init();
+// looks up, for `device` (current), the address of the array the allocation-free SpMM keeps its scratch in
+int spmm_static_setup(int device);
 bool is_initialised();     // has any call brought the device up yet
 int set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int num_cus();

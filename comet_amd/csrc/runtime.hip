@@ -79,6 +79,7 @@ static int do_init(int device)
     COMET_HIPCHK(hipStreamCreate(&g_aux));
     COMET_HIPCHK(hipEventCreateWithFlags(&g_fork, hipEventDisableTiming));
     COMET_HIPCHK(hipEventCreateWithFlags(&g_join, hipEventDisableTiming));
+    COMET_CHK(spmm_static_setup(device));
     g_device = device;
     g_inited = true;
     return COMET_HIP_OK;

@@ -1319,6 +1319,91 @@ static int spmm_chunks(Csr *a, int64_t K, const double *B, int64_t ldb, double *
 }
 
 // ---------------------------------------------------------------------------
+// SpMM for callers that cannot allocate (code under graph capture, serving loops that forbid hipMalloc): the
+// chunk kernel and its fix-up with their scratch - the chunk -> row table and the carry slots of rows cut by a
+// chunk boundary - in one array that lives in the library's image instead of in allocated workspaces.  Every
+// device holds its own copy at its own address; the address is looked up once per device, when the library is
+// initialised there, and host code uses that pointer, never the array's name.
+// ---------------------------------------------------------------------------
+constexpr int64_t SPMM_STATIC_SLOTS = 8192;      // (64-column tiles of K) x (chunks of 256 nonzeros) the array has room for
+constexpr size_t SPMM_STATIC_TABLE_BYTES = sizeof(int32_t) * (size_t)SPMM_STATIC_SLOTS;
+constexpr size_t SPMM_STATIC_CARRY_BYTES = sizeof(double) * 2 * 64 * (size_t)SPMM_STATIC_SLOTS;
+static __device__ __align__(256) unsigned char spmm_static_scratch[SPMM_STATIC_TABLE_BYTES + SPMM_STATIC_CARRY_BYTES];
+constexpr int SPMM_STATIC_MAX_DEVICES = 64;
+static unsigned char *g_spmm_static_ptr[SPMM_STATIC_MAX_DEVICES];     // device address of the array, per device
+
+namespace comet {
+int spmm_static_setup(int device)
+{
+    if (device < 0 || device >= SPMM_STATIC_MAX_DEVICES)
+        return set_error(COMET_HIP_ERR_ARG, "device %d has no slot for the static SpMM scratch", device);
+    unsigned char *ptr = nullptr;
+    COMET_HIPCHK(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(spmm_static_scratch)));
+    g_spmm_static_ptr[device] = ptr;
+    return COMET_HIP_OK;
+}
+}  // namespace comet
+
+extern "C" int comet_hip_spmm_csr_f64_noalloc(int64_t csr, int64_t K, int64_t b_dptr, int64_t ldb, int64_t c_dptr,
+                                              int64_t ldc, int accumulate)
+{
+    if (!is_initialised())       // bringing the device up creates streams: the caller does that beforehand
+        return set_error(COMET_HIP_ERR_ARG, "comet_hip_spmm_csr_f64_noalloc: call comet_hip_init first");
+    Csr *a = csr_from_handle(csr);
+    if (!a)
+        return COMET_HIP_ERR_HANDLE;
+    if (K < 0 || ldb < K || ldc < K)
+        return set_error(COMET_HIP_ERR_ARG, "bad K/ldb/ldc (%lld, %lld, %lld)", (long long)K, (long long)ldb,
+                         (long long)ldc);
+    if (K == 0 || a->nrows == 0)
+        return COMET_HIP_OK;
+    if (!c_dptr || (a->nnz > 0 && !b_dptr))
+        return set_error(COMET_HIP_ERR_ARG, "null matrix passed to a sparse-dense matrix product");
+    const int64_t tiles = ceil_div(K, 64), nchunks = ceil_div(a->nnz, SPMM_CH);
+    if (tiles > 65535 || tiles * nchunks > SPMM_STATIC_SLOTS)
+        return set_error(COMET_HIP_ERR_SIZE,
+                         "comet_hip_spmm_csr_f64_noalloc: ceil(K/64) * ceil(nnz/%d) = %lld exceeds the %lld slots of the "
+                         "static scratch (nnz up to %lld at K <= 64); use comet_hip_spmm_csr_f64",
+                         SPMM_CH, (long long)(tiles * nchunks), (long long)SPMM_STATIC_SLOTS,
+                         (long long)(SPMM_STATIC_SLOTS * SPMM_CH));
+    int device = -1;
+    COMET_HIPCHK(hipGetDevice(&device));
+    unsigned char *scratch = device >= 0 && device < SPMM_STATIC_MAX_DEVICES ? g_spmm_static_ptr[device] : nullptr;
+    if (!scratch)
+        return set_error(COMET_HIP_ERR_ARG, "the static SpMM scratch was not set up on device %d", device);
+    double *C = (double *)c_dptr;
+    if (a->nnz == 0) {
+        if (!accumulate) {
+            const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div(a->nrows * K, 256), 65536);
+            fill_rows_f64<<<dim3(blocks), dim3(256), 0, stream()>>>(C, a->nrows, K, ldc, 0.0);
+            COMET_HIPCHK(hipGetLastError());
+        }
+        return COMET_HIP_OK;
+    }
+    // Every word the kernels read from the array is written earlier in the same call (the table in full, a carry
+    // slot by the chunk that leaves a piece of a row in it), so nothing has to be cleared between calls.
+    int32_t *chunk_row = reinterpret_cast<int32_t *>(scratch);
+    double *carry = reinterpret_cast<double *>(scratch + SPMM_STATIC_TABLE_BYTES);
+    spmm_chunk_rows<<<dim3((unsigned)ceil_div(nchunks, 256)), dim3(256), 0, stream()>>>(a->pos, a->nrows, nchunks,
+                                                                                         chunk_row);
+    const dim3 grid((unsigned)ceil_div(nchunks, SPMM_WAVES), (unsigned)tiles), block(SPMM_WAVES * 64);
+    const double *B = (const double *)b_dptr;
+    if (accumulate) {
+        spmm_csr_nnzsplit<true><<<grid, block, 0, stream()>>>(a->pos, a->crd, a->val, a->nnz, a->nrows, chunk_row,
+                                                              nchunks, B, ldb, C, ldc, K, carry, nullptr);
+        spmm_csr_fixup<true><<<grid, block, 0, stream()>>>(a->pos, a->nnz, chunk_row, nchunks, C, ldc, K, carry,
+                                                           nullptr);
+    } else {
+        spmm_csr_nnzsplit<false><<<grid, block, 0, stream()>>>(a->pos, a->crd, a->val, a->nnz, a->nrows, chunk_row,
+                                                               nchunks, B, ldb, C, ldc, K, carry, nullptr);
+        spmm_csr_fixup<false><<<grid, block, 0, stream()>>>(a->pos, a->nnz, chunk_row, nchunks, C, ldc, K, carry,
+                                                            nullptr);
+    }
+    COMET_HIPCHK(hipGetLastError());
+    return COMET_HIP_OK;
+}
+
+// ---------------------------------------------------------------------------
 // Dense operand on the left: y[j] (+)= sum_i x[i] * B[i,j] and
 // C[a,c] (+)= sum_b A[a,b] * B[b,c] with B in CSR.  The reference's nests run
 // over the dense index outermost and scatter into the output

@@ -76,6 +76,7 @@ SIGNATURES = {
     "comet_hip_csr_destroy": (_int, [_i64]),
     "comet_hip_spmv_csr_f64": (_int, [_i64, _i64, _i64, _int]),
     "comet_hip_spmm_csr_f64": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
+    "comet_hip_spmm_csr_f64_noalloc": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
     "comet_hip_spgemm_csr_symbolic": (_int, [_i64, _i64, _i64, _i64, _pi64]),
     "comet_hip_spgemm_csr_numeric": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64]),
     "comet_hip_spgemm_csr": (_i64, [_i64, _i64, _i64]),

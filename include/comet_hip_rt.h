@@ -102,6 +102,18 @@ int comet_hip_spmv_csr_f64(int64_t csr, int64_t x_dptr, int64_t y_dptr, int accu
 int comet_hip_spmm_csr_f64(int64_t csr, int64_t K, int64_t b_dptr, int64_t ldb,
                            int64_t c_dptr, int64_t ldc, int accumulate);
 
+/* The same product for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops and harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  Nothing is allocated or freed: the scratch
+ * of its kernels (chunk table and carry slots) is an 8 MiB array in the
+ * library's image, one copy per device.  Limits: comet_hip_init must have run;
+ * ceil(K/64) * ceil(nnz/256) <= 8192 (nnz <= 2,097,152 at K <= 64), larger
+ * products return COMET_HIP_ERR_SIZE.  Rows are summed exactly as
+ * comet_hip_spmm_csr_f64 sums them for a matrix below its long-row threshold.
+ * All calls on one device share the array: calls that overlap in time race. */
+int comet_hip_spmm_csr_f64_noalloc(int64_t csr, int64_t K, int64_t b_dptr, int64_t ldb,
+                                   int64_t c_dptr, int64_t ldc, int accumulate);
+
 /* ---- SpGEMM  C = A * B, CSR x CSR -> CSR, optional structural mask ---------
  * Symbolic phase: per-row count of distinct output columns and the row
  * pointer, replacing the mark-array nest of
