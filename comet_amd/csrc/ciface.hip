@@ -45,17 +45,31 @@ int64_t g_pending_c = 0;
 
 }  // namespace
 
-extern "C" void _mlir_ciface_comet_hip_spmv_csr_f64_i64(comet_memref_1d *pos, comet_memref_1d *crd,
-                                                         comet_memref_1d *val, comet_memref_1d *x, comet_memref_1d *y)
+void comet::forget_pending_product() { g_pending_c = 0; }
+
+// Every entry point exists for both index widths: i64 is what the CPU lowering passes, i32 what lowered code
+// built with --target=GPU passes (frontends/comet_dsl/comet.cpp:817-823 switches the index memrefs to i32).
+namespace {
+
+template <typename I>
+int64_t upload(int64_t nrows, int64_t ncols, const I *pos, const I *crd, const double *val)
 {
-    const char *who = "comet_hip_spmv_csr_f64_i64";
+    if constexpr (sizeof(I) == 8)
+        return comet_hip_csr_upload_i64(nrows, ncols, (const int64_t *)pos, (const int64_t *)crd, val);
+    else
+        return comet_hip_csr_upload_i32(nrows, ncols, (const int32_t *)pos, (const int32_t *)crd, val);
+}
+
+template <typename I>
+void spmv_ciface(const char *who, comet_memref_1d *pos, comet_memref_1d *crd, comet_memref_1d *val,
+                 comet_memref_1d *x, comet_memref_1d *y)
+{
     const int64_t nrows = pos->sizes[0] - 1, ncols = x->sizes[0];
     if (nrows < 0 || y->sizes[0] != nrows) {
         set_error(COMET_HIP_ERR_ARG, "y has %lld entries, A has %lld rows", (long long)y->sizes[0], (long long)nrows);
         die(who);
     }
-    int64_t a = comet_hip_csr_upload_i64(nrows, ncols, data1<int64_t>(pos, who), data1<int64_t>(crd, who),
-                                         data1<double>(val, who));
+    int64_t a = upload<I>(nrows, ncols, data1<I>(pos, who), data1<I>(crd, who), data1<double>(val, who));
     if (!a)
         die(who);
     DeviceBuf dx(ncols * 8), dy(nrows * 8);
@@ -69,10 +83,10 @@ extern "C" void _mlir_ciface_comet_hip_spmv_csr_f64_i64(comet_memref_1d *pos, co
     (void)comet_hip_csr_destroy(a);
 }
 
-extern "C" void _mlir_ciface_comet_hip_spmm_csr_f64_i64(comet_memref_1d *pos, comet_memref_1d *crd,
-                                                         comet_memref_1d *val, comet_memref_2d *B, comet_memref_2d *C)
+template <typename I>
+void spmm_ciface(const char *who, comet_memref_1d *pos, comet_memref_1d *crd, comet_memref_1d *val,
+                 comet_memref_2d *B, comet_memref_2d *C)
 {
-    const char *who = "comet_hip_spmm_csr_f64_i64";
     if (!B || !C || !B->aligned || !C->aligned) {
         set_error(COMET_HIP_ERR_ARG, "null memref");
         die(who);
@@ -83,8 +97,7 @@ extern "C" void _mlir_ciface_comet_hip_spmm_csr_f64_i64(comet_memref_1d *pos, co
         set_error(COMET_HIP_ERR_ARG, "B/C must be contiguous row-major with matching shapes");
         die(who);
     }
-    int64_t a = comet_hip_csr_upload_i64(nrows, ncols, data1<int64_t>(pos, who), data1<int64_t>(crd, who),
-                                         data1<double>(val, who));
+    int64_t a = upload<I>(nrows, ncols, data1<I>(pos, who), data1<I>(crd, who), data1<double>(val, who));
     if (!a)
         die(who);
     DeviceBuf db(ncols * K * 8), dc(nrows * K * 8);
@@ -97,12 +110,11 @@ extern "C" void _mlir_ciface_comet_hip_spmm_csr_f64_i64(comet_memref_1d *pos, co
     (void)comet_hip_csr_destroy(a);
 }
 
-extern "C" void _mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i64(
-    int64_t nrowsA, int64_t ncolsB, comet_memref_1d *Apos, comet_memref_1d *Acrd, comet_memref_1d *Aval,
-    comet_memref_1d *Bpos, comet_memref_1d *Bcrd, comet_memref_1d *Bval, comet_memref_1d *Mpos,
-    comet_memref_1d *Mcrd, comet_memref_1d *sizes)
+template <typename I>
+void spgemm_sizes_ciface(const char *who, int64_t nrowsA, int64_t ncolsB, comet_memref_1d *Apos, comet_memref_1d *Acrd,
+                         comet_memref_1d *Aval, comet_memref_1d *Bpos, comet_memref_1d *Bcrd, comet_memref_1d *Bval,
+                         comet_memref_1d *Mpos, comet_memref_1d *Mcrd, comet_memref_1d *sizes)
 {
-    const char *who = "comet_hip_spgemm_csr_sizes_f64_i64";
     const int64_t nrowsB = Bpos->sizes[0] - 1;
     if (Apos->sizes[0] - 1 != nrowsA || !sizes || sizes->sizes[0] < 1) {
         set_error(COMET_HIP_ERR_ARG, "inconsistent row counts or missing sizes memref");
@@ -112,17 +124,14 @@ extern "C" void _mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i64(
         (void)comet_hip_csr_destroy(g_pending_c);
         g_pending_c = 0;
     }
-    int64_t a = comet_hip_csr_upload_i64(nrowsA, nrowsB, data1<int64_t>(Apos, who), data1<int64_t>(Acrd, who),
-                                         data1<double>(Aval, who));
-    int64_t b = a ? comet_hip_csr_upload_i64(nrowsB, ncolsB, data1<int64_t>(Bpos, who), data1<int64_t>(Bcrd, who),
-                                             data1<double>(Bval, who))
-                  : 0;
+    int64_t a = upload<I>(nrowsA, nrowsB, data1<I>(Apos, who), data1<I>(Acrd, who), data1<double>(Aval, who));
+    int64_t b = a ? upload<I>(nrowsB, ncolsB, data1<I>(Bpos, who), data1<I>(Bcrd, who), data1<double>(Bval, who)) : 0;
     int64_t m = 0;
     if (a && b && Mpos && Mpos->sizes[0] > 0) {
         // a mask carries structure only; its device value array is all zeros
         const int64_t mnnz = Mcrd->sizes[0];
         double *zeros = (double *)calloc((size_t)(mnnz > 0 ? mnnz : 1), sizeof(double));
-        m = comet_hip_csr_upload_i64(nrowsA, ncolsB, data1<int64_t>(Mpos, who), data1<int64_t>(Mcrd, who), zeros);
+        m = zeros ? upload<I>(nrowsA, ncolsB, data1<I>(Mpos, who), data1<I>(Mcrd, who), zeros) : 0;
         free(zeros);
         if (!m)
             die(who);
@@ -134,17 +143,16 @@ extern "C" void _mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i64(
         die(who);
     int64_t nnz = 0;
     (void)comet_hip_csr_dims(g_pending_c, nullptr, nullptr, &nnz);
-    ((int64_t *)sizes->aligned + sizes->offset)[0] = nnz;
+    ((int64_t *)sizes->aligned + sizes->offset)[0] = nnz;       // sizes are `index` values for either width
     (void)comet_hip_csr_destroy(a);
     (void)comet_hip_csr_destroy(b);
     if (m)
         (void)comet_hip_csr_destroy(m);
 }
 
-extern "C" void _mlir_ciface_comet_hip_spgemm_csr_fill_f64_i64(comet_memref_1d *Cpos, comet_memref_1d *Ccrd,
-                                                                comet_memref_1d *Cval)
+template <typename I>
+void spgemm_fill_ciface(const char *who, comet_memref_1d *Cpos, comet_memref_1d *Ccrd, comet_memref_1d *Cval)
 {
-    const char *who = "comet_hip_spgemm_csr_fill_f64_i64";
     if (!g_pending_c) {
         set_error(COMET_HIP_ERR_ARG, "fill called without a preceding sizes call");
         die(who);
@@ -156,20 +164,24 @@ extern "C" void _mlir_ciface_comet_hip_spgemm_csr_fill_f64_i64(comet_memref_1d *
                   (long long)nnz);
         die(who);
     }
-    if (comet_hip_csr_download_i64(g_pending_c, (int64_t *)data1<int64_t>(Cpos, who),
-                                   (int64_t *)data1<int64_t>(Ccrd, who), (double *)data1<double>(Cval, who)))
+    int rc;
+    if constexpr (sizeof(I) == 8)
+        rc = comet_hip_csr_download_i64(g_pending_c, (int64_t *)data1<I>(Cpos, who), (int64_t *)data1<I>(Ccrd, who),
+                                        (double *)data1<double>(Cval, who));
+    else
+        rc = comet_hip_csr_download_i32(g_pending_c, (int32_t *)data1<I>(Cpos, who), (int32_t *)data1<I>(Ccrd, who),
+                                        (double *)data1<double>(Cval, who));
+    if (rc)
         die(who);
     (void)comet_hip_csr_destroy(g_pending_c);
     g_pending_c = 0;
 }
 
-extern "C" double _mlir_ciface_comet_hip_tricount_f64_i64(int64_t ncols, comet_memref_1d *pos, comet_memref_1d *crd,
-                                                           comet_memref_1d *val)
+template <typename I>
+double tricount_ciface(const char *who, int64_t ncols, comet_memref_1d *pos, comet_memref_1d *crd, comet_memref_1d *val)
 {
-    const char *who = "comet_hip_tricount_f64_i64";
     const int64_t nrows = pos->sizes[0] - 1;
-    int64_t l = comet_hip_csr_upload_i64(nrows, ncols, data1<int64_t>(pos, who), data1<int64_t>(crd, who),
-                                         data1<double>(val, who));
+    int64_t l = upload<I>(nrows, ncols, data1<I>(pos, who), data1<I>(crd, who), data1<double>(val, who));
     if (!l)
         die(who);
     double out = 0.0;
@@ -177,6 +189,69 @@ extern "C" double _mlir_ciface_comet_hip_tricount_f64_i64(int64_t ncols, comet_m
         die(who);
     (void)comet_hip_csr_destroy(l);
     return out;
+}
+
+}  // namespace
+
+extern "C" void _mlir_ciface_comet_hip_spmv_csr_f64_i64(comet_memref_1d *pos, comet_memref_1d *crd,
+                                                         comet_memref_1d *val, comet_memref_1d *x, comet_memref_1d *y)
+{
+    spmv_ciface<int64_t>("comet_hip_spmv_csr_f64_i64", pos, crd, val, x, y);
+}
+extern "C" void _mlir_ciface_comet_hip_spmv_csr_f64_i32(comet_memref_1d *pos, comet_memref_1d *crd,
+                                                         comet_memref_1d *val, comet_memref_1d *x, comet_memref_1d *y)
+{
+    spmv_ciface<int32_t>("comet_hip_spmv_csr_f64_i32", pos, crd, val, x, y);
+}
+
+extern "C" void _mlir_ciface_comet_hip_spmm_csr_f64_i64(comet_memref_1d *pos, comet_memref_1d *crd,
+                                                         comet_memref_1d *val, comet_memref_2d *B, comet_memref_2d *C)
+{
+    spmm_ciface<int64_t>("comet_hip_spmm_csr_f64_i64", pos, crd, val, B, C);
+}
+extern "C" void _mlir_ciface_comet_hip_spmm_csr_f64_i32(comet_memref_1d *pos, comet_memref_1d *crd,
+                                                         comet_memref_1d *val, comet_memref_2d *B, comet_memref_2d *C)
+{
+    spmm_ciface<int32_t>("comet_hip_spmm_csr_f64_i32", pos, crd, val, B, C);
+}
+
+extern "C" void _mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i64(
+    int64_t nrowsA, int64_t ncolsB, comet_memref_1d *Apos, comet_memref_1d *Acrd, comet_memref_1d *Aval,
+    comet_memref_1d *Bpos, comet_memref_1d *Bcrd, comet_memref_1d *Bval, comet_memref_1d *Mpos,
+    comet_memref_1d *Mcrd, comet_memref_1d *sizes)
+{
+    spgemm_sizes_ciface<int64_t>("comet_hip_spgemm_csr_sizes_f64_i64", nrowsA, ncolsB, Apos, Acrd, Aval, Bpos, Bcrd,
+                                 Bval, Mpos, Mcrd, sizes);
+}
+extern "C" void _mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i32(
+    int64_t nrowsA, int64_t ncolsB, comet_memref_1d *Apos, comet_memref_1d *Acrd, comet_memref_1d *Aval,
+    comet_memref_1d *Bpos, comet_memref_1d *Bcrd, comet_memref_1d *Bval, comet_memref_1d *Mpos,
+    comet_memref_1d *Mcrd, comet_memref_1d *sizes)
+{
+    spgemm_sizes_ciface<int32_t>("comet_hip_spgemm_csr_sizes_f64_i32", nrowsA, ncolsB, Apos, Acrd, Aval, Bpos, Bcrd,
+                                 Bval, Mpos, Mcrd, sizes);
+}
+
+extern "C" void _mlir_ciface_comet_hip_spgemm_csr_fill_f64_i64(comet_memref_1d *Cpos, comet_memref_1d *Ccrd,
+                                                                comet_memref_1d *Cval)
+{
+    spgemm_fill_ciface<int64_t>("comet_hip_spgemm_csr_fill_f64_i64", Cpos, Ccrd, Cval);
+}
+extern "C" void _mlir_ciface_comet_hip_spgemm_csr_fill_f64_i32(comet_memref_1d *Cpos, comet_memref_1d *Ccrd,
+                                                                comet_memref_1d *Cval)
+{
+    spgemm_fill_ciface<int32_t>("comet_hip_spgemm_csr_fill_f64_i32", Cpos, Ccrd, Cval);
+}
+
+extern "C" double _mlir_ciface_comet_hip_tricount_f64_i64(int64_t ncols, comet_memref_1d *pos, comet_memref_1d *crd,
+                                                           comet_memref_1d *val)
+{
+    return tricount_ciface<int64_t>("comet_hip_tricount_f64_i64", ncols, pos, crd, val);
+}
+extern "C" double _mlir_ciface_comet_hip_tricount_f64_i32(int64_t ncols, comet_memref_1d *pos, comet_memref_1d *crd,
+                                                           comet_memref_1d *val)
+{
+    return tricount_ciface<int32_t>("comet_hip_tricount_f64_i32", ncols, pos, crd, val);
 }
 
 // ---------------------------------------------------------------------------

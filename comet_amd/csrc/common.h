@@ -25,6 +25,9 @@ int spmm_static_setup(int device);
 bool is_initialised();     // has any call brought the device up yet
 int set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int num_cus();
+// comet_hip_finalize destroys every handle: the two places that keep one between calls drop theirs
+void forget_pending_reads();       // formats.hip: reader "sizes" call -> "read" call
+void forget_pending_product();     // ciface.hip: SpGEMM "sizes" call -> "fill" call
 
 #define COMET_HIPCHK(call)                                                                   \
     do {                                                                                     \

@@ -12,9 +12,11 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <cstring>
 #include <rocprim/device/device_radix_sort.hpp>
 
+#include <exception>
 #include <map>
 #include <string>
 #include <utility>
@@ -87,9 +89,18 @@ static int parse_mtx(const char *path, HostCoo *out)
             out->nrows = a;
             out->ncols = b;
             declared = array ? a * b : (symmetric ? 2 * c : c);
-            out->row.reserve((size_t)declared);
-            out->col.reserve((size_t)declared);
-            out->val.reserve((size_t)declared);
+            // every entry takes at least two bytes of text ("1\n" in an array file), so a count beyond the file's
+            // size is a corrupt size line, not a reason to reserve memory for it
+            if (declared > (int64_t)text.size() || declared >= (1ll << 32))
+                return set_error(COMET_HIP_ERR_SIZE, "%s: the size line declares %lld entries, the file holds %lld bytes",
+                                 path, (long long)declared, (long long)text.size());
+            try {
+                out->row.reserve((size_t)declared);
+                out->col.reserve((size_t)declared);
+                out->val.reserve((size_t)declared);
+            } catch (const std::exception &) {
+                return set_error(COMET_HIP_ERR_SIZE, "%s: no host memory for %lld entries", path, (long long)declared);
+            }
             have_sizes = true;
             continue;
         }
@@ -462,6 +473,8 @@ static bool known_mode(int mode) { return mode >= COMET_READ_DEFAULT && mode <= 
 // ---------------------------------------------------------------------------
 static std::map<std::pair<int32_t, int32_t>, int64_t> g_pending_reads;
 
+void comet::forget_pending_reads() { g_pending_reads.clear(); }
+
 static int file_name_of(int32_t file_id, std::string *out)
 {
     const char *v = nullptr;
@@ -561,7 +574,14 @@ extern "C" int64_t comet_hip_csr_from_coo_i64(int64_t nrows, int64_t ncols, int6
                   (long long)nrows, (long long)ncols, (long long)nnz, read_mode);
         return 0;
     }
-    std::vector<int32_t> r32((size_t)nnz), c32((size_t)nnz);
+    std::vector<int32_t> r32, c32;
+    try {
+        r32.resize((size_t)nnz);
+        c32.resize((size_t)nnz);
+    } catch (const std::exception &) {
+        set_error(COMET_HIP_ERR_SIZE, "no host memory to stage %lld tuples", (long long)nnz);
+        return 0;
+    }
     for (int64_t e = 0; e < nnz; ++e) {
         if (row[e] < 0 || row[e] >= nrows || col[e] < 0 || col[e] >= ncols) {
             set_error(COMET_HIP_ERR_ARG, "tuple %lld = (%lld,%lld) lies outside %lld x %lld", (long long)e,
@@ -600,7 +620,13 @@ extern "C" int64_t comet_hip_csr_from_dcsr_i64(int64_t nrows, int64_t ncols, int
         return 0;
     }
     // expand the stored-row list into one pointer per row; the arrays of the second level are CSR's already
-    std::vector<int64_t> pos((size_t)nrows + 1, 0);
+    std::vector<int64_t> pos;
+    try {
+        pos.assign((size_t)nrows + 1, 0);
+    } catch (const std::exception &) {
+        set_error(COMET_HIP_ERR_SIZE, "no host memory for the row pointers of %lld rows", (long long)nrows);
+        return 0;
+    }
     int64_t prev = -1;
     for (int64_t s = 0; s < nrows_stored; ++s) {
         const int64_t r = a1crd[s];
@@ -758,20 +784,17 @@ extern "C" void comet_hip_read_input_sizes_2D_f64(int32_t file_id, int32_t a1for
     s[10] = ncols;
 }
 
-extern "C" void comet_hip_read_input_2D_f64_i64(int32_t file_id, int32_t a1format, int32_t a1_tile_format,
-                                                int32_t a2format, int32_t a2_tile_format, int a1pos_rank,
-                                                void *a1pos_desc, int a1crd_rank, void *a1crd_desc,
-                                                int a1tile_pos_rank, void *a1tile_pos_desc, int a1tile_crd_rank,
-                                                void *a1tile_crd_desc, int a2pos_rank, void *a2pos_desc,
-                                                int a2crd_rank, void *a2crd_desc, int a2tile_pos_rank,
-                                                void *a2tile_pos_desc, int a2tile_crd_rank, void *a2tile_crd_desc,
-                                                int aval_rank, void *aval_desc, int32_t read_mode)
+// I = int64_t for the CPU lowering, int32_t for lowered code built with --target=GPU, which switches every index
+// memref to i32 (frontends/comet_dsl/comet.cpp:817-823); the reference's reader is one template over both
+// (SparseUtils.cpp:2403-2447).
+template <typename I>
+static void read_input_2D_impl(const char *who, int32_t file_id, int32_t a1format, int32_t a1_tile_format,
+                               int32_t a2format, int32_t a2_tile_format, void *a1pos_desc, void *a1crd_desc,
+                               void *a1tile_pos_desc, void *a1tile_crd_desc, void *a2pos_desc, void *a2crd_desc,
+                               void *a2tile_pos_desc, void *a2tile_crd_desc, void *aval_desc, int32_t read_mode)
 {
-    const char *who = "comet_hip_read_input_2D_f64_i64";
-    (void)a1pos_rank; (void)a1crd_rank; (void)a1tile_pos_rank; (void)a1tile_crd_rank; (void)a2pos_rank;
-    (void)a2crd_rank; (void)a2tile_pos_rank; (void)a2tile_crd_rank; (void)aval_rank;
-    int64_t *a1pos = memref_data<int64_t>(a1pos_desc), *a1crd = memref_data<int64_t>(a1crd_desc);
-    int64_t *a2pos = memref_data<int64_t>(a2pos_desc), *a2crd = memref_data<int64_t>(a2crd_desc);
+    I *a1pos = memref_data<I>(a1pos_desc), *a1crd = memref_data<I>(a1crd_desc);
+    I *a2pos = memref_data<I>(a2pos_desc), *a2crd = memref_data<I>(a2crd_desc);
     double *aval = memref_data<double>(aval_desc);
     const Layout lay = layout_of(a1format, a1_tile_format, a2format, a2_tile_format);
     if (lay == LAYOUT_OTHER || !a1pos || !a1crd || !a2pos || !a2crd || !aval) {
@@ -785,7 +808,7 @@ extern "C" void comet_hip_read_input_2D_f64_i64(int32_t file_id, int32_t a1forma
     void *all[8] = {a1pos_desc, a1crd_desc, a2pos_desc, a2crd_desc,
                     a1tile_pos_desc, a1tile_crd_desc, a2tile_pos_desc, a2tile_crd_desc};
     for (void *d : all) {
-        int64_t *p = memref_data<int64_t>(d);
+        I *p = memref_data<I>(d);
         if (p && ((comet_memref_1d *)d)->sizes[0] > 0)
             p[0] = -1;
     }
@@ -795,20 +818,95 @@ extern "C" void comet_hip_read_input_2D_f64_i64(int32_t file_id, int32_t a1forma
     int64_t nrows = 0, nnz = 0;
     (void)comet_hip_csr_dims(h, &nrows, nullptr, &nnz);
     int rc = COMET_HIP_OK;
-    if (lay == LAYOUT_CSR) {            // :1898-1936
-        a1pos[0] = nrows;
-        rc = comet_hip_csr_download_i64(h, a2pos, a2crd, aval);
-    } else if (lay == LAYOUT_COO) {     // :1855-1896
-        a1pos[0] = 0;
-        a1pos[1] = nnz;
-        rc = comet_hip_csr_to_coo_i64(h, a1crd, a2crd, aval);
-    } else {                            // DCSR :1983-2010
-        int64_t stored = 0;
-        rc = comet_hip_csr_to_dcsr_i64(h, &stored, a1crd, a2pos, a2crd, aval);
-        a1pos[0] = 0;
-        a1pos[1] = stored;
+    if constexpr (sizeof(I) == 8) {
+        int64_t *p1 = (int64_t *)a1pos, *c1 = (int64_t *)a1crd, *p2 = (int64_t *)a2pos, *c2 = (int64_t *)a2crd;
+        if (lay == LAYOUT_CSR) {            // :1898-1936
+            p1[0] = nrows;
+            rc = comet_hip_csr_download_i64(h, p2, c2, aval);
+        } else if (lay == LAYOUT_COO) {     // :1855-1896
+            p1[0] = 0;
+            p1[1] = nnz;
+            rc = comet_hip_csr_to_coo_i64(h, c1, c2, aval);
+        } else {                            // DCSR :1983-2010
+            int64_t stored = 0;
+            rc = comet_hip_csr_to_dcsr_i64(h, &stored, c1, p2, c2, aval);
+            p1[0] = 0;
+            p1[1] = stored;
+        }
+    } else {
+        int32_t *p1 = (int32_t *)a1pos, *c1 = (int32_t *)a1crd, *p2 = (int32_t *)a2pos, *c2 = (int32_t *)a2crd;
+        if (nnz > INT32_MAX) {
+            set_error(COMET_HIP_ERR_SIZE, "%lld entries do not fit 32-bit positions", (long long)nnz);
+            rc = COMET_HIP_ERR_SIZE;
+        } else if (lay == LAYOUT_CSR) {
+            p1[0] = (int32_t)nrows;
+            rc = comet_hip_csr_download_i32(h, p2, c2, aval);
+        } else {
+            // the COO and DCSR conversions produce 64-bit host arrays: narrow them here
+            std::vector<int64_t> w1, w2, wp;
+            try {
+                w1.resize((size_t)std::max<int64_t>(lay == LAYOUT_COO ? nnz : nrows, 1));
+                w2.resize((size_t)std::max<int64_t>(nnz, 1));
+                wp.resize((size_t)nrows + 1);
+            } catch (const std::exception &) {
+                set_error(COMET_HIP_ERR_SIZE, "no host memory to stage %lld entries", (long long)nnz);
+                die_reader(who);
+            }
+            if (lay == LAYOUT_COO) {
+                p1[0] = 0;
+                p1[1] = (int32_t)nnz;
+                rc = comet_hip_csr_to_coo_i64(h, w1.data(), w2.data(), aval);
+                for (int64_t e = 0; rc == COMET_HIP_OK && e < nnz; ++e) {
+                    c1[e] = (int32_t)w1[(size_t)e];
+                    c2[e] = (int32_t)w2[(size_t)e];
+                }
+            } else {
+                int64_t stored = 0;
+                rc = comet_hip_csr_to_dcsr_i64(h, &stored, w1.data(), wp.data(), w2.data(), aval);
+                p1[0] = 0;
+                p1[1] = (int32_t)stored;
+                for (int64_t r = 0; rc == COMET_HIP_OK && r < stored; ++r)
+                    c1[r] = (int32_t)w1[(size_t)r];
+                for (int64_t r = 0; rc == COMET_HIP_OK && r <= stored; ++r)
+                    p2[r] = (int32_t)wp[(size_t)r];
+                for (int64_t e = 0; rc == COMET_HIP_OK && e < nnz; ++e)
+                    c2[e] = (int32_t)w2[(size_t)e];
+            }
+        }
     }
     (void)comet_hip_csr_destroy(h);
     if (rc)
         die_reader(who);
+}
+
+extern "C" void comet_hip_read_input_2D_f64_i64(int32_t file_id, int32_t a1format, int32_t a1_tile_format,
+                                                int32_t a2format, int32_t a2_tile_format, int a1pos_rank,
+                                                void *a1pos_desc, int a1crd_rank, void *a1crd_desc,
+                                                int a1tile_pos_rank, void *a1tile_pos_desc, int a1tile_crd_rank,
+                                                void *a1tile_crd_desc, int a2pos_rank, void *a2pos_desc,
+                                                int a2crd_rank, void *a2crd_desc, int a2tile_pos_rank,
+                                                void *a2tile_pos_desc, int a2tile_crd_rank, void *a2tile_crd_desc,
+                                                int aval_rank, void *aval_desc, int32_t read_mode)
+{
+    (void)a1pos_rank; (void)a1crd_rank; (void)a1tile_pos_rank; (void)a1tile_crd_rank; (void)a2pos_rank;
+    (void)a2crd_rank; (void)a2tile_pos_rank; (void)a2tile_crd_rank; (void)aval_rank;
+    read_input_2D_impl<int64_t>("comet_hip_read_input_2D_f64_i64", file_id, a1format, a1_tile_format, a2format,
+                                a2_tile_format, a1pos_desc, a1crd_desc, a1tile_pos_desc, a1tile_crd_desc, a2pos_desc,
+                                a2crd_desc, a2tile_pos_desc, a2tile_crd_desc, aval_desc, read_mode);
+}
+
+extern "C" void comet_hip_read_input_2D_f64_i32(int32_t file_id, int32_t a1format, int32_t a1_tile_format,
+                                                int32_t a2format, int32_t a2_tile_format, int a1pos_rank,
+                                                void *a1pos_desc, int a1crd_rank, void *a1crd_desc,
+                                                int a1tile_pos_rank, void *a1tile_pos_desc, int a1tile_crd_rank,
+                                                void *a1tile_crd_desc, int a2pos_rank, void *a2pos_desc,
+                                                int a2crd_rank, void *a2crd_desc, int a2tile_pos_rank,
+                                                void *a2tile_pos_desc, int a2tile_crd_rank, void *a2tile_crd_desc,
+                                                int aval_rank, void *aval_desc, int32_t read_mode)
+{
+    (void)a1pos_rank; (void)a1crd_rank; (void)a1tile_pos_rank; (void)a1tile_crd_rank; (void)a2pos_rank;
+    (void)a2crd_rank; (void)a2tile_pos_rank; (void)a2tile_crd_rank; (void)aval_rank;
+    read_input_2D_impl<int32_t>("comet_hip_read_input_2D_f64_i32", file_id, a1format, a1_tile_format, a2format,
+                                a2_tile_format, a1pos_desc, a1crd_desc, a1tile_pos_desc, a1tile_crd_desc, a2pos_desc,
+                                a2crd_desc, a2tile_pos_desc, a2tile_crd_desc, aval_desc, read_mode);
 }

@@ -480,6 +480,61 @@ static int validate_host_csr(int64_t nrows, int64_t ncols, const I *pos, const I
         if (crd[p] < 0 || (int64_t)crd[p] >= ncols)
             return set_error(COMET_HIP_ERR_ARG, "crd[%lld] = %lld outside [0,%lld)", (long long)p,
                              (long long)crd[p], (long long)ncols);
+    // The kernels bisect rows and index on-chip windows with (column - window start): a row whose columns
+    // go down would put entries outside those windows.  Equal neighbours (duplicates) are fine.
+    for (int64_t i = 0; i < nrows; ++i)
+        for (int64_t p = (int64_t)pos[i] + 1; p < (int64_t)pos[i + 1]; ++p)
+            if (crd[p] < crd[p - 1])
+                return set_error(COMET_HIP_ERR_ARG,
+                                 "row %lld: column %lld follows column %lld; the columns of a row must not decrease "
+                                 "(comet_hip_csr_from_coo_i64 orders tuples)",
+                                 (long long)i, (long long)crd[p], (long long)crd[p - 1]);
+    return COMET_HIP_OK;
+}
+
+// The same checks for arrays that already sit in HBM: one wavefront per row.  *bad becomes non-zero if pos does
+// not start at 0, decreases, does not end at nnz, or a column is out of range or smaller than its left neighbour.
+__global__ __launch_bounds__(256) void csr_check_device(int64_t nrows, int64_t ncols, int64_t nnz,
+                                                        const int64_t *__restrict__ pos,
+                                                        const int32_t *__restrict__ crd, int32_t *__restrict__ bad)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+    if (wave == 0 && lane == 0 && (pos[0] != 0 || pos[nrows] != nnz))
+        *bad = 1;
+    for (int64_t r = wave; r < nrows; r += nwaves) {
+        const int64_t s = pos[r], e = pos[r + 1];
+        if (s < 0 || e < s || e > nnz) {        // entries of such a row are not touched
+            if (lane == 0)
+                *bad = 1;
+            continue;
+        }
+        for (int64_t p = s + lane; p < e; p += 64) {
+            const int32_t c = crd[p];
+            if (c < 0 || c >= ncols || (p > s && c < crd[p - 1]))
+                *bad = 1;
+        }
+    }
+}
+
+static Workspace g_check_flag;
+
+static int validate_device_csr(const Csr *c)
+{
+    COMET_CHK(g_check_flag.ensure(sizeof(int32_t), false));
+    int32_t *flag = (int32_t *)g_check_flag.ptr;
+    COMET_HIPCHK(hipMemsetAsync(flag, 0, sizeof(int32_t), stream()));
+    const unsigned blocks = (unsigned)std::min<int64_t>(std::max<int64_t>(ceil_div(c->nrows, 4), 1), 16384);
+    csr_check_device<<<dim3(blocks), dim3(256), 0, stream()>>>(c->nrows, c->ncols, c->nnz, c->pos, c->crd, flag);
+    COMET_HIPCHK(hipGetLastError());
+    int32_t bad = 0;
+    COMET_HIPCHK(hipMemcpyAsync(&bad, flag, sizeof(int32_t), hipMemcpyDeviceToHost, stream()));
+    COMET_HIPCHK(hipStreamSynchronize(stream()));
+    if (bad)
+        return set_error(COMET_HIP_ERR_ARG,
+                         "device CSR arrays are not a valid matrix: pos must start at 0, never decrease and end at nnz; "
+                         "columns must lie in [0, ncols) and must not decrease inside a row");
     return COMET_HIP_OK;
 }
 
@@ -504,6 +559,8 @@ int comet_hip_finalize(void)
     if (!g_inited)
         return COMET_HIP_OK;
     (void)hipStreamSynchronize(g_stream);
+    forget_pending_reads();       // handles kept between a "sizes" call and its "fill" call die with the rest
+    forget_pending_product();
     for (Csr *c : g_live)
         csr_release(c);
     g_live.clear();
@@ -707,6 +764,11 @@ int64_t comet_hip_csr_wrap(int64_t nrows, int64_t ncols, int64_t nnz, int64_t po
     c->crd = (int32_t *)crd_dptr;
     c->val = (double *)val_dptr;
     c->owns = false;
+    // an out-of-range column or row pointer would send the kernels outside their buffers: look once, now
+    if (validate_device_csr(c) != COMET_HIP_OK) {
+        csr_release(c);
+        return 0;
+    }
     return csr_register(c);
 }
 
@@ -791,7 +853,7 @@ int comet_hip_csr_invalidate(int64_t csr)
         return COMET_HIP_ERR_HANDLE;
     COMET_HIPCHK(hipStreamSynchronize(stream()));
     csr_drop_plans(c);
-    return COMET_HIP_OK;
+    return validate_device_csr(c);      // the arrays were rewritten: they are looked at again
 }
 
 int comet_hip_csr_destroy(int64_t csr)

@@ -516,7 +516,25 @@ extern "C" int comet_hip_ttgt_contract(const comet_ttgt_plan *plan, const int64_
         return set_error(COMET_HIP_ERR_ARG, "null argument to comet_hip_ttgt_contract");
     if (beta != 0.0 && beta != 1.0)
         return set_error(COMET_HIP_ERR_ARG, "beta must be 0 or 1 (got %g)", beta);
+    // the plan may come from anywhere: ranks index 8-entry arrays and each perm must be a permutation
+    auto is_perm = [](const int32_t *perm, int rank) {
+        unsigned seen = 0;
+        for (int i = 0; i < rank; ++i) {
+            if (perm[i] < 0 || perm[i] >= rank || (seen >> perm[i] & 1u))
+                return false;
+            seen |= 1u << perm[i];
+        }
+        return true;
+    };
+    if (plan->rankA < 1 || plan->rankA > 8 || plan->rankB < 1 || plan->rankB > 8 || plan->rankC < 1 || plan->rankC > 8)
+        return set_error(COMET_HIP_ERR_ARG, "plan ranks (%d, %d, %d) outside 1..8", plan->rankA, plan->rankB,
+                         plan->rankC);
+    if ((plan->transA && !is_perm(plan->permA, plan->rankA)) || (plan->transB && !is_perm(plan->permB, plan->rankB)) ||
+        (plan->transC && !is_perm(plan->permC, plan->rankC)))
+        return set_error(COMET_HIP_ERR_ARG, "a transpose of the plan is not a permutation of its tensor's dimensions");
     const int64_t M = plan->M, N = plan->N, K = plan->K;
+    if (M < 0 || N < 0 || K < 0)
+        return set_error(COMET_HIP_ERR_ARG, "negative GEMM extent in the plan");
     int64_t ta = 1, tb = 1, tc = 1;
     for (int i = 0; i < plan->rankA; ++i) ta *= a_shape[i];
     for (int i = 0; i < plan->rankB; ++i) tb *= b_shape[i];

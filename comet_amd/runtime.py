@@ -102,6 +102,7 @@ SIGNATURES = {
     "comet_hip_mtx_read_csr": (_i64, [C.c_char_p, _int]),
     "comet_hip_read_input_sizes_2D_f64": (None, [_i32, _i32, _i32, _i32, _i32, _int, _vp, _i32]),
     "comet_hip_read_input_2D_f64_i64": (None, [_i32, _i32, _i32, _i32, _i32] + [_int, _vp] * 9 + [_i32]),
+    "comet_hip_read_input_2D_f64_i32": (None, [_i32, _i32, _i32, _i32, _i32] + [_int, _vp] * 9 + [_i32]),
     "comet_hip_read_input_2D_handle": (_i64, [_i32, _i32]),
     "comet_hip_csr_from_coo_i64": (_i64, [_i64, _i64, _i64, _vp, _vp, _vp, _int]),
     "comet_hip_csr_from_coo_device": (_i64, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
@@ -128,6 +129,11 @@ SIGNATURES = {
     "_mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i64": (None, [_i64, _i64, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _m1]),
     "_mlir_ciface_comet_hip_spgemm_csr_fill_f64_i64": (None, [_m1, _m1, _m1]),
     "_mlir_ciface_comet_hip_tricount_f64_i64": (_f64, [_i64, _m1, _m1, _m1]),
+    "_mlir_ciface_comet_hip_spmv_csr_f64_i32": (None, [_m1, _m1, _m1, _m1, _m1]),
+    "_mlir_ciface_comet_hip_spmm_csr_f64_i32": (None, [_m1, _m1, _m1, _m2, _m2]),
+    "_mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i32": (None, [_i64, _i64, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _m1]),
+    "_mlir_ciface_comet_hip_spgemm_csr_fill_f64_i32": (None, [_m1, _m1, _m1]),
+    "_mlir_ciface_comet_hip_tricount_f64_i32": (_f64, [_i64, _m1, _m1, _m1]),
 }
 
 _lib = None

@@ -77,7 +77,10 @@ int64_t comet_hip_csr_upload_i32(int64_t nrows, int64_t ncols, const int32_t *po
  * the handle does not own them.  The kernels keep what they derive from a
  * matrix in its handle (re-ordered copies, block pointers, the transpose), so
  * after writing into wrapped arrays call comet_hip_csr_invalidate before the
- * handle is used again. */
+ * handle is used again.  Both calls look at the arrays once on the device
+ * (pos starts at 0, never decreases, ends at nnz; columns inside [0, ncols) and
+ * not decreasing inside a row) and refuse anything else: wrap returns 0,
+ * invalidate COMET_HIP_ERR_ARG. */
 int64_t comet_hip_csr_wrap(int64_t nrows, int64_t ncols, int64_t nnz,
                            int64_t pos_dptr, int64_t crd_dptr, int64_t val_dptr);
 int comet_hip_csr_dims(int64_t csr, int64_t *nrows, int64_t *ncols, int64_t *nnz);
@@ -240,6 +243,19 @@ void comet_hip_read_input_2D_f64_i64(int32_t file_id, int32_t a1format, int32_t 
                                      int a2tile_pos_rank, void *a2tile_pos_desc,
                                      int a2tile_crd_rank, void *a2tile_crd_desc,
                                      int aval_rank, void *aval_desc, int32_t read_mode);
+/* The reader for lowered code built with --target=GPU, whose index memrefs
+ * hold int32 (frontends/comet_dsl/comet.cpp:817-823): read_input_2D_f64_i32,
+ * SparseUtils.cpp:2403-2425.  Same protocol; the sizes call is shared (sizes are
+ * `index` values for either width). */
+void comet_hip_read_input_2D_f64_i32(int32_t file_id, int32_t a1format, int32_t a1_tile_format,
+                                     int32_t a2format, int32_t a2_tile_format,
+                                     int a1pos_rank, void *a1pos_desc, int a1crd_rank, void *a1crd_desc,
+                                     int a1tile_pos_rank, void *a1tile_pos_desc,
+                                     int a1tile_crd_rank, void *a1tile_crd_desc,
+                                     int a2pos_rank, void *a2pos_desc, int a2crd_rank, void *a2crd_desc,
+                                     int a2tile_pos_rank, void *a2tile_pos_desc,
+                                     int a2tile_crd_rank, void *a2tile_crd_desc,
+                                     int aval_rank, void *aval_desc, int32_t read_mode);
 /* The same read for lowered code that keeps tensors on the device: the CSR
  * handle itself (0 on failure), no host arrays.  Consumes what a preceding
  * sizes call for the same id and mode built, or reads the file now. */
@@ -256,7 +272,7 @@ int64_t comet_hip_read_input_2D_handle(int32_t file_id, int32_t read_mode);
 int64_t comet_hip_csr_from_coo_i64(int64_t nrows, int64_t ncols, int64_t nnz, const int64_t *row,
                                    const int64_t *col, const double *val, int read_mode);
 /* The same for tuples that already sit in HBM: int32 rows and columns, float64
- * values; indices must lie inside the matrix (not checked). */
+ * values; a tuple outside the matrix is refused (checked on the device). */
 int64_t comet_hip_csr_from_coo_device(int64_t nrows, int64_t ncols, int64_t nnz, int64_t row_dptr,
                                       int64_t col_dptr, int64_t val_dptr, int read_mode);
 int64_t comet_hip_csr_from_dcsr_i64(int64_t nrows, int64_t ncols, int64_t nrows_stored,
@@ -366,6 +382,22 @@ void _mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i64(int64_t nrowsA, int64_t nco
 void _mlir_ciface_comet_hip_spgemm_csr_fill_f64_i64(comet_memref_1d *Cpos, comet_memref_1d *Ccrd,
                                                     comet_memref_1d *Cval);
 double _mlir_ciface_comet_hip_tricount_f64_i64(int64_t ncols, comet_memref_1d *pos, comet_memref_1d *crd,
+                                               comet_memref_1d *val);
+
+/* The same five entry points for index memrefs of int32 (pos, crd and the mask's
+ * arrays; `sizes` stays int64): what lowered code built with --target=GPU passes
+ * (frontends/comet_dsl/comet.cpp:817-823). */
+void _mlir_ciface_comet_hip_spmv_csr_f64_i32(comet_memref_1d *pos, comet_memref_1d *crd, comet_memref_1d *val,
+                                             comet_memref_1d *x, comet_memref_1d *y);
+void _mlir_ciface_comet_hip_spmm_csr_f64_i32(comet_memref_1d *pos, comet_memref_1d *crd, comet_memref_1d *val,
+                                             comet_memref_2d *B, comet_memref_2d *C);
+void _mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i32(int64_t nrowsA, int64_t ncolsB,
+        comet_memref_1d *Apos, comet_memref_1d *Acrd, comet_memref_1d *Aval,
+        comet_memref_1d *Bpos, comet_memref_1d *Bcrd, comet_memref_1d *Bval,
+        comet_memref_1d *Mpos, comet_memref_1d *Mcrd, comet_memref_1d *sizes);
+void _mlir_ciface_comet_hip_spgemm_csr_fill_f64_i32(comet_memref_1d *Cpos, comet_memref_1d *Ccrd,
+                                                    comet_memref_1d *Cval);
+double _mlir_ciface_comet_hip_tricount_f64_i32(int64_t ncols, comet_memref_1d *pos, comet_memref_1d *crd,
                                                comet_memref_1d *val);
 
 /* ---- host utilities of the reference's runtime ----------------------------

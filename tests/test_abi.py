@@ -146,3 +146,13 @@ def test_host_utilities_print_sort_and_time(tmp_path):
                         "data = \n9,1,3,7,8,2,\n"
                         "data = \n1,2,3,4,5,\n"
                         "ELAPSED_TIME = 2.500000\n")
+
+
+def test_corrupt_size_lines_and_plans_are_refused_without_a_gpu(tmp_path):
+    """Sizes taken from a file or a caller are bounded before anything is reserved or indexed with them."""
+    L = rt.lib()
+    path = str(tmp_path / "big.mtx")
+    with open(path, "w") as f:
+        f.write("%%MatrixMarket matrix coordinate real general\n3 3 4000000000000\n1 1 1.0\n")
+    assert L.comet_hip_mtx_read_csr(path.encode(), 1) == 0
+    assert b"declares" in L.comet_hip_last_error() or b"HIP device" in L.comet_hip_last_error()

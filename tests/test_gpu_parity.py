@@ -63,6 +63,13 @@ def test_bad_inputs_are_rejected():
         rt.CsrMatrix.from_arrays((2, 2), pos, np.zeros(1, dtype=np.int64), np.zeros(1))
     with pytest.raises(rt.CometHipError):      # column out of range
         rt.CsrMatrix.from_arrays((1, 2), np.array([0, 1]), np.array([5]), np.ones(1))
+    with pytest.raises(rt.CometHipError) as e:   # columns of a row must not decrease (duplicates may stay)
+        rt.CsrMatrix.from_arrays((2, 4), np.array([0, 3, 4]), np.array([0, 2, 1, 3]), np.ones(4))
+    assert "must not decrease" in str(e.value)
+    rt.CsrMatrix.from_arrays((2, 4), np.array([0, 3, 4]), np.array([1, 1, 2, 0]), np.ones(4))
+    with pytest.raises(rt.CometHipError):
+        rt.CsrMatrix.from_arrays((2, 4), np.array([0, 3, 4], dtype=np.int32), np.array([3, 2, 2, 0], dtype=np.int32),
+                                 np.ones(4))
     assert rt.lib().comet_hip_spmv_csr_f64(12345, 0, 0, 0) != 0      # unknown handle
     A = rt.CsrMatrix.from_arrays((1, 2), np.array([0, 1]), np.array([1]), np.ones(1))
     B = rt.CsrMatrix.from_arrays((3, 2), np.array([0, 0, 0, 0]), np.zeros(0, dtype=np.int64), np.zeros(0))
@@ -478,6 +485,64 @@ def test_spgemm_rows_with_more_entries_than_lanes(wide, monkeypatch):
     _spgemm_check(a, b, m)
 
 
+def test_spgemm_rmat_scale16_row_blocks_vs_checker():
+    """C = A*A on the benchmark's own generator at scale 16, edge factor 16 (65,536 vertices, 1.8 M entries,
+    1.24e9 products): the symbolic phase over all rows, the numeric phase on sampled blocks of 64 rows - the block
+    with the heaviest row, the hub rows at the low ids, the tail, and random ones - against the checker.  Real
+    R-MAT rows of every class (values in a slab, several column blocks per visit, one block per visit) go through
+    the kernel that serves their class."""
+    scale = 16
+    n = 1 << scale
+    pos, crd, val = gen.rmat_symmetric_csr(scale=scale, edge_factor=16, seed=20)
+    deg = np.diff(pos)
+    rowprod = np.zeros(n, dtype=np.int64)
+    nz = deg > 0
+    rowprod[nz] = np.add.reduceat(deg[crd], pos[:-1][nz])
+    A = rt.CsrMatrix.from_arrays((n, n), pos, crd, val)
+    dpos, nnzC = rt.spgemm_symbolic(A, A)
+    hpos = dpos.to_numpy()
+    assert hpos[0] == 0 and hpos[-1] == nnzC and np.all(np.diff(hpos) >= 0)
+    rng = np.random.default_rng(5)
+    starts = {int(np.argmax(rowprod)) // 64 * 64, 0, 64, n - 64, n // 2}
+    starts |= {int(b) * 64 for b in rng.choice(n // 64, 10, replace=False)}
+    rt.profile_reset()
+    rt.profile_enable(True)
+    checked = 0
+    for r0 in sorted(starts):
+        r1 = r0 + 64
+        cp, cc, cv = orc.spgemm(pos, crd, val, pos, crd, val, n, rows=(r0, r1))
+        assert np.array_equal(cp, hpos[r0:r1 + 1] - hpos[r0]), f"row pointer of rows [{r0},{r1})"
+        cnt = int(hpos[r1] - hpos[r0])
+        dcrd, dval = rt.DeviceArray(max(cnt, 1), np.int32), rt.DeviceArray(max(cnt, 1))
+        rt.spgemm_numeric(A, A, dpos, r0, r1, dcrd, dval)
+        gc, gv = dcrd.to_numpy(cnt), dval.to_numpy(cnt)
+        assert np.array_equal(gc, cc), f"columns of rows [{r0},{r1})"
+        assert np.all(np.abs(gv - cv) <= RTOL * np.abs(cv)), f"values of rows [{r0},{r1})"      # all products positive
+        checked += int(rowprod[r0:r1].sum())
+    rt.sync()
+    fired = rt.profile_report()
+    rt.profile_enable(False)
+    for k in ("spgemm_numeric", "spgemm_numeric_span", "spgemm_numeric_dense"):
+        assert k in fired and fired[k][0] > 0, f"{k} never ran on these rows"
+    assert checked > 50_000_000
+    # the masked product C<A> = A*A on the same blocks (structure = mask entries that receive a product)
+    mpos, mnnz = rt.spgemm_symbolic(A, A, mask=A)
+    hm = mpos.to_numpy()
+    for r0 in sorted(starts)[:6]:
+        r1 = r0 + 64
+        cp, cc, cv = orc.spgemm(pos, crd, val, pos, crd, val, n, mask=(pos, crd), rows=(r0, r1))
+        assert np.array_equal(cp, hm[r0:r1 + 1] - hm[r0])
+        cnt = int(hm[r1] - hm[r0])
+        dcrd, dval = rt.DeviceArray(max(cnt, 1), np.int32), rt.DeviceArray(max(cnt, 1))
+        rt.spgemm_numeric(A, A, mpos, r0, r1, dcrd, dval, mask=A)
+        assert np.array_equal(dcrd.to_numpy(cnt), cc)
+        assert np.all(np.abs(dval.to_numpy(cnt) - cv) <= RTOL * np.abs(cv))
+    # and the triangle count of the same graph
+    lpos, lcrd, lval = gen.strictly_lower(pos, crd, np.ones_like(val))
+    L = rt.CsrMatrix.from_arrays((n, n), lpos, lcrd, lval)
+    assert rt.triangle_count(L) == orc.tricount_masked(lpos, lcrd, lval)
+
+
 def test_spgemm_empty_and_repeatable():
     Z = rt.CsrMatrix.from_arrays((3, 3), np.zeros(4, dtype=np.int64), np.zeros(0, dtype=np.int64), np.zeros(0))
     p, c, v = rt.spgemm(Z, Z).to_arrays()
@@ -611,29 +676,41 @@ def test_ttgt_benchmark_contraction_scaled_down():
 
 
 # ----------------------------------------------------------------- memref entry points
-def test_mlir_ciface_entry_points(golden, golden_dir):
+@pytest.mark.parametrize("idt", [np.int64, np.int32])
+def test_mlir_ciface_entry_points(golden, golden_dir, idt):
+    """The memref-descriptor forms for both index widths: i64 (CPU lowering) and i32 (what --target=GPU makes
+    the lowered code pass, frontends/comet_dsl/comet.cpp:817-823)."""
+    sfx = "i64" if idt == np.int64 else "i32"
+    fn = lambda name: getattr(rt.lib(), f"_mlir_ciface_comet_hip_{name}_f64_{sfx}")
     (nr, nc), pos, crd, val = _mtx(golden_dir, "test_rank2.mtx")
-    L = rt.lib()
+    pos, crd = pos.astype(idt), crd.astype(idt)
     x, y = np.full(nc, 1.7), np.zeros(nr)
-    L._mlir_ciface_comet_hip_spmv_csr_f64_i64(rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val), rt.memref1d(x),
-                                              rt.memref1d(y))
+    fn("spmv_csr")(rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val), rt.memref1d(x), rt.memref1d(y))
     assert orc.format_f64(y) == golden["spmv_csr"]["printed"]
     B, Cm = np.full((nc, 4), 1.7), np.zeros((nr, 4))
-    L._mlir_ciface_comet_hip_spmm_csr_f64_i64(rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val), rt.memref2d(B),
-                                              rt.memref2d(Cm))
+    fn("spmm_csr")(rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val), rt.memref2d(B), rt.memref2d(Cm))
     assert orc.format_f64(Cm) == golden["spmm_csr"]["printed"]
-    sizes = np.zeros(1, dtype=np.int64)
-    empty = np.zeros(0, dtype=np.int64)
-    L._mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i64(nr, nc, rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val),
-                                                      rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val),
-                                                      rt.memref1d(empty), rt.memref1d(empty), rt.memref1d(sizes))
+    sizes = np.zeros(1, dtype=np.int64)          # sizes are `index` values for either width
+    empty = np.zeros(0, dtype=idt)
+    fn("spgemm_csr_sizes")(nr, nc, rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val),
+                           rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val),
+                           rt.memref1d(empty), rt.memref1d(empty), rt.memref1d(sizes))
     assert sizes[0] == 9
-    cp, cc, cv = np.zeros(nr + 1, dtype=np.int64), np.zeros(9, dtype=np.int64), np.zeros(9)
-    L._mlir_ciface_comet_hip_spgemm_csr_fill_f64_i64(rt.memref1d(cp), rt.memref1d(cc), rt.memref1d(cv))
+    cp, cc, cv = np.zeros(nr + 1, dtype=idt), np.zeros(9, dtype=idt), np.zeros(9)
+    fn("spgemm_csr_fill")(rt.memref1d(cp), rt.memref1d(cc), rt.memref1d(cv))
     g = golden["spgemm_csr"]
     assert cp.tolist() == g["pos"] and cc.tolist() == g["crd"] and orc.format_f64(cv) == g["printed_val"]
+    # the masked product through the same pair of calls (mask = B, the reference's masked golden)
+    fn("spgemm_csr_sizes")(nr, nc, rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val),
+                           rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val),
+                           rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(sizes))
+    gm = golden["spgemm_csr_masked"]
+    assert sizes[0] == len(gm["crd"])
+    cp, cc, cv = np.zeros(nr + 1, dtype=idt), np.zeros(int(sizes[0]), dtype=idt), np.zeros(int(sizes[0]))
+    fn("spgemm_csr_fill")(rt.memref1d(cp), rt.memref1d(cc), rt.memref1d(cv))
+    assert cp.tolist() == gm["pos"] and cc.tolist() == gm["crd"] and orc.format_f64(cv) == gm["printed_val"]
     (tr, tc), tpos, tcrd, tval = _mtx(golden_dir, "tc.mtx", 2)
-    assert L._mlir_ciface_comet_hip_tricount_f64_i64(tc, rt.memref1d(tpos), rt.memref1d(tcrd), rt.memref1d(tval)) == 5.0
+    assert fn("tricount")(tc, rt.memref1d(tpos.astype(idt)), rt.memref1d(tcrd.astype(idt)), rt.memref1d(tval)) == 5.0
 
 
 # ----------------------------------------------------------------- input side and other layouts
@@ -656,15 +733,18 @@ def _desc(a):
     return m, C.cast(C.pointer(m), C.c_void_p)
 
 
-def _memref_i64(n):
-    a = np.full(max(n, 1), 7, dtype=np.int64)
+def _memref_idx(n, idt=np.int64):
+    a = np.full(max(n, 1), 7, dtype=idt)
     return (a,) + _desc(a)
 
 
+@pytest.mark.parametrize("idt", [np.int64, np.int32])
 @pytest.mark.parametrize("layout", ["CSR", "COO", "DCSR"])
-def test_reader_file_id_protocol(golden, golden_dir, monkeypatch, layout):
-    """The two reader calls with the reference's argument lists, for the three layouts its matrix tests use."""
+def test_reader_file_id_protocol(golden, golden_dir, monkeypatch, layout, idt):
+    """The two reader calls with the reference's argument lists, for the three layouts its matrix tests use and
+    both index widths (read_input_2D_f64_i64 / _i32, lib/ExecutionEngine/SparseUtils.cpp:2403-2447)."""
     L = rt.lib()
+    read = L.comet_hip_read_input_2D_f64_i64 if idt == np.int64 else L.comet_hip_read_input_2D_f64_i32
     monkeypatch.setenv("SPARSE_FILE_NAME3", os.path.join(golden_dir, "test_rank2.mtx"))
     fmt = {"CSR": (0, 0, 1, 0), "COO": (2, 0, 3, 0), "DCSR": (1, 0, 1, 0)}[layout]
     for mode in (1, 3):
@@ -681,13 +761,13 @@ def test_reader_file_id_protocol(golden, golden_dir, monkeypatch, layout):
         else:
             stored = len(want[1])
             assert sizes[:11].tolist() == [2, stored, 0, 0, stored + 1, len(crd), 0, 0, len(crd), nr, nc]
-        arrs = [_memref_i64(int(sizes[i])) for i in range(8)]
+        arrs = [_memref_idx(int(sizes[i]), idt) for i in range(8)]
         aval = np.zeros(max(int(sizes[8]), 1))
         args = []
         for i in (0, 1, 2, 3, 4, 5, 6, 7):
             args += [1, arrs[i][2]]
         aval_m, aval_p = _desc(aval)
-        L.comet_hip_read_input_2D_f64_i64(3, *fmt, *args, 1, aval_p, mode)
+        read(3, *fmt, *args, 1, aval_p, mode)
         a1pos, a1crd, a2pos, a2crd = (arrs[i][0] for i in (0, 1, 4, 5))
         assert arrs[2][0][0] == -1 and arrs[3][0][0] == -1 and arrs[6][0][0] == -1 and arrs[7][0][0] == -1
         assert np.array_equal(aval[:len(val)], val)
@@ -960,6 +1040,65 @@ def test_vecmat_densemat_vs_checker(n, m, M, density, seed):
     out = rt.eltwise_mult_dense(B, dD, rt.DeviceArray.from_numpy(keep)).to_numpy()
     keep[np.repeat(np.arange(n), np.diff(pos)), crd] = v
     assert np.array_equal(out, keep)
+
+
+def test_ttgt_refuses_a_plan_that_is_not_one():
+    """A plan handed in by the caller is checked before its ranks and permutations index anything."""
+    import copy
+    A = rt.DeviceArray.from_numpy(gen.dense((4, 5, 6), seed=1))
+    B = rt.DeviceArray.from_numpy(gen.dense((6, 5, 3), seed=2))
+    plan = rt.ttgt_plan("abc", "cbd", "ad", {"a": 4, "b": 5, "c": 6, "d": 3}, 1)
+    good, _ = rt.ttgt_contract("abc", "cbd", "ad", A, B, plan=plan)
+    assert good.to_numpy().shape == (4, 3)
+    for field, value in (("rankC", 9), ("rankA", 0), ("permA", (0, 0, 2)), ("permB", (0, 1, 7))):
+        bad = copy.copy(plan)
+        if field.startswith("perm"):
+            setattr(bad, "trans" + field[-1], 1)
+            arr = getattr(bad, field)
+            for i, v in enumerate(value):
+                arr[i] = v
+        else:
+            setattr(bad, field, value)
+        with pytest.raises(rt.CometHipError):
+            rt.ttgt_contract("abc", "cbd", "ad", A, B, plan=bad)
+
+
+def test_wrapped_device_arrays_are_checked():
+    """comet_hip_csr_wrap and comet_hip_csr_invalidate look at caller-filled device arrays once and refuse what
+    would send a kernel outside its buffers; nothing here launches a product on bad data."""
+    L = rt.lib()
+    good = (np.array([0, 2, 2, 5], dtype=np.int64), np.array([0, 3, 1, 1, 2], dtype=np.int32), np.ones(5))
+
+    def wrap(pos, crd, nnz=5, ncols=4):
+        dpos, dcrd, dval = rt.DeviceArray.from_numpy(pos), rt.DeviceArray.from_numpy(crd), rt.DeviceArray.from_numpy(good[2])
+        return L.comet_hip_csr_wrap(3, ncols, nnz, dpos.ptr, dcrd.ptr, dval.ptr), (dpos, dcrd, dval)
+
+    h, keep = wrap(good[0], good[1])
+    assert h != 0
+    for pos, crd, kw in [
+        (good[0], np.array([0, 4, 1, 1, 2], dtype=np.int32), {}),                    # column == ncols
+        (good[0], np.array([0, -1, 1, 1, 2], dtype=np.int32), {}),                   # negative column
+        (good[0], np.array([3, 0, 1, 1, 2], dtype=np.int32), {}),                    # columns go down inside row 0
+        (np.array([0, 3, 2, 5], dtype=np.int64), good[1], {}),                       # pos decreases
+        (np.array([1, 2, 2, 5], dtype=np.int64), good[1], {}),                       # pos[0] != 0
+        (good[0], good[1], {"nnz": 4}),                                              # pos[nrows] != nnz
+        (np.array([0, 2, 9, 5], dtype=np.int64), good[1], {}),                       # a row pointer past nnz
+    ]:
+        bad, _keep = wrap(pos, crd, **kw)
+        assert bad == 0
+        assert b"not a valid matrix" in L.comet_hip_last_error()
+    # arrays rewritten in place: invalidate looks again
+    keep[1].free()
+    assert L.comet_hip_csr_destroy(h) == 0
+    dpos, dcrd, dval = (rt.DeviceArray.from_numpy(a) for a in good)
+    h = L.comet_hip_csr_wrap(3, 4, 5, dpos.ptr, dcrd.ptr, dval.ptr)
+    assert h != 0
+    worse = np.array([0, 3, 1, 7, 2], dtype=np.int32)
+    assert L.comet_hip_memcpy(dcrd.ptr, worse.ctypes.data, worse.nbytes, 0) == 0
+    assert L.comet_hip_csr_invalidate(h) == 1           # COMET_HIP_ERR_ARG
+    assert L.comet_hip_memcpy(dcrd.ptr, good[1].ctypes.data, good[1].nbytes, 0) == 0
+    assert L.comet_hip_csr_invalidate(h) == 0
+    assert L.comet_hip_csr_destroy(h) == 0
 
 
 def test_wrapped_arrays_changed_in_place_need_invalidate():
