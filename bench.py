@@ -1,12 +1,14 @@
 #!/usr/bin/env python3
 """Benchmark of the index-tree kernel path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload spmm|spmv|sddmm|ttgt|tricount|spgemm|coo2csr]
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+                    [--workload headline|spmm|spgemm|tricount|spmv|ttgt|sddmm|coo2csr|copy|gather]
 
 A step is one pass of the kernel over one batch of seeded synthetic input that is already
 resident in HBM.  The default workload is the one the headline metric is quoted on: CSR SpMM,
-A 500,000 x 500,000 with power-law rows (mean 16, cap 4096), B 500,000 x 64 fp64.
-Prints ONE JSON line.  `roofline` describes the dominant kernel: algorithmic bytes (or flops)
+A 500,000 x 500,000 with power-law rows (mean 16, cap 4096), B 500,000 x 64 fp64; the default run adds, under
+"also", short runs of the other workloads the metric names (SpGEMM and masked SpGEMM at R-MAT scale 20) and of
+SpMV and the TTGT contraction.  Prints ONE JSON line.  `roofline` describes the dominant kernel: algorithmic bytes (or flops)
 per launch divided by that kernel's average duration, measured here with HIP events on the
 library's stream.  `cpu_baseline` is the CPU checker (oracle/, a restatement of the loop nests
 COMET generates) timed on this machine's host cores on a bounded sample of the same workload.
@@ -24,14 +26,55 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP64_MFMA_PEAK_TFLOPS = 78.6  # MI355X dense fp64 matrix, published
-# HBM bytes per SpMM product (all of its kernels) on the default workload, from rocprofv3 --pmc FETCH_SIZE (x 2.000)
-# and WRITE_SIZE (x 1.000), factors from a 1 GiB copy kernel; see profiles/spmm_kernels__spmm_zipf_500k_k64.txt
-SPMM_TRAFFIC_BYTES = int((436_260 * 2.000 + 272_815 * 1.000) * 1024)
-# the same two counters for the other workloads at their default sizes (per step; profiles/*.txt hold the tables)
-SPMV_TRAFFIC_BYTES = int((124_163 * 2.000 + 31_250 * 1.000) * 1024)            # four column-block passes
-SDDMM_TRAFFIC_BYTES = int((2_288_233 * 2.000 + 312_341 * 1.000) * 1024)        # kernel + transpose of D
-TRICOUNT_TRAFFIC_BYTES = int((20_166_583 * 2.000 + 37_909 * 1.000) * 1024)     # both masked-sum kernels
-SPGEMM_TRAFFIC_BYTES = int((566_358_591 * 2.000 + 281_840_080 * 1.000) * 1024)  # symbolic + the numeric kernels of 6 blocks
+
+
+def _sha12(path):
+    import hashlib
+    with open(os.path.join(ROOT, path), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:12]
+
+
+def measured_traffic(workload):
+    """HBM-side bytes per step from the rocprofv3 --pmc runs recorded in profiles/*.txt, or None.
+
+    A profile summary carries one line per workload,
+        TRAFFIC workload=<name> bytes=<per step> ... sources=<file>:<sha256[:12]>[,<file>:<sha>...]
+    naming the kernel sources the counters were read on.  The figure is reported only while those files are
+    unchanged: after any edit of a kernel source it is null until the counters are read again."""
+    import glob
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.txt"))):
+        with open(path) as f:
+            for line in f:
+                if not line.startswith("TRAFFIC "):
+                    continue
+                kv = dict(tok.split("=", 1) for tok in line.split()[1:] if "=" in tok)
+                if kv.get("workload") != workload:
+                    continue
+                try:
+                    same = all(_sha12(src) == sha for src, sha in (t.rsplit(":", 1) for t in kv["sources"].split(",")))
+                except (OSError, KeyError, ValueError):
+                    same = False
+                return (int(kv["bytes"]), os.path.basename(path)) if same else (None, os.path.basename(path) + " (stale: kernel sources changed since the counters were read)")
+    return None, None
+
+
+def mem_free(rt):
+    import ctypes as C
+    f, t = C.c_int64(), C.c_int64()
+    rt._check(rt.lib().comet_hip_mem_info(C.byref(f), C.byref(t)), "comet_hip_mem_info")
+    return f.value
+
+
+def first_call(rt, fn):
+    """Wall time of the first call of `fn` (device drained before and after) and the device memory it keeps:
+    what a program that multiplies once pays on top of a steady-state step (plans cached in the handle,
+    workspaces)."""
+    rt.sync()
+    free0 = mem_free(rt)
+    t0 = time.perf_counter()
+    fn()
+    rt.sync()
+    return (time.perf_counter() - t0) * 1e3, free0 - mem_free(rt)
 
 
 _T0 = time.perf_counter()
@@ -103,19 +146,18 @@ def bench_spmm(rt, orc, gen, args):
     dB = rt.DeviceArray.from_numpy(B)
     dC = rt.DeviceArray((n, K))
     step = lambda: rt.spmm(A, dB, dC, accumulate=False)
-    step()
-    rt.sync()
+    first_ms, kept_bytes = first_call(rt, step)
     wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
     kt = kernel_times(rt, step, args.steps)
     flops = 2.0 * nnz * K
     ib = 4
     alg_bytes = nnz * (8 + ib) + (n + 1) * ib + 8 * n * K + 8 * n * K
-    # one product = the column sweep over the long rows + the chunk kernel over the rest (+ two small
-    # kernels that stitch rows together); the algorithmic bytes are those of the whole product, so the
-    # roofline is taken over the sum of their launch durations
-    parts = [k for k in ("spmm_heavy_sweep", "spmm_csr_nnzsplit", "spmm_heavy_combine", "spmm_csr_fixup") if k in kt]
-    dom = " + ".join(parts)
-    dom_ms = sum(kt[k]["avg_ms"] * kt[k]["launches"] for k in parts) / args.steps
+    # one product = several kernels (sweep, chunk kernel, the kernels that stitch rows together, fills); the
+    # algorithmic bytes are those of the whole product, so the roofline is taken over the timed step
+    dom = " + ".join(sorted(kt))
+    dom_ms = dev_ms
+    kernel_sum_ms = sum(v["avg_ms"] * v["launches"] for v in kt.values()) / args.steps
+    traffic, traffic_src = measured_traffic("spmm_csr_zipf") if (n, K) == (500_000, 64) else (None, None)
     # parity of what was just timed, on a sample of rows (full check lives in tests/)
     got = dC.to_numpy()
     rows = np.random.default_rng(0).choice(n, 2000, replace=False)
@@ -142,9 +184,13 @@ def bench_spmm(rt, orc, gen, args):
                    "index_bytes": ib, "accumulate": False},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": alg_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": SPMM_TRAFFIC_BYTES if (n, K) == (500_000, 64) else None,
-                     "kernel": dom, "kernel_avg_ms": dom_ms, "algorithmic_bytes": int(alg_bytes),
+                     "traffic": traffic, "traffic_source": traffic_src,
+                     "kernel": dom, "kernel_avg_ms": dom_ms, "kernel_sum_ms": kernel_sum_ms,
+                     "algorithmic_bytes": int(alg_bytes),
                      "gather_inclusive_bytes": int(nnz * 8 * K + nnz * (8 + ib) + 8 * n * K)},
+        "plan": {"first_call_ms": first_ms, "plan_ms": max(first_ms - dev_ms, 0.0), "kept_device_bytes": int(kept_bytes),
+                 "note": "first product on a new matrix minus a steady-state product; bytes = device memory the "
+                         "first call keeps (lists of the long rows, the other rows re-packed, workspaces)"},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
     }
 
@@ -186,7 +232,7 @@ def bench_sddmm(rt, orc, gen, args):
                    "index_bytes": ib},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (dev_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": alg_bytes / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": SDDMM_TRAFFIC_BYTES if (n, K) == (500_000, 64) else None,
+                     "traffic": measured_traffic("sddmm_csr_zipf")[0] if (n, K) == (500_000, 64) else None,
                      "kernel": dom + " (+ transpose of D: the whole step is timed)",
                      "kernel_avg_ms": dom_ms, "algorithmic_bytes": int(alg_bytes)},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
@@ -202,7 +248,7 @@ def bench_spmv(rt, orc, gen, args):
     dx = rt.DeviceArray.from_numpy(x)
     dy = rt.DeviceArray(n)
     step = lambda: rt.spmv(A, dx, dy, accumulate=False)
-    step()
+    first_ms, kept_bytes = first_call(rt, step)
     wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
     kt = kernel_times(rt, step, args.steps)
     parity_ok = bool(np.array_equal(dy.to_numpy(), orc.spmv(pos, crd, val, x)))
@@ -227,9 +273,12 @@ def bench_spmv(rt, orc, gen, args):
                    "column_block_passes": passes},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": alg_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": SPMV_TRAFFIC_BYTES if n == 1_000_000 else None,
+                     "traffic": measured_traffic("spmv_csr_poisson")[0] if n == 1_000_000 else None,
                      "kernel": dom, "kernel_avg_ms": dom_ms, "launches_per_step": passes,
                      "algorithmic_bytes": int(alg_bytes)},
+        "plan": {"first_call_ms": first_ms, "plan_ms": max(first_ms - dev_ms, 0.0), "kept_device_bytes": int(kept_bytes),
+                 "note": "first product on a new matrix minus a steady-state product; bytes = the column-blocked "
+                         "copy of the matrix the first call keeps"},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
     }
 
@@ -266,6 +315,16 @@ def bench_ttgt(rt, orc, gen, args):
         cpu = {"value": 2.0 * m ** 3 / t / 1e12, "unit": "TFLOP/s", "cores": host_threads(), "kind": "port",
                "sample": f"naive i-j-k GEMM {m}^3 (OpenMP over i), best of {reps} runs, {t:.2f} s each; the 4096^3 "
                          f"GEMM would take about {2.0 * 4096 ** 3 / (2.0 * m ** 3 / t):.0f} s at that rate"}
+        # the strong baseline: the host BLAS numpy is linked against, on a size it finishes in about a second
+        mb = 2048
+        Ab, Bb = gen.dense((mb, mb), seed=9), gen.dense((mb, mb), seed=10)
+        tb, repsb = cpu_time(lambda: Ab @ Bb, budget_s=6.0, min_reps=2)
+        cpu["blas_dgemm"] = {"value": 2.0 * mb ** 3 / tb / 1e12, "unit": "TFLOP/s",
+                             "sample": f"numpy matmul {mb}^3, best of {repsb} runs, {tb * 1e3:.0f} ms each, "
+                                       f"{host_threads()} threads at most"}
+    import ctypes as C
+    peak = C.c_double()
+    rt._check(rt.lib().comet_hip_mfma_f64_peak(20000, C.byref(peak)), "comet_hip_mfma_f64_peak")
     perm_bytes = 2 * 8 * e ** 4 * (plan.transA + plan.transB + plan.transC)
     return {
         "metric": "TTGT contraction TFLOP/s (fp64 MFMA GEMM + LDS-tiled transposes) on 1 MI355X",
@@ -274,7 +333,10 @@ def bench_ttgt(rt, orc, gen, args):
                    "transposes": {"A": plan.transA, "B": plan.transB, "C": plan.transC}, "beta": 0.0},
         "roofline": {"bound": "mfma", "achieved": flops / (dom_ms * 1e-3) / 1e12, "peak": FP64_MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": flops / (dom_ms * 1e-3) / 1e12 / FP64_MFMA_PEAK_TFLOPS, "traffic": None,
-                     "kernel": dom, "kernel_avg_ms": dom_ms, "transpose_bytes": int(perm_bytes)},
+                     "kernel": dom, "kernel_avg_ms": dom_ms, "transpose_bytes": int(perm_bytes),
+                     "measured_peak": peak.value,
+                     "measured_peak_note": "back-to-back v_mfma_f64_16x16x4_f64 on registers, 8 wavefronts per CU",
+                     "frac_of_measured_peak": flops / (dom_ms * 1e-3) / 1e12 / peak.value},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
     }
 
@@ -302,7 +364,7 @@ def bench_tricount(rt, orc, gen, args):
     L = rt.CsrMatrix.from_arrays((n, n), lpos, lcrd, lval)
     out = {}
     step = lambda: out.__setitem__("count", rt.triangle_count(L))
-    step()
+    first_ms, kept_bytes = first_call(rt, step)
     wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
     kt = kernel_times(rt, step, args.steps)
     # rows with many products take a workgroup each, the others a wavefront each: two kernels that run side by side
@@ -322,7 +384,7 @@ def bench_tricount(rt, orc, gen, args):
         parity = bool(want == out["count"])
         cpu = {"value": flops / t / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
                "sample": f"the full workload once, {t:.1f} s, single thread (the reference never parallelises "
-                         f"sparse-output loops)", "count": want}
+                         f"sparse-output loops)", "count": want, "seconds": t}
     return {
         "metric": "masked SpGEMM triangle count GFLOP/s (2 flops per masked-candidate product) on 1 MI355X",
         "value": flops / (dev_ms * 1e-3) / 1e9, "unit": "GFLOP/s", "ms_per_step": dev_ms, "dtype": "f64",
@@ -330,9 +392,11 @@ def bench_tricount(rt, orc, gen, args):
                    "products": nprod, "triangles": out["count"], "seed": 20},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": alg_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": TRICOUNT_TRAFFIC_BYTES if scale == 20 else None, "kernel": dom,
+                     "traffic": measured_traffic("tricount_rmat")[0] if scale == 20 else None, "kernel": dom,
                      "kernel_avg_ms": dom_ms, "algorithmic_bytes": int(alg_bytes)},
-        "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity,
+        "plan": {"first_call_ms": first_ms, "plan_ms": max(first_ms - dev_ms, 0.0), "kept_device_bytes": int(kept_bytes)},
+        "cpu_baseline": cpu, "speedup_vs_cpu": (cpu["seconds"] / (dev_ms * 1e-3)) if cpu else None,
+        "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity,
     }
 
 
@@ -382,6 +446,8 @@ def bench_spgemm(rt, orc, gen, args):
             state["vsum"] = vsum
 
     # every step is seconds long: per-kernel event timing stays on during the timed steps
+    first_ms, kept_bytes = first_call(rt, step)
+    kept_bytes -= 12 * state["cap"]          # the output block buffers are the caller's, not the library's
     step(check=True)
     for _ in range(args.warmup):
         step()
@@ -439,7 +505,8 @@ def bench_spgemm(rt, orc, gen, args):
         parity["sampled_blocks_bit_exact_structure_and_1e-12_values"] = struct_ok
         cpu = {"value": 2.0 * acc / t / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
                "sample": f"{len(picks)} blocks of 256 rows holding {acc} of {nprod} products, symbolic + numeric, "
-                         f"{t:.1f} s, single thread; extrapolated whole-job time {t * nprod / acc:.0f} s"}
+                         f"{t:.1f} s, single thread; extrapolated whole-job time {t * nprod / acc:.0f} s",
+               "extrapolated_seconds": t * nprod / acc}
     return {
         "metric": "Gustavson SpGEMM GFLOP/s (2 flops per product, symbolic + numeric) on 1 MI355X",
         "value": flops / (dev_ms * 1e-3) / 1e9, "unit": "GFLOP/s", "ms_per_step": dev_ms, "dtype": "f64",
@@ -448,11 +515,15 @@ def bench_spgemm(rt, orc, gen, args):
                    "seed": 20},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / ((sym_ms + num_ms) * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": alg_bytes / ((sym_ms + num_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": SPGEMM_TRAFFIC_BYTES if (scale, args.budget_gb) == (20, 48.0) else None,
+                     "traffic": measured_traffic("spgemm_rmat_AxA")[0] if (scale, args.budget_gb) == (20, 48.0) else None,
                      "kernel": "spgemm_symbolic + spgemm_numeric + spgemm_numeric_dense + spgemm_numeric_span",
                      "kernel_avg_ms": sym_ms + num_ms,
                      "symbolic_ms": sym_ms, "numeric_ms": num_ms, "algorithmic_bytes": int(alg_bytes)},
-        "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity,
+        "plan": {"first_call_ms": first_ms, "plan_ms": max(first_ms - dev_ms, 0.0), "kept_device_bytes": int(kept_bytes),
+                 "note": "first product minus a steady-state product; bytes = block pointers of the right operand, "
+                         "row lists and the slabs and bitmaps the library caches"},
+        "cpu_baseline": cpu, "speedup_vs_cpu": (cpu["extrapolated_seconds"] / (dev_ms * 1e-3)) if cpu else None,
+        "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity,
     }
 
 
@@ -521,7 +592,65 @@ def bench_coo2csr(rt, orc, gen, args):
     }
 
 
-WORKLOADS = {"copy": bench_copy, "spmm": bench_spmm, "spmv": bench_spmv, "sddmm": bench_sddmm, "ttgt": bench_ttgt, "tricount": bench_tricount,
+def bench_gather(rt, orc, gen, args):
+    """How fast the CUs take rows of 512 bytes out of the L2 when nothing else is done with them: the ceiling of
+    the SpMM sweep, whose long rows need nnz x 512 bytes of such gathers.  Every workgroup (16 wavefronts, one per
+    CU) draws its rows from the part of the table that belongs to its XCD (4 MiB or less: L2 hits)."""
+    import ctypes as C
+    rows_per_xcd = args.n or 4096
+    wgs, per_wave = 256, 4096
+    rng = np.random.Generator(np.random.PCG64(7))
+    xcd = (np.arange(wgs * 16) // 16) % 8
+    idx = (xcd[:, None] * rows_per_xcd + rng.integers(0, rows_per_xcd, (wgs * 16, per_wave))).astype(np.int32)
+    d_idx = rt.DeviceArray.from_numpy(idx)
+    table = rt.DeviceArray((8 * rows_per_xcd, 64), zero=True)
+    out = rt.DeviceArray(wgs * 1024)
+    step = lambda: rt._check(rt.lib().comet_hip_gather_rows_bench(wgs, per_wave, d_idx.ptr, table.ptr,
+                                                                  8 * rows_per_xcd, out.ptr), "gather bench")
+    step()
+    wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
+    kt = kernel_times(rt, step, args.steps)
+    dom_ms = kt["gather_rows_bench"]["avg_ms"]
+    nbytes = float(idx.size) * 512
+    return {
+        "metric": "rows of 512 B gathered from the L2, TB/s (ceiling of the SpMM sweep)", "value": nbytes / (dev_ms * 1e-3) / 1e12,
+        "unit": "TB/s", "ms_per_step": dev_ms, "dtype": "f64",
+        "config": {"workload": "gather_rows_l2", "table_rows_per_xcd": rows_per_xcd, "table_bytes_per_xcd": rows_per_xcd * 512,
+                   "gathers": int(idx.size), "workgroups": wgs, "wavefronts_per_workgroup": 16, "loads_in_flight": 16},
+        "roofline": {"bound": "l2 -> CU", "achieved": nbytes / (dom_ms * 1e-3) / 1e9, "peak": None, "unit": "GB/s",
+                     "frac": None, "traffic": None, "kernel": "gather_rows_bench", "kernel_avg_ms": dom_ms,
+                     "rows_per_second": idx.size / (dom_ms * 1e-3),
+                     "bytes_per_clock_per_cu_at_2.4GHz": nbytes / (dom_ms * 1e-3) / 256 / 2.4e9},
+        "cpu_baseline": None, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": None,
+    }
+
+
+def bench_headline(rt, orc, gen, args):
+    """The metric names SpMM and SpGEMM: the SpMM line carries, under "also", the SpGEMM and masked-SpGEMM
+    (triangle count) workloads at R-MAT scale 20 with their own roofline, CPU baseline and parity, plus SpMV and the
+    TTGT contraction - each a short run of its own workload function."""
+    import copy
+    import gc
+    res = bench_spmm(rt, orc, gen, args)
+    also = {}
+    for name, fn, steps, warmup in (("spgemm_rmat20", bench_spgemm, 2, 0), ("tricount_rmat20", bench_tricount, 5, 1),
+                                    ("spmv_poisson_1m", bench_spmv, 20, 3), ("ttgt_64x4", bench_ttgt, 5, 1)):
+        gc.collect()
+        sub_args = copy.copy(args)
+        sub_args.steps, sub_args.warmup, sub_args.n = steps, warmup, 0
+        log(f"also: {name}")
+        try:
+            sub = fn(rt, orc, gen, sub_args)
+            sub["steps"], sub["warmup"] = steps, warmup
+            sub.pop("kernels", None)
+            also[name] = sub
+        except Exception as exc:          # a failing side workload is reported, the headline line still prints
+            also[name] = {"error": f"{type(exc).__name__}: {exc}"}
+    res["also"] = also
+    return res
+
+
+WORKLOADS = {"headline": bench_headline, "gather": bench_gather, "copy": bench_copy, "spmm": bench_spmm, "spmv": bench_spmv, "sddmm": bench_sddmm, "ttgt": bench_ttgt, "tricount": bench_tricount,
              "spgemm": bench_spgemm, "coo2csr": bench_coo2csr}
 
 
@@ -530,7 +659,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="spmm")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="headline",
+                    help="headline (default): SpMM as the value, SpGEMM / triangle count / SpMV / TTGT under \"also\"")
     ap.add_argument("--n", type=int, default=0, help="override the problem size (rows, or extent for ttgt)")
     ap.add_argument("--scale", type=int, default=0, help="R-MAT scale for tricount / spgemm (default 20)")
     ap.add_argument("--candidate", type=int, default=-1, help="force a TTGT candidate (default: cost rule)")

@@ -879,6 +879,16 @@ int comet_hip_reduce_sum_f64(int64_t dptr, int64_t n, double *out)
     return comet::reduce_sum_device((const double *)dptr, n, out);
 }
 
+int comet_hip_mem_info(int64_t *free_bytes, int64_t *total_bytes)
+{
+    COMET_CHK(ensure_init());
+    size_t f = 0, t = 0;
+    COMET_HIPCHK(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = (int64_t)f;
+    if (total_bytes) *total_bytes = (int64_t)t;
+    return COMET_HIP_OK;
+}
+
 int comet_hip_copy_f64(int64_t dst_dptr, int64_t src_dptr, int64_t n)
 {
     COMET_CHK(ensure_init());

@@ -1319,6 +1319,55 @@ static int spmm_chunks(Csr *a, int64_t K, const double *B, int64_t ldb, double *
 }
 
 // ---------------------------------------------------------------------------
+// Yardstick for the sweep: how fast the CUs can take rows of a dense operand out of the L2 when nothing else is
+// done with them.  Every wavefront walks a list of row numbers; a half-wavefront fetches one row of 64 doubles,
+// 16 bytes per lane (the sweep's load shape), sixteen loads in flight, and only sums what arrives.  Workgroup w
+// (on XCD w mod 8) draws its rows from the w-mod-8-th eighth of the table, so with a table of at most 4 MiB per
+// XCD every gather after the first touch is an L2 hit.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void gather_rows_bench_kernel(const int32_t *__restrict__ idx, int64_t per_wave,
+                                                                 const double *__restrict__ table,
+                                                                 double *__restrict__ out)
+{
+    const int lane = threadIdx.x & 63, half = lane >> 5, sub = lane & 31;
+    const int64_t wave = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 6);
+    const int32_t *my = idx + wave * per_wave;
+    double2 acc = make_double2(0.0, 0.0);
+    for (int64_t i = 0; i < per_wave; i += 32) {
+        double2 b[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int64_t j = my[i + 2 * u + half];
+            b[u] = *reinterpret_cast<const double2 *>(table + j * 64 + sub * 2);
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            acc.x += b[u].x;
+            acc.y += b[u].y;
+        }
+    }
+    out[wave * 64 + lane] = acc.x + acc.y;
+}
+
+// idx[w * per_wave + i]: row of `table` (rows of 64 doubles) that wavefront w fetches i-th; 16 wavefronts per
+// workgroup, `workgroups` workgroups; per_wave a multiple of 32; out holds workgroups * 1024 doubles.
+extern "C" int comet_hip_gather_rows_bench(int64_t workgroups, int64_t per_wave, int64_t idx_dptr, int64_t table_dptr,
+                                           int64_t table_rows, int64_t out_dptr)
+{
+    COMET_CHK(ensure_init());
+    if (workgroups <= 0 || workgroups > 65535 || per_wave <= 0 || (per_wave & 31) || !idx_dptr || !table_dptr ||
+        table_rows <= 0 || !out_dptr)
+        return set_error(COMET_HIP_ERR_ARG, "bad arguments to comet_hip_gather_rows_bench");
+    {
+        KernelTimer t("gather_rows_bench");
+        gather_rows_bench_kernel<<<dim3((unsigned)workgroups), dim3(1024), 0, stream()>>>(
+            (const int32_t *)idx_dptr, per_wave, (const double *)table_dptr, (double *)out_dptr);
+    }
+    COMET_HIPCHK(hipGetLastError());
+    return COMET_HIP_OK;
+}
+
+// ---------------------------------------------------------------------------
 // SpMM for callers that cannot allocate (code under graph capture, serving loops that forbid hipMalloc): the
 // chunk kernel and its fix-up with their scratch - the chunk -> row table and the carry slots of rows cut by a
 // chunk boundary - in one array that lives in the library's image instead of in allocated workspaces.  Every

@@ -507,6 +507,58 @@ extern "C" int comet_hip_ttgt_plan(int32_t rankA, const int32_t *a_lab, int32_t 
     return make_plan(rankA, a_lab, rankB, b_lab, rankC, c_lab, extent, which, plan);
 }
 
+// Yardstick for the GEMM: back-to-back v_mfma_f64_16x16x4_f64 on registers only, sixteen independent
+// accumulators per wavefront (more than the instruction's latency needs), two wavefronts per SIMD on every CU.
+__global__ __launch_bounds__(256, 2) void mfma_f64_peak_kernel(int64_t iters, double *__restrict__ out)
+{
+    double4_t acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        acc[i] = (double4_t){0.0, 0.0, 0.0, 0.0};
+    const double a = 1.0 + threadIdx.x * 1e-9, b = 1.0 - threadIdx.x * 1e-9;
+    for (int64_t it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, acc[i], 0, 0, 0);
+    }
+    double4_t s = acc[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i)
+        s += acc[i];
+    out[(int64_t)blockIdx.x * blockDim.x + threadIdx.x] = s[0] + s[1] + s[2] + s[3];
+}
+
+static Workspace g_peak_out;
+
+extern "C" int comet_hip_mfma_f64_peak(int64_t iters, double *tflops)
+{
+    COMET_CHK(ensure_init());
+    if (iters <= 0 || iters > (1ll << 24) || !tflops)
+        return set_error(COMET_HIP_ERR_ARG, "bad arguments to comet_hip_mfma_f64_peak");
+    const int blocks = num_cus() * 2;        // 8 wavefronts per CU: two per SIMD
+    COMET_CHK(g_peak_out.ensure(sizeof(double) * 256 * (size_t)blocks, false));
+    hipEvent_t e0, e1;
+    COMET_HIPCHK(hipEventCreate(&e0));
+    COMET_HIPCHK(hipEventCreate(&e1));
+    float best = 0.f;
+    for (int rep = 0; rep < 4; ++rep) {      // the first launch warms the clocks up
+        COMET_HIPCHK(hipEventRecord(e0, stream()));
+        mfma_f64_peak_kernel<<<dim3((unsigned)blocks), dim3(256), 0, stream()>>>(iters, (double *)g_peak_out.ptr);
+        COMET_HIPCHK(hipEventRecord(e1, stream()));
+        COMET_HIPCHK(hipEventSynchronize(e1));
+        float ms = 0.f;
+        COMET_HIPCHK(hipEventElapsedTime(&ms, e0, e1));
+        if (rep > 0 && (best == 0.f || ms < best))
+            best = ms;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    COMET_HIPCHK(hipGetLastError());
+    const double flops = 2.0 * 16 * 16 * 4 * 16.0 * (double)iters * 4.0 * blocks;      // per MFMA x 16 x iters x waves
+    *tflops = flops / ((double)best * 1e-3) / 1e12;
+    return COMET_HIP_OK;
+}
+
 extern "C" int comet_hip_ttgt_contract(const comet_ttgt_plan *plan, const int64_t *a_shape, const int64_t *b_shape,
                                        const int64_t *c_shape, int64_t a_dptr, int64_t b_dptr, int64_t c_dptr,
                                        double beta)

@@ -124,6 +124,9 @@ SIGNATURES = {
     "comet_hip_profile_query": (_int, [C.c_char_p, _pi64, C.POINTER(_f64)]),
     "comet_hip_profile_name": (_int, [_i32, C.c_char_p, _i64]),
     "comet_hip_copy_f64": (_int, [_i64, _i64, _i64]),
+    "comet_hip_mem_info": (_int, [C.POINTER(_i64), C.POINTER(_i64)]),
+    "comet_hip_mfma_f64_peak": (_int, [_i64, C.POINTER(C.c_double)]),
+    "comet_hip_gather_rows_bench": (_int, [_i64, _i64, _i64, _i64, _i64, _i64]),
     "_mlir_ciface_comet_hip_spmv_csr_f64_i64": (None, [_m1, _m1, _m1, _m1, _m1]),
     "_mlir_ciface_comet_hip_spmm_csr_f64_i64": (None, [_m1, _m1, _m1, _m2, _m2]),
     "_mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i64": (None, [_i64, _i64, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _m1]),

@@ -358,6 +358,20 @@ int comet_hip_profile_query(const char *name, int64_t *launches, double *total_m
 int comet_hip_profile_name(int32_t index, char *buf, int64_t cap);
 /* Plain device-to-device copy kernel (used to calibrate hardware counters). */
 int comet_hip_copy_f64(int64_t dst_dptr, int64_t src_dptr, int64_t n);
+/* Free and total device memory (hipMemGetInfo): lets a caller see what a first
+ * call kept (plans cached in a handle, workspaces). */
+int comet_hip_mem_info(int64_t *free_bytes, int64_t *total_bytes);
+/* Two yardsticks the measurements are set against, neither has a counterpart in
+ * the reference.  mfma_f64_peak: TFLOP/s of back-to-back v_mfma_f64_16x16x4_f64
+ * on registers (`iters` x 16 per wavefront, 8 wavefronts per CU), the rate the
+ * TTGT GEMM is compared with.  gather_rows_bench: every wavefront fetches
+ * per_wave rows of 64 doubles named by idx (int32, one list per wavefront, 16
+ * wavefronts per workgroup) from `table`, half a wavefront per row and 16 bytes
+ * per lane as the SpMM sweep does, and sums them into out (workgroups x 1024
+ * doubles): the rate at which the CUs can take rows out of the L2. */
+int comet_hip_mfma_f64_peak(int64_t iters, double *tflops);
+int comet_hip_gather_rows_bench(int64_t workgroups, int64_t per_wave, int64_t idx_dptr,
+                                int64_t table_dptr, int64_t table_rows, int64_t out_dptr);
 
 /* ---- memref-descriptor forms ----------------------------------------------
  * What `func.call` sites in lowered code bind to (llvm.emit_c_interface):
