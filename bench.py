@@ -416,11 +416,13 @@ def bench_spgemm(rt, orc, gen, args):
     budget = int(args.budget_gb * (1 << 30)) // 12          # entries per block
     state = {}
 
+    mask = A if args.masked else None      # C<A> = A*A: the output holds the stored entries of A that receive a product
+
     def step(check=False):
         # the whole product: symbolic over all rows, numeric block by block into the same buffers.  With `check`
         # every block is also summed before it is dropped; that pass is the bench's own and stays out of the
         # timed steps (it reads each block once more: 47 ms at scale 20).
-        dpos, nnzC = rt.spgemm_symbolic(A, A)
+        dpos, nnzC = rt.spgemm_symbolic(A, A, mask=mask)
         log(f"symbolic done: nnz(C) = {nnzC}")
         hpos = dpos.to_numpy()
         maxrow = int(np.diff(hpos).max()) if n else 0
@@ -435,7 +437,7 @@ def bench_spgemm(rt, orc, gen, args):
         while rb < n:
             re = int(np.searchsorted(hpos, hpos[rb] + cap, side="right")) - 1
             re = min(max(re, rb + 1), n)
-            rt.spgemm_numeric(A, A, dpos, rb, re, dcrd, dval)
+            rt.spgemm_numeric(A, A, dpos, rb, re, dcrd, dval, mask=mask)
             if check:
                 vsum += rt.reduce_sum(dval, int(hpos[re] - hpos[rb]))
             log(f"numeric rows [{rb},{re}): {int(hpos[re] - hpos[rb])} entries")
@@ -461,9 +463,9 @@ def bench_spgemm(rt, orc, gen, args):
     flops = 2.0 * nprod
     ib = 4
     alg_bytes = nnzA * (8 + ib) + (n + 1) * ib + nnzC * (8 + ib) + 8 * (n + 1)
-    sym_ms = kt["spgemm_symbolic"]["avg_ms"] * kt["spgemm_symbolic"]["launches"] / args.steps
-    num_ms = sum(kt[k]["avg_ms"] * kt[k]["launches"] for k in
-                 ("spgemm_numeric", "spgemm_numeric_dense", "spgemm_numeric_span", "spgemm_row_products", "radix_sort_pairs") if k in kt) / args.steps
+    sym_ms = sum(v["avg_ms"] * v["launches"] for k, v in kt.items() if k.startswith("spgemm_symbolic")) / args.steps
+    num_ms = sum(v["avg_ms"] * v["launches"] for k, v in kt.items()
+                 if k.startswith("spgemm_numeric") or k in ("spgemm_row_products", "radix_sort_pairs")) / args.steps
     # sum of all values is a size-independent invariant: sum(C) = sum_k colsum(A)[k] * rowsum(A)[k]
     rowsum = np.add.reduceat(val, pos[:-1][np.diff(pos) > 0])
     rs = np.zeros(n)
@@ -471,7 +473,7 @@ def bench_spgemm(rt, orc, gen, args):
     cs = np.bincount(crd, weights=val, minlength=n)
     invariant = float(np.dot(cs, rs))
     cpu = None
-    parity = {"sum_values_rel_err": abs(state["vsum"] - invariant) / invariant}
+    parity = {"sum_values_rel_err": abs(state["vsum"] - invariant) / invariant} if not args.masked else {}
     if not args.no_cpu:
         # CPU checker on a row sample holding about args.cpu_products products, both phases, single thread
         rng = np.random.default_rng(0)
@@ -493,12 +495,13 @@ def bench_spgemm(rt, orc, gen, args):
         log(f"CPU checker on {len(picks)} row blocks ({acc} products)")
         for (r0, r1) in picks:
             t0 = time.perf_counter()
-            cp, cc, cv = orc.spgemm(pos, crd, val, pos, crd, val, n, rows=(r0, r1))
+            cp, cc, cv = orc.spgemm(pos, crd, val, pos, crd, val, n, rows=(r0, r1),
+                                    mask=(pos, crd) if args.masked else None)
             t += time.perf_counter() - t0
             struct_ok &= bool(np.array_equal(cp, hpos[r0:r1 + 1] - hpos[r0]))
             cnt = int(hpos[r1] - hpos[r0])
             if cnt <= state["cap"]:
-                rt.spgemm_numeric(A, A, state["dpos"], r0, r1, state["dcrd"], state["dval"])
+                rt.spgemm_numeric(A, A, state["dpos"], r0, r1, state["dcrd"], state["dval"], mask=mask)
                 gc, gv = state["dcrd"].to_numpy(cnt), state["dval"].to_numpy(cnt)
                 struct_ok &= bool(np.array_equal(gc, cc)) and bool(np.all(np.abs(gv - cv) <= 1e-12 * np.abs(cv)))
             log(f"  rows [{r0},{r1}): {cnt} entries checked, CPU time so far {t:.1f} s, ok = {struct_ok}")
@@ -510,12 +513,13 @@ def bench_spgemm(rt, orc, gen, args):
     return {
         "metric": "Gustavson SpGEMM GFLOP/s (2 flops per product, symbolic + numeric) on 1 MI355X",
         "value": flops / (dev_ms * 1e-3) / 1e9, "unit": "GFLOP/s", "ms_per_step": dev_ms, "dtype": "f64",
-        "config": {"workload": "spgemm_rmat_AxA", "scale": scale, "edge_factor": 16, "nnz_A": int(nnzA),
+        "config": {"workload": "spgemm_rmat_AxA_masked_by_A" if args.masked else "spgemm_rmat_AxA", "scale": scale, "edge_factor": 16, "nnz_A": int(nnzA),
                    "products": nprod, "nnz_C": nnzC, "row_blocks": state["blocks"], "block_budget_gb": args.budget_gb,
                    "seed": 20},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / ((sym_ms + num_ms) * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": alg_bytes / ((sym_ms + num_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": measured_traffic("spgemm_rmat_AxA")[0] if (scale, args.budget_gb) == (20, 48.0) else None,
+                     "traffic": measured_traffic("spgemm_rmat_AxA_masked_by_A" if args.masked else "spgemm_rmat_AxA")[0]
+                     if (scale, args.budget_gb) == (20, 48.0) else None,
                      "kernel": "spgemm_symbolic + spgemm_numeric + spgemm_numeric_dense + spgemm_numeric_span",
                      "kernel_avg_ms": sym_ms + num_ms,
                      "symbolic_ms": sym_ms, "numeric_ms": num_ms, "algorithmic_bytes": int(alg_bytes)},
@@ -666,6 +670,7 @@ def main():
     ap.add_argument("--candidate", type=int, default=-1, help="force a TTGT candidate (default: cost rule)")
     ap.add_argument("--budget-gb", type=float, default=48.0, help="spgemm: output bytes per numeric row block")
     ap.add_argument("--cpu-products", type=int, default=1_500_000_000, help="spgemm: products in the CPU sample")
+    ap.add_argument("--masked", action="store_true", help="spgemm: the masked product C<A> = A*A, materialised")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -317,6 +317,10 @@ __device__ inline double key_f64(unsigned long long k)
     return __longlong_as_double((long long)u);
 }
 extern __shared__ uint32_t sg_dyn_lds[];
+// Hash table of a masked product's mask row (see spgemm_numeric_kernel): values first (8-byte aligned), keys after.
+constexpr int SG_HASH_LOG = 13, SG_HASH_SLOTS = 1 << SG_HASH_LOG;
+constexpr int SG_HASH_FILL = SG_HASH_SLOTS * 3 / 4;          // longest mask row that goes into the table
+constexpr size_t SG_HASH_LDS = (size_t)SG_HASH_SLOTS * (8 + 4);
 
 // ---------------------------------------------------------------------------
 // Symbolic phase.  Unmasked: set the bit of every reachable column, count the
@@ -427,20 +431,30 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
 {
     __shared__ int64_t row_slot;
     __shared__ int wave_tot[SG_WAVES];
-    uint32_t *bm;
-    if constexpr (BM_LDS)
+    // Two bitmaps: the columns of the output row (bm) and, for a masked product, the mask row (mbm).  One of
+    // them fits LDS.  Unmasked, that is bm.  Masked, it is the mask: every product probes it, while only the
+    // products that fall on a mask entry touch bm, which then lives in HBM with the slab and, like the slab,
+    // is reached through L2 atomics only.
+    constexpr bool OUT_LDS = BM_LDS && !MASKED, MASK_LDS = BM_LDS && MASKED;
+    uint32_t *bm, *mbm = nullptr;
+    if constexpr (OUT_LDS)
         bm = sg_dyn_lds;
     else
         bm = gbm + (size_t)blockIdx.x * (size_t)(SG_T * ((1 << logW) + 1));
-    uint32_t *mbm = MASKED ? gmask + (size_t)blockIdx.x * (size_t)(SG_T * ((1 << logW) + 1)) : nullptr;
+    if constexpr (MASK_LDS)
+        mbm = sg_dyn_lds;
+    else if constexpr (MASKED)
+        mbm = gmask + (size_t)blockIdx.x * (size_t)(SG_T * ((1 << logW) + 1));
     double *slab = slabs + (size_t)blockIdx.x * (size_t)ncols;
     const BmAddr ad{logW};
     const int W = 1 << logW;
     const int nwords = SG_T * ((1 << logW) + 1);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     if constexpr (BM_LDS) {
-        for (int w = threadIdx.x; w < nwords; w += SG_T)
-            bm[w] = 0;
+        // the bitmap and, for a masked product, the hash table that shares its place
+        const int lds_words = MASKED && nwords < (int)(SG_HASH_LDS / 4) ? (int)(SG_HASH_LDS / 4) : nwords;
+        for (int w = threadIdx.x; w < lds_words; w += SG_T)
+            sg_dyn_lds[w] = 0;
     }
     __syncthreads();
     const int64_t out0 = Cpos[row_begin];
@@ -451,7 +465,114 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
         const int64_t i = row_begin + list.rows[t];
         const int64_t as = Apos[i], ae = Apos[i + 1];
         const int64_t ob = Cpos[i], oe = Cpos[i + 1];
-        if (as != ae && ob != oe) {
+        bool hashed = false;
+        if constexpr (MASK_LDS)
+            hashed = __builtin_amdgcn_readfirstlane((int)(Mpos[i + 1] - Mpos[i] <= SG_HASH_FILL)) != 0;
+        if (as != ae && ob != oe && hashed) {
+            // A mask row of at most SG_HASH_FILL entries (nearly every row) goes into a hash table in LDS, column
+            // -> slot, and the slot holds the value: a product probes the table (one LDS read for the 96 % that
+            // miss), a product that falls on a mask entry adds into the slot with an LDS atomic, and nothing of
+            // the row touches the L2.  A slot's key is column + 1, bit 31 says that a product has arrived.
+            uint32_t *hkey = sg_dyn_lds + 2 * SG_HASH_SLOTS;
+            double *hval = reinterpret_cast<double *>(sg_dyn_lds);
+            unsigned long long *hbits = reinterpret_cast<unsigned long long *>(sg_dyn_lds);
+            const auto slot_of = [&](int j) -> int {          // the slot that holds column j, or -1
+                uint32_t sl = ((uint32_t)j * 2654435761u) >> (32 - SG_HASH_LOG);
+                for (;;) {
+                    const uint32_t k = hkey[sl];
+                    if ((k & 0x7fffffffu) == (uint32_t)j + 1u)
+                        return (int)sl;
+                    if (k == 0u)
+                        return -1;
+                    sl = (sl + 1) & (SG_HASH_SLOTS - 1);
+                }
+            };
+            const int64_t ms = Mpos[i], mlen = Mpos[i + 1] - ms;
+            for (int64_t e = ms + threadIdx.x; e < ms + mlen; e += SG_T) {
+                const uint32_t key = (uint32_t)Mcrd[e] + 1u;
+                uint32_t sl = ((uint32_t)Mcrd[e] * 2654435761u) >> (32 - SG_HASH_LOG);
+                for (;;) {
+                    const uint32_t old = atomicCAS(&hkey[sl], 0u, key);
+                    if (old == 0u || old == key)
+                        break;
+                    sl = (sl + 1) & (SG_HASH_SLOTS - 1);
+                }
+            }
+            __syncthreads();
+            for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, [&](int j, int64_t q, double a, int64_t p, int64_t bs) {
+                const int sl = slot_of(j);
+                if (sl < 0)
+                    return;
+                if (!(hkey[sl] >> 31))
+                    atomicOr(&hkey[sl], 0x80000000u);
+                if constexpr (SEMI) {
+                    if (reduce_op == SR_ANY) {
+                        const unsigned long long key = ((unsigned long long)(p - as + 1) << 32) | (unsigned long long)(q - bs);
+                        __hip_atomic_fetch_max(&hbits[sl], key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    } else {
+                        const double e = semiring_mult(mult_op, a, Bval[q]);
+                        if (reduce_op == SR_PLUS)
+                            __hip_atomic_fetch_add(&hval[sl], e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        else
+                            __hip_atomic_fetch_max(&hbits[sl], reduce_op == SR_MIN ? ~f64_key(e) : f64_key(e),
+                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    }
+                } else {
+                    __hip_atomic_fetch_add(&hval[sl], a * Bval[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+            });
+            __syncthreads();
+            // the mask row is sorted: thread t takes a run of its entries, counts the ones a product reached, and
+            // after a prefix sum over the workgroup writes them in place
+            const int64_t per = (mlen + SG_T - 1) / SG_T;
+            const int64_t e0 = ms + (int64_t)threadIdx.x * per;
+            const int64_t e1 = e0 + per < ms + mlen ? e0 + per : ms + mlen;
+            int mine = 0;
+            for (int64_t e = e0; e < e1; ++e) {
+                const int j = Mcrd[e];
+                if (e > ms && Mcrd[e - 1] == j)
+                    continue;          // a column stored twice in the mask row is one output entry
+                mine += (int)(hkey[slot_of(j)] >> 31);
+            }
+            const int inc = wave_inclusive_scan(mine);
+            if (lane == 63)
+                wave_tot[wave] = inc;
+            __syncthreads();
+            int64_t off = ob - out0 + (inc - mine);
+            for (int w = 0; w < wave; ++w)
+                off += wave_tot[w];
+            for (int64_t e = e0; e < e1; ++e) {
+                const int j = Mcrd[e];
+                if (e > ms && Mcrd[e - 1] == j)
+                    continue;
+                const int sl = slot_of(j);
+                if (!(hkey[sl] >> 31))
+                    continue;
+                Ccrd[off] = j;
+                double out = hval[sl];
+                if (SEMI && reduce_op != SR_PLUS) {
+                    const unsigned long long v = hbits[sl];
+                    if (reduce_op == SR_MIN) {
+                        out = key_f64(~v);
+                    } else if (reduce_op == SR_MAX) {
+                        out = v < f64_key(0.0) ? 0.0 : key_f64(v);
+                    } else {
+                        const int64_t pp = as + (int64_t)(v >> 32) - 1;
+                        const int64_t qq = Bpos[Acrd[pp]] + (int64_t)(v & 0xffffffffull);
+                        out = semiring_mult(mult_op, Aval[pp], Bval[qq]);
+                    }
+                }
+                Cval[off] = out;
+                ++off;
+            }
+            __syncthreads();           // everybody has found its slots: now they are emptied (keys last used above)
+            for (int sl = threadIdx.x; sl < SG_HASH_SLOTS; sl += SG_T)
+                if (hkey[sl]) {
+                    hkey[sl] = 0u;
+                    hbits[sl] = 0ull;
+                }
+        }
+        if (as != ae && ob != oe && !hashed) {
         if constexpr (MASKED) {
             for (int64_t t = Mpos[i] + threadIdx.x; t < Mpos[i + 1]; t += SG_T)
                 atomicOr(&mbm[ad.word(Mcrd[t])], ad.bit(Mcrd[t]));
@@ -460,7 +581,10 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
         for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, [&](int j, int64_t q, double a, int64_t p, int64_t bs) {
             const int w = ad.word(j);
             const uint32_t b = ad.bit(j);
-            if constexpr (MASKED) {
+            if constexpr (MASK_LDS) {
+                if (!(mbm[w] & b))       // the mask row was set before the barrier above and does not change
+                    return;
+            } else if constexpr (MASKED) {
                 if (!(atomicOr(&mbm[w], 0u) & b))
                     return;
             }
@@ -483,10 +607,64 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
             }
         });
         __syncthreads();
+        if constexpr (MASK_LDS) {
+            // (rows whose mask row fits the hash table never come here: see below)
+            // The output row is a subset of the mask row: walk that (it is sorted) instead of the bitmap.  Thread t
+            // takes a run of consecutive mask entries, counts those whose bit a product has set, and after a prefix
+            // sum over the workgroup writes them in place; value and bit are fetched and cleared on the way.
+            const int64_t ms = Mpos[i], mlen = Mpos[i + 1] - ms;
+            const int64_t per = (mlen + SG_T - 1) / SG_T;
+            const int64_t e0 = ms + (int64_t)threadIdx.x * per;
+            const int64_t e1 = e0 + per < ms + mlen ? e0 + per : ms + mlen;
+            int mine = 0;
+            for (int64_t e = e0; e < e1; ++e) {
+                const int j = Mcrd[e];
+                if (e > ms && Mcrd[e - 1] == j)
+                    continue;          // a column stored twice in the mask row is one output entry
+                mine += (atomicOr(&bm[ad.word(j)], 0u) & ad.bit(j)) ? 1 : 0;
+            }
+            int inc = wave_inclusive_scan(mine);
+            if (lane == 63)
+                wave_tot[wave] = inc;
+            __syncthreads();           // also: every bit has been read before the first one is cleared below
+            int64_t off = ob - out0 + (inc - mine);
+            for (int w = 0; w < wave; ++w)
+                off += wave_tot[w];
+            for (int64_t e = e0; e < e1; ++e) {
+                const int j = Mcrd[e];
+                if ((e > ms && Mcrd[e - 1] == j) || !(atomicOr(&bm[ad.word(j)], 0u) & ad.bit(j)))
+                    continue;
+                Ccrd[off] = j;
+                if (SEMI && reduce_op != SR_PLUS) {
+                    const unsigned long long v = __hip_atomic_exchange((unsigned long long *)&slab[j], 0ull,
+                                                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    double out;
+                    if (reduce_op == SR_MIN) {
+                        out = key_f64(~v);
+                    } else if (reduce_op == SR_MAX) {
+                        out = v < f64_key(0.0) ? 0.0 : key_f64(v);
+                    } else {
+                        const int64_t pp = as + (int64_t)(v >> 32) - 1;
+                        const int64_t qq = Bpos[Acrd[pp]] + (int64_t)(v & 0xffffffffull);
+                        out = semiring_mult(mult_op, Aval[pp], Bval[qq]);
+                    }
+                    Cval[off] = out;
+                } else {
+                    Cval[off] = __hip_atomic_exchange(&slab[j], 0.0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+                ++off;
+            }
+            __syncthreads();           // all reads of the bits are done
+            for (int64_t e = e0; e < e1; ++e) {
+                const int j = Mcrd[e];
+                atomicAnd(&bm[ad.word(j)], ~ad.bit(j));
+                atomicAnd(&mbm[ad.word(j)], 0u);
+            }
+        } else {
         // extraction: my words hold my columns in ascending order
         int mine = 0;
         for (int k = 0; k < W; ++k)
-            mine += __popc(BM_LDS ? bm[threadIdx.x * (W + 1) + k] : atomicOr(&bm[threadIdx.x * (W + 1) + k], 0u));
+            mine += __popc(OUT_LDS ? bm[threadIdx.x * (W + 1) + k] : atomicOr(&bm[threadIdx.x * (W + 1) + k], 0u));
         int inc = mine;
         for (int d = 1; d < 64; d <<= 1) {
             const int o = __shfl_up(inc, d, 64);
@@ -501,7 +679,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
             off += wave_tot[w];
         for (int k = 0; k < W; ++k) {
             uint32_t word;
-            if constexpr (BM_LDS) {
+            if constexpr (OUT_LDS) {
                 word = bm[threadIdx.x * (W + 1) + k];
                 bm[threadIdx.x * (W + 1) + k] = 0;
             } else {
@@ -537,6 +715,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
             for (int64_t t = Mpos[i] + threadIdx.x; t < Mpos[i + 1]; t += SG_T)
                 atomicAnd(&mbm[ad.word(Mcrd[t])], 0u);
         }
+        }   // extraction over the bitmap
         }   // row with output
         t = draw_row(ticket, t_first, &row_slot);     // its barriers also close this row's clean-up
     }
@@ -1629,21 +1808,23 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
     const int64_t wide = sg_wide_threshold(nblk) > dense_threshold ? sg_wide_threshold(nblk) : dense_threshold;
     COMET_CHK(sg_row_list(a, b, rb, re, dense_threshold, dense ? wide : SG_NO_DENSE, &list));
     uint32_t *gbm = nullptr, *gmask = nullptr;
-    if (!g.lds) {
+    if (!g.lds || m) {          // the output row's bitmap is in HBM when LDS holds the mask row instead
         COMET_CHK(g_sg.gbm.ensure(sizeof(uint32_t) * g.bm_words * (size_t)g.groups, true));
         gbm = (uint32_t *)g_sg.gbm.ptr;
     }
-    if (m) {
+    if (m && !g.lds) {
         COMET_CHK(g_sg.gmask.ensure(sizeof(uint32_t) * g.bm_words * (size_t)g.groups, true));
         gmask = (uint32_t *)g_sg.gmask.ptr;
     }
     COMET_CHK(g_sg.slabs.ensure(sizeof(double) * (size_t)(b->ncols > 0 ? b->ncols : 1) * (size_t)g.groups, true));
     const dim3 grid((unsigned)g.groups), block(SG_T);
+    // a masked product keeps either the mask row's bitmap or its hash table in LDS, whichever the row needs
+    const size_t num_lds = m && g.lds && g.lds_bytes < SG_HASH_LDS ? SG_HASH_LDS : g.lds_bytes;
 #define LAUNCH_NUM(L, M, S)                                                                                \
     do {                                                                                                   \
-        COMET_CHK(sg_allow_lds(spgemm_numeric_kernel<L, M, S>, g.lds_bytes));                              \
+        COMET_CHK(sg_allow_lds(spgemm_numeric_kernel<L, M, S>, num_lds));                                  \
         KernelTimer t(S ? "spgemm_numeric_semiring" : M ? "spgemm_numeric_masked" : "spgemm_numeric");    \
-        spgemm_numeric_kernel<L, M, S><<<grid, block, g.lds_bytes, stream()>>>(                            \
+        spgemm_numeric_kernel<L, M, S><<<grid, block, num_lds, stream()>>>(                                \
             rb, re, b->ncols, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m ? m->pos : nullptr,        \
             m ? m->crd : nullptr, g.logW, gbm, gmask, (double *)g_sg.slabs.ptr,                            \
             (unsigned long long *)g_sg.ticket.ptr, list, 1, reduce_op, mult_op, Cpos, Ccrd, Cval);         \
