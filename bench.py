@@ -417,6 +417,7 @@ def bench_spgemm(rt, orc, gen, args):
     state = {}
 
     mask = A if args.masked else None      # C<A> = A*A: the output holds the stored entries of A that receive a product
+    semiring = tuple(args.semiring.split(",")) if args.semiring else None       # e.g. min,plus
 
     def step(check=False):
         # the whole product: symbolic over all rows, numeric block by block into the same buffers.  With `check`
@@ -437,7 +438,7 @@ def bench_spgemm(rt, orc, gen, args):
         while rb < n:
             re = int(np.searchsorted(hpos, hpos[rb] + cap, side="right")) - 1
             re = min(max(re, rb + 1), n)
-            rt.spgemm_numeric(A, A, dpos, rb, re, dcrd, dval, mask=mask)
+            rt.spgemm_numeric(A, A, dpos, rb, re, dcrd, dval, mask=mask, semiring=semiring)
             if check:
                 vsum += rt.reduce_sum(dval, int(hpos[re] - hpos[rb]))
             log(f"numeric rows [{rb},{re}): {int(hpos[re] - hpos[rb])} entries")
@@ -473,7 +474,7 @@ def bench_spgemm(rt, orc, gen, args):
     cs = np.bincount(crd, weights=val, minlength=n)
     invariant = float(np.dot(cs, rs))
     cpu = None
-    parity = {"sum_values_rel_err": abs(state["vsum"] - invariant) / invariant} if not args.masked else {}
+    parity = {"sum_values_rel_err": abs(state["vsum"] - invariant) / invariant} if not (args.masked or semiring) else {}
     if not args.no_cpu:
         # CPU checker on a row sample holding about args.cpu_products products, both phases, single thread
         rng = np.random.default_rng(0)
@@ -496,12 +497,12 @@ def bench_spgemm(rt, orc, gen, args):
         for (r0, r1) in picks:
             t0 = time.perf_counter()
             cp, cc, cv = orc.spgemm(pos, crd, val, pos, crd, val, n, rows=(r0, r1),
-                                    mask=(pos, crd) if args.masked else None)
+                                    mask=(pos, crd) if args.masked else None, semiring=semiring)
             t += time.perf_counter() - t0
             struct_ok &= bool(np.array_equal(cp, hpos[r0:r1 + 1] - hpos[r0]))
             cnt = int(hpos[r1] - hpos[r0])
             if cnt <= state["cap"]:
-                rt.spgemm_numeric(A, A, state["dpos"], r0, r1, state["dcrd"], state["dval"], mask=mask)
+                rt.spgemm_numeric(A, A, state["dpos"], r0, r1, state["dcrd"], state["dval"], mask=mask, semiring=semiring)
                 gc, gv = state["dcrd"].to_numpy(cnt), state["dval"].to_numpy(cnt)
                 struct_ok &= bool(np.array_equal(gc, cc)) and bool(np.all(np.abs(gv - cv) <= 1e-12 * np.abs(cv)))
             log(f"  rows [{r0},{r1}): {cnt} entries checked, CPU time so far {t:.1f} s, ok = {struct_ok}")
@@ -513,7 +514,8 @@ def bench_spgemm(rt, orc, gen, args):
     return {
         "metric": "Gustavson SpGEMM GFLOP/s (2 flops per product, symbolic + numeric) on 1 MI355X",
         "value": flops / (dev_ms * 1e-3) / 1e9, "unit": "GFLOP/s", "ms_per_step": dev_ms, "dtype": "f64",
-        "config": {"workload": "spgemm_rmat_AxA_masked_by_A" if args.masked else "spgemm_rmat_AxA", "scale": scale, "edge_factor": 16, "nnz_A": int(nnzA),
+        "config": {"workload": ("spgemm_rmat_AxA_masked_by_A" if args.masked else "spgemm_rmat_AxA") +
+                               ("_" + "_".join(semiring) if semiring else ""), "scale": scale, "edge_factor": 16, "nnz_A": int(nnzA),
                    "products": nprod, "nnz_C": nnzC, "row_blocks": state["blocks"], "block_budget_gb": args.budget_gb,
                    "seed": 20},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / ((sym_ms + num_ms) * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
@@ -671,6 +673,7 @@ def main():
     ap.add_argument("--budget-gb", type=float, default=48.0, help="spgemm: output bytes per numeric row block")
     ap.add_argument("--cpu-products", type=int, default=1_500_000_000, help="spgemm: products in the CPU sample")
     ap.add_argument("--masked", action="store_true", help="spgemm: the masked product C<A> = A*A, materialised")
+    ap.add_argument("--semiring", default="", help="spgemm: reduce,mult of another semiring, e.g. min,plus")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -316,6 +316,40 @@ __device__ inline double key_f64(unsigned long long k)
     const unsigned long long u = (k >> 63) ? (k & 0x7fffffffffffffffull) : ~k;
     return __longlong_as_double((long long)u);
 }
+// One product of a semiring into an accumulator in LDS.  plus adds; min, max and any keep a 64-bit key and take the
+// larger one, so the result does not depend on the order of the products: min the complement of the value's key,
+// max the key, any the place (pa, q) of the product - pa counts the entries of the row of A from 1, q is the place
+// in B - so that the product the reference's sequential loop reaches last wins.  An accumulator that received
+// nothing is all-zero whatever the semiring.
+__device__ __forceinline__ void semiring_lds_add(double *slot, int reduce_op, int mult_op, double a, double b, int pa,
+                                                 int64_t q)
+{
+    unsigned long long *key = reinterpret_cast<unsigned long long *>(slot);
+    if (reduce_op == SR_ANY) {
+        __hip_atomic_fetch_max(key, ((unsigned long long)(uint32_t)pa << 32) | (unsigned long long)(uint32_t)q,
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    } else {
+        const double e = semiring_mult(mult_op, a, b);
+        if (reduce_op == SR_PLUS)
+            __hip_atomic_fetch_add(slot, e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        else
+            __hip_atomic_fetch_max(key, reduce_op == SR_MIN ? ~f64_key(e) : f64_key(e), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+}
+// The value such an accumulator stands for (as = where the row of A begins).  max starts from 0, as the reference's
+// accumulator does, and so never returns less.
+__device__ __forceinline__ double semiring_lds_value(unsigned long long v, int reduce_op, int mult_op, int64_t as,
+                                                     const double *__restrict__ Aval, const double *__restrict__ Bval)
+{
+    if (reduce_op == SR_PLUS)
+        return __longlong_as_double((long long)v);
+    if (reduce_op == SR_MIN)
+        return key_f64(~v);
+    if (reduce_op == SR_MAX)
+        return v < f64_key(0.0) ? 0.0 : key_f64(v);
+    return semiring_mult(mult_op, Aval[as + (int64_t)(v >> 32) - 1], Bval[(int64_t)(v & 0xffffffffull)]);
+}
 extern __shared__ uint32_t sg_dyn_lds[];
 // Hash table of a masked product's mask row (see spgemm_numeric_kernel): values first (8-byte aligned), keys after.
 constexpr int SG_HASH_LOG = 13, SG_HASH_SLOTS = 1 << SG_HASH_LOG;
@@ -800,9 +834,10 @@ __device__ __forceinline__ int visit_flag(int *flags, int visit, int touched, in
     return __builtin_amdgcn_readfirstlane(flags[visit]);
 }
 
-// Visits the products of one slice per lane: f(j, x) for the entries [lo, hi) of a row of B (the part of it inside
-// the column block or blocks being swept), j the column and x = a times the entry's value (0 without VALUES,
-// when the value array is not read).  Returns whether this wavefront had anything to visit.
+// Visits the products of one slice per lane: f(j, a, b, pa, q) for the entries [lo, hi) of a row of B (the part of
+// it inside the column block or blocks being swept), j the column, a the entry of A (and pa the tag the caller
+// gave it: its place in the row of A, which only the `any` semiring needs), b the entry of B (0 without VALUES,
+// when the value array is not read) and q its place in B.  Returns whether this wavefront had anything to visit.
 
 constexpr int SG_SHORT = 32;                      // slices shorter than this are taken by 16 lanes, the others by 64
 constexpr int SG_SHORT_LOADS = SG_SHORT / 16;     // entries of a short slice per lane
@@ -812,7 +847,7 @@ constexpr int SG_LONG_LOADS = 4;                  // entries of a long slice per
 // entries o + 64 x < len, x < SG_LONG_LOADS (o = l for the first turn of a slice).  All loads are issued before
 // the first visit, and a load that no lane needs is skipped.
 template <bool VALUES, typename F>
-__device__ __forceinline__ void turn_of_slice(int64_t s, int64_t o, int64_t len, double at,
+__device__ __forceinline__ void turn_of_slice(int64_t s, int64_t o, int64_t len, double at, int pt,
                                               const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval, F f)
 {
     int64_t q[SG_LONG_LOADS];
@@ -833,11 +868,11 @@ __device__ __forceinline__ void turn_of_slice(int64_t s, int64_t o, int64_t len,
 #pragma unroll
     for (int x = 0; x < SG_LONG_LOADS; ++x)
         if (ok[x])
-            f(j[x], at * v[x]);
+            f(j[x], at, v[x], pt, q[x]);
 }
 
 template <bool VALUES, typename F>
-__device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double a, int lane,
+__device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double a, int pa, int lane,
                                                   const int32_t *__restrict__ Bcrd,
                                                   const double *__restrict__ Bval, F f)
 {
@@ -858,6 +893,7 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
         big &= big - 1;
         const int64_t s = readlane_i64(lo, t), len = readlane_i64(hi, t) - s;
         const double at = readlane_d(a, t);
+        const int pt = __builtin_amdgcn_readlane(pa, t);
         int64_t o = lane;
         if (len >= 64 * SG_LONG_LOADS) {
             // turns in which every lane has all its entries run without predicates, and the loads of the next
@@ -881,7 +917,7 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
                     vn[x] = VALUES ? Bval[s + o + 64 * (SG_LONG_LOADS + x)] : 0.0;
 #pragma unroll
                 for (int x = 0; x < SG_LONG_LOADS; ++x) {
-                    f(j[x], at * v[x]);
+                    f(j[x], at, v[x], pt, s + o + 64 * x);
                 }
 #pragma unroll
                 for (int x = 0; x < SG_LONG_LOADS; ++x) {
@@ -892,12 +928,12 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
             }
 #pragma unroll
             for (int x = 0; x < SG_LONG_LOADS; ++x) {
-                f(j[x], at * v[x]);
+                f(j[x], at, v[x], pt, s + o + 64 * x);
             }
             o += 64 * SG_LONG_LOADS;
         }
         if (o < len)
-            turn_of_slice<VALUES>(s, o, len, at, Bcrd, Bval, f);
+            turn_of_slice<VALUES>(s, o, len, at, pt, Bcrd, Bval, f);
     }
     const int quarter = lane >> 4, sub = lane & 15;
     while (todo) {              // four short slices per turn, one to a quarter, SG_SHORT_LOADS entries per lane
@@ -914,6 +950,7 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
         const int64_t e = ((int64_t)__shfl((int)(hi >> 32), src, 64) << 32) |
                           (uint32_t)__shfl((int)(hi & 0xffffffff), src, 64);
         const double at = __hiloint2double(__shfl(__double2hiint(a), src, 64), __shfl(__double2loint(a), src, 64));
+        const int pt = __shfl(pa, src, 64);
         int64_t q[SG_SHORT_LOADS];
         bool ok[SG_SHORT_LOADS];
 #pragma unroll
@@ -932,19 +969,21 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
 #pragma unroll
         for (int x = 0; x < SG_SHORT_LOADS; ++x) {
             if (ok[x]) {
-                f(j[x], at * v[x]);
+                f(j[x], at, v[x], pt, q[x]);
             }
         }
     }
     return touched;
 }
 
+template <bool SEMI>
 __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
     int64_t row_begin, int64_t row_end, const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd,
     const double *__restrict__ Aval, const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval,
     const int64_t *__restrict__ blkptr, int nblk,
     unsigned long long *ticket, RowList list,
-    const int64_t *__restrict__ Cpos, int32_t *__restrict__ Ccrd, double *__restrict__ Cval)
+    const int64_t *__restrict__ Cpos, int32_t *__restrict__ Ccrd, double *__restrict__ Cval, int reduce_op,
+    int mult_op)
 {
     __shared__ int64_t row_slot;
     __shared__ int wave_tot[SG_WAVES];
@@ -977,6 +1016,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
             const int held = __builtin_amdgcn_readfirstlane((int)(ae - as <= SG_T));
             int64_t h_lo = 0, h_hi = 0;
             double h_a = 0.0;
+            int h_pa = 0;
             const int64_t *h_bp = nullptr;
             if (held) {
                 const int64_t p = as + wave + (int64_t)lane * SG_WAVES;
@@ -985,21 +1025,35 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                     h_lo = h_bp[0];
                     h_hi = h_bp[1];
                     h_a = Aval[p];
+                    h_pa = (int)(p - as + 1);
                 }
             }
             for (int cb = 0; cb < nblk; ++cb) {
                 const int col0 = cb << SG_CB_LOG;
                 int touched = 0;     // did this wavefront add anything to the block
-                const auto add = [&](int j, double x) {
+                const auto add = [&](int j, double a, double b, int pa, int64_t q) {
                     j -= col0;
                     atomicOr(&bm[j >> 5], 1u << (j & 31));
-                    __hip_atomic_fetch_add(&acc[j], x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    if constexpr (SEMI)
+                        semiring_lds_add(&acc[j], reduce_op, mult_op, a, b, pa, q);
+                    else
+                        __hip_atomic_fetch_add(&acc[j], a * b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                };
+                const auto take = [&](int j) -> double {         // the block's value of column j, which is cleared
+                    double out;
+                    if constexpr (SEMI)
+                        out = semiring_lds_value(reinterpret_cast<unsigned long long *>(acc)[j], reduce_op, mult_op, as,
+                                                 Aval, Bval);
+                    else
+                        out = acc[j];
+                    acc[j] = 0.0;
+                    return out;
                 };
                 if (held) {
                     int64_t next = h_hi;
                     if (h_bp && cb + 1 < nblk)
                         next = h_bp[cb + 2];
-                    touched = for_each_in_slices<true>(h_lo, h_hi, h_a, lane, Bcrd, Bval, add);
+                    touched = for_each_in_slices<true>(h_lo, h_hi, h_a, h_pa, lane, Bcrd, Bval, add);
                     h_lo = h_hi;
                     h_hi = next;
                 }
@@ -1008,14 +1062,16 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                     const int cnt = (int)(left < 64 ? left : 64);
                     int64_t lo = 0, hi = 0;
                     double a = 0.0;
+                    int pa = 0;
                     if (lane < cnt) {
                         const int64_t p = base + (int64_t)lane * SG_WAVES;
                         const int64_t *bp = blkptr + (int64_t)Acrd[p] * (nblk + 1) + cb;
                         lo = bp[0];
                         hi = bp[1];
                         a = Aval[p];
+                        pa = (int)(p - as + 1);
                     }
-                    touched |= for_each_in_slices<true>(lo, hi, a, lane, Bcrd, Bval, add);
+                    touched |= for_each_in_slices<true>(lo, hi, a, pa, lane, Bcrd, Bval, add);
                 }
                 const int any = visit_flag(block_touched, visit, touched, lane);
                 visit = visit == 2 ? 0 : visit + 1;
@@ -1054,8 +1110,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                     for (int q = threadIdx.x; q < total; q += SG_T) {
                         const int j = emit_col[q];
                         store_streaming(&Ccrd[off + q], col0 + j);
-                        store_streaming(&Cval[off + q], acc[j]);
-                        acc[j] = 0.0;
+                        store_streaming(&Cval[off + q], take(j));
                     }
                     lds_barrier();
                 } else {
@@ -1073,8 +1128,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                     for (int q = threadIdx.x; q < n; q += SG_T) {
                         const int j = emit_col[q];
                         store_streaming(&Ccrd[off + c0 + q], col0 + j);
-                        store_streaming(&Cval[off + c0 + q], acc[j]);
-                        acc[j] = 0.0;
+                        store_streaming(&Cval[off + c0 + q], take(j));
                     }
                     lds_barrier();
                 }
@@ -1108,12 +1162,14 @@ constexpr size_t SG_SPAN_LDS = (size_t)SP_CAP * 8 + (size_t)SP_WORDS * 4 + (size
 static_assert(SP_WORDS % SG_T == 0 && SP_BLOCK_WORDS % SP_WPT == 0 && SP_CAP >= SG_CB && SP_CAP <= 65535,
               "a thread's words lie in one block, one block fits the value array, ranks fit 16 bits");
 
+template <bool SEMI>
 __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
     int64_t row_begin, int64_t row_end, const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd,
     const double *__restrict__ Aval, const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval,
     const int64_t *__restrict__ blkptr, int nblk,
     unsigned long long *ticket, RowList list,
-    const int64_t *__restrict__ Cpos, int32_t *__restrict__ Ccrd, double *__restrict__ Cval)
+    const int64_t *__restrict__ Cpos, int32_t *__restrict__ Ccrd, double *__restrict__ Cval, int reduce_op,
+    int mult_op)
 {
     __shared__ int64_t row_slot;
     __shared__ int wave_tot[SG_WAVES];
@@ -1148,7 +1204,14 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
             const double a = Aval[as];
             for (int64_t q = threadIdx.x; q < len; q += SG_T) {
                 store_streaming(&Ccrd[off + q], Bcrd[bs + q]);
-                store_streaming(&Cval[off + q], 0.0 + a * Bval[bs + q]);
+                if constexpr (SEMI) {        // what the reference's accumulator holds after this one product
+                    const double e = semiring_mult(mult_op, a, Bval[bs + q]);
+                    store_streaming(&Cval[off + q], reduce_op == SR_PLUS  ? 0.0 + e
+                                                    : reduce_op == SR_MAX ? (f64_key(e) < f64_key(0.0) ? 0.0 : e)
+                                                                          : e);
+                } else {
+                    store_streaming(&Cval[off + q], 0.0 + a * Bval[bs + q]);
+                }
             }
         } else if (as != ae) {
             int64_t off = Cpos[i] - out0;
@@ -1160,6 +1223,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
             const int held = __builtin_amdgcn_readfirstlane((int)(ae - as <= SG_T));
             const int small = __builtin_amdgcn_readfirstlane((int)(ae - as <= 64));
             double h_a = 0.0;
+            int h_pa = 0;
             const int64_t *h_bp = nullptr;
             int64_t h_lo = 0, h_hi = 0;
             if (held) {
@@ -1167,6 +1231,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
                 if (p < ae) {
                     h_bp = blkptr + (int64_t)Acrd[p] * (nblk + 1);
                     h_a = Aval[p];
+                    h_pa = (int)(p - as + 1);
                     h_lo = h_bp[0];
                     h_hi = h_bp[nblk < SP_BLOCKS ? nblk : SP_BLOCKS];
                 }
@@ -1186,24 +1251,26 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
                         const int c = g - (__builtin_amdgcn_readlane(upto, e) - __builtin_amdgcn_readlane(mine, e));
                         const int64_t s = readlane_i64(held_lo, e) + (int64_t)c * SP_CHUNK;
                         const int64_t left = readlane_i64(held_hi, e) - s;
-                        turn_of_slice<VALUES>(s, lane, left < SP_CHUNK ? left : SP_CHUNK, readlane_d(h_a, e), Bcrd,
-                                              Bval, f);
+                        turn_of_slice<VALUES>(s, lane, left < SP_CHUNK ? left : SP_CHUNK, readlane_d(h_a, e),
+                                              __builtin_amdgcn_readlane(h_pa, e), Bcrd, Bval, f);
                     }
                 } else if (held)
-                    touched = for_each_in_slices<VALUES>(held_lo, held_hi, h_a, lane, Bcrd, Bval, f);
+                    touched = for_each_in_slices<VALUES>(held_lo, held_hi, h_a, h_pa, lane, Bcrd, Bval, f);
                 for (int64_t base = as + wave; !held && base < ae; base += (int64_t)SG_WAVES * 64) {
                     const int64_t left = (ae - base + SG_WAVES - 1) / SG_WAVES;
                     const int cnt = (int)(left < 64 ? left : 64);
                     int64_t lo = 0, hi = 0;
                     double a = 0.0;
+                    int pa = 0;
                     if (lane < cnt) {
                         const int64_t p = base + (int64_t)lane * SG_WAVES;
                         const int64_t *bp = blkptr + (int64_t)Acrd[p] * (nblk + 1);
                         lo = bp[cbf];
                         hi = bp[cbt];
                         a = Aval[p];
+                        pa = (int)(p - as + 1);
                     }
-                    touched |= for_each_in_slices<VALUES>(lo, hi, a, lane, Bcrd, Bval, f);
+                    touched |= for_each_in_slices<VALUES>(lo, hi, a, pa, lane, Bcrd, Bval, f);
                 }
                 return touched;
             };
@@ -1214,7 +1281,8 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
                 int64_t h_next = h_hi;      // where the span after this one ends
                 if (h_bp && cb + nbv < nblk)
                     h_next = h_bp[cb + nbv + SP_BLOCKS < nblk ? cb + nbv + SP_BLOCKS : nblk];
-                const int touched = walk(cb, cb + nbv, h_lo, h_hi, std::false_type{}, [&](int j, double) {
+                const int touched = walk(cb, cb + nbv, h_lo, h_hi, std::false_type{},
+                                         [&](int j, double, double, int, int64_t) {
                     j -= col0;
                     atomicOr(&bm[j >> 5], 1u << (j & 31));
                 });
@@ -1259,15 +1327,24 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
                             h_next = h_bp[cb + nb + SP_BLOCKS < nblk ? cb + nb + SP_BLOCKS : nblk];
                         }
                     }
-                    walk(cb, cb + nb, h_lo, h_hi, std::true_type{}, [&](int j, double x) {
+                    walk(cb, cb + nb, h_lo, h_hi, std::true_type{}, [&](int j, double a, double b, int pa, int64_t q) {
                         j -= col0;
                         const uint32_t below = bm[j >> 5] & ((1u << (j & 31)) - 1u);
                         const int r = pre[j >> 5] + __popc(below);
-                        __hip_atomic_fetch_add(&val[r], x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        if constexpr (SEMI)
+                            semiring_lds_add(&val[r], reduce_op, mult_op, a, b, pa, q);
+                        else
+                            __hip_atomic_fetch_add(&val[r], a * b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                     });
                     lds_barrier();
-                    for (int q = threadIdx.x; q < total; q += SG_T)
-                        store_streaming(&Cval[off + q], val[q]);
+                    for (int q = threadIdx.x; q < total; q += SG_T) {
+                        if constexpr (SEMI)
+                            store_streaming(&Cval[off + q],
+                                            semiring_lds_value(reinterpret_cast<unsigned long long *>(val)[q], reduce_op,
+                                                               mult_op, as, Aval, Bval));
+                        else
+                            store_streaming(&Cval[off + q], val[q]);
+                    }
                     lds_barrier();
                     // the values are out: their array now takes the list of the columns, so that these leave
                     // through coalesced stores too (from their owners they would scatter, four bytes per lane)
@@ -1800,7 +1877,8 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
     COMET_CHK(sg_reset_ticket());
     // rows with many products go to the LDS-accumulator kernel (unmasked products only)
     const int nblk = (int)ceil_div(b->ncols > 0 ? b->ncols : 1, SG_CB);
-    const bool dense = !m && !semi && nblk <= SG_DENSE_MAX_BLOCKS;
+    // (the `any` semiring keeps a product's place in B in 32 bits of its accumulator)
+    const bool dense = !m && nblk <= SG_DENSE_MAX_BLOCKS && (reduce_op != COMET_SR_ANY || b->nnz < (1ll << 32));
     const int64_t dense_threshold = dense ? SG_DENSE_PER_BLOCK * nblk : SG_NO_DENSE;
     if (dense)
         COMET_CHK(sg_plan_blocks(b));
@@ -1843,21 +1921,36 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
     COMET_HIPCHK(hipGetLastError());
     if (dense) {
         COMET_CHK(sg_reset_ticket());
-        COMET_CHK(sg_allow_lds(spgemm_numeric_dense_kernel, SG_DENSE_LDS));
         KernelTimer t("spgemm_numeric_dense");
-        spgemm_numeric_dense_kernel<<<dim3((unsigned)(num_cus() > 0 ? num_cus() : 256)), block, SG_DENSE_LDS,
-                                      stream()>>>(rb, re, a->pos, a->crd, a->val, b->crd, b->val, b->sg_blkptr,
-                                                  nblk, (unsigned long long *)g_sg.ticket.ptr, list, Cpos, Ccrd,
-                                                  Cval);
+        const dim3 cus((unsigned)(num_cus() > 0 ? num_cus() : 256));
+        if (semi) {
+            COMET_CHK(sg_allow_lds(spgemm_numeric_dense_kernel<true>, SG_DENSE_LDS));
+            spgemm_numeric_dense_kernel<true><<<cus, block, SG_DENSE_LDS, stream()>>>(
+                rb, re, a->pos, a->crd, a->val, b->crd, b->val, b->sg_blkptr, nblk,
+                (unsigned long long *)g_sg.ticket.ptr, list, Cpos, Ccrd, Cval, reduce_op, mult_op);
+        } else {
+            COMET_CHK(sg_allow_lds(spgemm_numeric_dense_kernel<false>, SG_DENSE_LDS));
+            spgemm_numeric_dense_kernel<false><<<cus, block, SG_DENSE_LDS, stream()>>>(
+                rb, re, a->pos, a->crd, a->val, b->crd, b->val, b->sg_blkptr, nblk,
+                (unsigned long long *)g_sg.ticket.ptr, list, Cpos, Ccrd, Cval, reduce_op, mult_op);
+        }
         COMET_HIPCHK(hipGetLastError());
     }
     if (dense) {
         COMET_CHK(sg_reset_ticket());
-        COMET_CHK(sg_allow_lds(spgemm_numeric_span_kernel, SG_SPAN_LDS));
         KernelTimer t("spgemm_numeric_span");
-        spgemm_numeric_span_kernel<<<dim3((unsigned)(num_cus() > 0 ? num_cus() : 256)), block, SG_SPAN_LDS,
-                                     stream()>>>(rb, re, a->pos, a->crd, a->val, b->crd, b->val, b->sg_blkptr, nblk,
-                                                 (unsigned long long *)g_sg.ticket.ptr, list, Cpos, Ccrd, Cval);
+        const dim3 cus((unsigned)(num_cus() > 0 ? num_cus() : 256));
+        if (semi) {
+            COMET_CHK(sg_allow_lds(spgemm_numeric_span_kernel<true>, SG_SPAN_LDS));
+            spgemm_numeric_span_kernel<true><<<cus, block, SG_SPAN_LDS, stream()>>>(
+                rb, re, a->pos, a->crd, a->val, b->crd, b->val, b->sg_blkptr, nblk,
+                (unsigned long long *)g_sg.ticket.ptr, list, Cpos, Ccrd, Cval, reduce_op, mult_op);
+        } else {
+            COMET_CHK(sg_allow_lds(spgemm_numeric_span_kernel<false>, SG_SPAN_LDS));
+            spgemm_numeric_span_kernel<false><<<cus, block, SG_SPAN_LDS, stream()>>>(
+                rb, re, a->pos, a->crd, a->val, b->crd, b->val, b->sg_blkptr, nblk,
+                (unsigned long long *)g_sg.ticket.ptr, list, Cpos, Ccrd, Cval, reduce_op, mult_op);
+        }
         COMET_HIPCHK(hipGetLastError());
     }
     return COMET_HIP_OK;

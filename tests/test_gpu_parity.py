@@ -473,6 +473,46 @@ def test_spgemm_rows_of_every_class(m, long_len, wide, monkeypatch):
     assert np.array_equal(first[1], second[1])
 
 
+@pytest.mark.parametrize("semiring", [("min", "plus"), ("max", "times"), ("any", "second"), ("any", "pair"),
+                                      ("plus", "first"), ("min", "div")])
+@pytest.mark.parametrize("m,long_len,wide", [(200_000, 2000, None), (40_000, 1200, 1 << 40), (200_000, 2000, 0)])
+def test_spgemm_semiring_rows_of_every_class(semiring, m, long_len, wide, monkeypatch):
+    # the rows of test_spgemm_rows_of_every_class under other semirings: the kernels that keep a row's values in
+    # LDS hold keys there instead of sums (min, max: order-preserving keys; any: the place of the product)
+    if wide is not None:
+        monkeypatch.setenv("COMET_HIP_SPGEMM_WIDE", str(wide))
+    rng = np.random.default_rng(29)
+    k = 400
+    bpos, bcrd, bval = _rows_of_lengths(rng, [long_len] * 200 + [10] * 200, m)
+    bval = np.where(bval < 0, bval - 0.25, bval + 0.25)          # keeps div finite
+    long_rows, short_rows = np.arange(200), np.arange(200, 400)
+    lengths, picks = [], []
+    for n_long, n_short in [(0, 0), (0, 5), (1, 0), (3, 2), (10, 0), (25, 40), (40, 0), (120, 3), (200, 200), (0, 200),
+                            (2, 0), (60, 0), (0, 1), (7, 7)] * 2:
+        lengths.append(n_long + n_short)
+        picks.append(np.sort(np.concatenate([rng.choice(long_rows, n_long, replace=False),
+                                             rng.choice(short_rows, n_short, replace=False)])))
+    apos = np.zeros(len(lengths) + 1, dtype=np.int64)
+    np.cumsum(lengths, out=apos[1:])
+    acrd = np.concatenate(picks).astype(np.int64)
+    aval = rng.uniform(-1, 1, len(acrd))
+    A = rt.CsrMatrix.from_arrays((len(lengths), k), apos, acrd, aval)
+    B = rt.CsrMatrix.from_arrays((k, m), bpos, bcrd, bval)
+    wp, wc, wv = orc.spgemm(apos, acrd, aval, bpos, bcrd, bval, m, semiring=semiring)
+    for _ in range(2):          # twice: the accumulators are left clean
+        p, c, v = rt.spgemm(A, B, semiring=semiring).to_arrays()
+        assert np.array_equal(p, wp) and np.array_equal(c, wc)
+        if semiring[0] == "plus":
+            _, _, bound = orc.spgemm(apos, acrd, np.abs(aval), bpos, bcrd, np.abs(bval), m, semiring=semiring)
+            assert np.all(np.abs(v - wv) <= RTOL * bound)
+        else:
+            assert np.array_equal(v, wv)
+    p, c, v = rt.spgemm(A, B).to_arrays()          # and a plus-times product after them finds nothing left behind
+    _, _, pv = orc.spgemm(apos, acrd, aval, bpos, bcrd, bval, m)
+    _, _, bound = orc.spgemm(apos, acrd, np.abs(aval), bpos, bcrd, np.abs(bval), m)
+    assert np.array_equal(c, wc) and np.all(np.abs(v - pv) <= RTOL * bound)
+
+
 @pytest.mark.parametrize("wide", [1 << 40, 0])
 def test_spgemm_rows_with_more_entries_than_lanes(wide, monkeypatch):
     # more than 1024 entries in a row of A: the LDS kernels then fetch the row's entries again at every visit
