@@ -84,14 +84,74 @@ struct BmAddr {
 // turn costs about one trip to memory, so each turn issues all of its loads (up
 // to four per lane; a load no lane needs is skipped) before the visitor runs.
 constexpr int FEP_SHORT = 32, FEP_SHORT_LOADS = FEP_SHORT / 16, FEP_LONG_LOADS = 4;
-template <bool VALUES, typename F>
-__device__ inline void for_each_product(int64_t as, int64_t ae, const int32_t *__restrict__ Acrd,
-                                        const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
-                                        const int32_t *__restrict__ Bcrd, F f)
+// what the look-up and fetch steps of a masked product's visitor hand to the visit itself: where the column's
+// value lives (negative: the mask does not hold the column) and B's value, fetched for hits only
+struct MaskHit {
+    int at;
+    double b;
+};
+// four consecutive entries of an index array that lies at any 4-byte boundary
+typedef int sg_i4u __attribute__((ext_vector_type(4), aligned(4)));
+// With WIDE, a lane takes four consecutive entries in a turn in which every lane has all its entries - one 16-byte
+// load instead of four loads 64 entries apart - and f4(j, q, a, p, s) visits the entries q .. q + 3 of B_k at once
+// (their columns in j).  That pays where the visitor can treat neighbouring columns together (the symbolic phase:
+// 78 -> 64 ms on A*A of an R-MAT graph of scale 20); a visitor that probes a hash table per product is slower with
+// it (masked numeric phase, 247 -> 300 ms).
+// A visitor that looks its column up in LDS first (a mask's bitmap or hash table) and fetches B's value only on a
+// hit hands these two steps in as pre(j) and mid(j, q, what pre returned), and f gets what mid returned as a sixth
+// argument.  The walk runs pre for all the entries of a turn together, then mid for all of them (inside f each
+// step would sit behind the branch of the entry before it: four trips to LDS and four to memory per turn, one
+// after the other) - and it visits a turn's entries one turn late, after the next turn's columns have arrived and
+// its look-ups are out, so that the trip to memory for the values of the hits overlaps with the next turn's instead
+// of standing alone (a wavefront runs its turns one after the other, and nothing else hides that trip).  The
+// look-ups of a turn therefore run before the visits of the turn before it: they must not depend on them.
+template <bool VALUES, bool WIDE, typename PRE, typename MID, typename F, typename F4>
+__device__ inline void for_each_product_impl(int64_t as, int64_t ae, const int32_t *__restrict__ Acrd,
+                                             const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
+                                             const int32_t *__restrict__ Bcrd, PRE pre, MID mid, F f, F4 f4)
 {
+    using T1 = decltype(pre(0));
+    using T2 = decltype(mid(0, (int64_t)0, T1()));
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int quarter = lane >> 4, sub = lane & 15;
+    // the entries of the turn before: visited once the next turn's look-ups are out
+    constexpr int NP = FEP_LONG_LOADS > FEP_SHORT_LOADS ? FEP_LONG_LOADS : FEP_SHORT_LOADS;
+    bool w_ok[NP];
+    int w_j[NP];
+    int64_t w_q[NP], w_p[NP], w_s[NP];
+    double w_a[NP];
+    T2 w_md[NP];
+#pragma unroll
+    for (int x = 0; x < NP; ++x)
+        w_ok[x] = false;
+    const auto visit_pending = [&]() {
+#pragma unroll
+        for (int x = 0; x < NP; ++x)
+            if (w_ok[x])
+                f(w_j[x], w_q[x], w_a[x], w_p[x], w_s[x], w_md[x]);
+    };
+    // one turn: up to N entries per lane (ok[x]: the lane has entry x), columns j, places q in B
+    const auto turn = [&](auto n_tag, const bool *ok, const int *j, const int64_t *q, double at, int64_t p, int64_t s) {
+        constexpr int N = decltype(n_tag)::value;
+        T1 tk[N];
+#pragma unroll
+        for (int x = 0; x < N; ++x)
+            tk[x] = ok[x] ? pre(j[x]) : T1();
+        visit_pending();
+#pragma unroll
+        for (int x = 0; x < NP; ++x) {
+            w_ok[x] = x < N ? ok[x] : false;
+            if (x < N) {
+                w_j[x] = j[x];
+                w_q[x] = q[x];
+                w_a[x] = at;
+                w_p[x] = p;
+                w_s[x] = s;
+                w_md[x] = ok[x] ? mid(j[x], q[x], tk[x]) : T2();
+            }
+        }
+    };
     for (int64_t base = as + wave; base < ae; base += (int64_t)SG_WAVES * 64) {
         const int64_t left = (ae - base + SG_WAVES - 1) / SG_WAVES;     // my entries from here on
         const int cnt = (int)(left < 64 ? left : 64);
@@ -114,14 +174,35 @@ __device__ inline void for_each_product(int64_t as, int64_t ae, const int32_t *_
             const double at = VALUES ? readlane_d(a, t) : 0.0;
             const int64_t p = base + (int64_t)t * SG_WAVES;
             int64_t o = lane;
-            if (len >= 64 * FEP_LONG_LOADS) {
-                // Turns in which every lane has all its entries: straight-line code, so that the visitors'
-                // LDS operations are issued together as well, and the loads of the next turn are in flight
-                // while the visitor works on this one.
+            if (WIDE && len >= 64 * FEP_LONG_LOADS) {
+                // Turns in which every lane has all its entries: a lane takes four consecutive ones, a single
+                // 16-byte load, and the loads of the next turn are in flight while the visitor works on this one.
+                static_assert(FEP_LONG_LOADS == 4, "a lane's entries of a full turn are one 16-byte load");
+                int64_t c = s + 4 * (int64_t)lane;
+                sg_i4u j = *reinterpret_cast<const sg_i4u *>(Bcrd + c);
+                int64_t done = 0;
+                for (int64_t full = 64 * FEP_LONG_LOADS; full + 64 * FEP_LONG_LOADS <= len;
+                     full += 64 * FEP_LONG_LOADS) {
+                    const sg_i4u jn = *reinterpret_cast<const sg_i4u *>(Bcrd + c + 64 * FEP_LONG_LOADS);
+                    f4(j, c, at, p, s);
+                    j = jn;
+                    c += 64 * FEP_LONG_LOADS;
+                    done += 64 * FEP_LONG_LOADS;
+                }
+                f4(j, c, at, p, s);
+                o += done + 64 * FEP_LONG_LOADS;
+            }
+            if (!WIDE && len >= 64 * FEP_LONG_LOADS) {
+                // Turns in which every lane has all its entries: no predicates, and the loads of the next such
+                // turn are in flight while this one's look-ups and the visits of the turn before it run.
+                bool all[FEP_LONG_LOADS];
                 int j[FEP_LONG_LOADS];
+                int64_t q[FEP_LONG_LOADS];
 #pragma unroll
-                for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                for (int x = 0; x < FEP_LONG_LOADS; ++x) {
+                    all[x] = true;
                     j[x] = Bcrd[s + o + 64 * x];
+                }
                 for (int64_t full = 64 * FEP_LONG_LOADS; full + 64 * FEP_LONG_LOADS <= len;
                      full += 64 * FEP_LONG_LOADS) {
                     int jn[FEP_LONG_LOADS];
@@ -130,7 +211,8 @@ __device__ inline void for_each_product(int64_t as, int64_t ae, const int32_t *_
                         jn[x] = Bcrd[s + o + 64 * (FEP_LONG_LOADS + x)];
 #pragma unroll
                     for (int x = 0; x < FEP_LONG_LOADS; ++x)
-                        f(j[x], s + o + 64 * x, at, p, s);
+                        q[x] = s + o + 64 * x;
+                    turn(std::integral_constant<int, FEP_LONG_LOADS>(), all, j, q, at, p, s);
 #pragma unroll
                     for (int x = 0; x < FEP_LONG_LOADS; ++x)
                         j[x] = jn[x];
@@ -138,22 +220,23 @@ __device__ inline void for_each_product(int64_t as, int64_t ae, const int32_t *_
                 }
 #pragma unroll
                 for (int x = 0; x < FEP_LONG_LOADS; ++x)
-                    f(j[x], s + o + 64 * x, at, p, s);
+                    q[x] = s + o + 64 * x;
+                turn(std::integral_constant<int, FEP_LONG_LOADS>(), all, j, q, at, p, s);
                 o += 64 * FEP_LONG_LOADS;
             }
             if (o < len) {          // the rest of the row: fewer than 64 * FEP_LONG_LOADS entries
                 bool ok[FEP_LONG_LOADS];
                 int j[FEP_LONG_LOADS];
+                int64_t q[FEP_LONG_LOADS];
 #pragma unroll
-                for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                for (int x = 0; x < FEP_LONG_LOADS; ++x) {
                     ok[x] = o + 64 * x < len;
+                    q[x] = s + o + 64 * x;
+                }
 #pragma unroll
                 for (int x = 0; x < FEP_LONG_LOADS; ++x)
-                    j[x] = ok[x] ? Bcrd[s + o + 64 * x] : 0;
-#pragma unroll
-                for (int x = 0; x < FEP_LONG_LOADS; ++x)
-                    if (ok[x])
-                        f(j[x], s + o + 64 * x, at, p, s);
+                    j[x] = ok[x] ? Bcrd[q[x]] : 0;
+                turn(std::integral_constant<int, FEP_LONG_LOADS>(), ok, j, q, at, p, s);
             }
         }
         while (todo) {
@@ -174,18 +257,47 @@ __device__ inline void for_each_product(int64_t as, int64_t ae, const int32_t *_
             const int64_t p = base + (int64_t)src * SG_WAVES;
             bool ok[FEP_SHORT_LOADS];
             int j[FEP_SHORT_LOADS];
+            int64_t q[FEP_SHORT_LOADS];
 #pragma unroll
-            for (int x = 0; x < FEP_SHORT_LOADS; ++x)
+            for (int x = 0; x < FEP_SHORT_LOADS; ++x) {
                 ok[x] = pick >= 0 && s + sub + 16 * x < e;
+                q[x] = s + sub + 16 * x;
+            }
 #pragma unroll
             for (int x = 0; x < FEP_SHORT_LOADS; ++x)
-                j[x] = ok[x] ? Bcrd[s + sub + 16 * x] : 0;
-#pragma unroll
-            for (int x = 0; x < FEP_SHORT_LOADS; ++x)
-                if (ok[x])
-                    f(j[x], s + sub + 16 * x, at, p, s);
+                j[x] = ok[x] ? Bcrd[q[x]] : 0;
+            turn(std::integral_constant<int, FEP_SHORT_LOADS>(), ok, j, q, at, p, s);
         }
     }
+    visit_pending();
+}
+
+template <bool VALUES, typename F>
+__device__ inline void for_each_product(int64_t as, int64_t ae, const int32_t *__restrict__ Acrd,
+                                        const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
+                                        const int32_t *__restrict__ Bcrd, F f)
+{
+    for_each_product_impl<VALUES, false>(
+        as, ae, Acrd, Aval, Bpos, Bcrd, [](int) { return 0u; }, [](int, int64_t, uint32_t) { return 0u; },
+        [&](int j, int64_t q, double a, int64_t p, int64_t s, uint32_t) { f(j, q, a, p, s); },
+        [](sg_i4u, int64_t, double, int64_t, int64_t) {});
+}
+template <bool VALUES, typename PRE, typename MID, typename F>
+__device__ inline void for_each_product_probed(int64_t as, int64_t ae, const int32_t *__restrict__ Acrd,
+                                               const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
+                                               const int32_t *__restrict__ Bcrd, PRE pre, MID mid, F f)
+{
+    for_each_product_impl<VALUES, false>(as, ae, Acrd, Aval, Bpos, Bcrd, pre, mid, f,
+                                         [](sg_i4u, int64_t, double, int64_t, int64_t) {});
+}
+template <bool VALUES, typename F, typename F4>
+__device__ inline void for_each_product(int64_t as, int64_t ae, const int32_t *__restrict__ Acrd,
+                                        const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
+                                        const int32_t *__restrict__ Bcrd, F f, F4 f4)
+{
+    for_each_product_impl<VALUES, true>(
+        as, ae, Acrd, Aval, Bpos, Bcrd, [](int) { return 0u; }, [](int, int64_t, uint32_t) { return 0u; },
+        [&](int j, int64_t q, double a, int64_t p, int64_t s, uint32_t) { f(j, q, a, p, s); }, f4);
 }
 
 __device__ inline int wave_sum_i32(int v)
@@ -353,8 +465,18 @@ __device__ __forceinline__ double semiring_lds_value(unsigned long long v, int r
 extern __shared__ uint32_t sg_dyn_lds[];
 // Hash table of a masked product's mask row (see spgemm_numeric_kernel): values first (8-byte aligned), keys after.
 constexpr int SG_HASH_LOG = 13, SG_HASH_SLOTS = 1 << SG_HASH_LOG;
-constexpr int SG_HASH_FILL = SG_HASH_SLOTS * 3 / 4;          // longest mask row that goes into the table
+#ifndef COMET_SG_HASH_FILL
+#define COMET_SG_HASH_FILL (SG_HASH_SLOTS * 3 / 4)
+#endif
+constexpr int SG_HASH_FILL = COMET_SG_HASH_FILL;          // longest mask row that goes into the table
 constexpr size_t SG_HASH_LDS = (size_t)SG_HASH_SLOTS * (8 + 4);
+// The first slot a column is looked for in.  (Keeping groups of 32 neighbouring columns together, so that the
+// look-ups of a wavefront walking a sorted row fall into neighbouring LDS banks, was slower: 370 against 240 ms on
+// A*A masked by A at R-MAT scale 20 - a miss that lands in such a group walks to its end.)
+__device__ inline uint32_t sg_hash_slot(int j)
+{
+    return ((uint32_t)j * 2654435761u) >> (32 - SG_HASH_LOG);
+}
 
 // ---------------------------------------------------------------------------
 // Symbolic phase.  Unmasked: set the bit of every reachable column, count the
@@ -411,6 +533,37 @@ __global__ __launch_bounds__(SG_T) void spgemm_symbolic_kernel(
             } else {                                // the bits are counted when the bitmap is cleared
                 const uint32_t old = atomicOr(&bm[ad.word(j)], b);
                 count += (old & b) ? 0 : 1;
+            }
+        }, [&](sg_i4u j, int64_t, double, int64_t, int64_t) {
+            // four consecutive entries of a sorted row: the bits that fall into one word go there together
+            if constexpr (BM_LDS && !MASKED) {
+                int w = ad.word(j.x);
+                uint32_t b = ad.bit(j.x);
+                const int js[3] = {j.y, j.z, j.w};
+#pragma unroll
+                for (int x = 0; x < 3; ++x) {
+                    const int wx = ad.word(js[x]);
+                    if (wx != w) {
+                        atomicOr(&bm[w], b);
+                        w = wx;
+                        b = 0u;
+                    }
+                    b |= ad.bit(js[x]);
+                }
+                atomicOr(&bm[w], b);
+            } else {
+                const int js[4] = {j.x, j.y, j.z, j.w};
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    const uint32_t b = ad.bit(js[x]);
+                    if constexpr (MASKED) {
+                        const uint32_t old = atomicAnd(&bm[ad.word(js[x])], ~b);
+                        count += (old & b) ? 1 : 0;
+                    } else {
+                        const uint32_t old = atomicOr(&bm[ad.word(js[x])], b);
+                        count += (old & b) ? 0 : 1;
+                    }
+                }
             }
         });
         if constexpr (BM_LDS && !MASKED) {
@@ -511,7 +664,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
             double *hval = reinterpret_cast<double *>(sg_dyn_lds);
             unsigned long long *hbits = reinterpret_cast<unsigned long long *>(sg_dyn_lds);
             const auto slot_of = [&](int j) -> int {          // the slot that holds column j, or -1
-                uint32_t sl = ((uint32_t)j * 2654435761u) >> (32 - SG_HASH_LOG);
+                uint32_t sl = sg_hash_slot(j);
                 for (;;) {
                     const uint32_t k = hkey[sl];
                     if ((k & 0x7fffffffu) == (uint32_t)j + 1u)
@@ -524,7 +677,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
             const int64_t ms = Mpos[i], mlen = Mpos[i + 1] - ms;
             for (int64_t e = ms + threadIdx.x; e < ms + mlen; e += SG_T) {
                 const uint32_t key = (uint32_t)Mcrd[e] + 1u;
-                uint32_t sl = ((uint32_t)Mcrd[e] * 2654435761u) >> (32 - SG_HASH_LOG);
+                uint32_t sl = sg_hash_slot(Mcrd[e]);
                 for (;;) {
                     const uint32_t old = atomicCAS(&hkey[sl], 0u, key);
                     if (old == 0u || old == key)
@@ -533,8 +686,18 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
                 }
             }
             __syncthreads();
-            for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, [&](int j, int64_t q, double a, int64_t p, int64_t bs) {
-                const int sl = slot_of(j);
+            const auto first_slot = [](int j) { return sg_hash_slot(j); };
+            for_each_product_probed<true>(as, ae, Acrd, Aval, Bpos, Bcrd, [&](int j) { return hkey[first_slot(j)]; },
+                                          [&](int j, int64_t q, uint32_t k0) {
+                // k0 = the key in the column's first slot: nearly always that settles it
+                MaskHit h{-1, 0.0};
+                if (k0 != 0u)
+                    h.at = (k0 & 0x7fffffffu) == (uint32_t)j + 1u ? (int)first_slot(j) : slot_of(j);
+                if (h.at >= 0 && !(SEMI && reduce_op == SR_ANY))
+                    h.b = Bval[q];
+                return h;
+            }, [&](int j, int64_t q, double a, int64_t p, int64_t bs, MaskHit h) {
+                const int sl = h.at;
                 if (sl < 0)
                     return;
                 if (!(hkey[sl] >> 31))
@@ -544,7 +707,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
                         const unsigned long long key = ((unsigned long long)(p - as + 1) << 32) | (unsigned long long)(q - bs);
                         __hip_atomic_fetch_max(&hbits[sl], key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                     } else {
-                        const double e = semiring_mult(mult_op, a, Bval[q]);
+                        const double e = semiring_mult(mult_op, a, h.b);
                         if (reduce_op == SR_PLUS)
                             __hip_atomic_fetch_add(&hval[sl], e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                         else
@@ -552,7 +715,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                     }
                 } else {
-                    __hip_atomic_fetch_add(&hval[sl], a * Bval[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(&hval[sl], a * h.b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 }
             });
             __syncthreads();
@@ -612,16 +775,25 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
                 atomicOr(&mbm[ad.word(Mcrd[t])], ad.bit(Mcrd[t]));
             __syncthreads();
         }
-        for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, [&](int j, int64_t q, double a, int64_t p, int64_t bs) {
+        for_each_product_probed<true>(as, ae, Acrd, Aval, Bpos, Bcrd, [&](int j) {
+            if constexpr (MASK_LDS)
+                return mbm[ad.word(j)];      // the mask row was set before the barrier above and does not change
+            else
+                return 0u;
+        }, [&](int j, int64_t q, uint32_t mword) {
+            MaskHit h{0, 0.0};
+            if constexpr (MASK_LDS)
+                h.at = (mword & ad.bit(j)) ? 0 : -1;
+            else if constexpr (MASKED)
+                h.at = (atomicOr(&mbm[ad.word(j)], 0u) & ad.bit(j)) ? 0 : -1;
+            if (h.at >= 0 && !(SEMI && reduce_op == SR_ANY))
+                h.b = Bval[q];
+            return h;
+        }, [&](int j, int64_t q, double a, int64_t p, int64_t bs, MaskHit h) {
+            if (h.at < 0)
+                return;
             const int w = ad.word(j);
             const uint32_t b = ad.bit(j);
-            if constexpr (MASK_LDS) {
-                if (!(mbm[w] & b))       // the mask row was set before the barrier above and does not change
-                    return;
-            } else if constexpr (MASKED) {
-                if (!(atomicOr(&mbm[w], 0u) & b))
-                    return;
-            }
             atomicOr(&bm[w], b);
             if constexpr (SEMI) {
                 unsigned long long *slot = (unsigned long long *)&slab[j];
@@ -629,7 +801,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
                     const unsigned long long key = ((unsigned long long)(p - as + 1) << 32) | (unsigned long long)(q - bs);
                     __hip_atomic_fetch_max(slot, key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 } else {
-                    const double e = semiring_mult(mult_op, a, Bval[q]);
+                    const double e = semiring_mult(mult_op, a, h.b);
                     if (reduce_op == SR_PLUS)
                         __hip_atomic_fetch_add(&slab[j], e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                     else
@@ -637,7 +809,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_kernel(
                                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 }
             } else {
-                __hip_atomic_fetch_add(&slab[j], a * Bval[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(&slab[j], a * h.b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
         });
         __syncthreads();
@@ -768,8 +940,9 @@ constexpr int SG_CB_LOG = 14;
 constexpr int SG_CB = 1 << SG_CB_LOG;                                 // columns per block
 typedef uint16_t emit_t;                                              // a column of the block being written out
 constexpr int SG_EMIT = 8192;                                         // entries written out per turn of the emit
-constexpr size_t SG_DENSE_LDS = (size_t)SG_CB * 8 + (size_t)SG_CB / 8 + (size_t)SG_EMIT * sizeof(emit_t);  // accumulators, bitmap,
-                                                                      // list of the columns being written out
+constexpr size_t SG_DENSE_LDS = (size_t)SG_CB * 8 + (size_t)SG_CB / 8 + (size_t)SG_EMIT * sizeof(emit_t) +
+                                2 * (size_t)SG_CB / 8;               // accumulators, bitmap, list of the columns being
+                                                                      // written out, the mask row's bits (two blocks)
 
 // products[i - row_begin] = sum over k in A_i of nnz(B_k); one wavefront per row
 __global__ __launch_bounds__(256) void spgemm_row_products(int64_t row_begin, int64_t row_end,
@@ -898,39 +1071,43 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
         if (len >= 64 * SG_LONG_LOADS) {
             // turns in which every lane has all its entries run without predicates, and the loads of the next
             // such turn are in flight while this one's products go into LDS
-            int j[SG_LONG_LOADS];
-            double v[SG_LONG_LOADS];
-#pragma unroll
-            for (int x = 0; x < SG_LONG_LOADS; ++x)
-                j[x] = Bcrd[s + o + 64 * x];
-#pragma unroll
-            for (int x = 0; x < SG_LONG_LOADS; ++x)
-                v[x] = VALUES ? Bval[s + o + 64 * x] : 0.0;
+            // In a full turn a lane takes SG_LONG_LOADS consecutive entries: one 16-byte load of columns and two of
+            // values per lane instead of four loads of each, a stride of 64 entries apart.  (Entries of B lie at any
+            // 4- and 8-byte boundary: the loads are declared unaligned.)
+            static_assert(SG_LONG_LOADS == 4, "a lane's entries of a full turn are one 16-byte load of columns");
+            typedef double sg_d2u __attribute__((ext_vector_type(2), aligned(8)));
+            int64_t c = s + 4 * (int64_t)lane;          // this lane's first entry of the turn
+            sg_i4u j = *reinterpret_cast<const sg_i4u *>(Bcrd + c);
+            sg_d2u v0 = {0.0, 0.0}, v1 = {0.0, 0.0};
+            if constexpr (VALUES) {
+                v0 = *reinterpret_cast<const sg_d2u *>(Bval + c);
+                v1 = *reinterpret_cast<const sg_d2u *>(Bval + c + 2);
+            }
+            int64_t done = 0;
             for (int64_t full = 64 * SG_LONG_LOADS; full + 64 * SG_LONG_LOADS <= len; full += 64 * SG_LONG_LOADS) {
-                int jn[SG_LONG_LOADS];
-                double vn[SG_LONG_LOADS];
-#pragma unroll
-                for (int x = 0; x < SG_LONG_LOADS; ++x)
-                    jn[x] = Bcrd[s + o + 64 * (SG_LONG_LOADS + x)];
-#pragma unroll
-                for (int x = 0; x < SG_LONG_LOADS; ++x)
-                    vn[x] = VALUES ? Bval[s + o + 64 * (SG_LONG_LOADS + x)] : 0.0;
-#pragma unroll
-                for (int x = 0; x < SG_LONG_LOADS; ++x) {
-                    f(j[x], at, v[x], pt, s + o + 64 * x);
+                const int64_t cn = c + 64 * SG_LONG_LOADS;
+                const sg_i4u jn = *reinterpret_cast<const sg_i4u *>(Bcrd + cn);
+                sg_d2u v0n = {0.0, 0.0}, v1n = {0.0, 0.0};
+                if constexpr (VALUES) {
+                    v0n = *reinterpret_cast<const sg_d2u *>(Bval + cn);
+                    v1n = *reinterpret_cast<const sg_d2u *>(Bval + cn + 2);
                 }
-#pragma unroll
-                for (int x = 0; x < SG_LONG_LOADS; ++x) {
-                    j[x] = jn[x];
-                    v[x] = vn[x];
-                }
-                o += 64 * SG_LONG_LOADS;
+                f(j.x, at, v0.x, pt, c);
+                f(j.y, at, v0.y, pt, c + 1);
+                f(j.z, at, v1.x, pt, c + 2);
+                f(j.w, at, v1.y, pt, c + 3);
+                j = jn;
+                v0 = v0n;
+                v1 = v1n;
+                c = cn;
+                done += 64 * SG_LONG_LOADS;
             }
-#pragma unroll
-            for (int x = 0; x < SG_LONG_LOADS; ++x) {
-                f(j[x], at, v[x], pt, s + o + 64 * x);
-            }
-            o += 64 * SG_LONG_LOADS;
+            f(j.x, at, v0.x, pt, c);
+            f(j.y, at, v0.y, pt, c + 1);
+            f(j.z, at, v1.x, pt, c + 2);
+            f(j.w, at, v1.y, pt, c + 3);
+            done += 64 * SG_LONG_LOADS;
+            o += done;
         }
         if (o < len)
             turn_of_slice<VALUES>(s, o, len, at, pt, Bcrd, Bval, f);
@@ -976,10 +1153,16 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
     return touched;
 }
 
-template <bool SEMI>
+// MASKED (C<M> = A*B, for the rows whose mask row is too long for the slab kernel's hash table): every product is
+// added as without a mask - the LDS adds are not what this kernel waits for - and the mask row decides what leaves:
+// before a block's products are walked, the mask row's entries inside the block are set in a bitmap of their own
+// (the row is sorted, so they start where the block before ended), and when the block is written out the columns
+// outside it are dropped and their accumulators cleared.
+template <bool SEMI, bool MASKED>
 __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
     int64_t row_begin, int64_t row_end, const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd,
     const double *__restrict__ Aval, const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval,
+    const int64_t *__restrict__ Mpos, const int32_t *__restrict__ Mcrd,
     const int64_t *__restrict__ blkptr, int nblk,
     unsigned long long *ticket, RowList list,
     const int64_t *__restrict__ Cpos, int32_t *__restrict__ Ccrd, double *__restrict__ Cval, int reduce_op,
@@ -988,9 +1171,15 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
     __shared__ int64_t row_slot;
     __shared__ int wave_tot[SG_WAVES];
     __shared__ int block_touched[3];            // see visit_flag
+    __shared__ unsigned long long mask_next[2]; // where the mask row's entries of a block begin; blocks take turns
     double *acc = reinterpret_cast<double *>(sg_dyn_lds);
     uint32_t *bm = sg_dyn_lds + SG_CB * 2;
     emit_t *emit_col = reinterpret_cast<emit_t *>(bm + SG_CB / 32);
+    uint32_t *mbits = reinterpret_cast<uint32_t *>(emit_col + SG_EMIT);
+    if constexpr (MASKED) {
+        for (int w = threadIdx.x; w < 2 * (SG_CB / 32); w += SG_T)
+            mbits[w] = 0;
+    }
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     for (int j = threadIdx.x; j < SG_CB; j += SG_T)
@@ -1008,6 +1197,13 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
     while (t < t_end) {
         const int64_t i = row_begin + list.rows[t];
         const int64_t as = Apos[i], ae = Apos[i + 1];
+        int64_t me = 0;
+        if constexpr (MASKED) {
+            me = Mpos[i + 1];
+            if (threadIdx.x == 0)
+                mask_next[0] = mask_next[1] = (unsigned long long)Mpos[i];
+            lds_barrier();
+        }
         if (as != ae) {
             int64_t off = Cpos[i] - out0;
             // A row of at most one entry of A per lane (nearly all rows) keeps its entries in registers over
@@ -1030,6 +1226,24 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
             }
             for (int cb = 0; cb < nblk; ++cb) {
                 const int col0 = cb << SG_CB_LOG;
+                uint32_t *mb = mbits + (cb & 1) * (SG_CB / 32);
+                if constexpr (MASKED) {
+                    // The mask row's entries inside this block: they begin at mask_next[cb & 1], and where they end
+                    // goes to the other slot, for the next block (a slot is read in one block and written in the
+                    // next one, with the block's barrier in between; it only ever grows along a row).
+                    const int64_t lo = (int64_t)mask_next[cb & 1];
+                    const int col_end = col0 + SG_CB;
+                    if (threadIdx.x == 0)
+                        atomicMax(&mask_next[(cb + 1) & 1], (unsigned long long)lo);
+                    for (int64_t e = lo + threadIdx.x; e < me; e += SG_T) {
+                        const int j = Mcrd[e];
+                        if (j >= col_end)
+                            break;
+                        atomicOr(&mb[(j - col0) >> 5], 1u << ((j - col0) & 31));
+                        if (e + 1 == me || Mcrd[e + 1] >= col_end)
+                            atomicMax(&mask_next[(cb + 1) & 1], (unsigned long long)(e + 1));
+                    }
+                }
                 int touched = 0;     // did this wavefront add anything to the block
                 const auto add = [&](int j, double a, double b, int pa, int64_t q) {
                     j -= col0;
@@ -1082,7 +1296,18 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                 // wavefronts.  The counts of the two bytes are scanned together, packed into one word.
                 static_assert(SG_T * 16 == SG_CB && SG_WAVES <= 64, "one byte of each half of the bitmap per thread");
                 const uint8_t *bm8 = reinterpret_cast<const uint8_t *>(bm);
-                const uint32_t bits_a = bm8[threadIdx.x], bits_b = bm8[SG_CB / 16 + threadIdx.x];
+                uint32_t bits_a = bm8[threadIdx.x], bits_b = bm8[SG_CB / 16 + threadIdx.x];
+                const int jbase = (int)threadIdx.x << 3;
+                if constexpr (MASKED) {          // columns outside the mask row are dropped here
+                    const uint8_t *mb8 = reinterpret_cast<const uint8_t *>(mb);
+                    const uint32_t keep_a = mb8[threadIdx.x], keep_b = mb8[SG_CB / 16 + threadIdx.x];
+                    for (uint32_t w = bits_a & ~keep_a; w; w &= w - 1)
+                        acc[jbase + __ffs(w) - 1] = 0.0;
+                    for (uint32_t w = bits_b & ~keep_b; w; w &= w - 1)
+                        acc[SG_CB / 2 + jbase + __ffs(w) - 1] = 0.0;
+                    bits_a &= keep_a;
+                    bits_b &= keep_b;
+                }
                 const int mine = __popc(bits_a) | (__popc(bits_b) << 16);
                 const int inc = wave_inclusive_scan(mine);
                 if (lane == 63)
@@ -1093,12 +1318,14 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                 const int before = (wave ? __builtin_amdgcn_readlane(tots, wave - 1) : 0) + inc - mine;
                 const int total_a = all & 0xffff, total = total_a + (all >> 16);
                 const int first_a = before & 0xffff, first_b = total_a + (before >> 16);
-                if (threadIdx.x < SG_CB / 32)      // everybody has read its bytes: the bitmap is clean for the
+                if (threadIdx.x < SG_CB / 32) {    // everybody has read its bytes: the bitmap is clean for the
                     bm[threadIdx.x] = 0;           // next block, which nobody enters before the barrier below
+                    if constexpr (MASKED)
+                        mb[threadIdx.x] = 0;
+                }
                 // The owner of a byte knows where its columns go, but writing them from there would scatter
                 // every store over 64 cache lines.  So the columns are listed in LDS, SG_EMIT at a time, and
                 // then every lane writes the entry at its own place in the list: coalesced stores.
-                const int jbase = (int)threadIdx.x << 3;
                 if (total <= SG_EMIT) {         // the usual case: the whole block fits the list
                     int at = first_a;
                     for (uint32_t w = bits_a; w; w &= w - 1, ++at)
@@ -1134,7 +1361,10 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                 }
                 }
                 off += total;
-                }   // block received products
+                } else if constexpr (MASKED) {   // the block received no product
+                    if (threadIdx.x < SG_CB / 32)        // (the next block's bits go to the other half; the one after
+                        mb[threadIdx.x] = 0;             // that comes after the next block's barrier)
+                }
             }
         }
         t = draw_row<true>(ticket, t_first, &row_slot);
@@ -1415,14 +1645,21 @@ __global__ __launch_bounds__(SG_T) void spgemm_masked_sum_kernel(
             atomicOr(&bm[ad.word(Mcrd[t])], ad.bit(Mcrd[t]));
         __syncthreads();
         double part = 0.0;
-        for_each_product<true>(as, ae, Acrd, Aval, Bpos, Bcrd, [&](int j, int64_t q, double a, int64_t, int64_t) {
-            uint32_t word;
+        for_each_product_probed<true>(as, ae, Acrd, Aval, Bpos, Bcrd, [&](int j) {
             if constexpr (BM_LDS)
-                word = bm[ad.word(j)];
+                return bm[ad.word(j)];
             else
-                word = atomicOr(&bm[ad.word(j)], 0u);
-            if (word & ad.bit(j))
-                part += a * Bval[q];     // the value is fetched for hits only
+                return atomicOr(&bm[ad.word(j)], 0u);
+        }, [&](int j, int64_t q, uint32_t word) {
+            MaskHit h{-1, 0.0};
+            if (word & ad.bit(j)) {      // the value is fetched for hits only
+                h.at = 0;
+                h.b = Bval[q];
+            }
+            return h;
+        }, [&](int, int64_t, double a, int64_t, int64_t, MaskHit h) {
+            if (h.at >= 0)
+                part += a * h.b;
         });
         part = wave_sum_f64(part);
         if ((threadIdx.x & 63) == 0)
@@ -1724,13 +1961,18 @@ static int check_product_shapes(const Csr *a, const Csr *b, const Csr *m, const 
 }
 
 // keys that order rows by descending products; rows without products sort to the very end
-__global__ void sg_row_keys(int64_t n, const int64_t *__restrict__ rowprod, uint64_t *__restrict__ keys,
-                            uint32_t *__restrict__ idx)
+// With a mask (Mpos, already offset to the first row of the list), the rows whose mask row holds more than `fill`
+// entries sort in front of all others (keys below 2^61), whatever their number of products.
+__global__ void sg_row_keys(int64_t n, const int64_t *__restrict__ rowprod, const int64_t *__restrict__ Mpos,
+                            int64_t fill, uint64_t *__restrict__ keys, uint32_t *__restrict__ idx)
 {
     const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (r < n) {
         const int64_t p = rowprod[r];
-        keys[r] = p > 0 ? (uint64_t)((1ll << 62) - p) : ~0ull >> 1;
+        uint64_t key = p > 0 ? (uint64_t)((1ll << 62) - p) : ~0ull >> 1;
+        if (Mpos && p > 0 && Mpos[r + 1] - Mpos[r] > fill)
+            key = (uint64_t)((1ll << 61) - (p < (1ll << 61) ? p : (1ll << 61) - 1));
+        keys[r] = key;
         idx[r] = (uint32_t)r;
     }
 }
@@ -1763,7 +2005,8 @@ static SgRowLists g_rl;
 
 // Products per row of rows [rb, re) of A*B and the list of those rows by descending products.
 static int sg_row_list(const Csr *a, const Csr *b, int64_t rb, int64_t re, int64_t dense_threshold,
-                       int64_t wide_threshold, RowList *out)
+                       int64_t wide_threshold, RowList *out, const int64_t *long_mask_pos = nullptr,
+                       int64_t mask_fill = 0)
 {
     const int64_t n = re - rb;
     COMET_CHK(g_rl.rowprod.ensure(sizeof(int64_t) * (size_t)n, false));
@@ -1778,7 +2021,8 @@ static int sg_row_list(const Csr *a, const Csr *b, int64_t rb, int64_t re, int64
         spgemm_row_products<<<dim3((unsigned)ceil_div(n, 4)), dim3(256), 0, stream()>>>(rb, re, a->pos, a->crd, b->pos,
                                                                                         rowprod);
         sg_row_keys<<<dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, stream()>>>(
-            n, rowprod, (uint64_t *)g_rl.keys_in.ptr, (uint32_t *)g_rl.idx_in.ptr);
+            n, rowprod, long_mask_pos ? long_mask_pos + rb : nullptr, mask_fill, (uint64_t *)g_rl.keys_in.ptr,
+            (uint32_t *)g_rl.idx_in.ptr);
     }
     COMET_HIPCHK(hipGetLastError());
     COMET_CHK(sort_pairs_u64_u32((const uint64_t *)g_rl.keys_in.ptr, (uint64_t *)g_rl.keys_out.ptr,
@@ -1878,13 +2122,19 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
     // rows with many products go to the LDS-accumulator kernel (unmasked products only)
     const int nblk = (int)ceil_div(b->ncols > 0 ? b->ncols : 1, SG_CB);
     // (the `any` semiring keeps a product's place in B in 32 bits of its accumulator)
-    const bool dense = !m && nblk <= SG_DENSE_MAX_BLOCKS && (reduce_op != COMET_SR_ANY || b->nnz < (1ll << 32));
+    const bool lds_rows = nblk <= SG_DENSE_MAX_BLOCKS && (reduce_op != COMET_SR_ANY || b->nnz < (1ll << 32));
+    const bool dense = !m && lds_rows;
+    // masked: the rows whose mask row does not fit the slab kernel's hash table take the one-block kernel
+    const bool mdense = m && lds_rows && g.lds && getenv("COMET_HIP_SPGEMM_NO_MASKED_DENSE") == nullptr;
     const int64_t dense_threshold = dense ? SG_DENSE_PER_BLOCK * nblk : SG_NO_DENSE;
-    if (dense)
+    if (dense || mdense)
         COMET_CHK(sg_plan_blocks(b));
     RowList list;
     const int64_t wide = sg_wide_threshold(nblk) > dense_threshold ? sg_wide_threshold(nblk) : dense_threshold;
-    COMET_CHK(sg_row_list(a, b, rb, re, dense_threshold, dense ? wide : SG_NO_DENSE, &list));
+    if (mdense)         // those rows sort in front (sg_row_keys): bounds[0] = bounds[2] = their number
+        COMET_CHK(sg_row_list(a, b, rb, re, 1ll << 61, 1ll << 61, &list, m->pos, SG_HASH_FILL));
+    else
+        COMET_CHK(sg_row_list(a, b, rb, re, dense_threshold, dense ? wide : SG_NO_DENSE, &list));
     uint32_t *gbm = nullptr, *gmask = nullptr;
     if (!g.lds || m) {          // the output row's bitmap is in HBM when LDS holds the mask row instead
         COMET_CHK(g_sg.gbm.ensure(sizeof(uint32_t) * g.bm_words * (size_t)g.groups, true));
@@ -1919,21 +2169,24 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
 #undef LAUNCH_NUM_S
 #undef LAUNCH_NUM
     COMET_HIPCHK(hipGetLastError());
-    if (dense) {
+    if (dense || mdense) {
         COMET_CHK(sg_reset_ticket());
-        KernelTimer t("spgemm_numeric_dense");
+        KernelTimer t(mdense ? "spgemm_numeric_dense_masked" : "spgemm_numeric_dense");
         const dim3 cus((unsigned)(num_cus() > 0 ? num_cus() : 256));
-        if (semi) {
-            COMET_CHK(sg_allow_lds(spgemm_numeric_dense_kernel<true>, SG_DENSE_LDS));
-            spgemm_numeric_dense_kernel<true><<<cus, block, SG_DENSE_LDS, stream()>>>(
-                rb, re, a->pos, a->crd, a->val, b->crd, b->val, b->sg_blkptr, nblk,
-                (unsigned long long *)g_sg.ticket.ptr, list, Cpos, Ccrd, Cval, reduce_op, mult_op);
+#define LAUNCH_DENSE(S, M)                                                                                 \
+    do {                                                                                                   \
+        COMET_CHK(sg_allow_lds(spgemm_numeric_dense_kernel<S, M>, SG_DENSE_LDS));                          \
+        spgemm_numeric_dense_kernel<S, M><<<cus, block, SG_DENSE_LDS, stream()>>>(                         \
+            rb, re, a->pos, a->crd, a->val, b->crd, b->val, m ? m->pos : nullptr, m ? m->crd : nullptr,    \
+            b->sg_blkptr, nblk, (unsigned long long *)g_sg.ticket.ptr, list, Cpos, Ccrd, Cval, reduce_op,  \
+            mult_op);                                                                                      \
+    } while (0)
+        if (mdense) {
+            if (semi) LAUNCH_DENSE(true, true); else LAUNCH_DENSE(false, true);
         } else {
-            COMET_CHK(sg_allow_lds(spgemm_numeric_dense_kernel<false>, SG_DENSE_LDS));
-            spgemm_numeric_dense_kernel<false><<<cus, block, SG_DENSE_LDS, stream()>>>(
-                rb, re, a->pos, a->crd, a->val, b->crd, b->val, b->sg_blkptr, nblk,
-                (unsigned long long *)g_sg.ticket.ptr, list, Cpos, Ccrd, Cval, reduce_op, mult_op);
+            if (semi) LAUNCH_DENSE(true, false); else LAUNCH_DENSE(false, false);
         }
+#undef LAUNCH_DENSE
         COMET_HIPCHK(hipGetLastError());
     }
     if (dense) {

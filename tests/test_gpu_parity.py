@@ -513,6 +513,32 @@ def test_spgemm_semiring_rows_of_every_class(semiring, m, long_len, wide, monkey
     assert np.array_equal(c, wc) and np.all(np.abs(v - pv) <= RTOL * bound)
 
 
+@pytest.mark.parametrize("semiring", [None, ("min", "plus"), ("any", "first")])
+def test_spgemm_masked_long_mask_rows(semiring):
+    # mask rows of 0, 5, 6144 (the longest the hash table of the slab kernel takes), 6145, 20,000 and 70,000
+    # entries: the long ones take the one-block kernel, which adds every product and drops the columns outside
+    # the mask when a block is written out; the row pointers come from the masked symbolic phase
+    rng = np.random.default_rng(31)
+    k, m = 300, 100_000
+    bpos, bcrd, bval = _rows_of_lengths(rng, [3000] * 200 + [10] * 100, m, signed=False)
+    lengths = [50, 0, 7, 120, 300, 1, 64, 200] * 3
+    apos, acrd, aval = _rows_of_lengths(rng, lengths, k, signed=False)
+    mlens = [20_000, 70_000, 6145, 0, 6144, 5, 70_000, 30_000] * 3
+    mpos, mcrd, _ = _rows_of_lengths(rng, mlens, m)
+    A = rt.CsrMatrix.from_arrays((len(lengths), k), apos, acrd, aval)
+    B = rt.CsrMatrix.from_arrays((k, m), bpos, bcrd, bval)
+    Mk = rt.CsrMatrix.from_arrays((len(lengths), m), mpos, mcrd, np.ones(len(mcrd)))
+    wp, wc, wv = orc.spgemm(apos, acrd, aval, bpos, bcrd, bval, m, mask=(mpos, mcrd), semiring=semiring)
+    for _ in range(2):
+        p, c, v = rt.spgemm(A, B, Mk, semiring=semiring).to_arrays()
+        assert np.array_equal(p, wp) and np.array_equal(c, wc)
+        if semiring is None:
+            assert np.all(np.abs(v - wv) <= RTOL * np.abs(wv))       # positive values: no cancellation
+        else:
+            assert np.array_equal(v, wv)
+    _spgemm_check((apos, acrd, aval), (bpos, bcrd, bval), m)        # and nothing is left behind for a plain product
+
+
 @pytest.mark.parametrize("wide", [1 << 40, 0])
 def test_spgemm_rows_with_more_entries_than_lanes(wide, monkeypatch):
     # more than 1024 entries in a row of A: the LDS kernels then fetch the row's entries again at every visit
