@@ -90,6 +90,7 @@ struct Csr {
     int64_t *heavy_seg = nullptr;            // [8 * 512 + 1] list boundaries
     HeavyEnt *heavy_ent = nullptr;           // the lists, runs padded to even length
     int64_t heavy_rows = 0;
+    int heavy_groups = 0;                    // workgroups of the sweep per XCD the lists were made for
     int32_t *heavy_row = nullptr;            // [heavy_rows] row ids of the long rows
     int32_t *heavy_code = nullptr;           // [8][heavy_rows] wavefront * 8 + slot that holds the row on each XCD
     Csr *light = nullptr;

@@ -451,10 +451,16 @@ constexpr int SPMM_HW = 16;      // wavefronts per workgroup of the sweep
 constexpr int SPMM_HRB = COMET_SPMM_HR_BITS;         // bits of a list entry that name the owned row
 constexpr int SPMM_HR = 1 << SPMM_HRB;               // rows a wavefront can own
 constexpr int SPMM_HCOLB = 28 - SPMM_HRB;            // bits of a list entry left for the column
-constexpr int SPMM_HG = 32;      // workgroups per XCD: one per CU, so that all of them sweep together
-constexpr int SPMM_HBINS = SPMM_HG * SPMM_HW;        // wavefronts (= row bins) per XCD
-constexpr int SPMM_HSLOTS = SPMM_HBINS * SPMM_HR;    // slots for partial sums: 16 wavefronts x 8 rows per workgroup
-constexpr int SPMM_HROWS = SPMM_HG * (SPMM_HW - 1) * SPMM_HR;    // long rows the plan can hold
+// Workgroups of the sweep per XCD, one to a CU: all 32 CUs of an XCD when the sweep has the GPU to itself; fewer
+// when the rows that are neither long nor single hold enough of the matrix to be worth running beside it - the
+// chunk kernel that takes them waits on HBM, the sweep on the path from the L2 to the CU, and on the CUs the
+// sweep leaves free the chunk kernel is not starved by it (inside a CU the older wavefronts of the sweep win every
+// arbitration).  Measured on the benchmark matrix (ms per product): 32 and the kernels one after the other 0.329;
+// side by side with 28 workgroups per XCD 0.336, 26 0.348, 25 0.355, 24 0.311, 23 0.319, 22 0.325.
+constexpr int SPMM_HG_ALONE = 32, SPMM_HG_SHARED = 24;
+constexpr int spmm_hbins(int g) { return g * SPMM_HW; }               // wavefronts (= row bins) per XCD
+constexpr int spmm_hslots(int g) { return spmm_hbins(g) * SPMM_HR; }  // slots for partial sums per XCD
+constexpr int spmm_hrows(int g) { return g * (SPMM_HW - 1) * SPMM_HR; }    // long rows the plan can hold
 constexpr int SPMM_HEAVY_MIN_LEN = COMET_SPMM_HEAVY_MIN;              // a long row has at least this many nonzeros
 constexpr int SPMM_HCB = 32;                         // column blocks a wavefront's list is cut into
 
@@ -636,9 +642,8 @@ __device__ inline void single_rows(const spmm_v4i *__restrict__ list, int64_t n,
 template <bool SMALL, bool ACC>
 __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
     const int64_t *__restrict__ seg, const HeavyEnt *__restrict__ hent, const double *__restrict__ B, int64_t ldb,
-    int64_t K, double *__restrict__ partial, double *__restrict__ C, int64_t ldc)
+    int64_t K, double *__restrict__ partial, double *__restrict__ C, int64_t ldc, int G)
 {
-    constexpr int G = SPMM_HG;
     const int lane = threadIdx.x & 63, half = lane >> 5, sub = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int x = blockIdx.x & 7, g = blockIdx.x >> 3;
@@ -784,8 +789,8 @@ __global__ void heavy_count(int64_t nheavy, const int32_t *__restrict__ hrow, co
 
 __global__ void heavy_make_keys(int64_t nheavy, const int32_t *__restrict__ hrow, const int32_t *__restrict__ hcode,
                                 const int64_t *__restrict__ hstart, const int64_t *__restrict__ pos,
-                                const int32_t *__restrict__ crd, int64_t xcols, uint64_t *__restrict__ keys,
-                                uint32_t *__restrict__ idx)
+                                const int32_t *__restrict__ crd, int64_t xcols, int hbins,
+                                uint64_t *__restrict__ keys, uint32_t *__restrict__ idx)
 {
     const int64_t h = blockIdx.x;
     if (h >= nheavy)
@@ -796,7 +801,7 @@ __global__ void heavy_make_keys(int64_t nheavy, const int32_t *__restrict__ hrow
         const uint64_t x = c / (uint64_t)xcols;
         const uint64_t cb = (c - x * (uint64_t)xcols) * SPMM_HCB / (uint64_t)xcols;   // column block inside the range
         const uint64_t code = (uint64_t)hcode[x * nheavy + h];       // wavefront * SPMM_HR + slot on that XCD
-        keys[o + t] = ((((x * SPMM_HBINS + (code >> SPMM_HRB)) * SPMM_HCB + cb) * (2 * SPMM_HR) +
+        keys[o + t] = ((((x * hbins + (code >> SPMM_HRB)) * SPMM_HCB + cb) * (2 * SPMM_HR) +
                         (code & (SPMM_HR - 1))) << 28) | c;
         idx[o + t] = (uint32_t)(ps + t);
     }
@@ -805,8 +810,8 @@ __global__ void heavy_make_keys(int64_t nheavy, const int32_t *__restrict__ hrow
 // The rows with one nonzero, dealt round-robin to the last wavefronts of the workgroups of the XCD that sweeps
 // their column; these wavefronts own no long rows, so their lists are simply ordered by column.
 __global__ void single_make_keys(int64_t nsingle, const int32_t *__restrict__ srow, const int64_t *__restrict__ pos,
-                                 const int32_t *__restrict__ crd, int64_t xcols, uint64_t *__restrict__ keys,
-                                 uint32_t *__restrict__ idx)
+                                 const int32_t *__restrict__ crd, int64_t xcols, int groups,
+                                 uint64_t *__restrict__ keys, uint32_t *__restrict__ idx)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= nsingle)
@@ -814,8 +819,8 @@ __global__ void single_make_keys(int64_t nsingle, const int32_t *__restrict__ sr
     const uint64_t c = (uint64_t)(uint32_t)crd[pos[srow[i]]];
     const uint64_t x = c / (uint64_t)xcols;
     const uint64_t cb = (c - x * (uint64_t)xcols) * SPMM_HCB / (uint64_t)xcols;
-    const uint64_t bin = (uint64_t)(i % SPMM_HG) * SPMM_HW + SPMM_HWL;
-    keys[i] = ((((x * SPMM_HBINS + bin) * SPMM_HCB + cb) * (2 * SPMM_HR) + SPMM_HR) << 28) | c;
+    const uint64_t bin = (uint64_t)(i % groups) * SPMM_HW + SPMM_HWL;
+    keys[i] = ((((x * (uint64_t)spmm_hbins(groups) + bin) * SPMM_HCB + cb) * (2 * SPMM_HR) + SPMM_HR) << 28) | c;
     idx[i] = (uint32_t)i;
 }
 
@@ -882,10 +887,10 @@ __global__ void heavy_fill(int64_t n, const uint64_t *__restrict__ keys, const u
 
 // seg[b] = position in the padded list of the first entry whose (XCD, wavefront) number is >= b
 __global__ void heavy_segments(int64_t n, const uint64_t *__restrict__ keys, const int64_t *__restrict__ runs,
-                               const int64_t *__restrict__ pads, int64_t *__restrict__ seg)
+                               const int64_t *__restrict__ pads, int hbins, int64_t *__restrict__ seg)
 {
     const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (b > 8 * SPMM_HBINS)
+    if (b > 8 * hbins)
         return;
     int64_t lo = 0, hi = n;
     while (lo < hi) {
@@ -926,7 +931,7 @@ __global__ void light_copy(int64_t nlight, const int32_t *__restrict__ rowmap, c
 template <bool ACC>
 __global__ __launch_bounds__(256) void spmm_heavy_combine(int64_t nheavy, const int32_t *__restrict__ hrow,
                                                           const int32_t *__restrict__ hcode,
-                                                          const double *__restrict__ partial,
+                                                          const double *__restrict__ partial, int hslots,
                                                           double *__restrict__ C, int64_t ldc, int64_t K)
 {
     const int lane = threadIdx.x & 63;
@@ -937,7 +942,7 @@ __global__ __launch_bounds__(256) void spmm_heavy_combine(int64_t nheavy, const 
     const int64_t row = hrow[h];
     double acc = ACC ? C[row * ldc + col] : 0.0;
     for (int x = 0; x < 8; ++x)
-        acc = acc + partial[((int64_t)x * SPMM_HSLOTS + hcode[x * nheavy + h]) * K + col];
+        acc = acc + partial[((int64_t)x * hslots + hcode[x * nheavy + h]) * K + col];
     C[row * ldc + col] = acc;
 }
 
@@ -960,8 +965,26 @@ static int spmm_heavy_plan(Csr *a)
         if (pos[(size_t)r + 1] - pos[(size_t)r] >= SPMM_HEAVY_MIN_LEN)
             cand.emplace_back(-(pos[(size_t)r + 1] - pos[(size_t)r]), (int32_t)r);
     std::sort(cand.begin(), cand.end());
-    if ((int64_t)cand.size() > SPMM_HROWS)
-        cand.resize(SPMM_HROWS);
+    // How many CUs of an XCD the sweep takes: all of them, unless the rows that are neither long nor single (with
+    // the sweep at full size) hold at least a sixteenth of the matrix; COMET_HIP_SPMM_GROUPS overrides.
+    int G = SPMM_HG_ALONE;
+    {
+        int64_t long_nnz = 0, single = 0;
+        for (size_t k = 0; k < cand.size() && (int64_t)k < spmm_hrows(SPMM_HG_ALONE); ++k)
+            long_nnz -= cand[k].first;
+        for (int64_t r = 0; r < n; ++r)
+            single += pos[(size_t)r + 1] - pos[(size_t)r] == 1;
+        if ((a->nnz - long_nnz - single) * 16 >= a->nnz)
+            G = SPMM_HG_SHARED;
+        if (const char *e = getenv("COMET_HIP_SPMM_GROUPS")) {
+            const int g = atoi(e);
+            if (g >= 1 && g <= SPMM_HG_ALONE)
+                G = g;
+        }
+    }
+    const int hbins = spmm_hbins(G);
+    if ((int64_t)cand.size() > spmm_hrows(G))
+        cand.resize((size_t)spmm_hrows(G));
     const int64_t H = (int64_t)cand.size();
     int64_t hnnz = 0;
     for (auto &c : cand)
@@ -1036,7 +1059,7 @@ static int spmm_heavy_plan(Csr *a)
     HEAVY_TRY(hipMalloc((void **)&k_out, 8 * (size_t)nent));
     HEAVY_TRY(hipMalloc((void **)&i_in, 4 * (size_t)nent));
     HEAVY_TRY(hipMalloc((void **)&i_out, 4 * (size_t)nent));
-    HEAVY_TRY(hipMalloc((void **)&a->heavy_seg, 8 * (size_t)(8 * SPMM_HBINS + 1)));
+    HEAVY_TRY(hipMalloc((void **)&a->heavy_seg, 8 * (size_t)(8 * hbins + 1)));
     HEAVY_TRY(hipMalloc((void **)&a->heavy_row, 4 * (size_t)H));
     HEAVY_TRY(hipMalloc((void **)&a->heavy_code, 4 * (size_t)(8 * H)));
     HEAVY_TRY(hipMalloc((void **)&a->empty_rows, 4 * at_least_one(E)));
@@ -1069,8 +1092,8 @@ static int spmm_heavy_plan(Csr *a)
         static const double pace[4] = {1.0 / 1.12, 1.0 / 1.05, 1.0 / 0.96, 1.0 / 0.87};
         std::priority_queue<std::pair<double, int32_t>, std::vector<std::pair<double, int32_t>>,
                             std::greater<std::pair<double, int32_t>>> bins;
-        std::vector<int32_t> used(SPMM_HBINS, 0);
-        for (int32_t b = 0; b < SPMM_HBINS; ++b)
+        std::vector<int32_t> used((size_t)hbins, 0);
+        for (int32_t b = 0; b < hbins; ++b)
             if (b % SPMM_HW != SPMM_HWL)        // the last wavefront of a workgroup takes the rows with one nonzero
                 bins.push({0.0, b});
         for (auto &o : order) {
@@ -1086,10 +1109,10 @@ static int spmm_heavy_plan(Csr *a)
     {
         KernelTimer t("heavy_make_keys");
         heavy_make_keys<<<dim3((unsigned)H), dim3(256), 0, stream()>>>(H, a->heavy_row, a->heavy_code, d_hstart,
-                                                                       a->pos, a->crd, xcols, k_in, i_in);
+                                                                       a->pos, a->crd, xcols, hbins, k_in, i_in);
         if (S > 0)
             single_make_keys<<<dim3((unsigned)ceil_div(S, 256)), dim3(256), 0, stream()>>>(
-                S, d_srow, a->pos, a->crd, xcols, k_in + hnnz, i_in + hnnz);
+                S, d_srow, a->pos, a->crd, xcols, G, k_in + hnnz, i_in + hnnz);
     }
     if (sort_pairs_u64_u32(k_in, k_out, i_in, i_out, nent, 28 + (SPMM_HRB + 1) + 5 + 12) != COMET_HIP_OK) {
         cleanup(true);
@@ -1123,8 +1146,8 @@ static int spmm_heavy_plan(Csr *a)
         KernelTimer t("heavy_fill");
         heavy_fill<<<dim3((unsigned)ceil_div(nent, 256)), dim3(256), 0, stream()>>>(
             nent, k_out, i_out, a->val, a->pos, d_srow, d_first, d_runs, d_start, d_pads, a->heavy_ent);
-        heavy_segments<<<dim3((unsigned)ceil_div(8 * SPMM_HBINS + 1, 256)), dim3(256), 0, stream()>>>(
-            nent, k_out, d_runs, d_pads, a->heavy_seg);
+        heavy_segments<<<dim3((unsigned)ceil_div(8 * hbins + 1, 256)), dim3(256), 0, stream()>>>(
+            nent, k_out, d_runs, d_pads, hbins, a->heavy_seg);
     }
     // the rows of two and more nonzeros that are not long, as a matrix of their own
     light->nrows = L;
@@ -1154,6 +1177,7 @@ static int spmm_heavy_plan(Csr *a)
     a->light = light;
     a->heavy_nnz = hnnz;
     a->heavy_rows = H;
+    a->heavy_groups = G;
     a->nempty = E;
     a->heavy_state = 2;
     return COMET_HIP_OK;
@@ -1163,7 +1187,8 @@ static int spmm_heavy_plan(Csr *a)
 
 using namespace comet;
 
-static int spmm_chunks(Csr *a, int64_t K, const double *B, int64_t ldb, double *C, int64_t ldc, int accumulate);
+static int spmm_chunks(Csr *a, int64_t K, const double *B, int64_t ldb, double *C, int64_t ldc, int accumulate,
+                       hipStream_t on = nullptr);
 static int spmv_run(Csr *a, int64_t x_dptr, int64_t y_dptr, int accumulate);
 static int spmm_run(Csr *a, int64_t K, int64_t b_dptr, int64_t ldb, int64_t c_dptr, int64_t ldc, int accumulate);
 
@@ -1233,7 +1258,16 @@ static int spmm_run(Csr *a, int64_t K, int64_t b_dptr, int64_t ldb, int64_t c_dp
     if (a->heavy_state != 2 || !sweep_fits)
         return spmm_chunks(a, K, B, ldb, C, ldc, accumulate);
     // rows of two and more nonzeros that are not long: one wavefront per 256 nonzeros
-    if (a->light->nnz > 0)
+    // with CUs left free by the sweep, the chunk kernel of the rows in between runs beside it on a second stream
+    const int G = a->heavy_groups;
+    const bool overlap = a->light->nnz > 0 && G < SPMM_HG_ALONE;
+    if (overlap) {
+        // what the chunk kernel needs from stream() - its chunk table, its carry slots - is in place before the fork
+        COMET_CHK(spmm_plan(a->light));
+        COMET_CHK(g_spmm_carry.ensure(
+            sizeof(double) * (size_t)(ceil_div(K, 64) * a->light->spmm_nchunks * 2 * 64), false));
+        COMET_CHK(aux_fork());
+    } else if (a->light->nnz > 0)
         COMET_CHK(spmm_chunks(a->light, K, B, ldb, C, ldc, accumulate));
     const unsigned tiles = (unsigned)ceil_div(K, 64);
     if (!accumulate && a->nempty > 0) {
@@ -1242,47 +1276,54 @@ static int spmm_run(Csr *a, int64_t K, int64_t b_dptr, int64_t ldb, int64_t c_dp
         zero_listed_rows_f64<<<dim3(blocks), dim3(256), 0, stream()>>>(C, a->empty_rows, a->nempty, K, ldc);
     }
     // long rows (sums on chip, left in `partial`) and rows of one nonzero (stored to C)
-    COMET_CHK(g_heavy_partial.ensure(sizeof(double) * 8 * (size_t)SPMM_HSLOTS * (size_t)K, false));
+    COMET_CHK(g_heavy_partial.ensure(sizeof(double) * 8 * (size_t)spmm_hslots(G) * (size_t)K, false));
     double *partial = (double *)g_heavy_partial.ptr;
     {
         KernelTimer t("spmm_heavy_sweep");
         const bool small_b = a->ncols < (1 << 24) && ldb * 8 < (1 << 24) && a->ncols * ldb * 8 < (1ll << 32);
-        const dim3 grid(8 * SPMM_HG, tiles), block(SPMM_HW * 64);
+        const dim3 grid(8 * G, tiles), block(SPMM_HW * 64);
         if (small_b && accumulate)
             spmm_heavy_sweep<true, true><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K, partial,
-                                                                       C, ldc);
+                                                                       C, ldc, G);
         else if (small_b)
             spmm_heavy_sweep<true, false><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K, partial,
-                                                                        C, ldc);
+                                                                        C, ldc, G);
         else if (accumulate)
             spmm_heavy_sweep<false, true><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K, partial,
-                                                                        C, ldc);
+                                                                        C, ldc, G);
         else
             spmm_heavy_sweep<false, false><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K,
-                                                                         partial, C, ldc);
+                                                                         partial, C, ldc, G);
+    }
+    if (overlap) {      // the rows in between, on the CUs the sweep leaves free
+        COMET_CHK(spmm_chunks(a->light, K, B, ldb, C, ldc, accumulate, aux_stream()));
+        COMET_CHK(aux_join());
     }
     {
         KernelTimer t("spmm_heavy_combine");
         const dim3 grid((unsigned)ceil_div(a->heavy_rows, 4), tiles);
         if (accumulate)
             spmm_heavy_combine<true><<<grid, dim3(256), 0, stream()>>>(a->heavy_rows, a->heavy_row, a->heavy_code,
-                                                                       partial, C, ldc, K);
+                                                                       partial, spmm_hslots(G), C, ldc, K);
         else
             spmm_heavy_combine<false><<<grid, dim3(256), 0, stream()>>>(a->heavy_rows, a->heavy_row, a->heavy_code,
-                                                                        partial, C, ldc, K);
+                                                                        partial, spmm_hslots(G), C, ldc, K);
     }
     COMET_HIPCHK(hipGetLastError());
     return COMET_HIP_OK;
 }
 
-static int spmm_chunks(Csr *a, int64_t K, const double *B, int64_t ldb, double *C, int64_t ldc, int accumulate)
+static int spmm_chunks(Csr *a, int64_t K, const double *B, int64_t ldb, double *C, int64_t ldc, int accumulate,
+                       hipStream_t on)
 {
+    if (!on)
+        on = stream();
     const int64_t b_dptr = (int64_t)B;
     if (a->nnz == 0) {
         if (!accumulate) {
-            KernelTimer t("fill_rows_f64");
+            KernelTimer t("fill_rows_f64", on);
             unsigned blocks = (unsigned)std::min<int64_t>(ceil_div(a->nrows * K, 256), 65536);
-            fill_rows_f64<<<dim3(blocks), dim3(256), 0, stream()>>>(C, a->nrows, K, ldc, 0.0);
+            fill_rows_f64<<<dim3(blocks), dim3(256), 0, on>>>(C, a->nrows, K, ldc, 0.0);
             COMET_HIPCHK(hipGetLastError());
         }
         return COMET_HIP_OK;
@@ -1295,23 +1336,23 @@ static int spmm_chunks(Csr *a, int64_t K, const double *B, int64_t ldb, double *
     const dim3 grid((unsigned)ceil_div(nchunks, SPMM_WAVES), (unsigned)tiles);
     const dim3 block(SPMM_WAVES * 64);
     {
-        KernelTimer t("spmm_csr_nnzsplit");
+        KernelTimer t("spmm_csr_nnzsplit", on);
         if (accumulate)
-            spmm_csr_nnzsplit<true><<<grid, block, 0, stream()>>>(a->pos, a->crd, a->val, a->nnz, a->nrows,
+            spmm_csr_nnzsplit<true><<<grid, block, 0, on>>>(a->pos, a->crd, a->val, a->nnz, a->nrows,
                                                                   a->spmm_chunk_row, nchunks, (const double *)b_dptr,
                                                                   ldb, C, ldc, K, carry, a->rowmap);
         else
-            spmm_csr_nnzsplit<false><<<grid, block, 0, stream()>>>(a->pos, a->crd, a->val, a->nnz, a->nrows,
+            spmm_csr_nnzsplit<false><<<grid, block, 0, on>>>(a->pos, a->crd, a->val, a->nnz, a->nrows,
                                                                    a->spmm_chunk_row, nchunks, (const double *)b_dptr,
                                                                    ldb, C, ldc, K, carry, a->rowmap);
     }
     {
-        KernelTimer t("spmm_csr_fixup");
+        KernelTimer t("spmm_csr_fixup", on);
         if (accumulate)
-            spmm_csr_fixup<true><<<grid, block, 0, stream()>>>(a->pos, a->nnz, a->spmm_chunk_row, nchunks, C, ldc, K,
+            spmm_csr_fixup<true><<<grid, block, 0, on>>>(a->pos, a->nnz, a->spmm_chunk_row, nchunks, C, ldc, K,
                                                                carry, a->rowmap);
         else
-            spmm_csr_fixup<false><<<grid, block, 0, stream()>>>(a->pos, a->nnz, a->spmm_chunk_row, nchunks, C, ldc, K,
+            spmm_csr_fixup<false><<<grid, block, 0, on>>>(a->pos, a->nnz, a->spmm_chunk_row, nchunks, C, ldc, K,
                                                                 carry, a->rowmap);
     }
     COMET_HIPCHK(hipGetLastError());

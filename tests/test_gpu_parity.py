@@ -191,11 +191,19 @@ def test_spmm_golden(golden, golden_dir):
 
 
 def _long_rows(pos, K):
-    """The rows the library hands to the column sweep (its rule restated): at least 128 nonzeros, at most
-    the 3840 longest (ties: lower row first), and only if they hold a quarter of a matrix of >= 2^19 nonzeros."""
+    """The rows the library hands to the column sweep (its rule restated): at least 128 nonzeros, at most the
+    120 x g longest (ties: lower row first) with g = 32 workgroups of the sweep per XCD - or 24, leaving CUs to
+    the chunk kernel beside it, when the rows that are neither long (at g = 32) nor single hold a sixteenth of
+    the matrix; COMET_HIP_SPMM_GROUPS overrides g - and only if they hold a quarter of a matrix of >= 2^19
+    nonzeros."""
     lens = np.diff(pos)
     rows = np.flatnonzero(lens >= 128)
-    rows = rows[np.argsort(-lens[rows], kind="stable")][:3840]
+    rows = rows[np.argsort(-lens[rows], kind="stable")]
+    groups = 32
+    if (pos[-1] - lens[rows[:3840]].sum() - (lens == 1).sum()) * 16 >= pos[-1]:
+        groups = 24
+    groups = int(os.environ.get("COMET_HIP_SPMM_GROUPS", groups))
+    rows = rows[:120 * groups]
     if not (16 <= K <= 2048) or pos[-1] < (1 << 19) or 4 * lens[rows].sum() < pos[-1]:
         return rows[:0]
     return rows
@@ -1029,16 +1037,20 @@ def test_spmm_long_rows_sweep(K, acc, pad):
     assert nlong > 100 if (K % 2 == 0 and pad % 2 == 0) else nlong == 0
 
 
-def test_spmm_more_long_rows_than_the_sweep_holds():
-    """5000 rows of 300 nonzeros: the 3840 longest (ties: lowest row ids) sweep, the others stay on the
-    chunk kernel; an empty row and a short row sit between them."""
+@pytest.mark.parametrize("groups,held", [(None, 2880), (32, 3840), (16, 1920)])
+def test_spmm_more_long_rows_than_the_sweep_holds(groups, held, monkeypatch):
+    """5000 rows of 300 nonzeros: the longest the sweep has room for (ties: lowest row ids) sweep, the others
+    stay on the chunk kernel, which here holds enough of the matrix to run beside the sweep on CUs that it
+    leaves free (24 workgroups per XCD; 32 and 16 forced); an empty row and a short row sit between them."""
+    if groups is not None:
+        monkeypatch.setenv("COMET_HIP_SPMM_GROUPS", str(groups))
     rng = np.random.default_rng(31)
     n, m = 5002, 3000
     lens = np.full(n, 300); lens[17] = 0; lens[4000] = 3
     pos = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
     crd = np.concatenate([np.sort(rng.choice(m, l, replace=False)) for l in lens]).astype(np.int64)
     val = rng.uniform(-1, 1, len(crd))
-    assert _sweep_check(pos, crd, val, gen.dense((m, 64), seed=2)) == 3840
+    assert _sweep_check(pos, crd, val, gen.dense((m, 64), seed=2)) == held
 
 
 @pytest.mark.parametrize("acc", [False, True])
