@@ -450,7 +450,7 @@ constexpr int SPMM_HW = 16;      // wavefronts per workgroup of the sweep
 #endif
 constexpr int SPMM_HRB = COMET_SPMM_HR_BITS;         // bits of a list entry that name the owned row
 constexpr int SPMM_HR = 1 << SPMM_HRB;               // rows a wavefront can own
-constexpr int SPMM_HCOLB = 28 - SPMM_HRB;            // bits of a list entry left for the column
+constexpr int SPMM_HCOLB = 20;                       // bits of a list entry for the column, counted from the first column of its XCD's range
 // Workgroups of the sweep per XCD, one to a CU: all 32 CUs of an XCD when the sweep has the GPU to itself; fewer
 // when the rows that are neither long nor single hold enough of the matrix to be worth running beside it - the
 // chunk kernel that takes them waits on HBM, the sweep on the path from the L2 to the CU, and on the CUs the
@@ -498,11 +498,13 @@ constexpr int SPMM_HCB = 32;                         // column blocks a wavefron
 // flight; batches of 4 or 16 pairs: 0.25 ms) - with sixteen wavefronts per CU
 // the memory path is kept busy by the other wavefronts, and more requests
 // queued per wavefront only lengthen the queues.
-// Entry = column << SPMM_E_COL | real | first-of-run | owned row.
+// Entry = (column - first column of the XCD's range) << SPMM_E_COL | owned row << SPMM_E_ROW | first-of-run | real.
 constexpr int SPMM_HP = 8;       // pairs of entries per batch of gathers
-constexpr int SPMM_E_FIRST = SPMM_HR;          // the entry opens a run of one owned row
-constexpr int SPMM_E_REAL = 2 * SPMM_HR;       // not a pad
-constexpr int SPMM_E_COL = SPMM_HRB + 2;
+constexpr int SPMM_E_REAL = 1;                 // not a pad
+constexpr int SPMM_E_FIRST = 2;                // the entry opens a run of one owned row
+constexpr int SPMM_E_ROW = 3;                  // where the owned row (or, for a row kept in LDS, its slot) sits: 9 bits
+constexpr int SPMM_E_COL = 12;
+static_assert(SPMM_E_COL + SPMM_HCOLB <= 32 && SPMM_HRB <= SPMM_E_COL - SPMM_E_ROW, "an entry is 32 bits");
 constexpr int SPMM_HWL = SPMM_HW - 1;          // wavefronts of a workgroup that own long rows
 
 // SMALL: B spans less than 4 GiB and has fewer than 2^24 rows of fewer than 2^24 bytes, so the byte offset of a
@@ -536,7 +538,7 @@ __device__ inline void heavy_add(double (&accx)[SPMM_HR], double (&accy)[SPMM_HR
             if (e0 & SPMM_E_FIRST) {             // a run starts on an even entry
                 accx[run_slot] = run.x;
                 accy[run_slot] = run.y;
-                run_slot = e0 & (SPMM_HR - 1);
+                run_slot = (e0 >> SPMM_E_ROW) & (SPMM_HR - 1);
                 run.x = accx[run_slot];
                 run.y = accy[run_slot];
             }
@@ -642,11 +644,12 @@ __device__ inline void single_rows(const spmm_v4i *__restrict__ list, int64_t n,
 template <bool SMALL, bool ACC>
 __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
     const int64_t *__restrict__ seg, const HeavyEnt *__restrict__ hent, const double *__restrict__ B, int64_t ldb,
-    int64_t K, double *__restrict__ partial, double *__restrict__ C, int64_t ldc, int G)
+    int64_t K, double *__restrict__ partial, double *__restrict__ C, int64_t ldc, int G, int64_t xcols)
 {
     const int lane = threadIdx.x & 63, half = lane >> 5, sub = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int x = blockIdx.x & 7, g = blockIdx.x >> 3;
+    B += (int64_t)x * xcols * ldb;          // the entries count columns from the first one of this XCD's range
     int64_t col = (int64_t)blockIdx.y * 64 + 2 * sub;          // K is even: a lane's two columns exist or neither
     const bool active = col < K;
     if (!active)
@@ -856,7 +859,7 @@ __global__ void heavy_fill(int64_t n, const uint64_t *__restrict__ keys, const u
                            const double *__restrict__ val, const int64_t *__restrict__ pos,
                            const int32_t *__restrict__ srow, const int64_t *__restrict__ first,
                            const int64_t *__restrict__ runs, const int64_t *__restrict__ start,
-                           const int64_t *__restrict__ pads, HeavyEnt *__restrict__ hent)
+                           const int64_t *__restrict__ pads, int64_t xcols, HeavyEnt *__restrict__ hent)
 {
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= n)
@@ -865,7 +868,8 @@ __global__ void heavy_fill(int64_t n, const uint64_t *__restrict__ keys, const u
     const int64_t r = runs[e] + first[e] - 1;
     const int64_t p = e + pads[r];
     const bool direct = ((k >> 28) & SPMM_HR) != 0;
-    const uint32_t col = (uint32_t)(k & 0xfffffffull) << SPMM_E_COL;
+    const uint64_t c = k & 0xfffffffull;
+    const uint32_t col = (uint32_t)(c - (c / (uint64_t)xcols) * (uint64_t)xcols) << SPMM_E_COL;     // inside its XCD's range
     HeavyEnt out;
     if (direct) {
         out.ent = (int32_t)(col | SPMM_E_REAL);
@@ -873,7 +877,7 @@ __global__ void heavy_fill(int64_t n, const uint64_t *__restrict__ keys, const u
         out.val = val[pos[out.row]];
     } else {
         out.ent = (int32_t)(col | SPMM_E_REAL | (first[e] ? (uint32_t)SPMM_E_FIRST : 0u) |
-                            (uint32_t)((k >> 28) & (SPMM_HR - 1)));
+                            ((uint32_t)((k >> 28) & (SPMM_HR - 1)) << SPMM_E_ROW));
         out.row = 0;
         out.val = val[idx[e]];
     }
@@ -953,8 +957,8 @@ static int spmm_heavy_plan(Csr *a)
     if (a->heavy_state != 0)
         return COMET_HIP_OK;
     a->heavy_state = 1;
-    if (a->nnz < (1 << 19) || a->nnz >= (1ll << 32) || a->ncols >= (1ll << SPMM_HCOLB))
-        return COMET_HIP_OK;        // a list entry has SPMM_HCOLB bits for the column
+    if (a->nnz < (1 << 19) || a->nnz >= (1ll << 32) || ceil_div(a->ncols, 8) >= (1ll << SPMM_HCOLB))
+        return COMET_HIP_OK;        // a list entry has SPMM_HCOLB bits for the column inside an XCD's eighth
     const int64_t n = a->nrows;
     std::vector<int64_t> pos((size_t)n + 1);
     COMET_HIPCHK(hipMemcpyAsync(pos.data(), a->pos, sizeof(int64_t) * (size_t)(n + 1), hipMemcpyDeviceToHost,
@@ -1145,7 +1149,7 @@ static int spmm_heavy_plan(Csr *a)
     {
         KernelTimer t("heavy_fill");
         heavy_fill<<<dim3((unsigned)ceil_div(nent, 256)), dim3(256), 0, stream()>>>(
-            nent, k_out, i_out, a->val, a->pos, d_srow, d_first, d_runs, d_start, d_pads, a->heavy_ent);
+            nent, k_out, i_out, a->val, a->pos, d_srow, d_first, d_runs, d_start, d_pads, xcols, a->heavy_ent);
         heavy_segments<<<dim3((unsigned)ceil_div(8 * hbins + 1, 256)), dim3(256), 0, stream()>>>(
             nent, k_out, d_runs, d_pads, hbins, a->heavy_seg);
     }
@@ -1284,16 +1288,16 @@ static int spmm_run(Csr *a, int64_t K, int64_t b_dptr, int64_t ldb, int64_t c_dp
         const dim3 grid(8 * G, tiles), block(SPMM_HW * 64);
         if (small_b && accumulate)
             spmm_heavy_sweep<true, true><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K, partial,
-                                                                       C, ldc, G);
+                                                                       C, ldc, G, ceil_div(a->ncols, 8));
         else if (small_b)
             spmm_heavy_sweep<true, false><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K, partial,
-                                                                        C, ldc, G);
+                                                                        C, ldc, G, ceil_div(a->ncols, 8));
         else if (accumulate)
             spmm_heavy_sweep<false, true><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K, partial,
-                                                                        C, ldc, G);
+                                                                        C, ldc, G, ceil_div(a->ncols, 8));
         else
             spmm_heavy_sweep<false, false><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K,
-                                                                         partial, C, ldc, G);
+                                                                         partial, C, ldc, G, ceil_div(a->ncols, 8));
     }
     if (overlap) {      // the rows in between, on the CUs the sweep leaves free
         COMET_CHK(spmm_chunks(a->light, K, B, ldb, C, ldc, accumulate, aux_stream()));
