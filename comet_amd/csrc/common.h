@@ -91,6 +91,10 @@ struct Csr {
     HeavyEnt *heavy_ent = nullptr;           // the lists, runs padded to even length
     int64_t heavy_rows = 0;
     int heavy_groups = 0;                    // workgroups of the sweep per XCD the lists were made for
+    // rows of middling length that ride on the sweep with their sums in LDS: row m of the list is kept by workgroup
+    // m % heavy_groups of every XCD in slot m / heavy_groups
+    int64_t medium_rows = 0;
+    int32_t *medium_row = nullptr;           // [medium_rows] row ids
     int32_t *heavy_row = nullptr;            // [heavy_rows] row ids of the long rows
     int32_t *heavy_code = nullptr;           // [8][heavy_rows] wavefront * 8 + slot that holds the row on each XCD
     Csr *light = nullptr;

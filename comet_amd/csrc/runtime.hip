@@ -175,6 +175,9 @@ static void csr_drop_plans(Csr *c)
     (void)hipFree(c->heavy_ent);
     (void)hipFree(c->heavy_row);
     (void)hipFree(c->heavy_code);
+    (void)hipFree(c->medium_row);
+    c->medium_row = nullptr;
+    c->medium_rows = 0;
     c->heavy_seg = nullptr;
     c->heavy_ent = nullptr;
     c->heavy_row = c->heavy_code = nullptr;

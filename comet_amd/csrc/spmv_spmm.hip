@@ -461,6 +461,16 @@ constexpr int SPMM_HG_ALONE = 32, SPMM_HG_SHARED = 24;
 constexpr int spmm_hbins(int g) { return g * SPMM_HW; }               // wavefronts (= row bins) per XCD
 constexpr int spmm_hslots(int g) { return spmm_hbins(g) * SPMM_HR; }  // slots for partial sums per XCD
 constexpr int spmm_hrows(int g) { return g * (SPMM_HW - 1) * SPMM_HR; }    // long rows the plan can hold
+// Rows of middling length - too short for a register of their own over the whole sweep, long enough that eight
+// partial sums cost less than fetching their rows of B from beyond the L2 - keep their sums in the LDS of the
+// sweep's workgroups, 64 doubles per row and workgroup, and their entries ride in the lists of the wavefronts that
+// own long rows, so they move through the columns at the sweep's pace and find their rows of B in the L2.
+#ifndef COMET_SPMM_MED_MIN
+#define COMET_SPMM_MED_MIN 32
+#endif
+constexpr int SPMM_MED_MIN_LEN = COMET_SPMM_MED_MIN;   // such a row has at least this many nonzeros
+constexpr int SPMM_MSLOTS = 288;                        // sums a workgroup keeps in LDS: 144 KiB
+static_assert(SPMM_MSLOTS <= 512, "a list entry has nine bits for the slot");
 constexpr int SPMM_HEAVY_MIN_LEN = COMET_SPMM_HEAVY_MIN;              // a long row has at least this many nonzeros
 constexpr int SPMM_HCB = 32;                         // column blocks a wavefront's list is cut into
 
@@ -502,6 +512,7 @@ constexpr int SPMM_HCB = 32;                         // column blocks a wavefron
 constexpr int SPMM_HP = 8;       // pairs of entries per batch of gathers
 constexpr int SPMM_E_REAL = 1;                 // not a pad
 constexpr int SPMM_E_FIRST = 2;                // the entry opens a run of one owned row
+constexpr int SPMM_E_MED = 4;                  // the entry adds into a sum kept in LDS, in the slot its row field names
 constexpr int SPMM_E_ROW = 3;                  // where the owned row (or, for a row kept in LDS, its slot) sits: 9 bits
 constexpr int SPMM_E_COL = 12;
 static_assert(SPMM_E_COL + SPMM_HCOLB <= 32 && SPMM_HRB <= SPMM_E_COL - SPMM_E_ROW, "an entry is 32 bits");
@@ -527,14 +538,17 @@ __device__ inline void heavy_issue(double2 (&b)[SPMM_HP], int ents, int t0, int 
     }
 }
 
+extern __shared__ double spmm_medium_sums[];
 __device__ inline void heavy_add(double (&accx)[SPMM_HR], double (&accy)[SPMM_HR], double2 &run, int &run_slot,
-                                 const double2 (&b)[SPMM_HP], int ents, double vals, int t0, int npairs, int half)
+                                 const double2 (&b)[SPMM_HP], int ents, double vals, int t0, int npairs, int half,
+                                 int sub, bool active)
 {
 #pragma unroll
     for (int u = 0; u < SPMM_HP; ++u) {
         if (t0 + u < npairs) {
             const int t = t0 + u;
             const int e0 = __builtin_amdgcn_readlane(ents, 2 * t);
+            const bool med = (e0 & SPMM_E_MED) != 0;       // both entries of a pair are of the same kind
             if (e0 & SPMM_E_FIRST) {             // a run starts on an even entry
                 accx[run_slot] = run.x;
                 accy[run_slot] = run.y;
@@ -546,7 +560,16 @@ __device__ inline void heavy_add(double (&accx)[SPMM_HR], double (&accy)[SPMM_HR
             const double v = __hiloint2double(__shfl(__double2hiint(vals), 2 * t + half, 64),
                                               __shfl(__double2loint(vals), 2 * t + half, 64));
             const double px = v * b[u].x, py = v * b[u].y;
-            if (mine & SPMM_E_REAL) {            // a pad carries no value
+            if (med) {
+                // a row of middling length: its sum lives in LDS.  An add that returns nothing is issued and
+                // forgotten; all entries of such a row are in this wavefront's list, in column order, and the adds
+                // of one wavefront to one address are carried out in the order it issued them.
+                if ((mine & SPMM_E_REAL) && active) {
+                    double *sum = spmm_medium_sums + ((mine >> SPMM_E_ROW) & 511) * 64 + 2 * sub;
+                    __hip_atomic_fetch_add(sum, px, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(sum + 1, py, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+            } else if (mine & SPMM_E_REAL) {     // a pad carries no value
                 run.x = run.x + px;
                 run.y = run.y + py;
             }
@@ -644,7 +667,8 @@ __device__ inline void single_rows(const spmm_v4i *__restrict__ list, int64_t n,
 template <bool SMALL, bool ACC>
 __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
     const int64_t *__restrict__ seg, const HeavyEnt *__restrict__ hent, const double *__restrict__ B, int64_t ldb,
-    int64_t K, double *__restrict__ partial, double *__restrict__ C, int64_t ldc, int G, int64_t xcols)
+    int64_t K, double *__restrict__ partial, double *__restrict__ C, int64_t ldc, int G, int64_t xcols, int nslots,
+    double *__restrict__ partial_medium)
 {
     const int lane = threadIdx.x & 63, half = lane >> 5, sub = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -668,6 +692,9 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
 #pragma unroll
     for (int r = 0; r < SPMM_HR; ++r)
         accx[r] = accy[r] = 0.0;
+    // the sums in LDS whose entries this wavefront's list holds: slot mod SPMM_HWL = wavefront
+    for (int sl = wave; sl < nslots; sl += SPMM_HWL)
+        spmm_medium_sums[sl * 64 + lane] = 0.0;
     if (s < e) {
         double2 b[SPMM_HP];
         double2 run = make_double2(0.0, 0.0);
@@ -692,12 +719,12 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
                 n_val = __hiloint2double(q.w, q.z);
             }
             const int np = cnt >> 1;
-            heavy_add(accx, accy, run, run_slot, b, c_ent, c_val, 0, np, half);
+            heavy_add(accx, accy, run, run_slot, b, c_ent, c_val, 0, np, half, sub, active);
 #pragma unroll
             for (int t0 = SPMM_HP; t0 < 32; t0 += SPMM_HP)
                 if (np > t0) {
                     heavy_issue<SMALL>(b, c_ent, t0, np, half, B, ldb, col);
-                    heavy_add(accx, accy, run, run_slot, b, c_ent, c_val, t0, np, half);
+                    heavy_add(accx, accy, run, run_slot, b, c_ent, c_val, t0, np, half, sub, active);
                 }
             if (ncnt > 0)         // the first batch of the next 64 entries: in flight over the loop's back edge
                 heavy_issue<SMALL>(b, n_ent, 0, ncnt >> 1, half, B, ldb, col);
@@ -707,6 +734,13 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
         }
         accx[run_slot] = run.x;
         accy[run_slot] = run.y;
+    }
+    {   // this wavefront's sums in LDS: one partial sum per row and XCD, like the long rows'
+        const int64_t c1 = (int64_t)blockIdx.y * 64 + lane;
+        double *mout = partial_medium + ((int64_t)x * G + g) * nslots * K;
+        for (int sl = wave; sl < nslots; sl += SPMM_HWL)
+            if (c1 < K)
+                mout[(int64_t)sl * K + c1] = spmm_medium_sums[sl * 64 + lane];
     }
     // even entries + odd entries, then the lower half writes both columns
     double *out = partial + (((int64_t)x * G + g) * SPMM_HW + wave) * SPMM_HR * K;
@@ -827,6 +861,27 @@ __global__ void single_make_keys(int64_t nsingle, const int32_t *__restrict__ sr
     idx[i] = (uint32_t)i;
 }
 
+// The rows of middling length: row m of their list is kept by workgroup m % groups of every XCD, in slot
+// j = m / groups, and its entries go into the list of wavefront j % SPMM_HWL of that workgroup, behind the runs of
+// the wavefront's long rows in every column block.  idx = the entry's place among all such entries.
+__global__ void medium_make_keys(int64_t nmedium, const int32_t *__restrict__ mrow, const int64_t *__restrict__ mstart,
+                                 const int64_t *__restrict__ pos, const int32_t *__restrict__ crd, int64_t xcols,
+                                 int groups, uint64_t *__restrict__ keys, uint32_t *__restrict__ idx)
+{
+    const int64_t m = blockIdx.x;
+    if (m >= nmedium)
+        return;
+    const int64_t ps = pos[mrow[m]], len = pos[mrow[m] + 1] - ps, o = mstart[m];
+    const uint64_t bin = (uint64_t)(m % groups) * SPMM_HW + (uint64_t)((m / groups) % SPMM_HWL);
+    for (int64_t t = threadIdx.x; t < len; t += blockDim.x) {
+        const uint64_t c = (uint64_t)(uint32_t)crd[ps + t];
+        const uint64_t x = c / (uint64_t)xcols;
+        const uint64_t cb = (c - x * (uint64_t)xcols) * SPMM_HCB / (uint64_t)xcols;
+        keys[o + t] = ((((x * (uint64_t)spmm_hbins(groups) + bin) * SPMM_HCB + cb) * (2 * SPMM_HR) + SPMM_HR + 1) << 28) | c;
+        idx[o + t] = (uint32_t)(o + t);
+    }
+}
+
 // first[e] = 1 where entry e of the ordered list opens a run (another row, column block or wavefront)
 __global__ void heavy_mark_runs(int64_t n, const uint64_t *__restrict__ keys, int64_t *__restrict__ first)
 {
@@ -854,10 +909,12 @@ __global__ void heavy_run_odd(int64_t nruns, const int64_t *__restrict__ start, 
 }
 
 // Writes the list with every run padded to even length: entry e of run r lands at e + (pads in front of r).
-// idx is a position in val for a long row's entry, and a position in srow for a row with one nonzero.
+// idx is a position in val for a long row's entry, a position in srow for a row with one nonzero, and a place
+// among the entries of the rows of middling length for one of those.
 __global__ void heavy_fill(int64_t n, const uint64_t *__restrict__ keys, const uint32_t *__restrict__ idx,
                            const double *__restrict__ val, const int64_t *__restrict__ pos,
-                           const int32_t *__restrict__ srow, const int64_t *__restrict__ first,
+                           const int32_t *__restrict__ srow, int64_t nmedium, const int32_t *__restrict__ mrow,
+                           const int64_t *__restrict__ mstart, int groups, const int64_t *__restrict__ first,
                            const int64_t *__restrict__ runs, const int64_t *__restrict__ start,
                            const int64_t *__restrict__ pads, int64_t xcols, HeavyEnt *__restrict__ hent)
 {
@@ -871,7 +928,20 @@ __global__ void heavy_fill(int64_t n, const uint64_t *__restrict__ keys, const u
     const uint64_t c = k & 0xfffffffull;
     const uint32_t col = (uint32_t)(c - (c / (uint64_t)xcols) * (uint64_t)xcols) << SPMM_E_COL;     // inside its XCD's range
     HeavyEnt out;
-    if (direct) {
+    if (direct && ((k >> 28) & 1)) {          // a row of middling length: which one, from the entry's place
+        const int64_t at = idx[e];
+        int64_t lo = 0, hi = nmedium - 1;      // the last m with mstart[m] <= at
+        while (lo < hi) {
+            const int64_t mid = (lo + hi + 1) >> 1;
+            if (mstart[mid] <= at)
+                lo = mid;
+            else
+                hi = mid - 1;
+        }
+        out.ent = (int32_t)(col | SPMM_E_REAL | SPMM_E_MED | ((uint32_t)(lo / groups) << SPMM_E_ROW));
+        out.row = 0;
+        out.val = val[pos[mrow[lo]] + (at - mstart[lo])];
+    } else if (direct) {
         out.ent = (int32_t)(col | SPMM_E_REAL);
         out.row = srow[idx[e]];
         out.val = val[pos[out.row]];
@@ -936,13 +1006,23 @@ template <bool ACC>
 __global__ __launch_bounds__(256) void spmm_heavy_combine(int64_t nheavy, const int32_t *__restrict__ hrow,
                                                           const int32_t *__restrict__ hcode,
                                                           const double *__restrict__ partial, int hslots,
+                                                          int64_t nmedium, const int32_t *__restrict__ mrow, int groups,
+                                                          int nslots, const double *__restrict__ partial_medium,
                                                           double *__restrict__ C, int64_t ldc, int64_t K)
 {
     const int lane = threadIdx.x & 63;
     const int64_t h = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const int64_t col = (int64_t)blockIdx.y * 64 + lane;
-    if (h >= nheavy || col >= K)
+    if (h >= nheavy + nmedium || col >= K)
         return;
+    if (h >= nheavy) {          // a row of middling length: slot m / groups of workgroup m % groups of every XCD
+        const int64_t m = h - nheavy, row = mrow[m];
+        double acc = ACC ? C[row * ldc + col] : 0.0;
+        for (int x = 0; x < 8; ++x)
+            acc = acc + partial_medium[((((int64_t)x * groups + m % groups) * nslots) + m / groups) * K + col];
+        C[row * ldc + col] = acc;
+        return;
+    }
     const int64_t row = hrow[h];
     double acc = ACC ? C[row * ldc + col] : 0.0;
     for (int x = 0; x < 8; ++x)
@@ -950,7 +1030,17 @@ __global__ __launch_bounds__(256) void spmm_heavy_combine(int64_t nheavy, const 
     C[row * ldc + col] = acc;
 }
 
-static Workspace g_heavy_partial;
+static Workspace g_heavy_partial, g_medium_partial;
+
+// Launches the sweep with `lds` bytes of dynamic LDS, asking for more than the 64 KiB a kernel gets by default.
+template <typename Kern, typename... Args>
+static void sweep_launch(Kern kernel, dim3 grid, dim3 block, size_t lds, Args... args)
+{
+    if (lds > 64 * 1024)
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)lds);
+    kernel<<<grid, block, lds, stream()>>>(args...);
+}
 
 static int spmm_heavy_plan(Csr *a)
 {
@@ -965,10 +1055,20 @@ static int spmm_heavy_plan(Csr *a)
                                 stream()));
     COMET_HIPCHK(hipStreamSynchronize(stream()));
     std::vector<std::pair<int64_t, int32_t>> cand;       // (-length, row): sorts longest first, ties by row
-    for (int64_t r = 0; r < n; ++r)
-        if (pos[(size_t)r + 1] - pos[(size_t)r] >= SPMM_HEAVY_MIN_LEN)
-            cand.emplace_back(-(pos[(size_t)r + 1] - pos[(size_t)r]), (int32_t)r);
+    std::vector<std::pair<int64_t, int32_t>> mcand;      // the same for the rows of middling length
+    // Off unless COMET_HIP_SPMM_MEDIUM is set: on the benchmark matrix it takes 0.4 GB off the traffic past the L2
+    // (the rows of B these rows gather are hits) and costs time - an entry of such a row takes the sweep 11 ns of a
+    // CU, the chunk kernel beside the sweep 16, but the sweep is the longer of the two: 0.343 against 0.312 ms.
+    const bool medium_on = getenv("COMET_HIP_SPMM_MEDIUM") != nullptr;
+    for (int64_t r = 0; r < n; ++r) {
+        const int64_t len = pos[(size_t)r + 1] - pos[(size_t)r];
+        if (len >= SPMM_HEAVY_MIN_LEN)
+            cand.emplace_back(-len, (int32_t)r);
+        else if (medium_on && len >= SPMM_MED_MIN_LEN)
+            mcand.emplace_back(-len, (int32_t)r);
+    }
     std::sort(cand.begin(), cand.end());
+    std::sort(mcand.begin(), mcand.end());
     // How many CUs of an XCD the sweep takes: all of them, unless the rows that are neither long nor single (with
     // the sweep at full size) hold at least a sixteenth of the matrix; COMET_HIP_SPMM_GROUPS overrides.
     int G = SPMM_HG_ALONE;
@@ -987,6 +1087,21 @@ static int spmm_heavy_plan(Csr *a)
         }
     }
     const int hbins = spmm_hbins(G);
+    // rows of middling length: the long rows the sweep has no register for, then the rows below them, longest
+    // first, as many as the workgroups have slots in LDS
+    std::vector<int32_t> mrow;
+    std::vector<int64_t> mstart(1, 0);
+    if (medium_on) {
+        for (size_t k = (size_t)spmm_hrows(G); k < cand.size() && (int64_t)mrow.size() < (int64_t)G * SPMM_MSLOTS; ++k) {
+            mrow.push_back(cand[k].second);
+            mstart.push_back(mstart.back() - cand[k].first);
+        }
+        for (size_t k = 0; k < mcand.size() && (int64_t)mrow.size() < (int64_t)G * SPMM_MSLOTS; ++k) {
+            mrow.push_back(mcand[k].second);
+            mstart.push_back(mstart.back() - mcand[k].first);
+        }
+    }
+    const int64_t M = (int64_t)mrow.size(), mnnz = mstart.back();
     if ((int64_t)cand.size() > spmm_hrows(G))
         cand.resize((size_t)spmm_hrows(G));
     const int64_t H = (int64_t)cand.size();
@@ -997,7 +1112,9 @@ static int spmm_heavy_plan(Csr *a)
         return COMET_HIP_OK;        // the long rows hold too little of the matrix to pay for a second kernel
     std::vector<int32_t> hrow((size_t)H), hcode((size_t)(8 * H)), cnt((size_t)(8 * H));
     std::vector<int64_t> hstart((size_t)H + 1, 0);
-    std::vector<char> is_long((size_t)n, 0);
+    std::vector<char> is_long((size_t)n, 0);         // 1: long, 2: of middling length
+    for (int64_t m = 0; m < M; ++m)
+        is_long[(size_t)mrow[(size_t)m]] = 2;
     for (int64_t k = 0; k < H; ++k) {
         hrow[(size_t)k] = cand[(size_t)k].second;
         is_long[(size_t)hrow[(size_t)k]] = 1;
@@ -1012,9 +1129,9 @@ static int spmm_heavy_plan(Csr *a)
         (len == 0 ? erow : len == 1 ? srow : lrow).push_back((int32_t)r);
     }
     const int64_t S = (int64_t)srow.size(), E = (int64_t)erow.size(), L = (int64_t)lrow.size();
-    const int64_t nent = hnnz + S;          // entries of the lists before padding
+    const int64_t nent = hnnz + S + mnnz;          // entries of the lists before padding
     int32_t *d_cnt = nullptr, *d_srow = nullptr;
-    int64_t *d_hstart = nullptr, *d_len = nullptr;
+    int64_t *d_hstart = nullptr, *d_len = nullptr, *d_mstart = nullptr;
     int64_t *d_first = nullptr, *d_runs = nullptr, *d_start = nullptr, *d_odd = nullptr, *d_pads = nullptr;
     uint64_t *k_in = nullptr, *k_out = nullptr;
     uint32_t *i_in = nullptr, *i_out = nullptr;
@@ -1023,6 +1140,7 @@ static int spmm_heavy_plan(Csr *a)
         (void)hipFree(d_cnt);
         (void)hipFree(d_srow);
         (void)hipFree(d_hstart);
+        (void)hipFree(d_mstart);
         (void)hipFree(d_len);
         (void)hipFree(d_first);
         (void)hipFree(d_runs);
@@ -1038,6 +1156,8 @@ static int spmm_heavy_plan(Csr *a)
             (void)hipFree(a->heavy_ent);
             (void)hipFree(a->heavy_row);
             (void)hipFree(a->heavy_code);
+            (void)hipFree(a->medium_row);
+            a->medium_row = nullptr;
             (void)hipFree(a->empty_rows);
             a->heavy_seg = nullptr;
             a->heavy_ent = nullptr;
@@ -1058,6 +1178,11 @@ static int spmm_heavy_plan(Csr *a)
     HEAVY_TRY(hipMalloc((void **)&d_cnt, 4 * (size_t)(8 * H)));
     HEAVY_TRY(hipMalloc((void **)&d_srow, 4 * at_least_one(S)));
     HEAVY_TRY(hipMalloc((void **)&d_hstart, 8 * (size_t)(H + 1)));
+    HEAVY_TRY(hipMalloc((void **)&d_mstart, 8 * (size_t)(M + 1)));
+    HEAVY_TRY(hipMalloc((void **)&a->medium_row, 4 * at_least_one(M)));
+    if (M > 0)
+        HEAVY_TRY(hipMemcpyAsync(a->medium_row, mrow.data(), 4 * (size_t)M, hipMemcpyHostToDevice, stream()));
+    HEAVY_TRY(hipMemcpyAsync(d_mstart, mstart.data(), 8 * (size_t)(M + 1), hipMemcpyHostToDevice, stream()));
     HEAVY_TRY(hipMalloc((void **)&d_len, 8 * at_least_one(L)));
     HEAVY_TRY(hipMalloc((void **)&k_in, 8 * (size_t)nent));
     HEAVY_TRY(hipMalloc((void **)&k_out, 8 * (size_t)nent));
@@ -1117,6 +1242,9 @@ static int spmm_heavy_plan(Csr *a)
         if (S > 0)
             single_make_keys<<<dim3((unsigned)ceil_div(S, 256)), dim3(256), 0, stream()>>>(
                 S, d_srow, a->pos, a->crd, xcols, G, k_in + hnnz, i_in + hnnz);
+        if (M > 0)
+            medium_make_keys<<<dim3((unsigned)M), dim3(64), 0, stream()>>>(M, a->medium_row, d_mstart, a->pos, a->crd,
+                                                                          xcols, G, k_in + hnnz + S, i_in + hnnz + S);
     }
     if (sort_pairs_u64_u32(k_in, k_out, i_in, i_out, nent, 28 + (SPMM_HRB + 1) + 5 + 12) != COMET_HIP_OK) {
         cleanup(true);
@@ -1149,14 +1277,15 @@ static int spmm_heavy_plan(Csr *a)
     {
         KernelTimer t("heavy_fill");
         heavy_fill<<<dim3((unsigned)ceil_div(nent, 256)), dim3(256), 0, stream()>>>(
-            nent, k_out, i_out, a->val, a->pos, d_srow, d_first, d_runs, d_start, d_pads, xcols, a->heavy_ent);
+            nent, k_out, i_out, a->val, a->pos, d_srow, M, a->medium_row, d_mstart, G, d_first, d_runs, d_start, d_pads,
+            xcols, a->heavy_ent);
         heavy_segments<<<dim3((unsigned)ceil_div(8 * hbins + 1, 256)), dim3(256), 0, stream()>>>(
             nent, k_out, d_runs, d_pads, hbins, a->heavy_seg);
     }
     // the rows of two and more nonzeros that are not long, as a matrix of their own
     light->nrows = L;
     light->ncols = a->ncols;
-    light->nnz = a->nnz - hnnz - S;
+    light->nnz = a->nnz - hnnz - S - mnnz;
     light->owns = true;
     HEAVY_TRY(hipMalloc((void **)&light->pos, 8 * (size_t)(L + 1)));
     HEAVY_TRY(hipMalloc((void **)&light->crd, 4 * at_least_one(light->nnz)));
@@ -1182,6 +1311,7 @@ static int spmm_heavy_plan(Csr *a)
     a->heavy_nnz = hnnz;
     a->heavy_rows = H;
     a->heavy_groups = G;
+    a->medium_rows = M;
     a->nempty = E;
     a->heavy_state = 2;
     return COMET_HIP_OK;
@@ -1282,22 +1412,27 @@ static int spmm_run(Csr *a, int64_t K, int64_t b_dptr, int64_t ldb, int64_t c_dp
     // long rows (sums on chip, left in `partial`) and rows of one nonzero (stored to C)
     COMET_CHK(g_heavy_partial.ensure(sizeof(double) * 8 * (size_t)spmm_hslots(G) * (size_t)K, false));
     double *partial = (double *)g_heavy_partial.ptr;
+    // rows of middling length: ceil(rows / G) sums of 64 doubles in the LDS of every workgroup
+    const int nslots = (int)ceil_div(a->medium_rows, G);
+    const size_t medium_lds = sizeof(double) * 64 * (size_t)nslots;
+    COMET_CHK(g_medium_partial.ensure(sizeof(double) * 8 * (size_t)G * (size_t)(nslots > 0 ? nslots : 1) * (size_t)K, false));
+    double *partial_medium = (double *)g_medium_partial.ptr;
     {
         KernelTimer t("spmm_heavy_sweep");
         const bool small_b = a->ncols < (1 << 24) && ldb * 8 < (1 << 24) && a->ncols * ldb * 8 < (1ll << 32);
         const dim3 grid(8 * G, tiles), block(SPMM_HW * 64);
         if (small_b && accumulate)
-            spmm_heavy_sweep<true, true><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K, partial,
-                                                                       C, ldc, G, ceil_div(a->ncols, 8));
+            sweep_launch(spmm_heavy_sweep<true, true>, grid, block, medium_lds, a->heavy_seg, a->heavy_ent, B, ldb, K, partial, C, ldc,
+                         G, ceil_div(a->ncols, 8), nslots, partial_medium);
         else if (small_b)
-            spmm_heavy_sweep<true, false><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K, partial,
-                                                                        C, ldc, G, ceil_div(a->ncols, 8));
+            sweep_launch(spmm_heavy_sweep<true, false>, grid, block, medium_lds, a->heavy_seg, a->heavy_ent, B, ldb, K, partial, C, ldc,
+                         G, ceil_div(a->ncols, 8), nslots, partial_medium);
         else if (accumulate)
-            spmm_heavy_sweep<false, true><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K, partial,
-                                                                        C, ldc, G, ceil_div(a->ncols, 8));
+            sweep_launch(spmm_heavy_sweep<false, true>, grid, block, medium_lds, a->heavy_seg, a->heavy_ent, B, ldb, K, partial, C, ldc,
+                         G, ceil_div(a->ncols, 8), nslots, partial_medium);
         else
-            spmm_heavy_sweep<false, false><<<grid, block, 0, stream()>>>(a->heavy_seg, a->heavy_ent, B, ldb, K,
-                                                                         partial, C, ldc, G, ceil_div(a->ncols, 8));
+            sweep_launch(spmm_heavy_sweep<false, false>, grid, block, medium_lds, a->heavy_seg, a->heavy_ent, B, ldb, K, partial, C, ldc,
+                         G, ceil_div(a->ncols, 8), nslots, partial_medium);
     }
     if (overlap) {      // the rows in between, on the CUs the sweep leaves free
         COMET_CHK(spmm_chunks(a->light, K, B, ldb, C, ldc, accumulate, aux_stream()));
@@ -1305,13 +1440,15 @@ static int spmm_run(Csr *a, int64_t K, int64_t b_dptr, int64_t ldb, int64_t c_dp
     }
     {
         KernelTimer t("spmm_heavy_combine");
-        const dim3 grid((unsigned)ceil_div(a->heavy_rows, 4), tiles);
+        const dim3 grid((unsigned)ceil_div(a->heavy_rows + a->medium_rows, 4), tiles);
         if (accumulate)
             spmm_heavy_combine<true><<<grid, dim3(256), 0, stream()>>>(a->heavy_rows, a->heavy_row, a->heavy_code,
-                                                                       partial, spmm_hslots(G), C, ldc, K);
+                                                                       partial, spmm_hslots(G), a->medium_rows,
+                                                                       a->medium_row, G, nslots, partial_medium, C, ldc, K);
         else
             spmm_heavy_combine<false><<<grid, dim3(256), 0, stream()>>>(a->heavy_rows, a->heavy_row, a->heavy_code,
-                                                                        partial, spmm_hslots(G), C, ldc, K);
+                                                                        partial, spmm_hslots(G), a->medium_rows,
+                                                                       a->medium_row, G, nslots, partial_medium, C, ldc, K);
     }
     COMET_HIPCHK(hipGetLastError());
     return COMET_HIP_OK;

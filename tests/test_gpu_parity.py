@@ -190,8 +190,10 @@ def test_spmm_golden(golden, golden_dir):
     assert orc.format_f64(Cm.to_numpy()) == g["printed"]
 
 
-def _long_rows(pos, K):
-    """The rows the library hands to the column sweep (its rule restated): at least 128 nonzeros, at most the
+def _swept_rows(pos, K):
+    """The rows the library hands to the column sweep (its rule restated), as (long, middling).  Middling: the rows
+    of 32 to 127 nonzeros and the long rows the sweep has no register for, longest first, at most 288 x g; their
+    sums are kept in LDS.  Long: at least 128 nonzeros, at most the
     120 x g longest (ties: lower row first) with g = 32 workgroups of the sweep per XCD - or 24, leaving CUs to
     the chunk kernel beside it, when the rows that are neither long (at g = 32) nor single hold a sixteenth of
     the matrix; COMET_HIP_SPMM_GROUPS overrides g - and only if they hold a quarter of a matrix of >= 2^19
@@ -203,10 +205,17 @@ def _long_rows(pos, K):
     if (pos[-1] - lens[rows[:3840]].sum() - (lens == 1).sum()) * 16 >= pos[-1]:
         groups = 24
     groups = int(os.environ.get("COMET_HIP_SPMM_GROUPS", groups))
+    medium = np.concatenate([rows[120 * groups:], _by_length(lens, np.flatnonzero((lens >= 32) & (lens < 128)))])
+    if "COMET_HIP_SPMM_MEDIUM" not in os.environ:        # the library keeps such rows in LDS only when asked to
+        medium = medium[:0]
     rows = rows[:120 * groups]
     if not (16 <= K <= 2048) or pos[-1] < (1 << 19) or 4 * lens[rows].sum() < pos[-1]:
-        return rows[:0]
-    return rows
+        return rows[:0], rows[:0]
+    return rows, medium[:288 * groups]
+
+
+def _by_length(lens, rows):
+    return rows[np.argsort(-lens[rows], kind="stable")]
 
 
 def _bit_exact_rows(pos, K):
@@ -215,9 +224,10 @@ def _bit_exact_rows(pos, K):
     rows of at most one nonzero."""
     lens = np.diff(pos)
     light = lens.copy()
-    long_rows = _long_rows(pos, K)
+    long_rows, medium_rows = _swept_rows(pos, K)
     if len(long_rows):
         light[long_rows] = 0
+        light[medium_rows] = 0      # summed per XCD, then across: not the checker's order
         light[lens == 1] = 0        # these ride on the sweep: one product each
     lpos = np.concatenate([[0], np.cumsum(light)])
     return (lens <= 1) | ((light > 0) & (lpos[:-1] // 256 == (lpos[1:] - 1) // 256))
@@ -1017,7 +1027,7 @@ def _sweep_check(pos, crd, val, B, C0=None, ld_pad=0):
     want = orc.spmm(pos, crd, val, B, C0)
     bound = orc.spmm(pos, crd, np.abs(val), np.abs(B), None if C0 is None else np.abs(C0))
     assert np.all(np.abs(got - want) <= RTOL * bound)
-    long_rows = _long_rows(pos, K if swept else 0)
+    long_rows, _ = _swept_rows(pos, K if swept else 0)
     inside = _bit_exact_rows(pos, K if swept else 0)
     assert inside.sum() > 0 and np.array_equal(got[inside], want[inside])
     # a second call on the same handle reuses the plan and gives the same bits
@@ -1026,9 +1036,12 @@ def _sweep_check(pos, crd, val, B, C0=None, ld_pad=0):
     return len(long_rows)
 
 
+@pytest.mark.parametrize("medium", [False, True])
 @pytest.mark.parametrize("K,acc,pad", [(64, False, 0), (64, True, 0), (20, False, 4), (100, True, 6), (64, False, 3),
                                         (33, True, 0)])
-def test_spmm_long_rows_sweep(K, acc, pad):
+def test_spmm_long_rows_sweep(K, acc, pad, medium, monkeypatch):
+    if medium:      # rows of 32..127 nonzeros ride on the sweep too, their sums in LDS
+        monkeypatch.setenv("COMET_HIP_SPMM_MEDIUM", "1")
     pos, crd, val = gen.zipf_csr(n=40_000, mean=16.0, cap=4096, seed=7)
     assert len(crd) >= 1 << 19
     B = gen.dense((40_000, K), seed=8)
@@ -1044,6 +1057,7 @@ def test_spmm_more_long_rows_than_the_sweep_holds(groups, held, monkeypatch):
     leaves free (24 workgroups per XCD; 32 and 16 forced); an empty row and a short row sit between them."""
     if groups is not None:
         monkeypatch.setenv("COMET_HIP_SPMM_GROUPS", str(groups))
+        monkeypatch.setenv("COMET_HIP_SPMM_MEDIUM", "1")       # and the rows without a register keep their sums in LDS
     rng = np.random.default_rng(31)
     n, m = 5002, 3000
     lens = np.full(n, 300); lens[17] = 0; lens[4000] = 3
