@@ -75,6 +75,7 @@ struct Csr {
     // spmv_nb == 0: not decided yet; 1: run on the original arrays.
     int spmv_nb = 0;
     int64_t *spmv_bpos = nullptr;            // [spmv_nb][nrows + 1], relative to the block's base
+    int32_t *spmv_bpos32 = nullptr;          // the same in 32 bits (then spmv_bpos is null): what the passes read
     int32_t *spmv_bcrd = nullptr;
     double *spmv_bval = nullptr;
     std::vector<int64_t> spmv_base;          // first entry of each block in spmv_bcrd / spmv_bval

@@ -190,6 +190,8 @@ static void csr_drop_plans(Csr *c)
     c->sg_blkptr = nullptr;
     c->sg_nblk = 0;
     (void)hipFree(c->spmv_bpos);
+    (void)hipFree(c->spmv_bpos32);
+    c->spmv_bpos32 = nullptr;
     (void)hipFree(c->spmv_bcrd);
     (void)hipFree(c->spmv_bval);
     c->spmv_bpos = nullptr;

@@ -50,8 +50,10 @@ __device__ inline int64_t uniform_i64(int64_t v)
            (uint32_t)__builtin_amdgcn_readfirstlane((int)(v & 0xffffffff));
 }
 
-template <bool ACC>
-__global__ __launch_bounds__(SPMV_T) void spmv_csr_stream(const int64_t *__restrict__ pos,
+// P: the row pointers' type - int64 for a matrix as uploaded, int32 for the column blocks of the plan, whose row
+// pointers are read again by every pass
+template <bool ACC, typename P>
+__global__ __launch_bounds__(SPMV_T) void spmv_csr_stream(const P *__restrict__ pos,
                                                           const int32_t *__restrict__ crd,
                                                           const double *__restrict__ val,
                                                           const double *__restrict__ x,
@@ -65,9 +67,9 @@ __global__ __launch_bounds__(SPMV_T) void spmv_csr_stream(const int64_t *__restr
     const int64_t r0 = (int64_t)blockIdx.x * SPMV_T;
     const int64_t r = r0 + tid;
     const int64_t rlast = r0 + SPMV_T < nrows ? r0 + SPMV_T : nrows;
-    const int64_t ps = pos[r < nrows ? r : nrows];
-    const int64_t pe = pos[r + 1 < nrows ? r + 1 : nrows];
-    const int64_t bs = uniform_i64(pos[r0]), be = uniform_i64(pos[rlast]);
+    const int64_t ps = (int64_t)pos[r < nrows ? r : nrows];
+    const int64_t pe = (int64_t)pos[r + 1 < nrows ? r + 1 : nrows];
+    const int64_t bs = uniform_i64((int64_t)pos[r0]), be = uniform_i64((int64_t)pos[rlast]);
     double acc = 0.0;
     if (ACC && r < nrows)
         acc = y[r];
@@ -150,6 +152,13 @@ __device__ inline int64_t lower_bound_col(const int32_t *__restrict__ crd, int64
 }
 
 // cnt[b * nrows + r] = nonzeros of row r with column in block b
+__global__ void spmv_narrow_pos(const int64_t *__restrict__ in, int32_t *__restrict__ out, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        out[i] = (int32_t)in[i];
+}
+
 __global__ void spmv_split_count(const int64_t *__restrict__ pos, const int32_t *__restrict__ crd, int64_t nrows,
                                  int nb, int64_t block_cols, int64_t *__restrict__ cnt)
 {
@@ -260,6 +269,24 @@ static int spmv_plan(Csr *a)
     if (hipGetLastError() != hipSuccess) {
         cleanup();
         return set_error(COMET_HIP_ERR_HIP, "SpMV plan kernel launch failed");
+    }
+    // the blocks' row pointers are read by every pass: 32 bits are enough for them unless a block holds 2^31 nonzeros
+    bool narrow = true;
+    for (int b = 0; b < nb; ++b)
+        narrow = narrow && totals[b] < (1ll << 31);
+    if (narrow) {
+        int32_t *bpos32 = nullptr;
+        const int64_t count = (int64_t)nb * (n + 1);
+        if (hipMalloc((void **)&bpos32, sizeof(int32_t) * (size_t)count) == hipSuccess) {
+            spmv_narrow_pos<<<dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, stream()>>>(bpos, bpos32, count);
+            if (hipStreamSynchronize(stream()) == hipSuccess) {
+                a->spmv_bpos32 = bpos32;
+                (void)hipFree(bpos);
+                bpos = nullptr;
+            } else {
+                (void)hipFree(bpos32);
+            }
+        }
     }
     a->spmv_bpos = bpos;
     a->spmv_bcrd = bcrd;
@@ -1346,15 +1373,23 @@ static int spmv_run(Csr *a, int64_t x_dptr, int64_t y_dptr, int accumulate)
     const double *x = (const double *)x_dptr;
     double *y = (double *)y_dptr;
     for (int b = 0; b < a->spmv_nb; ++b) {
-        const int64_t *pos = a->spmv_nb == 1 ? a->pos : a->spmv_bpos + (int64_t)b * (a->nrows + 1);
         const int32_t *crd = a->spmv_nb == 1 ? a->crd : a->spmv_bcrd + a->spmv_base[b];
         const double *val = a->spmv_nb == 1 ? a->val : a->spmv_bval + a->spmv_base[b];
         const bool acc = accumulate || b > 0;   // later passes continue the row sums the earlier ones left in y
         KernelTimer t("spmv_csr_stream");
-        if (acc)
-            spmv_csr_stream<true><<<dim3(blocks), dim3(SPMV_T), 0, stream()>>>(pos, crd, val, x, y, a->nrows);
-        else
-            spmv_csr_stream<false><<<dim3(blocks), dim3(SPMV_T), 0, stream()>>>(pos, crd, val, x, y, a->nrows);
+        if (a->spmv_nb > 1 && a->spmv_bpos32) {
+            const int32_t *pos = a->spmv_bpos32 + (int64_t)b * (a->nrows + 1);
+            if (acc)
+                spmv_csr_stream<true, int32_t><<<dim3(blocks), dim3(SPMV_T), 0, stream()>>>(pos, crd, val, x, y, a->nrows);
+            else
+                spmv_csr_stream<false, int32_t><<<dim3(blocks), dim3(SPMV_T), 0, stream()>>>(pos, crd, val, x, y, a->nrows);
+        } else {
+            const int64_t *pos = a->spmv_nb == 1 ? a->pos : a->spmv_bpos + (int64_t)b * (a->nrows + 1);
+            if (acc)
+                spmv_csr_stream<true, int64_t><<<dim3(blocks), dim3(SPMV_T), 0, stream()>>>(pos, crd, val, x, y, a->nrows);
+            else
+                spmv_csr_stream<false, int64_t><<<dim3(blocks), dim3(SPMV_T), 0, stream()>>>(pos, crd, val, x, y, a->nrows);
+        }
     }
     COMET_HIPCHK(hipGetLastError());
     return COMET_HIP_OK;
