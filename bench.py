@@ -255,10 +255,11 @@ def bench_spmv(rt, orc, gen, args):
     flops = 2.0 * nnz
     ib = 4
     alg_bytes = nnz * (8 + ib) + (n + 1) * ib + 8 * n + 8 * n
-    dom = "spmv_csr_stream"     # one launch per column block of the plan: a step is all of them
+    # all column blocks of the plan in one launch, or (rows beyond what one resident grid holds) one launch per block
+    dom = "spmv_csr_blocks" if "spmv_csr_blocks" in kt else "spmv_csr_stream"
     passes = kt[dom]["launches"] // args.steps
-    # the passes are ~20 us each, short enough for an event pair per launch to add 25 % of its own; the step
-    # holds nothing but these passes, so the event pair around the timed steps is the kernel time
+    # the step holds nothing but these launches, and an event pair per launch adds several microseconds of its own to
+    # a kernel this short: the event pair around the timed steps is the kernel time
     dom_ms = dev_ms
     cpu = None
     if not args.no_cpu:
@@ -270,7 +271,7 @@ def bench_spmv(rt, orc, gen, args):
         "metric": "CSR SpMV GFLOP/s (+ achieved HBM GB/s as % of roofline) on 1 MI355X",
         "value": flops / (dev_ms * 1e-3) / 1e9, "unit": "GFLOP/s", "ms_per_step": dev_ms, "dtype": "f64",
         "config": {"workload": "spmv_csr_poisson", "rows": n, "cols": n, "nnz": int(nnz), "seed": 1, "index_bytes": ib,
-                   "column_block_passes": passes},
+                   "launches_per_step": passes},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (dom_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": alg_bytes / (dom_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "traffic": measured_traffic("spmv_csr_poisson")[0] if n == 1_000_000 else None,

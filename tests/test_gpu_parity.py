@@ -120,9 +120,13 @@ def test_spmv_poisson_shape_scaled_down():
     assert np.array_equal(got, orc.spmv(pos, crd, val, x))
 
 
-def test_spmv_column_blocked_plan_is_bit_exact():
-    # x larger than an L2: the library re-stores A in column blocks and runs one pass per block;
-    # the additions must still happen in the checker's order
+@pytest.mark.parametrize("per_block", [False, True])
+def test_spmv_column_blocked_plan_is_bit_exact(per_block, monkeypatch):
+    # x larger than an L2: the library re-stores A in column blocks and goes through them in order - in one launch
+    # with the row sums on chip, or (the switch; also what it does when one grid has no lanes for all rows) one
+    # launch per block with the sums going through y; the additions must still happen in the checker's order
+    if per_block:
+        monkeypatch.setenv("COMET_HIP_SPMV_LAUNCH_PER_BLOCK", "1")
     n = 600_000
     pos, crd, val = gen.poisson_csr(n=n, mean=4.0, seed=5)
     assert len(crd) > (1 << 20)
@@ -132,6 +136,47 @@ def test_spmv_column_blocked_plan_is_bit_exact():
     assert np.array_equal(rt.spmv(A, dx).to_numpy(), orc.spmv(pos, crd, val, x))
     assert np.array_equal(rt.spmv(A, dx, rt.DeviceArray.from_numpy(y0)).to_numpy(), orc.spmv(pos, crd, val, x, y0))
     assert np.array_equal(rt.spmv(A, dx).to_numpy(), orc.spmv(pos, crd, val, x))      # plan reused
+
+
+@pytest.mark.parametrize("n,m,mean", [(3000, 2_000_000, 400.0), (40_000, 700_000, 30.0), (1_300_000, 450_000, 1.0)])
+def test_spmv_column_blocked_plan_shapes(n, m, mean):
+    """The one-launch form deals the rows evenly to the workgroups the GPU holds at once: few rows (a part of the
+    lanes own one), rows of many nonzeros cut by the column blocks, more rows than lanes (several per lane)."""
+    rng = np.random.default_rng(n)
+    lens = rng.poisson(mean, n)
+    pos = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    crd = np.sort((rng.random(int(pos[-1])) * m).astype(np.int64) + np.repeat(np.arange(n, dtype=np.int64) * m, lens)) \
+        - np.repeat(np.arange(n, dtype=np.int64) * m, lens)       # sorted inside each row, repeats allowed
+    assert len(crd) > (1 << 20)
+    val, x, y0 = rng.uniform(-1, 1, len(crd)), rng.uniform(-1, 1, m), rng.uniform(-1, 1, n)
+    A = rt.CsrMatrix.from_arrays((n, m), pos, crd, val)
+    dx = rt.DeviceArray.from_numpy(x)
+    want = orc.spmv(pos, crd, val, x, y0)
+    got = rt.spmv(A, dx, rt.DeviceArray.from_numpy(y0)).to_numpy()
+    # a row's share of one column block has fewer than 128 products here, so every row is summed in its own order
+    assert np.array_equal(got, want)
+    assert np.array_equal(rt.spmv(A, dx).to_numpy(), orc.spmv(pos, crd, val, x))
+
+
+def test_spmv_column_blocked_plan_long_rows():
+    """Rows whose share of a column block is long (added by the whole workgroup, to rounding) next to short ones
+    (bit-exact) in a matrix that runs as column blocks, several rows per lane."""
+    rng = np.random.default_rng(23)
+    n, m = 700_000, 600_000
+    lens = rng.poisson(2.0, n)
+    for at, l in ((0, 5000), (1, 3), (2, 40_000), (255, 700), (256, 513), (300_000, 130_000), (n - 1, 2500)):
+        lens[at] = l
+    pos = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    off = np.repeat(np.arange(n, dtype=np.int64) * m, lens)
+    crd = np.sort((rng.random(int(pos[-1])) * m).astype(np.int64) + off) - off
+    val, x, y0 = rng.uniform(-1, 1, len(crd)), rng.uniform(-1, 1, m), rng.uniform(-1, 1, n)
+    A = rt.CsrMatrix.from_arrays((n, m), pos, crd, val)
+    got = rt.spmv(A, rt.DeviceArray.from_numpy(x), rt.DeviceArray.from_numpy(y0)).to_numpy()
+    want = orc.spmv(pos, crd, val, x, y0)
+    short = lens < 128
+    assert np.array_equal(got[short], want[short])
+    bound = orc.spmv(pos, crd, np.abs(val), np.abs(x), np.abs(y0))
+    assert np.all(np.abs(got - want) <= RTOL * bound)
 
 
 @pytest.mark.parametrize("acc", [False, True])
