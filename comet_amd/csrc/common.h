@@ -108,6 +108,10 @@ struct Csr {
     int32_t *entry_row = nullptr;
     // the transpose, built the first time a dense-times-sparse product needs it
     Csr *transposed = nullptr;
+    // the transpose of the structure with, as values, the place of every entry in this matrix (a mask's, for masked
+    // products taken pair by pair); dup_state: 0 not looked at, 1 no row holds a column twice, 2 some row does
+    Csr *transposed_index = nullptr;
+    int dup_state = 0;
 };
 
 Csr *csr_from_handle(int64_t h);           // nullptr (and error set) if unknown

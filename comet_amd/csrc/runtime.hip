@@ -164,7 +164,10 @@ static void csr_drop_plans(Csr *c)
         csr_release(c->light);
     if (c->transposed)
         csr_release(c->transposed);
-    c->light = c->transposed = nullptr;
+    if (c->transposed_index)
+        csr_release(c->transposed_index);
+    c->light = c->transposed = c->transposed_index = nullptr;
+    c->dup_state = 0;
     (void)hipFree(c->entry_row);
     c->entry_row = nullptr;
     (void)hipFree(c->rowmap);

@@ -1899,6 +1899,404 @@ __global__ void eltwise_mult_dense_kernel(int64_t nrows, const int64_t *__restri
 }
 
 // ------------------------------------------------------------------ host side
+// ---------------------------------------------------------------------------
+// Masked products as dot products over the mask.  C<M>[i][j] = sum over k of A[i][k] * B[k][j] is the dot product of
+// row i of A and column j of B; walking the products of row i (every entry of every B_k, k in A_i) costs |B_k|
+// look-ups per entry of A_i whatever the mask holds, the dot product of a stored pair (i, j) costs the shorter of
+// its two lists when that one is streamed against a table of the longer one.  So the pairs of the mask are split
+// by which list is longer.  One kernel serves both halves: a workgroup takes a row x of a matrix of pairs P,
+// puts the list T_x into its table, and for the pairs (x, y) of P_x that are its to do streams the list L_y
+// through the table.
+//   the row's half:     P = M,   T = A (rows),            L = B^T (columns of B);  pair (i, j) when |B^T_j| <= |A_i|
+//   the column's half:  P = M^T, T = B^T (columns of B),  L = A (rows);            pair (j, i) when |A_i| < |B^T_j|
+// The table is a bitmap over k in LDS with the number of set bits before every eighth word, so that a hit knows
+// its rank in T_x and with it where the value lies (a list in the table must not hold a column twice).  A pair's
+// products are added into a slot of LDS that belongs to the wavefront and the pair (64 pairs per wavefront at a
+// time) and leave, with the flag that says whether there was any, when the wavefront is through with its 64.
+// ---------------------------------------------------------------------------
+struct DotHit {
+    int hit;
+    double prod;
+};
+constexpr int DT_GROUP = 16;         // bitmap words per count
+constexpr int DT_WPT = 32;           // consecutive bitmap words a thread counts: SG_T * DT_WPT * 32 = 2^20 columns at most
+// The table of a list of at most SG_HASH_FILL entries is a hash table instead, key k + 1 and the value, in the same
+// LDS: nothing to count, and building and clearing it costs by the length of the list, not of the bitmap.
+// Words of LDS in front of the wavefronts' sums: the bitmap (one padding word after every 32, so that a thread's
+// 32 consecutive words lie in 32 banks) and the counts, or the hash table's keys and values, whichever is more
+constexpr int dot_bitmap_words(int words) { return words + words / 32 + words / DT_GROUP; }
+constexpr int dot_table_words(int words)
+{
+    return ((dot_bitmap_words(words) > 3 * SG_HASH_SLOTS ? dot_bitmap_words(words) : 3 * SG_HASH_SLOTS) + 1) & ~1;
+}
+constexpr size_t dot_lds_bytes(int words)
+{
+    return (size_t)dot_table_words(words) * 4 + (size_t)SG_WAVES * 64 * (8 + 4);
+}
+static_assert(dot_lds_bytes(SG_T * DT_WPT) <= 160 * 1024 - 256, "the table of 2^20 columns fits LDS");
+
+// The pairs [ms, me) of one row of P, dealt to the wavefronts like the entries of a row of A in
+// for_each_product_impl (the walk of a turn and its one-turn-late visits are the same); keep(y, len) says whether
+// a pair is this half's; f gets the pair's slot in the wavefront's batch; done(base, cnt, kept) ends a batch.
+template <typename KEEP, typename PRE, typename MID, typename F, typename DONE>
+__device__ inline void for_each_pair(int64_t ms, int64_t me, const int32_t *__restrict__ Pcrd,
+                                     const int64_t *__restrict__ Lpos, const int32_t *__restrict__ Lcrd, KEEP keep,
+                                     PRE pre, MID mid, F f, DONE done)
+{
+    using T1 = decltype(pre(0));
+    using T2 = decltype(mid(0, (int64_t)0, T1()));
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int quarter = lane >> 4, sub = lane & 15;
+    constexpr int NP = FEP_LONG_LOADS > FEP_SHORT_LOADS ? FEP_LONG_LOADS : FEP_SHORT_LOADS;
+    bool w_ok[NP];
+    int w_t[NP];
+    T2 w_md[NP];
+#pragma unroll
+    for (int x = 0; x < NP; ++x)
+        w_ok[x] = false;
+    const auto visit_pending = [&]() {
+#pragma unroll
+        for (int x = 0; x < NP; ++x)
+            if (w_ok[x])
+                f(w_t[x], w_md[x]);
+#pragma unroll
+        for (int x = 0; x < NP; ++x)
+            w_ok[x] = false;
+    };
+    const auto turn = [&](auto n_tag, const bool *ok, const int *k, const int64_t *q, int t) {
+        constexpr int N = decltype(n_tag)::value;
+        T1 tk[N];
+#pragma unroll
+        for (int x = 0; x < N; ++x)
+            tk[x] = ok[x] ? pre(k[x]) : T1();
+        visit_pending();
+#pragma unroll
+        for (int x = 0; x < N; ++x) {
+            w_ok[x] = ok[x];
+            w_t[x] = t;
+            w_md[x] = ok[x] ? mid(k[x], q[x], tk[x]) : T2();
+        }
+    };
+    for (int64_t base = ms + wave; base < me; base += (int64_t)SG_WAVES * 64) {
+        const int64_t left = (me - base + SG_WAVES - 1) / SG_WAVES;     // my pairs from here on
+        const int cnt = (int)(left < 64 ? left : 64);
+        int64_t bs = 0, be = 0;
+        bool kept = false;
+        if (lane < cnt) {
+            const int y = Pcrd[base + (int64_t)lane * SG_WAVES];
+            bs = Lpos[y];
+            be = Lpos[y + 1];
+            kept = keep(y, be - bs);
+            if (!kept)
+                be = bs;
+        }
+        unsigned long long big = __ballot(be - bs >= FEP_SHORT);
+        unsigned long long todo = __ballot(bs < be && be - bs < FEP_SHORT);
+        while (big) {
+            const int t = __builtin_ctzll(big);
+            big &= big - 1;
+            const int64_t s = readlane_i64(bs, t), len = readlane_i64(be, t) - s;
+            int64_t o = lane;
+            if (len >= 64 * FEP_LONG_LOADS) {
+                bool all[FEP_LONG_LOADS];
+                int k[FEP_LONG_LOADS];
+                int64_t q[FEP_LONG_LOADS];
+#pragma unroll
+                for (int x = 0; x < FEP_LONG_LOADS; ++x) {
+                    all[x] = true;
+                    k[x] = Lcrd[s + o + 64 * x];
+                }
+                for (int64_t full = 64 * FEP_LONG_LOADS; full + 64 * FEP_LONG_LOADS <= len;
+                     full += 64 * FEP_LONG_LOADS) {
+                    int kn[FEP_LONG_LOADS];
+#pragma unroll
+                    for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                        kn[x] = Lcrd[s + o + 64 * (FEP_LONG_LOADS + x)];
+#pragma unroll
+                    for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                        q[x] = s + o + 64 * x;
+                    turn(std::integral_constant<int, FEP_LONG_LOADS>(), all, k, q, t);
+#pragma unroll
+                    for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                        k[x] = kn[x];
+                    o += 64 * FEP_LONG_LOADS;
+                }
+#pragma unroll
+                for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                    q[x] = s + o + 64 * x;
+                turn(std::integral_constant<int, FEP_LONG_LOADS>(), all, k, q, t);
+                o += 64 * FEP_LONG_LOADS;
+            }
+            if (o < len) {
+                bool ok[FEP_LONG_LOADS];
+                int k[FEP_LONG_LOADS];
+                int64_t q[FEP_LONG_LOADS];
+#pragma unroll
+                for (int x = 0; x < FEP_LONG_LOADS; ++x) {
+                    ok[x] = o + 64 * x < len;
+                    q[x] = s + o + 64 * x;
+                }
+#pragma unroll
+                for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                    k[x] = ok[x] ? Lcrd[q[x]] : 0;
+                turn(std::integral_constant<int, FEP_LONG_LOADS>(), ok, k, q, t);
+            }
+        }
+        while (todo) {
+            int pick = -1;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int t = todo ? __builtin_ctzll(todo) : -1;
+                todo = todo ? (todo & (todo - 1)) : 0;
+                pick = quarter == g ? t : pick;
+            }
+            const int src = pick < 0 ? lane : pick;
+            const int64_t s = ((int64_t)__shfl((int)(bs >> 32), src, 64) << 32) |
+                              (uint32_t)__shfl((int)(bs & 0xffffffff), src, 64);
+            const int64_t e = ((int64_t)__shfl((int)(be >> 32), src, 64) << 32) |
+                              (uint32_t)__shfl((int)(be & 0xffffffff), src, 64);
+            bool ok[FEP_SHORT_LOADS];
+            int k[FEP_SHORT_LOADS];
+            int64_t q[FEP_SHORT_LOADS];
+#pragma unroll
+            for (int x = 0; x < FEP_SHORT_LOADS; ++x) {
+                ok[x] = pick >= 0 && s + sub + 16 * x < e;
+                q[x] = s + sub + 16 * x;
+            }
+#pragma unroll
+            for (int x = 0; x < FEP_SHORT_LOADS; ++x)
+                k[x] = ok[x] ? Lcrd[q[x]] : 0;
+            turn(std::integral_constant<int, FEP_SHORT_LOADS>(), ok, k, q, src);
+        }
+        visit_pending();
+        done(base, cnt, kept);
+    }
+}
+
+// strict: a pair is kept when its streamed list is shorter than the table's (otherwise: not longer).  [xlo, xhi):
+// the pairs' other index must lie in it (the rows of M being computed, for the column's half).  perm: where pair p
+// of P lies in the row-major order of the mask (nullptr: at p); out0 is taken off either.
+template <bool VALUES>
+__global__ __launch_bounds__(SG_T) void spgemm_dot_kernel(
+    int64_t row_begin, const int64_t *__restrict__ Tpos, const int32_t *__restrict__ Tcrd,
+    const double *__restrict__ Tval, const int64_t *__restrict__ Ppos, const int32_t *__restrict__ Pcrd,
+    const int64_t *__restrict__ Lpos, const int32_t *__restrict__ Lcrd, const double *__restrict__ Lval,
+    const double *__restrict__ perm, int64_t out0, int strict, int64_t xlo, int64_t xhi, int words,
+    unsigned long long *ticket, RowList list, double *__restrict__ pair_val, uint8_t *__restrict__ pair_hit)
+{
+    __shared__ int64_t row_slot;
+    __shared__ int wave_tot[SG_WAVES];
+    uint32_t *bm = sg_dyn_lds;
+    uint32_t *cnt_before = bm + words + words / 32;    // [words / DT_GROUP]
+    uint32_t *hkey = sg_dyn_lds;                       // [SG_HASH_SLOTS], over the bitmap
+    double *hval = reinterpret_cast<double *>(sg_dyn_lds + SG_HASH_SLOTS);        // [SG_HASH_SLOTS]
+    const int table_words = dot_table_words(words);
+    double *wacc = reinterpret_cast<double *>(sg_dyn_lds + table_words);           // [SG_WAVES][64]
+    int *whit = reinterpret_cast<int *>(wacc + SG_WAVES * 64);                     // [SG_WAVES][64]
+    const BmAddr ad{5};
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    for (int w = threadIdx.x; w < table_words; w += SG_T)
+        sg_dyn_lds[w] = 0;
+    wacc[threadIdx.x] = 0.0;
+    whit[threadIdx.x] = 0;
+    lds_barrier();
+    bool values_left = false;       // a hash table's values lie where bitmap words are: cleared before the next bitmap
+    int64_t t_first, t_end;
+    list_range(list, 2, &t_first, &t_end);
+    int64_t tk = draw_row<true>(ticket, t_first, &row_slot);
+    while (tk < t_end) {
+        const int64_t x = row_begin + list.rows[tk];
+        const int64_t ts = Tpos[x], te = Tpos[x + 1];
+        const int64_t ps = Ppos[x], pe = Ppos[x + 1];
+        const int64_t tlen = te - ts;
+        const auto keep = [&](int y, int64_t len) {
+            return len > 0 && (strict ? len < tlen : len <= tlen) && y >= xlo && y < xhi;
+        };
+        const auto add = [&](int t, DotHit h) {
+            if (h.hit) {
+                whit[wave * 64 + t] = 1;
+                if constexpr (VALUES)
+                    __hip_atomic_fetch_add(&wacc[wave * 64 + t], h.prod, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        };
+        const auto done = [&](int64_t base, int cnt, bool kept) {
+            // the slots belong to this wavefront, which has issued all its adds: LDS keeps a wavefront's order
+            if (lane < cnt && kept) {
+                const int64_t p = base + (int64_t)lane * SG_WAVES;
+                const int64_t at = (perm ? (int64_t)perm[p] : p) - out0;
+                pair_hit[at] = (uint8_t)whit[wave * 64 + lane];
+                if constexpr (VALUES)
+                    pair_val[at] = wacc[wave * 64 + lane];
+            }
+            wacc[wave * 64 + lane] = 0.0;
+            whit[wave * 64 + lane] = 0;
+        };
+        if (ts != te && ps != pe && tlen <= SG_HASH_FILL) {
+            for (int64_t t = ts + threadIdx.x; t < te; t += SG_T) {
+                const int k = Tcrd[t];
+                const uint32_t key = (uint32_t)k + 1u;
+                uint32_t sl = sg_hash_slot(k);
+                for (;;) {
+                    const uint32_t old = atomicCAS(&hkey[sl], 0u, key);
+                    if (old == 0u)
+                        break;
+                    sl = (sl + 1) & (SG_HASH_SLOTS - 1);
+                }
+                if constexpr (VALUES)
+                    hval[sl] = Tval[t];
+            }
+            values_left = VALUES;
+            lds_barrier();
+            for_each_pair(ps, pe, Pcrd, Lpos, Lcrd, keep,
+                [&](int k) { return hkey[sg_hash_slot(k)]; },
+                [&](int k, int64_t q, uint32_t k0) {
+                    DotHit h{0, 0.0};
+                    if (k0 != 0u) {
+                        uint32_t sl = sg_hash_slot(k);
+                        uint32_t key = k0;
+                        while (key != 0u && key != (uint32_t)k + 1u) {
+                            sl = (sl + 1) & (SG_HASH_SLOTS - 1);
+                            key = hkey[sl];
+                        }
+                        if (key != 0u) {
+                            h.hit = 1;
+                            if constexpr (VALUES)
+                                h.prod = hval[sl] * Lval[q];
+                        }
+                    }
+                    return h;
+                }, add, done);
+            lds_barrier();
+            for (int sl = threadIdx.x; sl < SG_HASH_SLOTS; sl += SG_T)
+                hkey[sl] = 0u;
+        } else if (ts != te && ps != pe) {
+            if (values_left) {
+                for (int w = SG_HASH_SLOTS + threadIdx.x; w < 3 * SG_HASH_SLOTS; w += SG_T)
+                    sg_dyn_lds[w] = 0;
+                values_left = false;
+                lds_barrier();
+            }
+            for (int64_t t = ts + threadIdx.x; t < te; t += SG_T) {
+                const int k = Tcrd[t];
+                atomicOr(&bm[ad.word(k)], ad.bit(k));
+            }
+            lds_barrier();
+            {   // bits before every group of words: a thread counts DT_WPT consecutive words
+                const int w0 = (int)threadIdx.x * DT_WPT;
+                int mine = 0;
+                if (w0 < words) {
+#pragma unroll
+                    for (int c = 0; c < DT_WPT; ++c)
+                        mine += __popc(bm[w0 + c + (w0 >> 5)]);
+                }
+                const int inc = wave_inclusive_scan(mine);
+                if (lane == 63)
+                    wave_tot[wave] = inc;
+                lds_barrier();
+                const int tots = wave_inclusive_scan(lane < SG_WAVES ? wave_tot[lane] : 0);
+                int run = (wave ? __builtin_amdgcn_readlane(tots, wave - 1) : 0) + inc - mine;
+                if (w0 < words) {
+#pragma unroll
+                    for (int c = 0; c < DT_WPT; ++c) {
+                        if (c % DT_GROUP == 0)
+                            cnt_before[(w0 + c) / DT_GROUP] = (uint32_t)run;
+                        run += __popc(bm[w0 + c + (w0 >> 5)]);
+                    }
+                }
+                lds_barrier();
+            }
+            for_each_pair(ps, pe, Pcrd, Lpos, Lcrd, keep,
+                [&](int k) { return bm[ad.word(k)]; },
+                [&](int k, int64_t q, uint32_t word) {
+                    DotHit h{0, 0.0};
+                    if (word & ad.bit(k)) {
+                        h.hit = 1;
+                        if constexpr (VALUES) {
+                            const int w = k >> 5, wg = w & ~(DT_GROUP - 1);
+                            int rank = (int)cnt_before[w / DT_GROUP] + __popc(word & (ad.bit(k) - 1u));
+                            for (int v = wg; v < w; ++v)
+                                rank += __popc(bm[v + (v >> 5)]);
+                            h.prod = Tval[ts + rank] * Lval[q];
+                        }
+                    }
+                    return h;
+                }, add, done);
+            lds_barrier();
+            for (int64_t t = ts + threadIdx.x; t < te; t += SG_T)
+                bm[ad.word(Tcrd[t])] = 0;
+        }
+        tk = draw_row<true>(ticket, t_first, &row_slot);      // its barriers also close this row's clean-up
+    }
+}
+
+// rowcount[i - rb] = stored pairs of mask row i that met a product
+__global__ __launch_bounds__(256) void spgemm_dot_count(int64_t rb, int64_t re, const int64_t *__restrict__ Mpos,
+                                                        const uint8_t *__restrict__ pair_hit,
+                                                        int64_t *__restrict__ rowcount)
+{
+    const int64_t i = rb + (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= re)
+        return;
+    const int lane = threadIdx.x & 63;
+    const int64_t out0 = Mpos[rb];
+    int n = 0;
+    for (int64_t p = Mpos[i] + lane; p < Mpos[i + 1]; p += 64)
+        n += pair_hit[p - out0];
+    n = wave_sum_i32(n);
+    if (lane == 0)
+        rowcount[i - rb] = n;
+}
+
+// the pairs that met a product, in the order of the mask row, to the place Cpos gives the row
+__global__ __launch_bounds__(256) void spgemm_dot_compact(int64_t rb, int64_t re, const int64_t *__restrict__ Mpos,
+                                                          const int32_t *__restrict__ Mcrd,
+                                                          const double *__restrict__ pair_val,
+                                                          const uint8_t *__restrict__ pair_hit,
+                                                          const int64_t *__restrict__ Cpos, int32_t *__restrict__ Ccrd,
+                                                          double *__restrict__ Cval)
+{
+    const int64_t i = rb + (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= re)
+        return;
+    const int lane = threadIdx.x & 63;
+    const int64_t in0 = Mpos[rb];
+    int64_t at = Cpos[i] - Cpos[rb];
+    for (int64_t base = Mpos[i]; base < Mpos[i + 1]; base += 64) {
+        const int64_t p = base + lane;
+        const bool hit = p < Mpos[i + 1] && pair_hit[p - in0];
+        const unsigned long long m = __ballot(hit);
+        if (hit) {
+            const int64_t o = at + __popcll(m & ((1ull << lane) - 1ull));
+            Ccrd[o] = Mcrd[p];
+            Cval[o] = pair_val[p - in0];
+        }
+        at += __popcll(m);
+    }
+}
+
+// flag[0] |= 1 when a row holds a column twice (rows are sorted); a wavefront per row
+__global__ __launch_bounds__(256) void csr_find_duplicates(int64_t nrows, const int64_t *__restrict__ pos,
+                                                           const int32_t *__restrict__ crd, int *__restrict__ flag)
+{
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= nrows)
+        return;
+    bool twice = false;
+    for (int64_t p = pos[r] + (threadIdx.x & 63); p + 1 < pos[r + 1]; p += 64)
+        twice = twice || crd[p] == crd[p + 1];
+    if (twice)
+        atomicOr(flag, 1);
+}
+
+__global__ void fill_iota_f64(int64_t n, double *__restrict__ out)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        out[i] = (double)i;
+}
+
 struct SgScratch {
     Workspace ticket;     // one 64-bit row counter
     Workspace rowcount;   // int64[nrows] / double[nrows]
@@ -2037,8 +2435,24 @@ static int sg_row_list(const Csr *a, const Csr *b, int64_t rb, int64_t re, int64
 
 constexpr int64_t SG_NO_DENSE = 1ll << 61;     // a threshold no row reaches: every row stays on the slab path
 
+static int dot_form_fits(const Csr *a, const Csr *b, const Csr *m, bool *fits);
+static int dot_pairs(const Csr *a, const Csr *b, const Csr *m, int64_t rb, int64_t re, bool values, double **pair_val,
+                     uint8_t **pair_hit);
+
 static int symbolic_counts(const Csr *a, const Csr *b, const Csr *m, int64_t *rowcount)
 {
+    bool dots = false;
+    COMET_CHK(dot_form_fits(a, b, m, &dots));
+    if (dots) {         // a masked product: which stored pairs of the mask meet a product
+        double *pair_val = nullptr;
+        uint8_t *pair_hit = nullptr;
+        COMET_CHK(dot_pairs(a, b, m, 0, a->nrows, false, &pair_val, &pair_hit));
+        KernelTimer t("spgemm_dot_count");
+        spgemm_dot_count<<<dim3((unsigned)ceil_div(a->nrows, 4)), dim3(256), 0, stream()>>>(0, a->nrows, m->pos, pair_hit,
+                                                                                            rowcount);
+        COMET_HIPCHK(hipGetLastError());
+        return COMET_HIP_OK;
+    }
     SgGeom g;
     COMET_CHK(sg_geometry(b->ncols, &g));
     COMET_CHK(sg_reset_ticket());
@@ -2110,12 +2524,154 @@ static int sg_plan_blocks(Csr *b)
     return COMET_HIP_OK;
 }
 
+// ---- masked products as dot products over the mask: the host side ----
+static Workspace g_dot_val, g_dot_hit, g_dot_flag;
+
+static int dot_transposed(const Csr *x, Csr **out)
+{
+    Csr *m = const_cast<Csr *>(x);           // what is kept in a handle is not part of the matrix
+    if (!m->transposed) {
+        m->transposed = csr_transposed_copy(m);
+        if (!m->transposed)
+            return COMET_HIP_ERR_HIP;
+    }
+    *out = m->transposed;
+    return COMET_HIP_OK;
+}
+
+// the transpose of the structure of x whose values say where each entry lies in x
+static int dot_transposed_index(const Csr *x, Csr **out)
+{
+    Csr *m = const_cast<Csr *>(x);
+    if (!m->transposed_index) {
+        double *iota = nullptr;
+        COMET_HIPCHK(hipMalloc((void **)&iota, sizeof(double) * (size_t)(m->nnz > 0 ? m->nnz : 1)));
+        if (m->nnz > 0)
+            fill_iota_f64<<<dim3((unsigned)ceil_div(m->nnz, 256)), dim3(256), 0, stream()>>>(m->nnz, iota);
+        Csr view;
+        view.nrows = m->nrows;
+        view.ncols = m->ncols;
+        view.nnz = m->nnz;
+        view.pos = m->pos;
+        view.crd = m->crd;
+        view.val = iota;
+        m->transposed_index = csr_transposed_copy(&view);
+        const hipError_t e = hipStreamSynchronize(stream());
+        (void)hipFree(iota);
+        if (!m->transposed_index || e != hipSuccess)
+            return set_error(COMET_HIP_ERR_HIP, "transposing the mask failed");
+    }
+    *out = m->transposed_index;
+    return COMET_HIP_OK;
+}
+
+// whether no row of x holds a column twice (looked at once per matrix)
+static int dot_no_duplicates(const Csr *x, bool *ok)
+{
+    Csr *m = const_cast<Csr *>(x);
+    if (m->dup_state == 0) {
+        COMET_CHK(g_dot_flag.ensure(sizeof(int), false));
+        COMET_HIPCHK(hipMemsetAsync(g_dot_flag.ptr, 0, sizeof(int), stream()));
+        if (m->nrows > 0)
+            csr_find_duplicates<<<dim3((unsigned)ceil_div(m->nrows, 4)), dim3(256), 0, stream()>>>(m->nrows, m->pos, m->crd,
+                                                                                                   (int *)g_dot_flag.ptr);
+        int flag = 0;
+        COMET_HIPCHK(hipMemcpyAsync(&flag, g_dot_flag.ptr, sizeof(int), hipMemcpyDeviceToHost, stream()));
+        COMET_HIPCHK(hipStreamSynchronize(stream()));
+        m->dup_state = flag ? 2 : 1;
+    }
+    *ok = m->dup_state == 1;
+    return COMET_HIP_OK;
+}
+
+// A masked product runs as dot products when the table over k fits LDS and no list that goes into a table holds a
+// column twice.  COMET_HIP_SPGEMM_NO_DOT keeps the walk over the products of every row (the tests run both).
+static int dot_form_fits(const Csr *a, const Csr *b, const Csr *m, bool *fits)
+{
+    *fits = false;
+    if (!m || a->ncols > (1ll << 20) || a->nrows >= (1ll << 31) || b->ncols >= (1ll << 31) || m->nnz >= (1ll << 52) ||
+        getenv("COMET_HIP_SPGEMM_NO_DOT") != nullptr)
+        return COMET_HIP_OK;
+    bool ok_a = false, ok_b = false, ok_m = false;
+    COMET_CHK(dot_no_duplicates(a, &ok_a));
+    COMET_CHK(dot_no_duplicates(b, &ok_b));
+    COMET_CHK(dot_no_duplicates(m, &ok_m));
+    *fits = ok_a && ok_b && ok_m;
+    return COMET_HIP_OK;
+}
+
+// pair_hit[p - Mpos[rb]] (and pair_val, with values) for every stored pair p of the mask rows [rb, re)
+static int dot_pairs(const Csr *a, const Csr *b, const Csr *m, int64_t rb, int64_t re, bool values, double **pair_val,
+                     uint8_t **pair_hit)
+{
+    Csr *bt = nullptr, *mt = nullptr;
+    COMET_CHK(dot_transposed(b, &bt));
+    COMET_CHK(dot_transposed_index(m, &mt));
+    int64_t ends[2] = {0, 0};
+    COMET_HIPCHK(hipMemcpyAsync(&ends[0], m->pos + rb, sizeof(int64_t), hipMemcpyDeviceToHost, stream()));
+    COMET_HIPCHK(hipMemcpyAsync(&ends[1], m->pos + re, sizeof(int64_t), hipMemcpyDeviceToHost, stream()));
+    COMET_HIPCHK(hipStreamSynchronize(stream()));
+    const int64_t out0 = ends[0], npairs = ends[1] - ends[0];
+    COMET_CHK(g_dot_hit.ensure((size_t)(npairs > 0 ? npairs : 1), false));
+    COMET_CHK(g_dot_val.ensure(sizeof(double) * (size_t)(npairs > 0 ? npairs : 1), false));
+    *pair_hit = (uint8_t *)g_dot_hit.ptr;
+    *pair_val = (double *)g_dot_val.ptr;
+    if (npairs == 0)
+        return COMET_HIP_OK;
+    COMET_HIPCHK(hipMemsetAsync(*pair_hit, 0, (size_t)npairs, stream()));
+    if (values)
+        COMET_HIPCHK(hipMemsetAsync(*pair_val, 0, sizeof(double) * (size_t)npairs, stream()));
+    int words = (int)ceil_div(a->ncols > 0 ? a->ncols : 1, 32);
+    words = (int)ceil_div(words, DT_WPT) * DT_WPT;
+    const size_t lds = dot_lds_bytes(words);
+    const dim3 grid((unsigned)(num_cus() > 0 ? num_cus() : 256)), block(SG_T);
+    const int64_t everywhere = 1ll << 62;
+    for (int half = 0; half < 2; ++half) {
+        // the row's half: tables of the rows of A, the columns of B streamed; the column's half the other way round
+        const Csr *T = half == 0 ? a : bt, *P = half == 0 ? m : mt, *L = half == 0 ? bt : a;
+        const int64_t first = half == 0 ? rb : 0, last = half == 0 ? re : mt->nrows;
+        RowList list;
+        COMET_CHK(sg_row_list(P, L, first, last, SG_NO_DENSE, SG_NO_DENSE, &list));
+        COMET_CHK(sg_reset_ticket());
+        KernelTimer t(half == 0 ? "spgemm_dot_rows" : "spgemm_dot_columns");
+        if (values) {
+            COMET_CHK(sg_allow_lds(spgemm_dot_kernel<true>, lds));
+            spgemm_dot_kernel<true><<<grid, block, lds, stream()>>>(
+                first, T->pos, T->crd, T->val, P->pos, P->crd, L->pos, L->crd, L->val, half == 0 ? nullptr : mt->val, out0,
+                half, half == 0 ? 0 : rb, half == 0 ? everywhere : re, words, (unsigned long long *)g_sg.ticket.ptr, list,
+                *pair_val, *pair_hit);
+        } else {
+            COMET_CHK(sg_allow_lds(spgemm_dot_kernel<false>, lds));
+            spgemm_dot_kernel<false><<<grid, block, lds, stream()>>>(
+                first, T->pos, T->crd, T->val, P->pos, P->crd, L->pos, L->crd, L->val, half == 0 ? nullptr : mt->val, out0,
+                half, half == 0 ? 0 : rb, half == 0 ? everywhere : re, words, (unsigned long long *)g_sg.ticket.ptr, list,
+                *pair_val, *pair_hit);
+        }
+        COMET_HIPCHK(hipGetLastError());
+    }
+    return COMET_HIP_OK;
+}
+
 static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos, int64_t rb, int64_t re,
                         int32_t *Ccrd, double *Cval, int reduce_op, int mult_op)
 {
     if (reduce_op < 0 || reduce_op > COMET_SR_ANY || mult_op < 0 || mult_op > COMET_OP_DIV)
         return set_error(COMET_HIP_ERR_ARG, "unknown semiring (reduce %d, mult %d)", reduce_op, mult_op);
     const bool semi = reduce_op != COMET_SR_PLUS || mult_op != COMET_OP_TIMES;
+    if (m && !semi && re > rb) {
+        bool dots = false;
+        COMET_CHK(dot_form_fits(a, b, m, &dots));
+        if (dots) {
+            double *pair_val = nullptr;
+            uint8_t *pair_hit = nullptr;
+            COMET_CHK(dot_pairs(a, b, m, rb, re, true, &pair_val, &pair_hit));
+            KernelTimer t("spgemm_dot_compact");
+            spgemm_dot_compact<<<dim3((unsigned)ceil_div(re - rb, 4)), dim3(256), 0, stream()>>>(
+                rb, re, m->pos, m->crd, pair_val, pair_hit, Cpos, Ccrd, Cval);
+            COMET_HIPCHK(hipGetLastError());
+            return COMET_HIP_OK;
+        }
+    }
     SgGeom g;
     COMET_CHK(sg_geometry(b->ncols, &g));
     COMET_CHK(sg_reset_ticket());

@@ -456,12 +456,70 @@ def test_spgemm_vs_checker(n, k, m, density, seed, signed):
     _spgemm_check(a, b, m)
 
 
+@pytest.mark.parametrize("dot", [True, False])
 @pytest.mark.parametrize("seed", [0, 1])
-def test_spgemm_masked_vs_checker(seed):
+def test_spgemm_masked_vs_checker(seed, dot, monkeypatch):
+    # a masked product is taken pair by pair of the mask (dot products) or, with the switch, row by row of A
+    if not dot:
+        monkeypatch.setenv("COMET_HIP_SPGEMM_NO_DOT", "1")
     rng = np.random.default_rng(seed)
     a = _rand_csr(rng, 400, 400, 0.04, signed=False)
     mk = _rand_csr(rng, 400, 400, 0.1, signed=False)
     _spgemm_check(a, a, 400, mask=(mk[0], mk[1]))
+
+
+@pytest.mark.parametrize("n,k,m,da,db,dm,seed", [(500, 300, 700, 0.05, 0.04, 0.08, 0), (64, 5000, 64, 0.3, 0.3, 0.9, 1),
+                                                 (3000, 33, 2000, 0.2, 0.1, 0.01, 2), (200, 40_000, 300, 0.01, 0.002, 0.5, 3),
+                                                 (50, 70, (1 << 20) + 999, 0.3, 0.00001, 0.00002, 4)])
+def test_spgemm_masked_dot_products(n, k, m, da, db, dm, seed):
+    """C<M> = A*B with three different rectangular matrices: rows of A against columns of B pair by pair of the mask,
+    the shorter list of a pair streamed against a table of the longer; whole and in row blocks; empty rows and
+    columns; an inner dimension that is no multiple of 32; more than 2^20 columns of B."""
+    rng = np.random.default_rng(100 + seed)
+    a = _rand_csr(rng, n, k, da, signed=True)
+    b = _rand_csr(rng, k, m, db, signed=True)
+    mk = _rand_csr(rng, n, m, dm, signed=False)
+    _spgemm_check(a, b, m, mask=(mk[0], mk[1]))
+    A = rt.CsrMatrix.from_arrays((n, k), *a)
+    B = rt.CsrMatrix.from_arrays((k, m), *b)
+    Mk = rt.CsrMatrix.from_arrays((n, m), mk[0], mk[1], np.ones(len(mk[1])))
+    dpos, nnz = rt.spgemm_symbolic(A, B, mask=Mk)
+    hp = dpos.to_numpy()
+    wp, wc, wv = orc.spgemm(*a, *b, m, mask=(mk[0], mk[1]))
+    _, _, bound = orc.spgemm(a[0], a[1], np.abs(a[2]), b[0], b[1], np.abs(b[2]), m, mask=(mk[0], mk[1]))
+    assert np.array_equal(hp, wp) and nnz == wp[-1]
+    for rb, re in ((0, n // 3), (n // 3, n // 3 + 1), (n // 3 + 1, n)):
+        cnt = int(hp[re] - hp[rb])
+        dc, dv = rt.DeviceArray(max(cnt, 1), np.int32), rt.DeviceArray(max(cnt, 1))
+        rt.spgemm_numeric(A, B, dpos, rb, re, dc, dv, mask=Mk)
+        assert np.array_equal(dc.to_numpy(cnt), wc[hp[rb]:hp[re]])
+        assert np.all(np.abs(dv.to_numpy(cnt) - wv[hp[rb]:hp[re]]) <= RTOL * bound[hp[rb]:hp[re]])
+
+
+def test_spgemm_masked_dot_products_hubs_and_repeats():
+    """Lists of very different lengths (a few rows of A and columns of B with thousands of entries among short ones:
+    each half of the pairs has work), and a matrix that holds a column twice in a row, which the tables cannot
+    take: that product is walked row by row as before."""
+    rng = np.random.default_rng(41)
+    n = k = m = 6000
+    la = rng.integers(0, 12, n); la[rng.choice(n, 8, replace=False)] = 4000
+    lb = rng.integers(0, 12, k); lb[rng.choice(k, 8, replace=False)] = 3000
+    a = _rows_of_lengths(rng, la, k)
+    bt = _rows_of_lengths(rng, lb, k)                    # rows here = columns of B: transpose on the host
+    rows_b = np.repeat(np.arange(m), lb)
+    order = np.lexsort((rows_b, bt[1]))
+    bpos = np.concatenate([[0], np.cumsum(np.bincount(bt[1], minlength=k))]).astype(np.int64)
+    b = (bpos, rows_b[order].astype(np.int64), bt[2][order])
+    lm = rng.integers(0, 40, n); lm[rng.choice(n, 5, replace=False)] = 5000
+    mk = _rows_of_lengths(rng, lm, m)
+    _spgemm_check(a, b, m, mask=(mk[0], mk[1]))
+    # the same product with an entry of A stored twice
+    apos, acrd, aval = a
+    r = int(np.argmax(la))
+    at = int(apos[r]) + 5
+    acrd2 = np.insert(acrd, at, acrd[at]); aval2 = np.insert(aval, at, 0.5)
+    apos2 = apos.copy(); apos2[r + 1:] += 1
+    _spgemm_check((apos2, acrd2, aval2), b, m, mask=(mk[0], mk[1]))
 
 
 def test_spgemm_wide_matrix_uses_global_bitmap():
@@ -576,11 +634,15 @@ def test_spgemm_semiring_rows_of_every_class(semiring, m, long_len, wide, monkey
     assert np.array_equal(c, wc) and np.all(np.abs(v - pv) <= RTOL * bound)
 
 
-@pytest.mark.parametrize("semiring", [None, ("min", "plus"), ("any", "first")])
-def test_spgemm_masked_long_mask_rows(semiring):
+@pytest.mark.parametrize("semiring", [None, "rows", ("min", "plus"), ("any", "first")])
+def test_spgemm_masked_long_mask_rows(semiring, monkeypatch):
     # mask rows of 0, 5, 6144 (the longest the hash table of the slab kernel takes), 6145, 20,000 and 70,000
     # entries: the long ones take the one-block kernel, which adds every product and drops the columns outside
     # the mask when a block is written out; the row pointers come from the masked symbolic phase
+    # (plus-times goes pair by pair of the mask unless told otherwise: "rows" is that product walked row by row)
+    if semiring == "rows":
+        monkeypatch.setenv("COMET_HIP_SPGEMM_NO_DOT", "1")
+        semiring = None
     rng = np.random.default_rng(31)
     k, m = 300, 100_000
     bpos, bcrd, bval = _rows_of_lengths(rng, [3000] * 200 + [10] * 100, m, signed=False)
