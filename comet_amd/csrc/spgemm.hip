@@ -944,21 +944,28 @@ constexpr size_t SG_DENSE_LDS = (size_t)SG_CB * 8 + (size_t)SG_CB / 8 + (size_t)
                                 2 * (size_t)SG_CB / 8;               // accumulators, bitmap, list of the columns being
                                                                       // written out, the mask row's bits (two blocks)
 
-// products[i - row_begin] = sum over k in A_i of nnz(B_k); one wavefront per row
+// products[i - row_begin] = sum over k in A_i of nnz(B_k); one wavefront per row.  With Tpos (the dot-product form of
+// a masked product, where row i's pairs k are shared out by which of the two lists is longer) only the k whose row
+// of B is shorter than row i of T (strict) or not longer (otherwise), and that lie in [xlo, xhi), count.
 __global__ __launch_bounds__(256) void spgemm_row_products(int64_t row_begin, int64_t row_end,
                                                            const int64_t *__restrict__ Apos,
                                                            const int32_t *__restrict__ Acrd,
                                                            const int64_t *__restrict__ Bpos,
-                                                           int64_t *__restrict__ products)
+                                                           int64_t *__restrict__ products,
+                                                           const int64_t *__restrict__ Tpos = nullptr, int strict = 0,
+                                                           int64_t xlo = 0, int64_t xhi = 0)
 {
     const int64_t i = row_begin + (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (i >= row_end)
         return;
     const int lane = threadIdx.x & 63;
+    const int64_t tlen = Tpos ? Tpos[i + 1] - Tpos[i] : 0;
     int64_t s = 0;
     for (int64_t p = Apos[i] + lane; p < Apos[i + 1]; p += 64) {
         const int k = Acrd[p];
-        s += Bpos[k + 1] - Bpos[k];
+        const int64_t len = Bpos[k + 1] - Bpos[k];
+        if (!Tpos || ((strict ? len < tlen : len <= tlen) && k >= xlo && k < xhi))
+            s += len;
     }
     for (int d = 32; d > 0; d >>= 1)
         s += __shfl_down(s, d, 64);
@@ -1938,13 +1945,19 @@ static_assert(dot_lds_bytes(SG_T * DT_WPT) <= 160 * 1024 - 256, "the table of 2^
 // The pairs [ms, me) of one row of P, dealt to the wavefronts like the entries of a row of A in
 // for_each_product_impl (the walk of a turn and its one-turn-late visits are the same); keep(y, len) says whether
 // a pair is this half's; f gets the pair's slot in the wavefront's batch; done(base, cnt, kept) ends a batch.
-template <typename KEEP, typename PRE, typename MID, typename F, typename DONE>
+// With VALUES the entries' values are loaded with their columns and handed to mid: in these products a fifth of the
+// look-ups hit, so nearly every cache line of the values is needed anyway, and fetched only for the hits they would
+// be a second trip to memory behind the first.
+// Without VALUES only whether a pair meets a product is asked, and decided(t) says that pair t of the wavefront's
+// batch already has: the rest of its list is then left out (a long list is through after a turn or two).
+template <bool VALUES, typename KEEP, typename PRE, typename MID, typename F, typename DONE, typename DECIDED>
 __device__ inline void for_each_pair(int64_t ms, int64_t me, const int32_t *__restrict__ Pcrd,
-                                     const int64_t *__restrict__ Lpos, const int32_t *__restrict__ Lcrd, KEEP keep,
-                                     PRE pre, MID mid, F f, DONE done)
+                                     const int64_t *__restrict__ Lpos, const int32_t *__restrict__ Lcrd,
+                                     const double *__restrict__ Lval, KEEP keep, PRE pre, MID mid, F f, DONE done,
+                                     DECIDED decided)
 {
     using T1 = decltype(pre(0));
-    using T2 = decltype(mid(0, (int64_t)0, T1()));
+    using T2 = decltype(mid(0, 0.0, T1()));
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int quarter = lane >> 4, sub = lane & 15;
@@ -1964,7 +1977,7 @@ __device__ inline void for_each_pair(int64_t ms, int64_t me, const int32_t *__re
         for (int x = 0; x < NP; ++x)
             w_ok[x] = false;
     };
-    const auto turn = [&](auto n_tag, const bool *ok, const int *k, const int64_t *q, int t) {
+    const auto turn = [&](auto n_tag, const bool *ok, const int *k, const double *v, int t) {
         constexpr int N = decltype(n_tag)::value;
         T1 tk[N];
 #pragma unroll
@@ -1975,7 +1988,7 @@ __device__ inline void for_each_pair(int64_t ms, int64_t me, const int32_t *__re
         for (int x = 0; x < N; ++x) {
             w_ok[x] = ok[x];
             w_t[x] = t;
-            w_md[x] = ok[x] ? mid(k[x], q[x], tk[x]) : T2();
+            w_md[x] = ok[x] ? mid(k[x], v[x], tk[x]) : T2();
         }
     };
     for (int64_t base = ms + wave; base < me; base += (int64_t)SG_WAVES * 64) {
@@ -2001,46 +2014,54 @@ __device__ inline void for_each_pair(int64_t ms, int64_t me, const int32_t *__re
             if (len >= 64 * FEP_LONG_LOADS) {
                 bool all[FEP_LONG_LOADS];
                 int k[FEP_LONG_LOADS];
-                int64_t q[FEP_LONG_LOADS];
+                double v[FEP_LONG_LOADS];
 #pragma unroll
                 for (int x = 0; x < FEP_LONG_LOADS; ++x) {
                     all[x] = true;
                     k[x] = Lcrd[s + o + 64 * x];
+                    v[x] = VALUES ? Lval[s + o + 64 * x] : 0.0;
                 }
+                bool enough = false;
                 for (int64_t full = 64 * FEP_LONG_LOADS; full + 64 * FEP_LONG_LOADS <= len;
                      full += 64 * FEP_LONG_LOADS) {
+                    if (!VALUES && decided(t)) {        // what earlier turns found (a turn's visits come one turn late)
+                        enough = true;
+                        break;
+                    }
                     int kn[FEP_LONG_LOADS];
+                    double vn[FEP_LONG_LOADS];
 #pragma unroll
-                    for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                    for (int x = 0; x < FEP_LONG_LOADS; ++x) {
                         kn[x] = Lcrd[s + o + 64 * (FEP_LONG_LOADS + x)];
+                        vn[x] = VALUES ? Lval[s + o + 64 * (FEP_LONG_LOADS + x)] : 0.0;
+                    }
+                    turn(std::integral_constant<int, FEP_LONG_LOADS>(), all, k, v, t);
 #pragma unroll
-                    for (int x = 0; x < FEP_LONG_LOADS; ++x)
-                        q[x] = s + o + 64 * x;
-                    turn(std::integral_constant<int, FEP_LONG_LOADS>(), all, k, q, t);
-#pragma unroll
-                    for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                    for (int x = 0; x < FEP_LONG_LOADS; ++x) {
                         k[x] = kn[x];
+                        v[x] = vn[x];
+                    }
                     o += 64 * FEP_LONG_LOADS;
                 }
-#pragma unroll
-                for (int x = 0; x < FEP_LONG_LOADS; ++x)
-                    q[x] = s + o + 64 * x;
-                turn(std::integral_constant<int, FEP_LONG_LOADS>(), all, k, q, t);
+                turn(std::integral_constant<int, FEP_LONG_LOADS>(), all, k, v, t);
                 o += 64 * FEP_LONG_LOADS;
+                if (enough)
+                    o = len;
             }
-            if (o < len) {
+            if (o < len && (VALUES || !decided(t))) {
                 bool ok[FEP_LONG_LOADS];
                 int k[FEP_LONG_LOADS];
-                int64_t q[FEP_LONG_LOADS];
-#pragma unroll
-                for (int x = 0; x < FEP_LONG_LOADS; ++x) {
-                    ok[x] = o + 64 * x < len;
-                    q[x] = s + o + 64 * x;
-                }
+                double v[FEP_LONG_LOADS];
 #pragma unroll
                 for (int x = 0; x < FEP_LONG_LOADS; ++x)
-                    k[x] = ok[x] ? Lcrd[q[x]] : 0;
-                turn(std::integral_constant<int, FEP_LONG_LOADS>(), ok, k, q, t);
+                    ok[x] = o + 64 * x < len;
+#pragma unroll
+                for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                    k[x] = ok[x] ? Lcrd[s + o + 64 * x] : 0;
+#pragma unroll
+                for (int x = 0; x < FEP_LONG_LOADS; ++x)
+                    v[x] = VALUES && ok[x] ? Lval[s + o + 64 * x] : 0.0;
+                turn(std::integral_constant<int, FEP_LONG_LOADS>(), ok, k, v, t);
             }
         }
         while (todo) {
@@ -2058,16 +2079,17 @@ __device__ inline void for_each_pair(int64_t ms, int64_t me, const int32_t *__re
                               (uint32_t)__shfl((int)(be & 0xffffffff), src, 64);
             bool ok[FEP_SHORT_LOADS];
             int k[FEP_SHORT_LOADS];
-            int64_t q[FEP_SHORT_LOADS];
-#pragma unroll
-            for (int x = 0; x < FEP_SHORT_LOADS; ++x) {
-                ok[x] = pick >= 0 && s + sub + 16 * x < e;
-                q[x] = s + sub + 16 * x;
-            }
+            double v[FEP_SHORT_LOADS];
 #pragma unroll
             for (int x = 0; x < FEP_SHORT_LOADS; ++x)
-                k[x] = ok[x] ? Lcrd[q[x]] : 0;
-            turn(std::integral_constant<int, FEP_SHORT_LOADS>(), ok, k, q, src);
+                ok[x] = pick >= 0 && s + sub + 16 * x < e;
+#pragma unroll
+            for (int x = 0; x < FEP_SHORT_LOADS; ++x)
+                k[x] = ok[x] ? Lcrd[s + sub + 16 * x] : 0;
+#pragma unroll
+            for (int x = 0; x < FEP_SHORT_LOADS; ++x)
+                v[x] = VALUES && ok[x] ? Lval[s + sub + 16 * x] : 0.0;
+            turn(std::integral_constant<int, FEP_SHORT_LOADS>(), ok, k, v, src);
         }
         visit_pending();
         done(base, cnt, kept);
@@ -2121,6 +2143,8 @@ __global__ __launch_bounds__(SG_T) void spgemm_dot_kernel(
                     __hip_atomic_fetch_add(&wacc[wave * 64 + t], h.prod, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
         };
+        // (uniform: t is; a wavefront's own LDS operations keep their order)
+        const auto decided = [&](int t) { return __builtin_amdgcn_readfirstlane(whit[wave * 64 + t]) != 0; };
         const auto done = [&](int64_t base, int cnt, bool kept) {
             // the slots belong to this wavefront, which has issued all its adds: LDS keeps a wavefront's order
             if (lane < cnt && kept) {
@@ -2149,9 +2173,9 @@ __global__ __launch_bounds__(SG_T) void spgemm_dot_kernel(
             }
             values_left = VALUES;
             lds_barrier();
-            for_each_pair(ps, pe, Pcrd, Lpos, Lcrd, keep,
+            for_each_pair<VALUES>(ps, pe, Pcrd, Lpos, Lcrd, Lval, keep,
                 [&](int k) { return hkey[sg_hash_slot(k)]; },
-                [&](int k, int64_t q, uint32_t k0) {
+                [&](int k, double lv, uint32_t k0) {
                     DotHit h{0, 0.0};
                     if (k0 != 0u) {
                         uint32_t sl = sg_hash_slot(k);
@@ -2163,11 +2187,11 @@ __global__ __launch_bounds__(SG_T) void spgemm_dot_kernel(
                         if (key != 0u) {
                             h.hit = 1;
                             if constexpr (VALUES)
-                                h.prod = hval[sl] * Lval[q];
+                                h.prod = hval[sl] * lv;
                         }
                     }
                     return h;
-                }, add, done);
+                }, add, done, decided);
             lds_barrier();
             for (int sl = threadIdx.x; sl < SG_HASH_SLOTS; sl += SG_T)
                 hkey[sl] = 0u;
@@ -2207,9 +2231,9 @@ __global__ __launch_bounds__(SG_T) void spgemm_dot_kernel(
                 }
                 lds_barrier();
             }
-            for_each_pair(ps, pe, Pcrd, Lpos, Lcrd, keep,
+            for_each_pair<VALUES>(ps, pe, Pcrd, Lpos, Lcrd, Lval, keep,
                 [&](int k) { return bm[ad.word(k)]; },
-                [&](int k, int64_t q, uint32_t word) {
+                [&](int k, double lv, uint32_t word) {
                     DotHit h{0, 0.0};
                     if (word & ad.bit(k)) {
                         h.hit = 1;
@@ -2218,11 +2242,11 @@ __global__ __launch_bounds__(SG_T) void spgemm_dot_kernel(
                             int rank = (int)cnt_before[w / DT_GROUP] + __popc(word & (ad.bit(k) - 1u));
                             for (int v = wg; v < w; ++v)
                                 rank += __popc(bm[v + (v >> 5)]);
-                            h.prod = Tval[ts + rank] * Lval[q];
+                            h.prod = Tval[ts + rank] * lv;
                         }
                     }
                     return h;
-                }, add, done);
+                }, add, done, decided);
             lds_barrier();
             for (int64_t t = ts + threadIdx.x; t < te; t += SG_T)
                 bm[ad.word(Tcrd[t])] = 0;
@@ -2402,9 +2426,14 @@ struct SgRowLists {
 static SgRowLists g_rl;
 
 // Products per row of rows [rb, re) of A*B and the list of those rows by descending products.
+struct SgPairFilter {          // see spgemm_row_products
+    const int64_t *tpos = nullptr;
+    int strict = 0;
+    int64_t xlo = 0, xhi = 0;
+};
 static int sg_row_list(const Csr *a, const Csr *b, int64_t rb, int64_t re, int64_t dense_threshold,
                        int64_t wide_threshold, RowList *out, const int64_t *long_mask_pos = nullptr,
-                       int64_t mask_fill = 0)
+                       int64_t mask_fill = 0, SgPairFilter filter = SgPairFilter())
 {
     const int64_t n = re - rb;
     COMET_CHK(g_rl.rowprod.ensure(sizeof(int64_t) * (size_t)n, false));
@@ -2416,8 +2445,8 @@ static int sg_row_list(const Csr *a, const Csr *b, int64_t rb, int64_t re, int64
     int64_t *rowprod = (int64_t *)g_rl.rowprod.ptr;
     {
         KernelTimer t("spgemm_row_products");
-        spgemm_row_products<<<dim3((unsigned)ceil_div(n, 4)), dim3(256), 0, stream()>>>(rb, re, a->pos, a->crd, b->pos,
-                                                                                        rowprod);
+        spgemm_row_products<<<dim3((unsigned)ceil_div(n, 4)), dim3(256), 0, stream()>>>(
+            rb, re, a->pos, a->crd, b->pos, rowprod, filter.tpos, filter.strict, filter.xlo, filter.xhi);
         sg_row_keys<<<dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, stream()>>>(
             n, rowprod, long_mask_pos ? long_mask_pos + rb : nullptr, mask_fill, (uint64_t *)g_rl.keys_in.ptr,
             (uint32_t *)g_rl.idx_in.ptr);
@@ -2630,8 +2659,13 @@ static int dot_pairs(const Csr *a, const Csr *b, const Csr *m, int64_t rb, int64
         // the row's half: tables of the rows of A, the columns of B streamed; the column's half the other way round
         const Csr *T = half == 0 ? a : bt, *P = half == 0 ? m : mt, *L = half == 0 ? bt : a;
         const int64_t first = half == 0 ? rb : 0, last = half == 0 ? re : mt->nrows;
-        RowList list;
-        COMET_CHK(sg_row_list(P, L, first, last, SG_NO_DENSE, SG_NO_DENSE, &list));
+        RowList list;        // the rows that have pairs of this half, by the entries these stream
+        SgPairFilter mine;
+        mine.tpos = T->pos;
+        mine.strict = half;
+        mine.xlo = half == 0 ? 0 : rb;
+        mine.xhi = half == 0 ? everywhere : re;
+        COMET_CHK(sg_row_list(P, L, first, last, SG_NO_DENSE, SG_NO_DENSE, &list, nullptr, 0, mine));
         COMET_CHK(sg_reset_ticket());
         KernelTimer t(half == 0 ? "spgemm_dot_rows" : "spgemm_dot_columns");
         if (values) {
