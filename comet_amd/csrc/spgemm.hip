@@ -2476,7 +2476,7 @@ static int symbolic_counts(const Csr *a, const Csr *b, const Csr *m, int64_t *ro
         double *pair_val = nullptr;
         uint8_t *pair_hit = nullptr;
         COMET_CHK(dot_pairs(a, b, m, 0, a->nrows, false, &pair_val, &pair_hit));
-        KernelTimer t("spgemm_dot_count");
+        KernelTimer t("spgemm_symbolic_dot_count");
         spgemm_dot_count<<<dim3((unsigned)ceil_div(a->nrows, 4)), dim3(256), 0, stream()>>>(0, a->nrows, m->pos, pair_hit,
                                                                                             rowcount);
         COMET_HIPCHK(hipGetLastError());
@@ -2667,7 +2667,8 @@ static int dot_pairs(const Csr *a, const Csr *b, const Csr *m, int64_t rb, int64
         mine.xhi = half == 0 ? everywhere : re;
         COMET_CHK(sg_row_list(P, L, first, last, SG_NO_DENSE, SG_NO_DENSE, &list, nullptr, 0, mine));
         COMET_CHK(sg_reset_ticket());
-        KernelTimer t(half == 0 ? "spgemm_dot_rows" : "spgemm_dot_columns");
+        KernelTimer t(values ? (half == 0 ? "spgemm_numeric_dot_rows" : "spgemm_numeric_dot_columns")
+                             : (half == 0 ? "spgemm_symbolic_dot_rows" : "spgemm_symbolic_dot_columns"));
         if (values) {
             COMET_CHK(sg_allow_lds(spgemm_dot_kernel<true>, lds));
             spgemm_dot_kernel<true><<<grid, block, lds, stream()>>>(
@@ -2699,7 +2700,7 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
             double *pair_val = nullptr;
             uint8_t *pair_hit = nullptr;
             COMET_CHK(dot_pairs(a, b, m, rb, re, true, &pair_val, &pair_hit));
-            KernelTimer t("spgemm_dot_compact");
+            KernelTimer t("spgemm_numeric_dot_compact");
             spgemm_dot_compact<<<dim3((unsigned)ceil_div(re - rb, 4)), dim3(256), 0, stream()>>>(
                 rb, re, m->pos, m->crd, pair_val, pair_hit, Cpos, Ccrd, Cval);
             COMET_HIPCHK(hipGetLastError());
