@@ -2858,6 +2858,57 @@ extern "C" int64_t comet_hip_spgemm_csr(int64_t ah, int64_t bh, int64_t mh)
     return comet_hip_spgemm_csr_semiring(ah, bh, mh, COMET_SR_PLUS, COMET_OP_TIMES);
 }
 
+// C<M> = A*B in one pass over the pairs of the mask: their values and which of them met a product come out of
+// the same walk, so the row pointers need no symbolic phase of their own.  *done says whether this form applied.
+static int64_t masked_product_one_pass(const Csr *a, const Csr *b, const Csr *m, bool *done)
+{
+    *done = false;
+    bool dots = false;
+    if (dot_form_fits(a, b, m, &dots) != COMET_HIP_OK)
+        return 0;
+    if (!dots || a->nrows == 0)
+        return 0;
+    *done = true;
+    double *pair_val = nullptr;
+    uint8_t *pair_hit = nullptr;
+    if (dot_pairs(a, b, m, 0, a->nrows, true, &pair_val, &pair_hit) != COMET_HIP_OK ||
+        g_sg.rowcount.ensure(sizeof(int64_t) * (size_t)a->nrows, false) != COMET_HIP_OK)
+        return 0;
+    Csr *c = new Csr();
+    c->nrows = a->nrows;
+    c->ncols = b->ncols;
+    c->owns = true;
+    const auto fail = [&](const char *what) -> int64_t {
+        if (what)
+            set_error(COMET_HIP_ERR_HIP, "%s", what);
+        csr_release(c);
+        return 0;
+    };
+    if (hipMalloc((void **)&c->pos, sizeof(int64_t) * (size_t)(a->nrows + 1)) != hipSuccess)
+        return fail("row pointer allocation failed");
+    {
+        KernelTimer t("spgemm_symbolic_dot_count");
+        spgemm_dot_count<<<dim3((unsigned)ceil_div(a->nrows, 4)), dim3(256), 0, stream()>>>(
+            0, a->nrows, m->pos, pair_hit, (int64_t *)g_sg.rowcount.ptr);
+    }
+    if (exclusive_scan_i64((const int64_t *)g_sg.rowcount.ptr, a->nrows, c->pos) != COMET_HIP_OK)
+        return fail(nullptr);
+    if (hipMemcpyAsync(&c->nnz, c->pos + a->nrows, sizeof(int64_t), hipMemcpyDeviceToHost, stream()) != hipSuccess ||
+        hipStreamSynchronize(stream()) != hipSuccess)
+        return fail("reading the size of the product failed");
+    if (hipMalloc((void **)&c->crd, sizeof(int32_t) * (size_t)(c->nnz > 0 ? c->nnz : 1)) != hipSuccess ||
+        hipMalloc((void **)&c->val, sizeof(double) * (size_t)(c->nnz > 0 ? c->nnz : 1)) != hipSuccess)
+        return fail("output allocation failed");
+    {
+        KernelTimer t("spgemm_numeric_dot_compact");
+        spgemm_dot_compact<<<dim3((unsigned)ceil_div(a->nrows, 4)), dim3(256), 0, stream()>>>(
+            0, a->nrows, m->pos, m->crd, pair_val, pair_hit, c->pos, c->crd, c->val);
+    }
+    if (hipGetLastError() != hipSuccess)
+        return fail("launching the compaction failed");
+    return csr_register(c);
+}
+
 extern "C" int64_t comet_hip_spgemm_csr_semiring(int64_t ah, int64_t bh, int64_t mh, int reduce_op, int mult_op)
 {
     if (ensure_init() != COMET_HIP_OK)
@@ -2867,6 +2918,12 @@ extern "C" int64_t comet_hip_spgemm_csr_semiring(int64_t ah, int64_t bh, int64_t
         return 0;
     if (check_product_shapes(a, b, m, "spgemm") != COMET_HIP_OK)
         return 0;
+    if (m && reduce_op == COMET_SR_PLUS && mult_op == COMET_OP_TIMES) {
+        bool done = false;
+        const int64_t h = masked_product_one_pass(a, b, m, &done);
+        if (done)
+            return h;
+    }
     int64_t *pos = nullptr;
     if (hipMalloc((void **)&pos, sizeof(int64_t) * (size_t)(a->nrows + 1)) != hipSuccess) {
         set_error(COMET_HIP_ERR_HIP, "row pointer allocation failed");
