@@ -2099,13 +2099,17 @@ __device__ inline void for_each_pair(int64_t ms, int64_t me, const int32_t *__re
 // strict: a pair is kept when its streamed list is shorter than the table's (otherwise: not longer).  [xlo, xhi):
 // the pairs' other index must lie in it (the rows of M being computed, for the column's half).  perm: where pair p
 // of P lies in the row-major order of the mask (nullptr: at p); out0 is taken off either.
-template <bool VALUES>
+// SEMI: another semiring than plus-times (reduce plus, min or max; `any` keeps the place of a product in B, which
+// this form does not have): a product is mult(a, b) with a the entry of A - the table's in the row's half, the
+// streamed one in the column's (swapped) - and a pair's slot holds a sum or the key of a minimum or maximum.
+template <bool VALUES, bool SEMI>
 __global__ __launch_bounds__(SG_T) void spgemm_dot_kernel(
     int64_t row_begin, const int64_t *__restrict__ Tpos, const int32_t *__restrict__ Tcrd,
     const double *__restrict__ Tval, const int64_t *__restrict__ Ppos, const int32_t *__restrict__ Pcrd,
     const int64_t *__restrict__ Lpos, const int32_t *__restrict__ Lcrd, const double *__restrict__ Lval,
     const double *__restrict__ perm, int64_t out0, int strict, int64_t xlo, int64_t xhi, int words,
-    unsigned long long *ticket, RowList list, double *__restrict__ pair_val, uint8_t *__restrict__ pair_hit)
+    unsigned long long *ticket, RowList list, double *__restrict__ pair_val, uint8_t *__restrict__ pair_hit,
+    int reduce_op, int mult_op, int swapped)
 {
     __shared__ int64_t row_slot;
     __shared__ int wave_tot[SG_WAVES];
@@ -2139,9 +2143,24 @@ __global__ __launch_bounds__(SG_T) void spgemm_dot_kernel(
         const auto add = [&](int t, DotHit h) {
             if (h.hit) {
                 whit[wave * 64 + t] = 1;
-                if constexpr (VALUES)
+                if constexpr (VALUES && SEMI) {
+                    if (reduce_op == SR_PLUS)
+                        __hip_atomic_fetch_add(&wacc[wave * 64 + t], h.prod, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    else
+                        __hip_atomic_fetch_max(reinterpret_cast<unsigned long long *>(&wacc[wave * 64 + t]),
+                                               reduce_op == SR_MIN ? ~f64_key(h.prod) : f64_key(h.prod), __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_WORKGROUP);
+                } else if constexpr (VALUES) {
                     __hip_atomic_fetch_add(&wacc[wave * 64 + t], h.prod, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
             }
+        };
+        // tv: the table's value, lv: the streamed entry's
+        const auto product = [&](double tv, double lv) {
+            if constexpr (SEMI)
+                return swapped ? semiring_mult(mult_op, lv, tv) : semiring_mult(mult_op, tv, lv);
+            else
+                return tv * lv;
         };
         // (uniform: t is; a wavefront's own LDS operations keep their order)
         const auto decided = [&](int t) { return __builtin_amdgcn_readfirstlane(whit[wave * 64 + t]) != 0; };
@@ -2151,7 +2170,10 @@ __global__ __launch_bounds__(SG_T) void spgemm_dot_kernel(
                 const int64_t p = base + (int64_t)lane * SG_WAVES;
                 const int64_t at = (perm ? (int64_t)perm[p] : p) - out0;
                 pair_hit[at] = (uint8_t)whit[wave * 64 + lane];
-                if constexpr (VALUES)
+                if constexpr (VALUES && SEMI)
+                    pair_val[at] = semiring_lds_value(reinterpret_cast<unsigned long long *>(wacc)[wave * 64 + lane],
+                                                      reduce_op, mult_op, 0, nullptr, nullptr);
+                else if constexpr (VALUES)
                     pair_val[at] = wacc[wave * 64 + lane];
             }
             wacc[wave * 64 + lane] = 0.0;
@@ -2187,7 +2209,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_dot_kernel(
                         if (key != 0u) {
                             h.hit = 1;
                             if constexpr (VALUES)
-                                h.prod = hval[sl] * lv;
+                                h.prod = product(hval[sl], lv);
                         }
                     }
                     return h;
@@ -2242,7 +2264,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_dot_kernel(
                             int rank = (int)cnt_before[w / DT_GROUP] + __popc(word & (ad.bit(k) - 1u));
                             for (int v = wg; v < w; ++v)
                                 rank += __popc(bm[v + (v >> 5)]);
-                            h.prod = Tval[ts + rank] * lv;
+                            h.prod = product(Tval[ts + rank], lv);
                         }
                     }
                     return h;
@@ -2466,7 +2488,7 @@ constexpr int64_t SG_NO_DENSE = 1ll << 61;     // a threshold no row reaches: ev
 
 static int dot_form_fits(const Csr *a, const Csr *b, const Csr *m, bool *fits);
 static int dot_pairs(const Csr *a, const Csr *b, const Csr *m, int64_t rb, int64_t re, bool values, double **pair_val,
-                     uint8_t **pair_hit);
+                     uint8_t **pair_hit, int reduce_op = COMET_SR_PLUS, int mult_op = COMET_OP_TIMES);
 
 static int symbolic_counts(const Csr *a, const Csr *b, const Csr *m, int64_t *rowcount)
 {
@@ -2631,8 +2653,9 @@ static int dot_form_fits(const Csr *a, const Csr *b, const Csr *m, bool *fits)
 
 // pair_hit[p - Mpos[rb]] (and pair_val, with values) for every stored pair p of the mask rows [rb, re)
 static int dot_pairs(const Csr *a, const Csr *b, const Csr *m, int64_t rb, int64_t re, bool values, double **pair_val,
-                     uint8_t **pair_hit)
+                     uint8_t **pair_hit, int reduce_op, int mult_op)
 {
+    const bool semi = reduce_op != COMET_SR_PLUS || mult_op != COMET_OP_TIMES;
     Csr *bt = nullptr, *mt = nullptr;
     COMET_CHK(dot_transposed(b, &bt));
     COMET_CHK(dot_transposed_index(m, &mt));
@@ -2669,19 +2692,22 @@ static int dot_pairs(const Csr *a, const Csr *b, const Csr *m, int64_t rb, int64
         COMET_CHK(sg_reset_ticket());
         KernelTimer t(values ? (half == 0 ? "spgemm_numeric_dot_rows" : "spgemm_numeric_dot_columns")
                              : (half == 0 ? "spgemm_symbolic_dot_rows" : "spgemm_symbolic_dot_columns"));
-        if (values) {
-            COMET_CHK(sg_allow_lds(spgemm_dot_kernel<true>, lds));
-            spgemm_dot_kernel<true><<<grid, block, lds, stream()>>>(
-                first, T->pos, T->crd, T->val, P->pos, P->crd, L->pos, L->crd, L->val, half == 0 ? nullptr : mt->val, out0,
-                half, half == 0 ? 0 : rb, half == 0 ? everywhere : re, words, (unsigned long long *)g_sg.ticket.ptr, list,
-                *pair_val, *pair_hit);
-        } else {
-            COMET_CHK(sg_allow_lds(spgemm_dot_kernel<false>, lds));
-            spgemm_dot_kernel<false><<<grid, block, lds, stream()>>>(
-                first, T->pos, T->crd, T->val, P->pos, P->crd, L->pos, L->crd, L->val, half == 0 ? nullptr : mt->val, out0,
-                half, half == 0 ? 0 : rb, half == 0 ? everywhere : re, words, (unsigned long long *)g_sg.ticket.ptr, list,
-                *pair_val, *pair_hit);
-        }
+#define LAUNCH_DOT(V, S)                                                                                   \
+    do {                                                                                                   \
+        COMET_CHK(sg_allow_lds(spgemm_dot_kernel<V, S>, lds));                                             \
+        spgemm_dot_kernel<V, S><<<grid, block, lds, stream()>>>(                                           \
+            first, T->pos, T->crd, T->val, P->pos, P->crd, L->pos, L->crd, L->val,                         \
+            half == 0 ? nullptr : mt->val, out0, half, half == 0 ? 0 : rb, half == 0 ? everywhere : re,    \
+            words, (unsigned long long *)g_sg.ticket.ptr, list, *pair_val, *pair_hit, reduce_op, mult_op,  \
+            half);                                                                                         \
+    } while (0)
+        if (!values)
+            LAUNCH_DOT(false, false);
+        else if (semi)
+            LAUNCH_DOT(true, true);
+        else
+            LAUNCH_DOT(true, false);
+#undef LAUNCH_DOT
         COMET_HIPCHK(hipGetLastError());
     }
     return COMET_HIP_OK;
@@ -2693,13 +2719,13 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
     if (reduce_op < 0 || reduce_op > COMET_SR_ANY || mult_op < 0 || mult_op > COMET_OP_DIV)
         return set_error(COMET_HIP_ERR_ARG, "unknown semiring (reduce %d, mult %d)", reduce_op, mult_op);
     const bool semi = reduce_op != COMET_SR_PLUS || mult_op != COMET_OP_TIMES;
-    if (m && !semi && re > rb) {
+    if (m && reduce_op != COMET_SR_ANY && re > rb) {
         bool dots = false;
         COMET_CHK(dot_form_fits(a, b, m, &dots));
         if (dots) {
             double *pair_val = nullptr;
             uint8_t *pair_hit = nullptr;
-            COMET_CHK(dot_pairs(a, b, m, rb, re, true, &pair_val, &pair_hit));
+            COMET_CHK(dot_pairs(a, b, m, rb, re, true, &pair_val, &pair_hit, reduce_op, mult_op));
             KernelTimer t("spgemm_numeric_dot_compact");
             spgemm_dot_compact<<<dim3((unsigned)ceil_div(re - rb, 4)), dim3(256), 0, stream()>>>(
                 rb, re, m->pos, m->crd, pair_val, pair_hit, Cpos, Ccrd, Cval);
@@ -2860,7 +2886,7 @@ extern "C" int64_t comet_hip_spgemm_csr(int64_t ah, int64_t bh, int64_t mh)
 
 // C<M> = A*B in one pass over the pairs of the mask: their values and which of them met a product come out of
 // the same walk, so the row pointers need no symbolic phase of their own.  *done says whether this form applied.
-static int64_t masked_product_one_pass(const Csr *a, const Csr *b, const Csr *m, bool *done)
+static int64_t masked_product_one_pass(const Csr *a, const Csr *b, const Csr *m, int reduce_op, int mult_op, bool *done)
 {
     *done = false;
     bool dots = false;
@@ -2871,7 +2897,7 @@ static int64_t masked_product_one_pass(const Csr *a, const Csr *b, const Csr *m,
     *done = true;
     double *pair_val = nullptr;
     uint8_t *pair_hit = nullptr;
-    if (dot_pairs(a, b, m, 0, a->nrows, true, &pair_val, &pair_hit) != COMET_HIP_OK ||
+    if (dot_pairs(a, b, m, 0, a->nrows, true, &pair_val, &pair_hit, reduce_op, mult_op) != COMET_HIP_OK ||
         g_sg.rowcount.ensure(sizeof(int64_t) * (size_t)a->nrows, false) != COMET_HIP_OK)
         return 0;
     Csr *c = new Csr();
@@ -2918,9 +2944,9 @@ extern "C" int64_t comet_hip_spgemm_csr_semiring(int64_t ah, int64_t bh, int64_t
         return 0;
     if (check_product_shapes(a, b, m, "spgemm") != COMET_HIP_OK)
         return 0;
-    if (m && reduce_op == COMET_SR_PLUS && mult_op == COMET_OP_TIMES) {
+    if (m && reduce_op >= 0 && reduce_op < COMET_SR_ANY && mult_op >= 0 && mult_op <= COMET_OP_DIV) {
         bool done = false;
-        const int64_t h = masked_product_one_pass(a, b, m, &done);
+        const int64_t h = masked_product_one_pass(a, b, m, reduce_op, mult_op, &done);
         if (done)
             return h;
     }

@@ -496,6 +496,34 @@ def test_spgemm_masked_dot_products(n, k, m, da, db, dm, seed):
         assert np.all(np.abs(dv.to_numpy(cnt) - wv[hp[rb]:hp[re]]) <= RTOL * bound[hp[rb]:hp[re]])
 
 
+@pytest.mark.parametrize("semiring", [("min", "plus"), ("max", "times"), ("plus", "first"), ("min", "div"), ("max", "minus"),
+                                      ("plus", "pair"), ("any", "second")])
+def test_spgemm_masked_dot_products_semirings(semiring):
+    """The dot-product form under other semirings: the order of the two operands of `mult` is A's entry first in
+    both halves; min and max are exact, sums to rounding; `any` takes the walk by rows."""
+    rng = np.random.default_rng(77)
+    n, k, m = 700, 900, 800
+    a = _rand_csr(rng, n, k, 0.05, signed=True)
+    b = _rand_csr(rng, k, m, 0.04, signed=True)
+    b = (b[0], b[1], np.where(b[2] < 0, b[2] - 0.25, b[2] + 0.25))          # keeps div finite
+    la = np.diff(a[0])
+    mk = _rand_csr(rng, n, m, 0.2, signed=False)
+    A = rt.CsrMatrix.from_arrays((n, k), *a)
+    B = rt.CsrMatrix.from_arrays((k, m), *b)
+    Mk = rt.CsrMatrix.from_arrays((n, m), mk[0], mk[1], np.ones(len(mk[1])))
+    wp, wc, wv = orc.spgemm(*a, *b, m, mask=(mk[0], mk[1]), semiring=semiring)
+    for _ in range(2):
+        p, c, v = rt.spgemm(A, B, Mk, semiring=semiring).to_arrays()
+        assert np.array_equal(p, wp) and np.array_equal(c, wc)
+        if semiring[0] == "plus":
+            _, _, bound = orc.spgemm(a[0], a[1], np.abs(a[2]), b[0], b[1], np.abs(b[2]), m, mask=(mk[0], mk[1]),
+                                     semiring=semiring)
+            assert np.all(np.abs(v - wv) <= RTOL * np.maximum(bound, 1.0))
+        else:
+            assert np.array_equal(v, wv)
+    _spgemm_check(a, b, m, mask=(mk[0], mk[1]))        # plus-times afterwards finds nothing left behind
+
+
 def test_spgemm_masked_dot_products_hubs_and_repeats():
     """Lists of very different lengths (a few rows of A and columns of B with thousands of entries among short ones:
     each half of the pairs has work), and a matrix that holds a column twice in a row, which the tables cannot
