@@ -558,7 +558,6 @@ constexpr int spmm_hrows(int g) { return g * (SPMM_HW - 1) * SPMM_HR; }    // lo
 #endif
 constexpr int SPMM_MED_MIN_LEN = COMET_SPMM_MED_MIN;   // such a row has at least this many nonzeros
 constexpr int SPMM_MSLOTS = 288;                        // sums a workgroup keeps in LDS: 144 KiB
-static_assert(SPMM_MSLOTS <= 512, "a list entry has nine bits for the slot");
 constexpr int SPMM_HEAVY_MIN_LEN = COMET_SPMM_HEAVY_MIN;              // a long row has at least this many nonzeros
 constexpr int SPMM_HCB = 32;                         // column blocks a wavefront's list is cut into
 
@@ -596,14 +595,16 @@ constexpr int SPMM_HCB = 32;                         // column blocks a wavefron
 // flight; batches of 4 or 16 pairs: 0.25 ms) - with sixteen wavefronts per CU
 // the memory path is kept busy by the other wavefronts, and more requests
 // queued per wavefront only lengthen the queues.
-// Entry = (column - first column of the XCD's range) << SPMM_E_COL | owned row << SPMM_E_ROW | first-of-run | real.
+// Entry = column - first column of the XCD's range (the low 24 bits, so that the byte offset of the row of B is one
+// 24-bit multiply-add on the entry as it is) | real, first-of-run, kept-in-LDS | owned row << SPMM_E_ROW.  The slot of
+// a row kept in LDS is the entry's second word.
 constexpr int SPMM_HP = 8;       // pairs of entries per batch of gathers
-constexpr int SPMM_E_REAL = 1;                 // not a pad
-constexpr int SPMM_E_FIRST = 2;                // the entry opens a run of one owned row
-constexpr int SPMM_E_MED = 4;                  // the entry adds into a sum kept in LDS, in the slot its row field names
-constexpr int SPMM_E_ROW = 3;                  // where the owned row (or, for a row kept in LDS, its slot) sits: 9 bits
-constexpr int SPMM_E_COL = 12;
-static_assert(SPMM_E_COL + SPMM_HCOLB <= 32 && SPMM_HRB <= SPMM_E_COL - SPMM_E_ROW, "an entry is 32 bits");
+constexpr int SPMM_E_REAL = 1 << 24;           // not a pad
+constexpr int SPMM_E_FIRST = 1 << 25;          // the entry opens a run of one owned row
+constexpr int SPMM_E_MED = 1 << 26;            // the entry adds into a sum kept in LDS, in the slot its second word names
+constexpr int SPMM_E_ROW = 27;                 // where the owned row sits
+constexpr unsigned SPMM_E_COLMASK = 0xffffffu;
+static_assert(SPMM_HCOLB <= 24 && SPMM_E_ROW + SPMM_HRB <= 32, "an entry is 32 bits");
 constexpr int SPMM_HWL = SPMM_HW - 1;          // wavefronts of a workgroup that own long rows
 
 // SMALL: B spans less than 4 GiB and has fewer than 2^24 rows of fewer than 2^24 bytes, so the byte offset of a
@@ -617,10 +618,10 @@ __device__ inline void heavy_issue(double2 (&b)[SPMM_HP], int ents, int t0, int 
         const int t = t0 + u < npairs ? t0 + u : npairs - 1;     // past the end: reload the last one, never used
         const unsigned mine = (unsigned)__shfl(ents, 2 * t + half, 64);       // each half its own entry
         if constexpr (SMALL) {
-            const unsigned off = __umul24(mine >> SPMM_E_COL, (unsigned)ldb * 8u) + (unsigned)col * 8u;
+            const unsigned off = __umul24(mine, (unsigned)ldb * 8u) + (unsigned)col * 8u;
             b[u] = *reinterpret_cast<const double2 *>(reinterpret_cast<const char *>(B) + off);
         } else {
-            const int64_t j = (int64_t)(mine >> SPMM_E_COL);
+            const int64_t j = (int64_t)(mine & SPMM_E_COLMASK);
             b[u] = *reinterpret_cast<const double2 *>(B + j * ldb + col);
         }
     }
@@ -628,8 +629,8 @@ __device__ inline void heavy_issue(double2 (&b)[SPMM_HP], int ents, int t0, int 
 
 extern __shared__ double spmm_medium_sums[];
 __device__ inline void heavy_add(double (&accx)[SPMM_HR], double (&accy)[SPMM_HR], double2 &run, int &run_slot,
-                                 const double2 (&b)[SPMM_HP], int ents, double vals, int t0, int npairs, int half,
-                                 int sub, bool active)
+                                 const double2 (&b)[SPMM_HP], int ents, int slots,
+                                 double vals, int t0, int npairs, int half, int sub, bool active)
 {
 #pragma unroll
     for (int u = 0; u < SPMM_HP; ++u) {
@@ -640,26 +641,31 @@ __device__ inline void heavy_add(double (&accx)[SPMM_HR], double (&accy)[SPMM_HR
             if (e0 & SPMM_E_FIRST) {             // a run starts on an even entry
                 accx[run_slot] = run.x;
                 accy[run_slot] = run.y;
-                run_slot = (e0 >> SPMM_E_ROW) & (SPMM_HR - 1);
+                run_slot = ((unsigned)e0 >> SPMM_E_ROW) & (SPMM_HR - 1);
                 run.x = accx[run_slot];
                 run.y = accy[run_slot];
             }
             const int mine = __shfl(ents, 2 * t + half, 64);
             const double v = __hiloint2double(__shfl(__double2hiint(vals), 2 * t + half, 64),
                                               __shfl(__double2loint(vals), 2 * t + half, 64));
-            const double px = v * b[u].x, py = v * b[u].y;
             if (med) {
+                const double px = v * b[u].x, py = v * b[u].y;
+                const int slot = __shfl(slots, 2 * t + half, 64);
                 // a row of middling length: its sum lives in LDS.  An add that returns nothing is issued and
                 // forgotten; all entries of such a row are in this wavefront's list, in column order, and the adds
                 // of one wavefront to one address are carried out in the order it issued them.
                 if ((mine & SPMM_E_REAL) && active) {
-                    double *sum = spmm_medium_sums + ((mine >> SPMM_E_ROW) & 511) * 64 + 2 * sub;
+                    double *sum = spmm_medium_sums + slot * 64 + 2 * sub;
                     __hip_atomic_fetch_add(sum, px, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                     __hip_atomic_fetch_add(sum + 1, py, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 }
             } else if (mine & SPMM_E_REAL) {     // a pad carries no value
-                run.x = run.x + px;
-                run.y = run.y + py;
+                // A branch over the lanes of a pad, not a select: two fused multiply-adds instead of two
+                // multiplications, two additions and four selects (a long row's sum is to rounding in any case:
+                // it is added from sixteen partial sums).
+                asm volatile("" ::: "memory");
+                run.x = __builtin_fma(v, b[u].x, run.x);
+                run.y = __builtin_fma(v, b[u].y, run.y);
             }
         }
     }
@@ -685,10 +691,10 @@ __device__ inline void single_issue(double2 (&b)[NB], double2 (&c)[NB], const sp
         const spmm_v4i q = ring_half[(KB + 2 * (t + u)) & 63];
         const unsigned mine = (unsigned)q.x;
         if constexpr (SMALL) {
-            const unsigned off = __umul24(mine >> SPMM_E_COL, (unsigned)ldb * 8u) + (unsigned)col * 8u;
+            const unsigned off = __umul24(mine, (unsigned)ldb * 8u) + (unsigned)col * 8u;
             b[u] = *reinterpret_cast<const double2 *>(reinterpret_cast<const char *>(B) + off);
         } else {
-            const int64_t j = (int64_t)(mine >> SPMM_E_COL);
+            const int64_t j = (int64_t)(mine & SPMM_E_COLMASK);
             b[u] = *reinterpret_cast<const double2 *>(B + j * ldb + col);
         }
         if constexpr (ACC)
@@ -788,35 +794,38 @@ __global__ __launch_bounds__(SPMM_HW * 64) void spmm_heavy_sweep(
         double2 run = make_double2(0.0, 0.0);
         int run_slot = 0;
         int cnt = (int)(e - s < 64 ? e - s : 64);
-        int c_ent = 0;
+        int c_ent = 0, c_slot = 0;
         double c_val = 0.0;
         if (lane < cnt) {
             const spmm_v4i q = __builtin_nontemporal_load(list + s + lane);
             c_ent = q.x;
+            c_slot = q.y;
             c_val = __hiloint2double(q.w, q.z);
         }
         heavy_issue<SMALL>(b, c_ent, 0, cnt >> 1, half, B, ldb, col);
         for (int64_t base = s; base < e; base += 64) {
             const int64_t left = e - base - 64;
             const int ncnt = (int)(left < 0 ? 0 : (left < 64 ? left : 64));
-            int n_ent = 0;
+            int n_ent = 0, n_slot = 0;
             double n_val = 0.0;
             if (lane < ncnt) {
                 const spmm_v4i q = __builtin_nontemporal_load(list + base + 64 + lane);
                 n_ent = q.x;
+                n_slot = q.y;
                 n_val = __hiloint2double(q.w, q.z);
             }
             const int np = cnt >> 1;
-            heavy_add(accx, accy, run, run_slot, b, c_ent, c_val, 0, np, half, sub, active);
+            heavy_add(accx, accy, run, run_slot, b, c_ent, c_slot, c_val, 0, np, half, sub, active);
 #pragma unroll
             for (int t0 = SPMM_HP; t0 < 32; t0 += SPMM_HP)
                 if (np > t0) {
                     heavy_issue<SMALL>(b, c_ent, t0, np, half, B, ldb, col);
-                    heavy_add(accx, accy, run, run_slot, b, c_ent, c_val, t0, np, half, sub, active);
+                    heavy_add(accx, accy, run, run_slot, b, c_ent, c_slot, c_val, t0, np, half, sub, active);
                 }
             if (ncnt > 0)         // the first batch of the next 64 entries: in flight over the loop's back edge
                 heavy_issue<SMALL>(b, n_ent, 0, ncnt >> 1, half, B, ldb, col);
             c_ent = n_ent;
+            c_slot = n_slot;
             c_val = n_val;
             cnt = ncnt;
         }
@@ -1014,7 +1023,7 @@ __global__ void heavy_fill(int64_t n, const uint64_t *__restrict__ keys, const u
     const int64_t p = e + pads[r];
     const bool direct = ((k >> 28) & SPMM_HR) != 0;
     const uint64_t c = k & 0xfffffffull;
-    const uint32_t col = (uint32_t)(c - (c / (uint64_t)xcols) * (uint64_t)xcols) << SPMM_E_COL;     // inside its XCD's range
+    const uint32_t col = (uint32_t)(c - (c / (uint64_t)xcols) * (uint64_t)xcols);     // inside its XCD's range
     HeavyEnt out;
     if (direct && ((k >> 28) & 1)) {          // a row of middling length: which one, from the entry's place
         const int64_t at = idx[e];
@@ -1026,8 +1035,8 @@ __global__ void heavy_fill(int64_t n, const uint64_t *__restrict__ keys, const u
             else
                 hi = mid - 1;
         }
-        out.ent = (int32_t)(col | SPMM_E_REAL | SPMM_E_MED | ((uint32_t)(lo / groups) << SPMM_E_ROW));
-        out.row = 0;
+        out.ent = (int32_t)(col | SPMM_E_REAL | SPMM_E_MED);
+        out.row = (int32_t)(lo / groups);
         out.val = val[pos[mrow[lo]] + (at - mstart[lo])];
     } else if (direct) {
         out.ent = (int32_t)(col | SPMM_E_REAL);
