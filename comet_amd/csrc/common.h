@@ -84,6 +84,7 @@ struct Csr {
     // found without searching.
     int64_t *sg_blkptr = nullptr;
     int sg_nblk = 0;
+    uint16_t *sg_crd16 = nullptr;            // the columns inside their block of 2^14 (null: not kept)
     // SpMM plan for long rows (heavy_state: 0 undecided, 1 not worth it, 2 in use): the long rows re-stored as
     // per-(XCD, wavefront) lists ordered by column for spmm_heavy_sweep, and the rest of the matrix as `light`.
     int heavy_state = 0;

@@ -190,7 +190,9 @@ static void csr_drop_plans(Csr *c)
     c->spmm_chunk_row = nullptr;
     c->spmm_nchunks = 0;
     (void)hipFree(c->sg_blkptr);
+    (void)hipFree(c->sg_crd16);
     c->sg_blkptr = nullptr;
+    c->sg_crd16 = nullptr;
     c->sg_nblk = 0;
     (void)hipFree(c->spmv_bpos);
     (void)hipFree(c->spmv_bpos32);

@@ -975,6 +975,14 @@ __global__ __launch_bounds__(256) void spgemm_row_products(int64_t row_begin, in
 
 // blkptr[k * (nblk + 1) + cb] = position in crd/val of the first entry of row k whose column is >= cb * SG_CB
 // (cb = nblk gives the end of the row): the slice of row k inside block cb is one 16-byte load away.
+// crd16[q] = the column of entry q inside its block of SG_CB columns
+__global__ void spgemm_block_columns(int64_t nnz, const int32_t *__restrict__ crd, uint16_t *__restrict__ crd16)
+{
+    const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (q < nnz)
+        crd16[q] = (uint16_t)(crd[q] & (SG_CB - 1));
+}
+
 __global__ void spgemm_block_pointers(int64_t nrows, const int64_t *__restrict__ pos,
                                       const int32_t *__restrict__ crd, int nblk, int64_t *__restrict__ blkptr)
 {
@@ -1026,9 +1034,24 @@ constexpr int SG_LONG_LOADS = 4;                  // entries of a long slice per
 // One turn of a wavefront over a slice that starts at entry s of B and has len entries: lane l visits the
 // entries o + 64 x < len, x < SG_LONG_LOADS (o = l for the first turn of a slice).  All loads are issued before
 // the first visit, and a load that no lane needs is skipped.
-template <bool VALUES, typename F>
+// The columns of B come as 32-bit numbers or (COL = uint16_t) as the 16-bit numbers inside their block of SG_CB
+// columns that the right-hand operand's plan keeps for the kernel that takes one block per visit: a third of the
+// bytes of an entry it only needs the column of.
+typedef unsigned short sg_h4u __attribute__((ext_vector_type(4), aligned(2)));
+template <typename COL>
+struct SgCol4;
+template <>
+struct SgCol4<int32_t> {
+    typedef sg_i4u type;
+};
+template <>
+struct SgCol4<uint16_t> {
+    typedef sg_h4u type;
+};
+
+template <bool VALUES, typename COL, typename F>
 __device__ __forceinline__ void turn_of_slice(int64_t s, int64_t o, int64_t len, double at, int pt,
-                                              const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval, F f)
+                                              const COL *__restrict__ Bcrd, const double *__restrict__ Bval, F f)
 {
     int64_t q[SG_LONG_LOADS];
     bool ok[SG_LONG_LOADS];
@@ -1041,7 +1064,7 @@ __device__ __forceinline__ void turn_of_slice(int64_t s, int64_t o, int64_t len,
     double v[SG_LONG_LOADS];
 #pragma unroll
     for (int x = 0; x < SG_LONG_LOADS; ++x)
-        j[x] = ok[x] ? Bcrd[q[x]] : 0;
+        j[x] = ok[x] ? (int)Bcrd[q[x]] : 0;
 #pragma unroll
     for (int x = 0; x < SG_LONG_LOADS; ++x)
         v[x] = VALUES && ok[x] ? Bval[q[x]] : 0.0;
@@ -1051,11 +1074,12 @@ __device__ __forceinline__ void turn_of_slice(int64_t s, int64_t o, int64_t len,
             f(j[x], at, v[x], pt, q[x]);
 }
 
-template <bool VALUES, typename F>
+template <bool VALUES, typename COL, typename F>
 __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double a, int pa, int lane,
-                                                  const int32_t *__restrict__ Bcrd,
+                                                  const COL *__restrict__ Bcrd,
                                                   const double *__restrict__ Bval, F f)
 {
+    typedef typename SgCol4<COL>::type col4;
     // Long slices take the whole wavefront, one at a time; short ones (a slice of one block often holds a
     // dozen entries) are handed to the four 16-lane quarters, four at a time.  A wavefront runs its turns
     // one after the other (there is room for one workgroup per CU, so nobody else hides the latency), and
@@ -1084,7 +1108,7 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
             static_assert(SG_LONG_LOADS == 4, "a lane's entries of a full turn are one 16-byte load of columns");
             typedef double sg_d2u __attribute__((ext_vector_type(2), aligned(8)));
             int64_t c = s + 4 * (int64_t)lane;          // this lane's first entry of the turn
-            sg_i4u j = *reinterpret_cast<const sg_i4u *>(Bcrd + c);
+            col4 j = *reinterpret_cast<const col4 *>(Bcrd + c);
             sg_d2u v0 = {0.0, 0.0}, v1 = {0.0, 0.0};
             if constexpr (VALUES) {
                 v0 = *reinterpret_cast<const sg_d2u *>(Bval + c);
@@ -1093,31 +1117,31 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
             int64_t done = 0;
             for (int64_t full = 64 * SG_LONG_LOADS; full + 64 * SG_LONG_LOADS <= len; full += 64 * SG_LONG_LOADS) {
                 const int64_t cn = c + 64 * SG_LONG_LOADS;
-                const sg_i4u jn = *reinterpret_cast<const sg_i4u *>(Bcrd + cn);
+                const col4 jn = *reinterpret_cast<const col4 *>(Bcrd + cn);
                 sg_d2u v0n = {0.0, 0.0}, v1n = {0.0, 0.0};
                 if constexpr (VALUES) {
                     v0n = *reinterpret_cast<const sg_d2u *>(Bval + cn);
                     v1n = *reinterpret_cast<const sg_d2u *>(Bval + cn + 2);
                 }
-                f(j.x, at, v0.x, pt, c);
-                f(j.y, at, v0.y, pt, c + 1);
-                f(j.z, at, v1.x, pt, c + 2);
-                f(j.w, at, v1.y, pt, c + 3);
+                f((int)j.x, at, v0.x, pt, c);
+                f((int)j.y, at, v0.y, pt, c + 1);
+                f((int)j.z, at, v1.x, pt, c + 2);
+                f((int)j.w, at, v1.y, pt, c + 3);
                 j = jn;
                 v0 = v0n;
                 v1 = v1n;
                 c = cn;
                 done += 64 * SG_LONG_LOADS;
             }
-            f(j.x, at, v0.x, pt, c);
-            f(j.y, at, v0.y, pt, c + 1);
-            f(j.z, at, v1.x, pt, c + 2);
-            f(j.w, at, v1.y, pt, c + 3);
+            f((int)j.x, at, v0.x, pt, c);
+            f((int)j.y, at, v0.y, pt, c + 1);
+            f((int)j.z, at, v1.x, pt, c + 2);
+            f((int)j.w, at, v1.y, pt, c + 3);
             done += 64 * SG_LONG_LOADS;
             o += done;
         }
         if (o < len)
-            turn_of_slice<VALUES>(s, o, len, at, pt, Bcrd, Bval, f);
+            turn_of_slice<VALUES, COL>(s, o, len, at, pt, Bcrd, Bval, f);
     }
     const int quarter = lane >> 4, sub = lane & 15;
     while (todo) {              // four short slices per turn, one to a quarter, SG_SHORT_LOADS entries per lane
@@ -1146,7 +1170,7 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
         double v[SG_SHORT_LOADS];
 #pragma unroll
         for (int x = 0; x < SG_SHORT_LOADS; ++x)
-            j[x] = (ok[x] ? Bcrd[q[x]] : 0);
+            j[x] = (ok[x] ? (int)Bcrd[q[x]] : 0);
 #pragma unroll
         for (int x = 0; x < SG_SHORT_LOADS; ++x)
             v[x] = (VALUES && ok[x] ? Bval[q[x]] : 0.0);
@@ -1165,10 +1189,11 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
 // before a block's products are walked, the mask row's entries inside the block are set in a bitmap of their own
 // (the row is sorted, so they start where the block before ended), and when the block is written out the columns
 // outside it are dropped and their accumulators cleared.
-template <bool SEMI, bool MASKED>
+// COL: B's columns as 32-bit numbers, or as 16-bit numbers inside their block (see turn_of_slice).
+template <bool SEMI, bool MASKED, typename COL>
 __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
     int64_t row_begin, int64_t row_end, const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd,
-    const double *__restrict__ Aval, const int32_t *__restrict__ Bcrd, const double *__restrict__ Bval,
+    const double *__restrict__ Aval, const COL *__restrict__ Bcrd, const double *__restrict__ Bval,
     const int64_t *__restrict__ Mpos, const int32_t *__restrict__ Mcrd,
     const int64_t *__restrict__ blkptr, int nblk,
     unsigned long long *ticket, RowList list,
@@ -1253,7 +1278,8 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                 }
                 int touched = 0;     // did this wavefront add anything to the block
                 const auto add = [&](int j, double a, double b, int pa, int64_t q) {
-                    j -= col0;
+                    if constexpr (sizeof(COL) == 4)
+                        j -= col0;
                     atomicOr(&bm[j >> 5], 1u << (j & 31));
                     if constexpr (SEMI)
                         semiring_lds_add(&acc[j], reduce_op, mult_op, a, b, pa, q);
@@ -2561,8 +2587,16 @@ static int sg_plan_blocks(Csr *b)
     if (b->sg_blkptr) {
         COMET_HIPCHK(hipStreamSynchronize(stream()));
         COMET_HIPCHK(hipFree(b->sg_blkptr));
+        (void)hipFree(b->sg_crd16);
         b->sg_blkptr = nullptr;
+        b->sg_crd16 = nullptr;
     }
+    static_assert(SG_CB <= 65536, "a column inside its block fits 16 bits");
+    if (hipMalloc((void **)&b->sg_crd16, sizeof(uint16_t) * (size_t)(b->nnz > 0 ? b->nnz : 1)) != hipSuccess)
+        b->sg_crd16 = nullptr;          // the kernel then reads the 32-bit columns
+    else if (b->nnz > 0)
+        spgemm_block_columns<<<dim3((unsigned)ceil_div(b->nnz, 256)), dim3(256), 0, stream()>>>(b->nnz, b->crd,
+                                                                                                 b->sg_crd16);
     COMET_HIPCHK(hipMalloc((void **)&b->sg_blkptr,
                            sizeof(int64_t) * (size_t)(nblk + 1) * (size_t)(b->nrows > 0 ? b->nrows : 1)));
     b->sg_nblk = nblk;
@@ -2790,19 +2824,27 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
         COMET_CHK(sg_reset_ticket());
         KernelTimer t(mdense ? "spgemm_numeric_dense_masked" : "spgemm_numeric_dense");
         const dim3 cus((unsigned)(num_cus() > 0 ? num_cus() : 256));
-#define LAUNCH_DENSE(S, M)                                                                                 \
+#define LAUNCH_DENSE_C(S, M, COL, CRD)                                                                     \
     do {                                                                                                   \
-        COMET_CHK(sg_allow_lds(spgemm_numeric_dense_kernel<S, M>, SG_DENSE_LDS));                          \
-        spgemm_numeric_dense_kernel<S, M><<<cus, block, SG_DENSE_LDS, stream()>>>(                         \
-            rb, re, a->pos, a->crd, a->val, b->crd, b->val, m ? m->pos : nullptr, m ? m->crd : nullptr,    \
+        COMET_CHK(sg_allow_lds(spgemm_numeric_dense_kernel<S, M, COL>, SG_DENSE_LDS));                     \
+        spgemm_numeric_dense_kernel<S, M, COL><<<cus, block, SG_DENSE_LDS, stream()>>>(                    \
+            rb, re, a->pos, a->crd, a->val, CRD, b->val, m ? m->pos : nullptr, m ? m->crd : nullptr,       \
             b->sg_blkptr, nblk, (unsigned long long *)g_sg.ticket.ptr, list, Cpos, Ccrd, Cval, reduce_op,  \
             mult_op);                                                                                      \
+    } while (0)
+#define LAUNCH_DENSE(S, M)                                                                                 \
+    do {                                                                                                   \
+        if (b->sg_crd16 && getenv("COMET_HIP_SPGEMM_WIDE_COLUMNS") == nullptr)                             \
+            LAUNCH_DENSE_C(S, M, uint16_t, b->sg_crd16);                                                   \
+        else                                                                                               \
+            LAUNCH_DENSE_C(S, M, int32_t, b->crd);                                                         \
     } while (0)
         if (mdense) {
             if (semi) LAUNCH_DENSE(true, true); else LAUNCH_DENSE(false, true);
         } else {
             if (semi) LAUNCH_DENSE(true, false); else LAUNCH_DENSE(false, false);
         }
+#undef LAUNCH_DENSE_C
 #undef LAUNCH_DENSE
         COMET_HIPCHK(hipGetLastError());
     }

@@ -592,17 +592,23 @@ def _rows_of_lengths(rng, lengths, ncols, pick=None, signed=True):
     return pos, crd.astype(np.int64), val
 
 
-@pytest.mark.parametrize("m,long_len,wide", [(200_000, 2000, None), (40_000, 1200, None), (40_000, 1200, 1 << 40),
-                                             (200_000, 2000, 1 << 40), (200_000, 2000, 0)])
-def test_spgemm_rows_of_every_class(m, long_len, wide, monkeypatch):
+@pytest.mark.parametrize("m,long_len,wide,cols32", [(200_000, 2000, None, False), (40_000, 1200, None, False),
+                                                    (40_000, 1200, 1 << 40, False), (200_000, 2000, 1 << 40, False),
+                                                    (200_000, 2000, 0, False), (200_000, 2000, 0, True),
+                                                    (1_000_000, 3000, None, False), (1_000_000, 3000, None, True)])
+def test_spgemm_rows_of_every_class(m, long_len, wide, cols32, monkeypatch):
     # Rows of B: 200 long ones and 200 of 10 entries.  Rows of A pick among them so that the product has rows
     # for each numeric kernel: no products, a few (values kept in a slab), thousands spread thinly over the
     # column blocks (several blocks per visit, values compact) and many per block (one block per visit).
     # `wide` moves the border between the last two: with 1 << 40 every heavy row takes the several-block
     # kernel, and with 40,000 columns the thick rows then exceed the compact array, so their visits are cut
     # short at a block boundary; with 0 every heavy row takes one block per visit.
+    # The one-block kernel reads B's columns as 16-bit numbers inside their block (a copy the library keeps with the
+    # block pointers), or with cols32 the 32-bit ones.
     if wide is not None:
         monkeypatch.setenv("COMET_HIP_SPGEMM_WIDE", str(wide))
+    if cols32:
+        monkeypatch.setenv("COMET_HIP_SPGEMM_WIDE_COLUMNS", "1")
     rng = np.random.default_rng(17)
     k = 400
     b = _rows_of_lengths(rng, [long_len] * 200 + [10] * 200, m)
