@@ -1027,8 +1027,11 @@ __device__ __forceinline__ int visit_flag(int *flags, int visit, int touched, in
 // gave it: its place in the row of A, which only the `any` semiring needs), b the entry of B (0 without VALUES,
 // when the value array is not read) and q its place in B.  Returns whether this wavefront had anything to visit.
 
-constexpr int SG_SHORT = 32;                      // slices shorter than this are taken by 16 lanes, the others by 64
-constexpr int SG_SHORT_LOADS = SG_SHORT / 16;     // entries of a short slice per lane
+#ifndef COMET_SG_SHORT
+#define COMET_SG_SHORT 32
+#endif
+constexpr int SG_SHORT = COMET_SG_SHORT;          // slices shorter than this are laid end to end, the others take turns of their own
+constexpr int SG_SHORT_LOADS = 2;                 // entries of the short slices per lane and batch
 constexpr int SG_LONG_LOADS = 4;                  // entries of a long slice per lane and turn
 
 // One turn of a wavefront over a slice that starts at entry s of B and has len entries: lane l visits the
@@ -1081,14 +1084,15 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
 {
     typedef typename SgCol4<COL>::type col4;
     // Long slices take the whole wavefront, one at a time; short ones (a slice of one block often holds a
-    // dozen entries) are handed to the four 16-lane quarters, four at a time.  A wavefront runs its turns
-    // one after the other (there is room for one workgroup per CU, so nobody else hides the latency), and
+    // dozen entries) are laid end to end and dealt to the lanes entry by entry (below).  A wavefront runs its
+    // turns one after the other (there is room for one workgroup per CU, so nobody else hides the latency), and
     // a turn costs about one trip to memory: so every turn issues all of its loads before the first LDS
     // operation waits for one, and a load that no lane needs is skipped.  Measured on A*A of an R-MAT
     // graph of scale 20: two loads per lane and turn of a long slice instead of four, +18 % time in this
-    // kernel, eight +2 %; two long slices or eight short ones per turn, +2..8 %; slices of up to 4 or 8
-    // entries left to their own lane (64 slices per turn, but every lane a cache line of its own), +4..6 %;
-    // the 16-lane path up to 64 or 128 entries, +1..5 %.
+    // kernel, eight +2 %; two long slices per turn, +2..8 %; slices of up to 4 or 8 entries left to their own
+    // lane (64 slices per turn, but every lane a cache line of its own), +4..6 %; the short slices one to a
+    // 16-lane quarter, four at a time, +1.7 % (up to 64 or 128 entries that way, +1..5 % more); laid end to
+    // end up to 128 or 256 entries instead of 32, +6 % and +22 %.
     unsigned long long big = __ballot(hi - lo >= SG_SHORT);
     unsigned long long todo = __ballot(lo < hi && hi - lo < SG_SHORT);
     const int touched = (big | todo) != 0;
@@ -1143,41 +1147,73 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
         if (o < len)
             turn_of_slice<VALUES, COL>(s, o, len, at, pt, Bcrd, Bval, f);
     }
-    const int quarter = lane >> 4, sub = lane & 15;
-    while (todo) {              // four short slices per turn, one to a quarter, SG_SHORT_LOADS entries per lane
-        int pick = -1;
+    // The short slices are laid end to end and dealt to the lanes entry by entry, 64 at a time, so that every load
+    // and every LDS operation has all its lanes (a quarter-wavefront per slice left two thirds of them idle: a
+    // slice of one block holds a dozen entries).  The lane that holds the slice an entry belongs to is found by
+    // bisection over the running sum of the slices' lengths.
+    if (todo) {
+        const int mylen = (todo >> lane) & 1ull ? (int)(hi - lo) : 0;
+        const int upto = wave_inclusive_scan(mylen);           // entries of the short slices of lanes 0..lane
+        const int total = __builtin_amdgcn_readlane(upto, 63);
+        // the entries e0 + 64 x + lane: where they lie in B, whose they are, and their loads
+        const auto fetch = [&](int e0, bool *ok, int64_t *q, double *at, int *pt, int *j, double *v) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int t = todo ? __builtin_ctzll(todo) : -1;
-            todo = todo ? (todo & (todo - 1)) : 0;
-            pick = quarter == g ? t : pick;
-        }
-        const int src = pick < 0 ? lane : pick;
-        const int64_t s = ((int64_t)__shfl((int)(lo >> 32), src, 64) << 32) |
-                          (uint32_t)__shfl((int)(lo & 0xffffffff), src, 64);
-        const int64_t e = ((int64_t)__shfl((int)(hi >> 32), src, 64) << 32) |
-                          (uint32_t)__shfl((int)(hi & 0xffffffff), src, 64);
-        const double at = __hiloint2double(__shfl(__double2hiint(a), src, 64), __shfl(__double2loint(a), src, 64));
-        const int pt = __shfl(pa, src, 64);
-        int64_t q[SG_SHORT_LOADS];
+            for (int x = 0; x < SG_SHORT_LOADS; ++x) {
+                const int e = e0 + 64 * x + lane;
+                ok[x] = e < total;
+                int l = 0, h = 63;                  // the first lane whose running sum exceeds e
+#pragma unroll
+                for (int step = 0; step < 6; ++step) {
+                    const int mid = (l + h) >> 1;
+                    const bool right = __shfl(upto, mid, 64) <= e;
+                    l = right ? mid + 1 : l;
+                    h = right ? h : mid;
+                }
+                const int t = ok[x] ? l : lane;
+                const int before = __shfl(upto - mylen, t, 64);
+                const int64_t s = ((int64_t)__shfl((int)(lo >> 32), t, 64) << 32) |
+                                  (uint32_t)__shfl((int)(lo & 0xffffffff), t, 64);
+                q[x] = ok[x] ? s + (e - before) : 0;
+                at[x] = __hiloint2double(__shfl(__double2hiint(a), t, 64), __shfl(__double2loint(a), t, 64));
+                pt[x] = __shfl(pa, t, 64);
+            }
+#pragma unroll
+            for (int x = 0; x < SG_SHORT_LOADS; ++x)
+                j[x] = (ok[x] ? (int)Bcrd[q[x]] : 0);
+#pragma unroll
+            for (int x = 0; x < SG_SHORT_LOADS; ++x)
+                v[x] = (VALUES && ok[x] ? Bval[q[x]] : 0.0);
+        };
         bool ok[SG_SHORT_LOADS];
+        int64_t q[SG_SHORT_LOADS];
+        double at[SG_SHORT_LOADS], v[SG_SHORT_LOADS];
+        int pt[SG_SHORT_LOADS], j[SG_SHORT_LOADS];
+        fetch(0, ok, q, at, pt, j, v);
+        for (int e0 = 0; e0 < total; e0 += 64 * SG_SHORT_LOADS) {
+            // the next batch's loads are in flight while this one's products go into LDS
+            bool okn[SG_SHORT_LOADS];
+            int64_t qn[SG_SHORT_LOADS];
+            double atn[SG_SHORT_LOADS], vn[SG_SHORT_LOADS];
+            int ptn[SG_SHORT_LOADS], jn[SG_SHORT_LOADS];
+            const bool more = e0 + 64 * SG_SHORT_LOADS < total;
+            if (more)
+                fetch(e0 + 64 * SG_SHORT_LOADS, okn, qn, atn, ptn, jn, vn);
 #pragma unroll
-        for (int x = 0; x < SG_SHORT_LOADS; ++x) {
-            ok[x] = pick >= 0 && s + sub + 16 * x < e;
-            q[x] = ok[x] ? s + sub + 16 * x : 0;
-        }
-        int j[SG_SHORT_LOADS];
-        double v[SG_SHORT_LOADS];
+            for (int x = 0; x < SG_SHORT_LOADS; ++x) {
+                if (ok[x]) {
+                    f(j[x], at[x], v[x], pt[x], q[x]);
+                }
+            }
+            if (more) {
 #pragma unroll
-        for (int x = 0; x < SG_SHORT_LOADS; ++x)
-            j[x] = (ok[x] ? (int)Bcrd[q[x]] : 0);
-#pragma unroll
-        for (int x = 0; x < SG_SHORT_LOADS; ++x)
-            v[x] = (VALUES && ok[x] ? Bval[q[x]] : 0.0);
-#pragma unroll
-        for (int x = 0; x < SG_SHORT_LOADS; ++x) {
-            if (ok[x]) {
-                f(j[x], at, v[x], pt, q[x]);
+                for (int x = 0; x < SG_SHORT_LOADS; ++x) {
+                    ok[x] = okn[x];
+                    q[x] = qn[x];
+                    at[x] = atn[x];
+                    v[x] = vn[x];
+                    pt[x] = ptn[x];
+                    j[x] = jn[x];
+                }
             }
         }
     }
