@@ -1969,7 +1969,10 @@ __global__ void eltwise_mult_dense_kernel(int64_t nrows, const int64_t *__restri
 
 // ------------------------------------------------------------------ host side
 // ---------------------------------------------------------------------------
-// Masked products as dot products over the mask.  C<M>[i][j] = sum over k of A[i][k] * B[k][j] is the dot product of
+// Masked products as dot products over the mask (the reference's masked Gustavson nest,
+// lib/Conversion/IndexTreeToSCF/IndexTreeToSCF.cpp:1083-1148 and :1327-1448, walks every product of row i and tests
+// its column against the mask row's mark array; C keeps the mask's entries that received a product, in mask order -
+// what comes out here is the same set and, per entry, the same sum).  C<M>[i][j] = sum over k of A[i][k] * B[k][j] is the dot product of
 // row i of A and column j of B; walking the products of row i (every entry of every B_k, k in A_i) costs |B_k|
 // look-ups per entry of A_i whatever the mask holds, the dot product of a stored pair (i, j) costs the shorter of
 // its two lists when that one is streamed against a table of the longer one.  So the pairs of the mask are split
