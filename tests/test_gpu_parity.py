@@ -524,6 +524,24 @@ def test_spgemm_masked_dot_products_semirings(semiring):
     _spgemm_check(a, b, m, mask=(mk[0], mk[1]))        # plus-times afterwards finds nothing left behind
 
 
+def test_spgemm_masked_inner_dimension_beyond_the_table():
+    """More than 2^20 columns of A (= rows of B): the table over k of the dot-product form does not fit LDS, and the
+    masked product is walked by rows."""
+    rng = np.random.default_rng(5)
+    n, k, m = 40, (1 << 20) + 77, 300
+    cols = np.sort(rng.choice(k, 2000, replace=False))            # the inner indices that are used at all
+    a = _rows_of_lengths(rng, rng.integers(0, 60, n), k, pick=cols)
+    lb = np.zeros(k, dtype=np.int64); lb[cols] = rng.integers(0, 8, len(cols))
+    b = _rows_of_lengths(rng, lb, m)
+    mk = _rand_csr(rng, n, m, 0.5, signed=False)
+    rt.profile_reset(); rt.profile_enable(True)
+    _spgemm_check(a, b, m, mask=(mk[0], mk[1]))
+    rt.sync()
+    fired = rt.profile_report()
+    rt.profile_enable(False)
+    assert not any("dot" in name for name in fired), sorted(fired)
+
+
 def test_spgemm_masked_dot_products_hubs_and_repeats():
     """Lists of very different lengths (a few rows of A and columns of B with thousands of entries among short ones:
     each half of the pairs has work), and a matrix that holds a column twice in a row, which the tables cannot
