@@ -1220,6 +1220,118 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
     return touched;
 }
 
+// One product a * b for column j of the block that begins at column col0 (j counts from there with 16-bit columns):
+// its bit is set and it is added to the column's accumulator in LDS.
+template <bool SEMI, typename COL>
+__device__ __forceinline__ void dense_add(double *acc, uint32_t *bm, int col0, int j, double a, double b, int pa,
+                                          int64_t q, int reduce_op, int mult_op)
+{
+    if constexpr (sizeof(COL) == 4)
+        j -= col0;
+    atomicOr(&bm[j >> 5], 1u << (j & 31));
+    if constexpr (SEMI)
+        semiring_lds_add(&acc[j], reduce_op, mult_op, a, b, pa, q);
+    else
+        __hip_atomic_fetch_add(&acc[j], a * b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+// the block's value of column j, which is cleared (as: where the row of A begins, for the semirings that keep places)
+template <bool SEMI>
+__device__ __forceinline__ double dense_take(double *acc, int j, int reduce_op, int mult_op, int64_t as,
+                                             const double *__restrict__ Aval, const double *__restrict__ Bval)
+{
+    double out;
+    if constexpr (SEMI)
+        out = semiring_lds_value(reinterpret_cast<unsigned long long *>(acc)[j], reduce_op, mult_op, as, Aval, Bval);
+    else
+        out = acc[j];
+    acc[j] = 0.0;
+    return out;
+}
+
+// Writes out the block of SG_CB columns a workgroup holds in LDS (bitmap bm, accumulators read and cleared through
+// take) as sorted entries of C and leaves the bitmap clean; returns how many.  place(total), which every thread
+// calls once the number of entries is known, says where in Ccrd / Cval the first of them goes.  With MASKED the
+// columns that are not set in mb are dropped and mb is cleared as well.
+template <bool MASKED, typename TAKE, typename PLACE>
+__device__ __forceinline__ int dense_emit_block(uint32_t *bm, uint32_t *mb, double *acc, emit_t *emit_col,
+                                                int *wave_tot, int lane, int wave, int col0,
+                                                int32_t *__restrict__ Ccrd, double *__restrict__ Cval, TAKE take,
+                                                PLACE place)
+{
+    // Thread t owns the columns [8t, 8t + 8) and [8192 + 8t, 8192 + 8t + 8): one byte from each half of the bitmap,
+    // so that the dense low columns of a half (the columns of a power-law graph thin out with the number of set
+    // bits of the id) are spread over all the wavefronts.  The counts of the two bytes are scanned together,
+    // packed into one word.
+    static_assert(SG_T * 16 == SG_CB && SG_WAVES <= 64, "one byte of each half of the bitmap per thread");
+    const uint8_t *bm8 = reinterpret_cast<const uint8_t *>(bm);
+    uint32_t bits_a = bm8[threadIdx.x], bits_b = bm8[SG_CB / 16 + threadIdx.x];
+    const int jbase = (int)threadIdx.x << 3;
+    if constexpr (MASKED) {          // columns outside the mask row are dropped here
+        const uint8_t *mb8 = reinterpret_cast<const uint8_t *>(mb);
+        const uint32_t keep_a = mb8[threadIdx.x], keep_b = mb8[SG_CB / 16 + threadIdx.x];
+        for (uint32_t w = bits_a & ~keep_a; w; w &= w - 1)
+            acc[jbase + __ffs(w) - 1] = 0.0;
+        for (uint32_t w = bits_b & ~keep_b; w; w &= w - 1)
+            acc[SG_CB / 2 + jbase + __ffs(w) - 1] = 0.0;
+        bits_a &= keep_a;
+        bits_b &= keep_b;
+    }
+    const int mine = __popc(bits_a) | (__popc(bits_b) << 16);
+    const int inc = wave_inclusive_scan(mine);
+    if (lane == 63)
+        wave_tot[wave] = inc;
+    lds_barrier();
+    const int tots = wave_inclusive_scan(lane < SG_WAVES ? wave_tot[lane] : 0);
+    const int all = __builtin_amdgcn_readlane(tots, SG_WAVES - 1);
+    const int before = (wave ? __builtin_amdgcn_readlane(tots, wave - 1) : 0) + inc - mine;
+    const int total_a = all & 0xffff, total = total_a + (all >> 16);
+    const int first_a = before & 0xffff, first_b = total_a + (before >> 16);
+    const int64_t off = place(total);
+    if (threadIdx.x < SG_CB / 32) {    // everybody has read its bytes: the bitmap is clean for the next block,
+        bm[threadIdx.x] = 0;           // which nobody enters before the barrier below
+        if constexpr (MASKED)
+            mb[threadIdx.x] = 0;
+    }
+    // The owner of a byte knows where its columns go, but writing them from there would scatter every store over
+    // 64 cache lines.  So the columns are listed in LDS, SG_EMIT at a time, and then every lane writes the entry
+    // at its own place in the list: coalesced stores.
+    if (total <= SG_EMIT) {         // the usual case: the whole block fits the list
+        int at = first_a;
+        for (uint32_t w = bits_a; w; w &= w - 1, ++at)
+            emit_col[at] = (emit_t)(jbase + __ffs(w) - 1);
+        at = first_b;
+        for (uint32_t w = bits_b; w; w &= w - 1, ++at)
+            emit_col[at] = (emit_t)(SG_CB / 2 + jbase + __ffs(w) - 1);
+        lds_barrier();
+        for (int q = threadIdx.x; q < total; q += SG_T) {
+            const int j = emit_col[q];
+            store_streaming(&Ccrd[off + q], col0 + j);
+            store_streaming(&Cval[off + q], take(j));
+        }
+        lds_barrier();
+    } else {
+        for (int c0 = 0; c0 < total; c0 += SG_EMIT) {
+            int at = first_a - c0;
+            for (uint32_t w = bits_a; w; w &= w - 1, ++at)
+                if (at >= 0 && at < SG_EMIT)
+                    emit_col[at] = (emit_t)(jbase + __ffs(w) - 1);
+            at = first_b - c0;
+            for (uint32_t w = bits_b; w; w &= w - 1, ++at)
+                if (at >= 0 && at < SG_EMIT)
+                    emit_col[at] = (emit_t)(SG_CB / 2 + jbase + __ffs(w) - 1);
+            lds_barrier();
+            const int n = total - c0 < SG_EMIT ? total - c0 : SG_EMIT;
+            for (int q = threadIdx.x; q < n; q += SG_T) {
+                const int j = emit_col[q];
+                store_streaming(&Ccrd[off + c0 + q], col0 + j);
+                store_streaming(&Cval[off + c0 + q], take(j));
+            }
+            lds_barrier();
+        }
+    }
+    return total;
+}
+
 // MASKED (C<M> = A*B, for the rows whose mask row is too long for the slab kernel's hash table): every product is
 // added as without a mask - the LDS adds are not what this kernel waits for - and the mask row decides what leaves:
 // before a block's products are walked, the mask row's entries inside the block are set in a bitmap of their own
@@ -1314,24 +1426,9 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                 }
                 int touched = 0;     // did this wavefront add anything to the block
                 const auto add = [&](int j, double a, double b, int pa, int64_t q) {
-                    if constexpr (sizeof(COL) == 4)
-                        j -= col0;
-                    atomicOr(&bm[j >> 5], 1u << (j & 31));
-                    if constexpr (SEMI)
-                        semiring_lds_add(&acc[j], reduce_op, mult_op, a, b, pa, q);
-                    else
-                        __hip_atomic_fetch_add(&acc[j], a * b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    dense_add<SEMI, COL>(acc, bm, col0, j, a, b, pa, q, reduce_op, mult_op);
                 };
-                const auto take = [&](int j) -> double {         // the block's value of column j, which is cleared
-                    double out;
-                    if constexpr (SEMI)
-                        out = semiring_lds_value(reinterpret_cast<unsigned long long *>(acc)[j], reduce_op, mult_op, as,
-                                                 Aval, Bval);
-                    else
-                        out = acc[j];
-                    acc[j] = 0.0;
-                    return out;
-                };
+                const auto take = [&](int j) { return dense_take<SEMI>(acc, j, reduce_op, mult_op, as, Aval, Bval); };
                 if (held) {
                     int64_t next = h_hi;
                     if (h_bp && cb + 1 < nblk)
@@ -1359,77 +1456,8 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                 const int any = visit_flag(block_touched, visit, touched, lane);
                 visit = visit == 2 ? 0 : visit + 1;
                 if (any) {
-                // Emit this block.  Thread t owns the columns [8t, 8t + 8) and [8192 + 8t, 8192 + 8t + 8): one
-                // byte from each half of the bitmap, so that the dense low columns of a half (the columns of a
-                // power-law graph thin out with the number of set bits of the id) are spread over all the
-                // wavefronts.  The counts of the two bytes are scanned together, packed into one word.
-                static_assert(SG_T * 16 == SG_CB && SG_WAVES <= 64, "one byte of each half of the bitmap per thread");
-                const uint8_t *bm8 = reinterpret_cast<const uint8_t *>(bm);
-                uint32_t bits_a = bm8[threadIdx.x], bits_b = bm8[SG_CB / 16 + threadIdx.x];
-                const int jbase = (int)threadIdx.x << 3;
-                if constexpr (MASKED) {          // columns outside the mask row are dropped here
-                    const uint8_t *mb8 = reinterpret_cast<const uint8_t *>(mb);
-                    const uint32_t keep_a = mb8[threadIdx.x], keep_b = mb8[SG_CB / 16 + threadIdx.x];
-                    for (uint32_t w = bits_a & ~keep_a; w; w &= w - 1)
-                        acc[jbase + __ffs(w) - 1] = 0.0;
-                    for (uint32_t w = bits_b & ~keep_b; w; w &= w - 1)
-                        acc[SG_CB / 2 + jbase + __ffs(w) - 1] = 0.0;
-                    bits_a &= keep_a;
-                    bits_b &= keep_b;
-                }
-                const int mine = __popc(bits_a) | (__popc(bits_b) << 16);
-                const int inc = wave_inclusive_scan(mine);
-                if (lane == 63)
-                    wave_tot[wave] = inc;
-                lds_barrier();
-                const int tots = wave_inclusive_scan(lane < SG_WAVES ? wave_tot[lane] : 0);
-                const int all = __builtin_amdgcn_readlane(tots, SG_WAVES - 1);
-                const int before = (wave ? __builtin_amdgcn_readlane(tots, wave - 1) : 0) + inc - mine;
-                const int total_a = all & 0xffff, total = total_a + (all >> 16);
-                const int first_a = before & 0xffff, first_b = total_a + (before >> 16);
-                if (threadIdx.x < SG_CB / 32) {    // everybody has read its bytes: the bitmap is clean for the
-                    bm[threadIdx.x] = 0;           // next block, which nobody enters before the barrier below
-                    if constexpr (MASKED)
-                        mb[threadIdx.x] = 0;
-                }
-                // The owner of a byte knows where its columns go, but writing them from there would scatter
-                // every store over 64 cache lines.  So the columns are listed in LDS, SG_EMIT at a time, and
-                // then every lane writes the entry at its own place in the list: coalesced stores.
-                if (total <= SG_EMIT) {         // the usual case: the whole block fits the list
-                    int at = first_a;
-                    for (uint32_t w = bits_a; w; w &= w - 1, ++at)
-                        emit_col[at] = (emit_t)(jbase + __ffs(w) - 1);
-                    at = first_b;
-                    for (uint32_t w = bits_b; w; w &= w - 1, ++at)
-                        emit_col[at] = (emit_t)(SG_CB / 2 + jbase + __ffs(w) - 1);
-                    lds_barrier();
-                    for (int q = threadIdx.x; q < total; q += SG_T) {
-                        const int j = emit_col[q];
-                        store_streaming(&Ccrd[off + q], col0 + j);
-                        store_streaming(&Cval[off + q], take(j));
-                    }
-                    lds_barrier();
-                } else {
-                for (int c0 = 0; c0 < total; c0 += SG_EMIT) {
-                    int at = first_a - c0;
-                    for (uint32_t w = bits_a; w; w &= w - 1, ++at)
-                        if (at >= 0 && at < SG_EMIT)
-                            emit_col[at] = (emit_t)(jbase + __ffs(w) - 1);
-                    at = first_b - c0;
-                    for (uint32_t w = bits_b; w; w &= w - 1, ++at)
-                        if (at >= 0 && at < SG_EMIT)
-                            emit_col[at] = (emit_t)(SG_CB / 2 + jbase + __ffs(w) - 1);
-                    lds_barrier();
-                    const int n = total - c0 < SG_EMIT ? total - c0 : SG_EMIT;
-                    for (int q = threadIdx.x; q < n; q += SG_T) {
-                        const int j = emit_col[q];
-                        store_streaming(&Ccrd[off + c0 + q], col0 + j);
-                        store_streaming(&Cval[off + c0 + q], take(j));
-                    }
-                    lds_barrier();
-                }
-                }
-                off += total;
+                    off += dense_emit_block<MASKED>(bm, mb, acc, emit_col, wave_tot, lane, wave, col0, Ccrd, Cval,
+                                                    take, [&](int) { return off; });
                 } else if constexpr (MASKED) {   // the block received no product
                     if (threadIdx.x < SG_CB / 32)        // (the next block's bits go to the other half; the one after
                         mb[threadIdx.x] = 0;             // that comes after the next block's barrier)
@@ -1437,6 +1465,210 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
             }
         }
         t = draw_row<true>(ticket, t_first, &row_slot);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// The same rows, block by block: the kernel above takes a row through its column blocks, so at any time the
+// workgroups of an XCD read the slices of every block and the long rows of B, which most products come from,
+// never stay in its L2 (a few hundred rows of an R-MAT graph make over half of the products, but they hold
+// tens of megabytes).  Here the tickets go over (column block, row) with the block outermost: all workgroups
+// are in the same block at the same time and what they share is that block's slices of the long rows only.
+// A row's entries inside a block then leave before the blocks ahead of it are counted, so where they go is
+// handed from block to block: before[r * nblk + cb] = the row's entries ahead of block cb, written by the
+// workgroup that counted block cb - 1 and awaited by the one that writes block cb.  That one holds a later
+// ticket, and a workgroup only ever waits for earlier tickets, which running workgroups hold: the one with the
+// earliest unfinished ticket waits for nobody.  The wait is bounded all the same (`patience` polls, after
+// which *gave_up is set and the row is wrong: the host then fails the call).
+// A ticket is DB_ROWS consecutive rows of the list, so that the loads which lead to a row's slices (its entries
+// of A, their block pointers) are issued while the row before is walked.
+// ---------------------------------------------------------------------------
+struct DenseRow {
+    int64_t as;         // first entry of the row of A
+    int64_t coff;       // first entry of the row of C, counted from the row block's
+    int32_t cnt;        // entries of the row of A
+    int32_t pad;
+};
+constexpr int DB_ROWS = 8;
+constexpr int DB_PATIENCE = 1 << 24;
+
+// rows[r] for the nd first rows of the list and before[] in its initial state: nothing ahead of block 0, the rest open
+__global__ void spgemm_dense_rows(int64_t row_begin, RowList list, int64_t nd, int nblk, const int64_t *__restrict__ Apos,
+                                  const int64_t *__restrict__ Cpos, DenseRow *__restrict__ rows,
+                                  int32_t *__restrict__ before)
+{
+    const int64_t x = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (x < nd * nblk)
+        before[x] = x % nblk == 0 ? 0 : -1;
+    if (x < nd) {
+        const int64_t i = row_begin + list.rows[x];
+        DenseRow r;
+        r.as = Apos[i];
+        r.cnt = (int32_t)(Apos[i + 1] - r.as < (1ll << 30) ? Apos[i + 1] - r.as : (1ll << 30));
+        r.coff = Cpos[i] - Cpos[row_begin];
+        r.pad = 0;
+        rows[x] = r;
+    }
+}
+
+template <bool SEMI, typename COL>
+__global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_blocks_kernel(
+    const DenseRow *__restrict__ rows, int64_t nd, const int32_t *__restrict__ Acrd, const double *__restrict__ Aval,
+    const COL *__restrict__ Bcrd, const double *__restrict__ Bval, const int64_t *__restrict__ blkptr, int nblk,
+    unsigned long long *ticket, int32_t *before, int patience, int *gave_up, int32_t *__restrict__ Ccrd,
+    double *__restrict__ Cval, int reduce_op, int mult_op)
+{
+    __shared__ int64_t row_slot;
+    __shared__ int wave_tot[SG_WAVES];
+    __shared__ int block_touched[3];            // see visit_flag
+    __shared__ int ahead_slot;                  // the row's entries ahead of the block
+    double *acc = reinterpret_cast<double *>(sg_dyn_lds);
+    uint32_t *bm = sg_dyn_lds + SG_CB * 2;
+    emit_t *emit_col = reinterpret_cast<emit_t *>(bm + SG_CB / 32);
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    for (int j = threadIdx.x; j < SG_CB; j += SG_T)
+        acc[j] = 0.0;
+    if (threadIdx.x < SG_CB / 32)
+        bm[threadIdx.x] = 0;
+    if (threadIdx.x < 3)
+        block_touched[threadIdx.x] = 0;
+    lds_barrier();
+    int visit = 0;
+    const int64_t nchunks = (nd + DB_ROWS - 1) / DB_ROWS;
+    const int64_t u_end = nchunks * nblk;
+    int64_t u = draw_row<true>(ticket, 0, &row_slot);
+    while (u < u_end) {
+        const int cb = (int)(u / nchunks);
+        const int64_t r0 = (u - cb * nchunks) * DB_ROWS;
+        const int nr = (int)(nd - r0 < DB_ROWS ? nd - r0 : DB_ROWS);
+        const int col0 = cb << SG_CB_LOG;
+        DenseRow mine;
+        mine.as = mine.coff = 0;
+        mine.cnt = 0;
+        if (lane < nr)
+            mine = rows[r0 + lane];
+        // the entry of A a lane holds of row x of the ticket (of its first SG_T entries: a longer row loads the others
+        // as it goes), and the slice of its row of B inside the block
+        const auto load_entry = [&](int x, int &k, double &a) {
+            k = -1;
+            a = 0.0;
+            if (x < nr) {
+                const int cnt = __builtin_amdgcn_readlane(mine.cnt, x);
+                const int p = wave + lane * SG_WAVES;
+                if (p < cnt) {
+                    const int64_t as = ((int64_t)__builtin_amdgcn_readlane((int)(mine.as >> 32), x) << 32) |
+                                       (uint32_t)__builtin_amdgcn_readlane((int)mine.as, x);
+                    k = Acrd[as + p];
+                    a = Aval[as + p];
+                }
+            }
+        };
+        const auto load_slice = [&](int k, int64_t &lo, int64_t &hi) {
+            lo = hi = 0;
+            if (k >= 0) {
+                const int64_t *bp = blkptr + (int64_t)k * (nblk + 1) + cb;
+                lo = bp[0];
+                hi = bp[1];
+            }
+        };
+        int k0, k1, k2;
+        double a0, a1, a2;
+        int64_t lo0, hi0, lo1, hi1;
+        load_entry(0, k0, a0);
+        load_entry(1, k1, a1);
+        load_slice(k0, lo0, hi0);
+        for (int x = 0; x < nr; ++x) {
+            load_slice(k1, lo1, hi1);
+            load_entry(x + 2, k2, a2);
+            const int cnt = __builtin_amdgcn_readlane(mine.cnt, x);
+            const int64_t as = ((int64_t)__builtin_amdgcn_readlane((int)(mine.as >> 32), x) << 32) |
+                               (uint32_t)__builtin_amdgcn_readlane((int)mine.as, x);
+            const int64_t coff = ((int64_t)__builtin_amdgcn_readlane((int)(mine.coff >> 32), x) << 32) |
+                                 (uint32_t)__builtin_amdgcn_readlane((int)mine.coff, x);
+            const auto add = [&](int j, double a, double b, int pa, int64_t q) {
+                dense_add<SEMI, COL>(acc, bm, col0, j, a, b, pa, q, reduce_op, mult_op);
+            };
+            const auto take = [&](int j) { return dense_take<SEMI>(acc, j, reduce_op, mult_op, as, Aval, Bval); };
+            // What lies ahead of this block comes from whoever counted the block before it.  That was many tickets
+            // ago as a rule, so the answer is asked for before the walk and the trip to memory it takes is over by
+            // the time the walk is; only if it was not there yet is it waited for, behind the walk.
+            int32_t *mark = before + (r0 + x) * nblk + cb;
+            int early = 0;
+            if (threadIdx.x == 0 && cb > 0)
+                early = __hip_atomic_fetch_max(mark, -1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int mine_p = wave + lane * SG_WAVES;          // the entry this lane holds of a batch of SG_T
+            int touched = for_each_in_slices<true>(lo0, hi0, a0, mine_p + 1, lane, Bcrd, Bval, add);
+            if (cnt > SG_T) {
+                // the entries of A beyond the first SG_T, SG_T at a time: a batch's entries are loaded two batches
+                // ahead and its slices one, so that a walk does not begin with two trips to memory
+                const auto load_more = [&](int base, int &k, double &a) {
+                    k = -1;
+                    a = 0.0;
+                    if (base + mine_p < cnt) {
+                        k = Acrd[as + base + mine_p];
+                        a = Aval[as + base + mine_p];
+                    }
+                };
+                int kb, kn;
+                double ab, an;
+                int64_t lob, hib;
+                load_more(SG_T, kb, ab);
+                load_more(2 * SG_T, kn, an);
+                load_slice(kb, lob, hib);
+                for (int base = SG_T; base < cnt; base += SG_T) {
+                    int64_t lon, hin;
+                    load_slice(kn, lon, hin);
+                    int k2;
+                    double a2;
+                    load_more(base + 2 * SG_T, k2, a2);
+                    touched |= for_each_in_slices<true>(lob, hib, ab, base + mine_p + 1, lane, Bcrd, Bval, add);
+                    lob = lon;
+                    hib = hin;
+                    ab = an;
+                    kn = k2;
+                    an = a2;
+                }
+            }
+            const int any = visit_flag(block_touched, visit, touched, lane);
+            visit = visit == 2 ? 0 : visit + 1;
+            const auto await = [&]() {
+                int ahead = early;
+                for (int polls = 1; ahead < 0 && polls < patience; ++polls) {
+                    __builtin_amdgcn_s_sleep(4);
+                    ahead = __hip_atomic_fetch_max(mark, -1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                if (ahead < 0) {
+                    __hip_atomic_store(gave_up, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ahead = 0;
+                }
+                return ahead;
+            };
+            const auto hand_on = [&](int ahead) {
+                if (cb + 1 < nblk)
+                    __hip_atomic_exchange(mark + 1, ahead, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            };
+            if (any) {
+                if (threadIdx.x == 0)
+                    ahead_slot = await();          // (read behind the first barrier of the write-out)
+                dense_emit_block<false>(bm, nullptr, acc, emit_col, wave_tot, lane, wave, col0, Ccrd, Cval, take,
+                                        [&](int total) {
+                                            const int ahead = ahead_slot;
+                                            if (threadIdx.x == 0)
+                                                hand_on(ahead + total);
+                                            return coff + ahead;
+                                        });
+            } else if (threadIdx.x == 0) {
+                hand_on(await());
+            }
+            k0 = k1;
+            a0 = a1;
+            lo0 = lo1;
+            hi0 = hi1;
+            k1 = k2;
+            a1 = a2;
+        }
+        u = draw_row<true>(ticket, 0, &row_slot);
     }
 }
 
@@ -2414,6 +2646,9 @@ struct SgScratch {
     Workspace gbm;        // global bitmaps (only when the bitmap does not fit LDS)
     Workspace gmask;      // global mask bitmaps (masked numeric)
     Workspace slabs;      // dense accumulators, zero between calls
+    Workspace dense_rows;     // DenseRow[] and before[] of spgemm_numeric_dense_blocks_kernel
+    Workspace dense_before;
+    Workspace gave_up;        // its flag, zero between calls
 };
 static SgScratch g_sg;
 
@@ -2859,7 +3094,49 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
 #undef LAUNCH_NUM_S
 #undef LAUNCH_NUM
     COMET_HIPCHK(hipGetLastError());
-    if (dense || mdense) {
+    // the rows of the one-block kernel block by block (COMET_HIP_SPGEMM_ROW_MAJOR keeps them row by row; the
+    // tests run both)
+    const bool by_blocks = dense && a->nnz < (1ll << 31) && getenv("COMET_HIP_SPGEMM_ROW_MAJOR") == nullptr;
+    bool ran_blocks = false;
+    if (by_blocks) {
+        int64_t nd = 0;
+        COMET_HIPCHK(hipMemcpyAsync(&nd, list.bounds + 2, sizeof(int64_t), hipMemcpyDeviceToHost, stream()));
+        COMET_HIPCHK(hipStreamSynchronize(stream()));
+        if (nd > 0) {
+            ran_blocks = true;
+            COMET_CHK(g_sg.dense_rows.ensure(sizeof(DenseRow) * (size_t)nd, false));
+            COMET_CHK(g_sg.dense_before.ensure(sizeof(int32_t) * (size_t)nd * (size_t)nblk, false));
+            COMET_CHK(g_sg.gave_up.ensure(sizeof(int), true));
+            COMET_CHK(sg_reset_ticket());
+            int patience = DB_PATIENCE;
+            if (const char *e = getenv("COMET_HIP_SPGEMM_PATIENCE"))
+                patience = atoi(e);
+            KernelTimer t("spgemm_numeric_dense_blocks");
+            const dim3 cus((unsigned)(num_cus() > 0 ? num_cus() : 256));
+            spgemm_dense_rows<<<dim3((unsigned)ceil_div(nd * nblk, 256)), dim3(256), 0, stream()>>>(
+                rb, list, nd, nblk, a->pos, Cpos, (DenseRow *)g_sg.dense_rows.ptr, (int32_t *)g_sg.dense_before.ptr);
+#define LAUNCH_BLOCKS_C(S, COL, CRD)                                                                       \
+    do {                                                                                                   \
+        COMET_CHK(sg_allow_lds(spgemm_numeric_dense_blocks_kernel<S, COL>, SG_DENSE_LDS));                 \
+        spgemm_numeric_dense_blocks_kernel<S, COL><<<cus, block, SG_DENSE_LDS, stream()>>>(                \
+            (const DenseRow *)g_sg.dense_rows.ptr, nd, a->crd, a->val, CRD, b->val, b->sg_blkptr, nblk,    \
+            (unsigned long long *)g_sg.ticket.ptr, (int32_t *)g_sg.dense_before.ptr, patience,             \
+            (int *)g_sg.gave_up.ptr, Ccrd, Cval, reduce_op, mult_op);                                      \
+    } while (0)
+#define LAUNCH_BLOCKS(S)                                                                                   \
+    do {                                                                                                   \
+        if (b->sg_crd16 && getenv("COMET_HIP_SPGEMM_WIDE_COLUMNS") == nullptr)                             \
+            LAUNCH_BLOCKS_C(S, uint16_t, b->sg_crd16);                                                     \
+        else                                                                                               \
+            LAUNCH_BLOCKS_C(S, int32_t, b->crd);                                                           \
+    } while (0)
+            if (semi) LAUNCH_BLOCKS(true); else LAUNCH_BLOCKS(false);
+#undef LAUNCH_BLOCKS_C
+#undef LAUNCH_BLOCKS
+            COMET_HIPCHK(hipGetLastError());
+        }
+    }
+    if ((dense && !by_blocks) || mdense) {
         COMET_CHK(sg_reset_ticket());
         KernelTimer t(mdense ? "spgemm_numeric_dense_masked" : "spgemm_numeric_dense");
         const dim3 cus((unsigned)(num_cus() > 0 ? num_cus() : 256));
@@ -2903,6 +3180,15 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
                 (unsigned long long *)g_sg.ticket.ptr, list, Cpos, Ccrd, Cval, reduce_op, mult_op);
         }
         COMET_HIPCHK(hipGetLastError());
+    }
+    if (ran_blocks) {           // did a workgroup stop waiting for the block before its own
+        int gave_up = 0;
+        COMET_HIPCHK(hipMemcpyAsync(&gave_up, g_sg.gave_up.ptr, sizeof(int), hipMemcpyDeviceToHost, stream()));
+        COMET_HIPCHK(hipStreamSynchronize(stream()));
+        if (gave_up) {
+            COMET_HIPCHK(hipMemsetAsync(g_sg.gave_up.ptr, 0, sizeof(int), stream()));
+            return set_error(COMET_HIP_ERR_HIP, "spgemm numeric: a column block's place in its row never arrived");
+        }
     }
     return COMET_HIP_OK;
 }

@@ -610,11 +610,12 @@ def _rows_of_lengths(rng, lengths, ncols, pick=None, signed=True):
     return pos, crd.astype(np.int64), val
 
 
+@pytest.mark.parametrize("row_major", [False, True])
 @pytest.mark.parametrize("m,long_len,wide,cols32", [(200_000, 2000, None, False), (40_000, 1200, None, False),
                                                     (40_000, 1200, 1 << 40, False), (200_000, 2000, 1 << 40, False),
                                                     (200_000, 2000, 0, False), (200_000, 2000, 0, True),
                                                     (1_000_000, 3000, None, False), (1_000_000, 3000, None, True)])
-def test_spgemm_rows_of_every_class(m, long_len, wide, cols32, monkeypatch):
+def test_spgemm_rows_of_every_class(m, long_len, wide, cols32, row_major, monkeypatch):
     # Rows of B: 200 long ones and 200 of 10 entries.  Rows of A pick among them so that the product has rows
     # for each numeric kernel: no products, a few (values kept in a slab), thousands spread thinly over the
     # column blocks (several blocks per visit, values compact) and many per block (one block per visit).
@@ -622,7 +623,10 @@ def test_spgemm_rows_of_every_class(m, long_len, wide, cols32, monkeypatch):
     # kernel, and with 40,000 columns the thick rows then exceed the compact array, so their visits are cut
     # short at a block boundary; with 0 every heavy row takes one block per visit.
     # The one-block kernel reads B's columns as 16-bit numbers inside their block (a copy the library keeps with the
-    # block pointers), or with cols32 the 32-bit ones.
+    # block pointers), or with cols32 the 32-bit ones.  It takes its rows block by block, all rows through block 0
+    # first (a row's place in C is handed from block to block), or with row_major each row through all its blocks.
+    if row_major:
+        monkeypatch.setenv("COMET_HIP_SPGEMM_ROW_MAJOR", "1")
     if wide is not None:
         monkeypatch.setenv("COMET_HIP_SPGEMM_WIDE", str(wide))
     if cols32:
@@ -716,15 +720,37 @@ def test_spgemm_masked_long_mask_rows(semiring, monkeypatch):
     _spgemm_check((apos, acrd, aval), (bpos, bcrd, bval), m)        # and nothing is left behind for a plain product
 
 
-@pytest.mark.parametrize("wide", [1 << 40, 0])
-def test_spgemm_rows_with_more_entries_than_lanes(wide, monkeypatch):
+@pytest.mark.parametrize("wide,row_major", [(1 << 40, False), (0, False), (0, True)])
+def test_spgemm_rows_with_more_entries_than_lanes(wide, row_major, monkeypatch):
     # more than 1024 entries in a row of A: the LDS kernels then fetch the row's entries again at every visit
-    # instead of holding one per lane; `wide` sends the rows through either kernel
+    # instead of holding one per lane; `wide` sends the rows through either kernel, row_major the one-block
+    # kernel's rows one after the other instead of block by block
     monkeypatch.setenv("COMET_HIP_SPGEMM_WIDE", str(wide))
+    if row_major:
+        monkeypatch.setenv("COMET_HIP_SPGEMM_ROW_MAJOR", "1")
     rng = np.random.default_rng(23)
     k, m = 3000, 40_000
     b = _rows_of_lengths(rng, rng.integers(0, 17, k), m)
-    a = _rows_of_lengths(rng, [2500, 1100, 30, 0, 1025, 3000], k)
+    a = _rows_of_lengths(rng, [2500, 1100, 30, 0, 1025, 3000, 2049], k)
+    _spgemm_check(a, b, m)
+
+
+def test_spgemm_block_by_block_wait_is_bounded(monkeypatch):
+    # Block by block, the workgroup that writes a row's entries of one column block waits for the count of the
+    # block before, which another workgroup publishes.  The wait gives up after a number of polls (here: one, so
+    # that it may well do so), the kernel then still ends and the call fails with an error instead of returning a
+    # wrong product; the next call, with the usual patience, is right.
+    rng = np.random.default_rng(41)
+    k, m = 64, 100_000
+    b = _rows_of_lengths(rng, [3000] * k, m)
+    a = _rows_of_lengths(rng, [40] * 300, k)
+    monkeypatch.setenv("COMET_HIP_SPGEMM_WIDE", "0")
+    monkeypatch.setenv("COMET_HIP_SPGEMM_PATIENCE", "1")
+    try:
+        _spgemm_check(a, b, m)
+    except RuntimeError as e:
+        assert "never arrived" in str(e)
+    monkeypatch.delenv("COMET_HIP_SPGEMM_PATIENCE")
     _spgemm_check(a, b, m)
 
 
@@ -765,7 +791,7 @@ def test_spgemm_rmat_scale16_row_blocks_vs_checker():
     rt.sync()
     fired = rt.profile_report()
     rt.profile_enable(False)
-    for k in ("spgemm_numeric", "spgemm_numeric_span", "spgemm_numeric_dense"):
+    for k in ("spgemm_numeric", "spgemm_numeric_span", "spgemm_numeric_dense_blocks"):
         assert k in fired and fired[k][0] > 0, f"{k} never ran on these rows"
     assert checked > 50_000_000
     # the masked product C<A> = A*A on the same blocks (structure = mask entries that receive a product)
