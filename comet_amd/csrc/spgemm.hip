@@ -2842,10 +2842,11 @@ constexpr int64_t SG_DENSE_PER_BLOCK = 8;
 
 // Heavy rows with at least this many products per column block of the matrix stay with the block kernel, the
 // others go to the span kernel (measured on A*A of an R-MAT graph of scale 20, 64 blocks, ms per product:
-// 512 per block 583, 1024 572, 2048 559, 4096 557, 8192 570, every heavy row to the span kernel 604, none 613).
+// 512 per block 583, 1024 572, 2048 559, 4096 557, 8192 570, every heavy row to the span kernel 604, none 613;
+// with the kernels as they are now 1024 per block 437, 2048 402, 4096 386, 6144 381, 8192 382, 12288 382, 16384 389).
 // COMET_HIP_SPGEMM_WIDE, a number of products per row, overrides the rule: either kernel is right for any row,
 // so the tests use it to send the same rows through both.
-constexpr int64_t SG_WIDE_PER_BLOCK = 4096;
+constexpr int64_t SG_WIDE_PER_BLOCK = 6144;
 static int64_t sg_wide_threshold(int nblk)
 {
     const char *e = getenv("COMET_HIP_SPGEMM_WIDE");
