@@ -23,6 +23,8 @@
 // (spgemm_numeric_dense_kernel, the widest rows).
 // The order in which the products of one (i,j) are added is therefore not the
 // reference's ascending-k order: values agree to rounding, structure exactly.
+#include <type_traits>
+
 #include "common.h"
 
 namespace comet {
@@ -1041,6 +1043,7 @@ constexpr int SG_LONG_LOADS = 4;                  // entries of a long slice per
 // columns that the right-hand operand's plan keeps for the kernel that takes one block per visit: a third of the
 // bytes of an entry it only needs the column of.
 typedef unsigned short sg_h4u __attribute__((ext_vector_type(4), aligned(2)));
+typedef double sg_d2u __attribute__((ext_vector_type(2), aligned(8)));
 template <typename COL>
 struct SgCol4;
 template <>
@@ -1077,12 +1080,42 @@ __device__ __forceinline__ void turn_of_slice(int64_t s, int64_t o, int64_t len,
             f(j[x], at, v[x], pt, q[x]);
 }
 
-template <bool VALUES, typename COL, typename F>
-__device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double a, int pa, int lane,
-                                                  const COL *__restrict__ Bcrd,
-                                                  const double *__restrict__ Bval, F f)
+// A turn in which every lane has all its entries, the lane taking SG_LONG_LOADS consecutive ones (see the full turns of
+// for_each_in_slices): f4(j, a, v0, v1, pa, q) for the entries q .. q + 3.
+template <bool VALUES, typename COL, typename F4>
+__device__ __forceinline__ void full_turn_of_slice(int64_t s, int lane, double at, int pt, const COL *__restrict__ Bcrd,
+                                                   const double *__restrict__ Bval, F4 f4)
 {
     typedef typename SgCol4<COL>::type col4;
+    const int64_t c = s + 4 * (int64_t)lane;
+    const col4 j = *reinterpret_cast<const col4 *>(Bcrd + c);
+    sg_d2u v0 = {0.0, 0.0}, v1 = {0.0, 0.0};
+    if constexpr (VALUES) {
+        v0 = *reinterpret_cast<const sg_d2u *>(Bval + c);
+        v1 = *reinterpret_cast<const sg_d2u *>(Bval + c + 2);
+    }
+    f4(j, at, v0, v1, pt, c);
+}
+
+struct SgOneByOne {};          // in place of f4: the four entries of a lane in a full turn go through f one by one
+template <bool VALUES, typename COL, typename F, typename F4 = SgOneByOne>
+__device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double a, int pa, int lane,
+                                                  const COL *__restrict__ Bcrd,
+                                                  const double *__restrict__ Bval, F f, F4 f4 = F4())
+{
+    typedef typename SgCol4<COL>::type col4;
+    // f4(j, a, v0, v1, pa, q): the four consecutive entries q .. q + 3 of one row of B, columns j, values v0.x, v0.y,
+    // v1.x, v1.y
+    const auto four = [&](col4 j, double at, auto v0, auto v1, int pt, int64_t c) {
+        if constexpr (std::is_same<F4, SgOneByOne>::value) {
+            f((int)j.x, at, v0.x, pt, c);
+            f((int)j.y, at, v0.y, pt, c + 1);
+            f((int)j.z, at, v1.x, pt, c + 2);
+            f((int)j.w, at, v1.y, pt, c + 3);
+        } else {
+            f4(j, at, v0, v1, pt, c);
+        }
+    };
     // Long slices take the whole wavefront, one at a time; short ones (a slice of one block often holds a
     // dozen entries) are laid end to end and dealt to the lanes entry by entry (below).  A wavefront runs its
     // turns one after the other (there is room for one workgroup per CU, so nobody else hides the latency), and
@@ -1110,7 +1143,6 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
             // values per lane instead of four loads of each, a stride of 64 entries apart.  (Entries of B lie at any
             // 4- and 8-byte boundary: the loads are declared unaligned.)
             static_assert(SG_LONG_LOADS == 4, "a lane's entries of a full turn are one 16-byte load of columns");
-            typedef double sg_d2u __attribute__((ext_vector_type(2), aligned(8)));
             int64_t c = s + 4 * (int64_t)lane;          // this lane's first entry of the turn
             col4 j = *reinterpret_cast<const col4 *>(Bcrd + c);
             sg_d2u v0 = {0.0, 0.0}, v1 = {0.0, 0.0};
@@ -1127,20 +1159,14 @@ __device__ __forceinline__ int for_each_in_slices(int64_t lo, int64_t hi, double
                     v0n = *reinterpret_cast<const sg_d2u *>(Bval + cn);
                     v1n = *reinterpret_cast<const sg_d2u *>(Bval + cn + 2);
                 }
-                f((int)j.x, at, v0.x, pt, c);
-                f((int)j.y, at, v0.y, pt, c + 1);
-                f((int)j.z, at, v1.x, pt, c + 2);
-                f((int)j.w, at, v1.y, pt, c + 3);
+                four(j, at, v0, v1, pt, c);
                 j = jn;
                 v0 = v0n;
                 v1 = v1n;
                 c = cn;
                 done += 64 * SG_LONG_LOADS;
             }
-            f((int)j.x, at, v0.x, pt, c);
-            f((int)j.y, at, v0.y, pt, c + 1);
-            f((int)j.z, at, v1.x, pt, c + 2);
-            f((int)j.w, at, v1.y, pt, c + 3);
+            four(j, at, v0, v1, pt, c);
             done += 64 * SG_LONG_LOADS;
             o += done;
         }
@@ -1233,6 +1259,39 @@ __device__ __forceinline__ void dense_add(double *acc, uint32_t *bm, int col0, i
         semiring_lds_add(&acc[j], reduce_op, mult_op, a, b, pa, q);
     else
         __hip_atomic_fetch_add(&acc[j], a * b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+// Four consecutive entries of a row of B at once (columns ascending): the bits that fall into one word of the bitmap
+// go there together - lanes that walk a dense slice otherwise pile up on that word, four times each.
+template <bool SEMI, typename COL, typename J4, typename V2>
+__device__ __forceinline__ void dense_add4(double *acc, uint32_t *bm, int col0, J4 j4, double a, V2 v0, V2 v1, int pa,
+                                           int64_t q, int reduce_op, int mult_op)
+{
+    int j[4] = {(int)j4.x, (int)j4.y, (int)j4.z, (int)j4.w};
+    const double b[4] = {v0.x, v0.y, v1.x, v1.y};
+    if constexpr (sizeof(COL) == 4) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+            j[x] -= col0;
+    }
+    int w = j[0] >> 5;
+    uint32_t bits = 1u << (j[0] & 31);
+#pragma unroll
+    for (int x = 1; x < 4; ++x) {
+        if ((j[x] >> 5) != w) {
+            atomicOr(&bm[w], bits);
+            w = j[x] >> 5;
+            bits = 0u;
+        }
+        bits |= 1u << (j[x] & 31);
+    }
+    atomicOr(&bm[w], bits);
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        if constexpr (SEMI)
+            semiring_lds_add(&acc[j[x]], reduce_op, mult_op, a, b[x], pa, q + x);
+        else
+            __hip_atomic_fetch_add(&acc[j[x]], a * b[x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
 }
 // the block's value of column j, which is cleared (as: where the row of A begins, for the semirings that keep places)
 template <bool SEMI>
@@ -1504,7 +1563,7 @@ __global__ void spgemm_dense_rows(int64_t row_begin, RowList list, int64_t nd, i
         const int64_t i = row_begin + list.rows[x];
         DenseRow r;
         r.as = Apos[i];
-        r.cnt = (int32_t)(Apos[i + 1] - r.as < (1ll << 30) ? Apos[i + 1] - r.as : (1ll << 30));
+        r.cnt = (int32_t)(Apos[i + 1] - r.as);         // (the host sends matrices of under 2^30 entries here)
         r.coff = Cpos[i] - Cpos[row_begin];
         r.pad = 0;
         rows[x] = r;
@@ -1589,6 +1648,9 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_blocks_kernel(
             const auto add = [&](int j, double a, double b, int pa, int64_t q) {
                 dense_add<SEMI, COL>(acc, bm, col0, j, a, b, pa, q, reduce_op, mult_op);
             };
+            const auto add4 = [&](auto j, double a, auto v0, auto v1, int pa, int64_t q) {
+                dense_add4<SEMI, COL>(acc, bm, col0, j, a, v0, v1, pa, q, reduce_op, mult_op);
+            };
             const auto take = [&](int j) { return dense_take<SEMI>(acc, j, reduce_op, mult_op, as, Aval, Bval); };
             // What lies ahead of this block comes from whoever counted the block before it.  That was many tickets
             // ago as a rule, so the answer is asked for before the walk and the trip to memory it takes is over by
@@ -1598,7 +1660,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_blocks_kernel(
             if (threadIdx.x == 0 && cb > 0)
                 early = __hip_atomic_fetch_max(mark, -1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             const int mine_p = wave + lane * SG_WAVES;          // the entry this lane holds of a batch of SG_T
-            int touched = for_each_in_slices<true>(lo0, hi0, a0, mine_p + 1, lane, Bcrd, Bval, add);
+            int touched = for_each_in_slices<true>(lo0, hi0, a0, mine_p + 1, lane, Bcrd, Bval, add, add4);
             if (cnt > SG_T) {
                 // the entries of A beyond the first SG_T, SG_T at a time: a batch's entries are loaded two batches
                 // ahead and its slices one, so that a walk does not begin with two trips to memory
@@ -1619,15 +1681,15 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_blocks_kernel(
                 for (int base = SG_T; base < cnt; base += SG_T) {
                     int64_t lon, hin;
                     load_slice(kn, lon, hin);
-                    int k2;
-                    double a2;
-                    load_more(base + 2 * SG_T, k2, a2);
-                    touched |= for_each_in_slices<true>(lob, hib, ab, base + mine_p + 1, lane, Bcrd, Bval, add);
+                    int kf;
+                    double af;
+                    load_more(base + 2 * SG_T, kf, af);
+                    touched |= for_each_in_slices<true>(lob, hib, ab, base + mine_p + 1, lane, Bcrd, Bval, add, add4);
                     lob = lon;
                     hib = hin;
                     ab = an;
-                    kn = k2;
-                    an = a2;
+                    kn = kf;
+                    an = af;
                 }
             }
             const int any = visit_flag(block_touched, visit, touched, lane);
@@ -1769,7 +1831,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
             }
             // f over the products of the row whose columns lie in the blocks [cbf, cbt); a held row's slice of these
             // blocks is [held_lo, held_hi)
-            const auto walk = [&](int cbf, int cbt, int64_t held_lo, int64_t held_hi, auto values, auto f) -> int {
+            const auto walk = [&](int cbf, int cbt, int64_t held_lo, int64_t held_hi, auto values, auto f, auto f4) -> int {
                 constexpr bool VALUES = decltype(values)::value;
                 int touched = 0;
                 if (small) {
@@ -1782,11 +1844,15 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
                         const int c = g - (__builtin_amdgcn_readlane(upto, e) - __builtin_amdgcn_readlane(mine, e));
                         const int64_t s = readlane_i64(held_lo, e) + (int64_t)c * SP_CHUNK;
                         const int64_t left = readlane_i64(held_hi, e) - s;
-                        turn_of_slice<VALUES>(s, lane, left < SP_CHUNK ? left : SP_CHUNK, readlane_d(h_a, e),
-                                              __builtin_amdgcn_readlane(h_pa, e), Bcrd, Bval, f);
+                        if (left >= SP_CHUNK)
+                            full_turn_of_slice<VALUES>(s, lane, readlane_d(h_a, e), __builtin_amdgcn_readlane(h_pa, e), Bcrd,
+                                                       Bval, f4);
+                        else
+                            turn_of_slice<VALUES>(s, lane, left, readlane_d(h_a, e), __builtin_amdgcn_readlane(h_pa, e),
+                                                  Bcrd, Bval, f);
                     }
                 } else if (held)
-                    touched = for_each_in_slices<VALUES>(held_lo, held_hi, h_a, h_pa, lane, Bcrd, Bval, f);
+                    touched = for_each_in_slices<VALUES>(held_lo, held_hi, h_a, h_pa, lane, Bcrd, Bval, f, f4);
                 for (int64_t base = as + wave; !held && base < ae; base += (int64_t)SG_WAVES * 64) {
                     const int64_t left = (ae - base + SG_WAVES - 1) / SG_WAVES;
                     const int cnt = (int)(left < 64 ? left : 64);
@@ -1801,7 +1867,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
                         a = Aval[p];
                         pa = (int)(p - as + 1);
                     }
-                    touched |= for_each_in_slices<VALUES>(lo, hi, a, pa, lane, Bcrd, Bval, f);
+                    touched |= for_each_in_slices<VALUES>(lo, hi, a, pa, lane, Bcrd, Bval, f, f4);
                 }
                 return touched;
             };
@@ -1816,6 +1882,21 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
                                          [&](int j, double, double, int, int64_t) {
                     j -= col0;
                     atomicOr(&bm[j >> 5], 1u << (j & 31));
+                }, [&](sg_i4u j4, double, sg_d2u, sg_d2u, int, int64_t) {
+                    // four consecutive entries of a sorted row: the bits that fall into one word go there together
+                    const int j[4] = {j4.x - col0, j4.y - col0, j4.z - col0, j4.w - col0};
+                    int w = j[0] >> 5;
+                    uint32_t bits = 1u << (j[0] & 31);
+#pragma unroll
+                    for (int x = 1; x < 4; ++x) {
+                        if ((j[x] >> 5) != w) {
+                            atomicOr(&bm[w], bits);
+                            w = j[x] >> 5;
+                            bits = 0u;
+                        }
+                        bits |= 1u << (j[x] & 31);
+                    }
+                    atomicOr(&bm[w], bits);
                 });
                 const int any = visit_flag(span_touched, visit, touched, lane);
                 visit = visit == 2 ? 0 : visit + 1;
@@ -1858,7 +1939,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
                             h_next = h_bp[cb + nb + SP_BLOCKS < nblk ? cb + nb + SP_BLOCKS : nblk];
                         }
                     }
-                    walk(cb, cb + nb, h_lo, h_hi, std::true_type{}, [&](int j, double a, double b, int pa, int64_t q) {
+                    const auto add_at_rank = [&](int j, double a, double b, int pa, int64_t q) {
                         j -= col0;
                         const uint32_t below = bm[j >> 5] & ((1u << (j & 31)) - 1u);
                         const int r = pre[j >> 5] + __popc(below);
@@ -1866,6 +1947,13 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_span_kernel(
                             semiring_lds_add(&val[r], reduce_op, mult_op, a, b, pa, q);
                         else
                             __hip_atomic_fetch_add(&val[r], a * b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    };
+                    walk(cb, cb + nb, h_lo, h_hi, std::true_type{}, add_at_rank,
+                         [&](sg_i4u j4, double a, sg_d2u v0, sg_d2u v1, int pa, int64_t q) {
+                        add_at_rank(j4.x, a, v0.x, pa, q);
+                        add_at_rank(j4.y, a, v0.y, pa, q + 1);
+                        add_at_rank(j4.z, a, v1.x, pa, q + 2);
+                        add_at_rank(j4.w, a, v1.y, pa, q + 3);
                     });
                     lds_barrier();
                     for (int q = threadIdx.x; q < total; q += SG_T) {
@@ -3097,7 +3185,7 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
     COMET_HIPCHK(hipGetLastError());
     // the rows of the one-block kernel block by block (COMET_HIP_SPGEMM_ROW_MAJOR keeps them row by row; the
     // tests run both)
-    const bool by_blocks = dense && a->nnz < (1ll << 31) && getenv("COMET_HIP_SPGEMM_ROW_MAJOR") == nullptr;
+    const bool by_blocks = dense && a->nnz < (1ll << 30) && getenv("COMET_HIP_SPGEMM_ROW_MAJOR") == nullptr;
     bool ran_blocks = false;
     if (by_blocks) {
         int64_t nd = 0;
