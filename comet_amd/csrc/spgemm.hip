@@ -1487,12 +1487,15 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                 const auto add = [&](int j, double a, double b, int pa, int64_t q) {
                     dense_add<SEMI, COL>(acc, bm, col0, j, a, b, pa, q, reduce_op, mult_op);
                 };
+                const auto add4 = [&](auto j, double a, auto v0, auto v1, int pa, int64_t q) {
+                    dense_add4<SEMI, COL>(acc, bm, col0, j, a, v0, v1, pa, q, reduce_op, mult_op);
+                };
                 const auto take = [&](int j) { return dense_take<SEMI>(acc, j, reduce_op, mult_op, as, Aval, Bval); };
                 if (held) {
                     int64_t next = h_hi;
                     if (h_bp && cb + 1 < nblk)
                         next = h_bp[cb + 2];
-                    touched = for_each_in_slices<true>(h_lo, h_hi, h_a, h_pa, lane, Bcrd, Bval, add);
+                    touched = for_each_in_slices<true>(h_lo, h_hi, h_a, h_pa, lane, Bcrd, Bval, add, add4);
                     h_lo = h_hi;
                     h_hi = next;
                 }
@@ -1510,7 +1513,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_numeric_dense_kernel(
                         a = Aval[p];
                         pa = (int)(p - as + 1);
                     }
-                    touched |= for_each_in_slices<true>(lo, hi, a, pa, lane, Bcrd, Bval, add);
+                    touched |= for_each_in_slices<true>(lo, hi, a, pa, lane, Bcrd, Bval, add, add4);
                 }
                 const int any = visit_flag(block_touched, visit, touched, lane);
                 visit = visit == 2 ? 0 : visit + 1;
