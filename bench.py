@@ -146,7 +146,10 @@ def bench_spmm(rt, orc, gen, args):
     dB = rt.DeviceArray.from_numpy(B)
     dC = rt.DeviceArray((n, K))
     step = lambda: rt.spmm(A, dB, dC, accumulate=False)
-    first_ms, kept_bytes = first_call(rt, step)
+    # the first product runs without a plan, the second one builds it (neither is timed as a step)
+    first_ms, kept_first = first_call(rt, step)
+    second_ms, kept_second = first_call(rt, step)
+    kept_bytes = kept_first + kept_second
     wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
     kt = kernel_times(rt, step, args.steps)
     flops = 2.0 * nnz * K
@@ -188,9 +191,11 @@ def bench_spmm(rt, orc, gen, args):
                      "kernel": dom, "kernel_avg_ms": dom_ms, "kernel_sum_ms": kernel_sum_ms,
                      "algorithmic_bytes": int(alg_bytes),
                      "gather_inclusive_bytes": int(nnz * 8 * K + nnz * (8 + ib) + 8 * n * K)},
-        "plan": {"first_call_ms": first_ms, "plan_ms": max(first_ms - dev_ms, 0.0), "kept_device_bytes": int(kept_bytes),
-                 "note": "first product on a new matrix minus a steady-state product; bytes = device memory the "
-                         "first call keeps (lists of the long rows, the other rows re-packed, workspaces)"},
+        "plan": {"first_call_ms": first_ms, "second_call_ms": second_ms, "plan_ms": max(second_ms - dev_ms, 0.0),
+                 "kept_device_bytes": int(kept_bytes),
+                 "note": "a matrix's first product runs without a plan (all rows through the chunk kernel), its second "
+                         "one builds the plan: plan_ms = second product minus a steady-state one; bytes = device "
+                         "memory the two calls keep (lists of the long rows, the other rows re-packed, workspaces)"},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
     }
 
@@ -248,7 +253,10 @@ def bench_spmv(rt, orc, gen, args):
     dx = rt.DeviceArray.from_numpy(x)
     dy = rt.DeviceArray(n)
     step = lambda: rt.spmv(A, dx, dy, accumulate=False)
-    first_ms, kept_bytes = first_call(rt, step)
+    # the first product runs on the matrix as it is, the second one makes the column-blocked copy (neither is a step)
+    first_ms, kept_first = first_call(rt, step)
+    second_ms, kept_second = first_call(rt, step)
+    kept_bytes = kept_first + kept_second
     wall_ms, dev_ms = timed_steps(rt, step, args.steps, args.warmup)
     kt = kernel_times(rt, step, args.steps)
     parity_ok = bool(np.array_equal(dy.to_numpy(), orc.spmv(pos, crd, val, x)))
@@ -277,9 +285,10 @@ def bench_spmv(rt, orc, gen, args):
                      "traffic": measured_traffic("spmv_csr_poisson")[0] if n == 1_000_000 else None,
                      "kernel": dom, "kernel_avg_ms": dom_ms, "launches_per_step": passes,
                      "algorithmic_bytes": int(alg_bytes)},
-        "plan": {"first_call_ms": first_ms, "plan_ms": max(first_ms - dev_ms, 0.0), "kept_device_bytes": int(kept_bytes),
-                 "note": "first product on a new matrix minus a steady-state product; bytes = the column-blocked "
-                         "copy of the matrix the first call keeps"},
+        "plan": {"first_call_ms": first_ms, "second_call_ms": second_ms, "plan_ms": max(second_ms - dev_ms, 0.0),
+                 "kept_device_bytes": int(kept_bytes),
+                 "note": "a matrix's first product runs on its own arrays, its second one makes the column-blocked "
+                         "copy: plan_ms = second product minus a steady-state one; bytes = that copy"},
         "cpu_baseline": cpu, "kernels": kt, "wall_ms_per_step": wall_ms, "parity_sample_ok": parity_ok,
     }
 

@@ -113,12 +113,16 @@ struct Csr {
     // products taken pair by pair); dup_state: 0 not looked at, 1 no row holds a column twice, 2 some row does
     Csr *transposed_index = nullptr;
     int dup_state = 0;
+    // products taken with this matrix on the left so far (0, 1, more): the SpMM and SpMV plans, which cost tens of
+    // products, are built when a matrix is multiplied for the second time (plan_at_once() builds them at the first)
+    int spmm_uses = 0, spmv_uses = 0;
 };
 
 Csr *csr_from_handle(int64_t h);           // nullptr (and error set) if unknown
 int64_t csr_register(Csr *c);              // takes ownership of the struct
 int csr_alloc(Csr *c, int64_t nrows, int64_t ncols, int64_t nnz);   // allocates pos/crd/val, owns = true
 void csr_release(Csr *c);                  // frees the arrays it owns, its plans and the struct
+bool plan_at_once();                       // COMET_HIP_PLAN_AT_ONCE is set
 int csr_entry_rows(Csr *a, const int32_t **rows);      // the row of every stored entry, kept in the handle
 Csr *csr_transposed_copy(const Csr *a);    // new unregistered struct holding the transpose (nullptr on failure)
 

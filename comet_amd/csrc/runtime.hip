@@ -158,6 +158,11 @@ int csr_alloc(Csr *c, int64_t nrows, int64_t ncols, int64_t nnz)
 }
 
 // Everything the kernels derived from the matrix and keep in its handle.
+bool plan_at_once()
+{
+    return getenv("COMET_HIP_PLAN_AT_ONCE") != nullptr;
+}
+
 static void csr_drop_plans(Csr *c)
 {
     if (c->light)
@@ -185,6 +190,7 @@ static void csr_drop_plans(Csr *c)
     c->heavy_ent = nullptr;
     c->heavy_row = c->heavy_code = nullptr;
     c->heavy_state = 0;
+    c->spmm_uses = c->spmv_uses = 0;
     c->heavy_nnz = c->heavy_rows = 0;
     (void)hipFree(c->spmm_chunk_row);
     c->spmm_chunk_row = nullptr;

@@ -1467,39 +1467,45 @@ static int spmv_run(Csr *a, int64_t x_dptr, int64_t y_dptr, int accumulate)
         return set_error(COMET_HIP_ERR_ARG, "null vector passed to a sparse matrix-vector product");
     if (a->nrows == 0)
         return COMET_HIP_OK;
-    COMET_CHK(spmv_plan(a));
+    // The column-blocked copy costs some twenty products: a matrix multiplied once runs on its own arrays, the copy
+    // is made when it is multiplied again.
+    const bool plan_now = a->spmv_uses > 0 || plan_at_once();
+    a->spmv_uses = a->spmv_uses < 2 ? a->spmv_uses + 1 : 2;
+    if (plan_now)
+        COMET_CHK(spmv_plan(a));
+    const int nb = a->spmv_nb > 0 ? a->spmv_nb : 1;
     const unsigned blocks = (unsigned)ceil_div(a->nrows, SPMV_T);
     const double *x = (const double *)x_dptr;
     double *y = (double *)y_dptr;
-    if (a->spmv_nb > 1 && a->spmv_bpos32 && getenv("COMET_HIP_SPMV_LAUNCH_PER_BLOCK") == nullptr) {
+    if (nb > 1 && a->spmv_bpos32 && getenv("COMET_HIP_SPMV_LAUNCH_PER_BLOCK") == nullptr) {
         // all column blocks in one launch, the row sums staying on chip - when the workgroups the GPU holds at once
         // have room for all rows
         int grid = 0, tile_rows = 0, tiles = 0;
         if (spmv_blocks_shape(a->nrows, &grid, &tile_rows, &tiles)) {
             SpmvBases base;
-            for (int b = 0; b < a->spmv_nb; ++b)
+            for (int b = 0; b < nb; ++b)
                 base.v[b] = a->spmv_base[b];
             KernelTimer t("spmv_csr_blocks");
             spmv_csr_blocks<int32_t><<<dim3((unsigned)grid), dim3(SPMV_T), sizeof(double) * SPMV_T * (size_t)tiles,
-                                       stream()>>>(a->spmv_bpos32, a->spmv_bcrd, a->spmv_bval, base, a->spmv_nb, x, y,
+                                       stream()>>>(a->spmv_bpos32, a->spmv_bcrd, a->spmv_bval, base, nb, x, y,
                                                    a->nrows, tile_rows, tiles, accumulate);
             COMET_HIPCHK(hipGetLastError());
             return COMET_HIP_OK;
         }
     }
-    for (int b = 0; b < a->spmv_nb; ++b) {
-        const int32_t *crd = a->spmv_nb == 1 ? a->crd : a->spmv_bcrd + a->spmv_base[b];
-        const double *val = a->spmv_nb == 1 ? a->val : a->spmv_bval + a->spmv_base[b];
+    for (int b = 0; b < nb; ++b) {
+        const int32_t *crd = nb == 1 ? a->crd : a->spmv_bcrd + a->spmv_base[b];
+        const double *val = nb == 1 ? a->val : a->spmv_bval + a->spmv_base[b];
         const bool acc = accumulate || b > 0;   // later passes continue the row sums the earlier ones left in y
         KernelTimer t("spmv_csr_stream");
-        if (a->spmv_nb > 1 && a->spmv_bpos32) {
+        if (nb > 1 && a->spmv_bpos32) {
             const int32_t *pos = a->spmv_bpos32 + (int64_t)b * (a->nrows + 1);
             if (acc)
                 spmv_csr_stream<true, int32_t><<<dim3(blocks), dim3(SPMV_T), 0, stream()>>>(pos, crd, val, x, y, a->nrows);
             else
                 spmv_csr_stream<false, int32_t><<<dim3(blocks), dim3(SPMV_T), 0, stream()>>>(pos, crd, val, x, y, a->nrows);
         } else {
-            const int64_t *pos = a->spmv_nb == 1 ? a->pos : a->spmv_bpos + (int64_t)b * (a->nrows + 1);
+            const int64_t *pos = nb == 1 ? a->pos : a->spmv_bpos + (int64_t)b * (a->nrows + 1);
             if (acc)
                 spmv_csr_stream<true, int64_t><<<dim3(blocks), dim3(SPMV_T), 0, stream()>>>(pos, crd, val, x, y, a->nrows);
             else
@@ -1537,7 +1543,11 @@ static int spmm_run(Csr *a, int64_t K, int64_t b_dptr, int64_t ldb, int64_t c_dp
     // (the sweep loads B and stores C sixteen bytes at a time: two columns per lane, rows aligned to that)
     const bool sweep_fits = K >= 16 && K <= 2048 && (K & 1) == 0 && (ldb & 1) == 0 && (b_dptr & 15) == 0 &&
                             (ldc & 1) == 0 && (c_dptr & 15) == 0 && getenv("COMET_SPMM_NO_SWEEP") == nullptr;
-    if (sweep_fits)
+    // The plan (the long rows as per-XCD lists, the rest re-packed) costs some forty products: a matrix multiplied
+    // once goes through the chunk kernel whole, the plan is made when it is multiplied again.
+    const bool plan_now = a->spmm_uses > 0 || plan_at_once();
+    a->spmm_uses = a->spmm_uses < 2 ? a->spmm_uses + 1 : 2;
+    if (sweep_fits && plan_now)
         COMET_CHK(spmm_heavy_plan(a));
     if (a->heavy_state != 2 || !sweep_fits)
         return spmm_chunks(a, K, B, ldb, C, ldc, accumulate);

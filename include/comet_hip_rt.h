@@ -101,7 +101,10 @@ int comet_hip_spmv_csr_f64(int64_t csr, int64_t x_dptr, int64_t y_dptr, int accu
 /* ---- SpMM  C[i,:] (+)= sum_p val[p] * B[crd[p],:] --------------------------
  * Same builders plus the dense inner loop (IndexTreeToSCF.cpp:476-489).
  * B is ncols x K with row stride ldb, C is nrows x K with row stride ldc
- * (elements).  accumulate as for SpMV. */
+ * (elements).  accumulate as for SpMV.
+ * Both products keep a plan in the handle (a re-ordered copy of parts of the
+ * matrix) that costs tens of products to build: it is built when a handle is
+ * multiplied for the second time, the first product runs without it. */
 int comet_hip_spmm_csr_f64(int64_t csr, int64_t K, int64_t b_dptr, int64_t ldb,
                            int64_t c_dptr, int64_t ldc, int accumulate);
 

@@ -23,3 +23,10 @@ def golden():
 @pytest.fixture(scope="session")
 def golden_dir():
     return GOLDEN
+
+
+@pytest.fixture(autouse=True)
+def plans_at_the_first_product(monkeypatch):
+    """The library builds its SpMM and SpMV plans when a matrix is multiplied for the second time; the tests
+    multiply once, so they ask for the plan at once (the tests of that rule take the switch away again)."""
+    monkeypatch.setenv("COMET_HIP_PLAN_AT_ONCE", "1")

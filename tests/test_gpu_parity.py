@@ -1235,6 +1235,43 @@ def test_spmm_long_rows_sweep(K, acc, pad, medium, monkeypatch):
     assert nlong > 100 if (K % 2 == 0 and pad % 2 == 0) else nlong == 0
 
 
+def test_spmm_plan_waits_for_the_second_product(monkeypatch):
+    # The plan of a matrix costs some forty products, so a matrix multiplied once (what a .ta program does) goes
+    # through the chunk kernel whole; the plan is made when the same handle is multiplied again, and kept.
+    monkeypatch.delenv("COMET_HIP_PLAN_AT_ONCE")
+    pos, crd, val = gen.zipf_csr(n=40_000, mean=16.0, cap=4096, seed=7)
+    assert len(crd) >= 1 << 19
+    B = gen.dense((40_000, 64), seed=8)
+    A = rt.CsrMatrix.from_arrays((40_000, 40_000), pos, crd, val)
+    dB, dC = rt.DeviceArray.from_numpy(B), rt.DeviceArray((40_000, 64))
+    want = orc.spmm(pos, crd, val, B)
+    bound = orc.spmm(pos, crd, np.abs(val), np.abs(B))
+    seen = []
+    for _ in range(3):
+        rep = _kernels_of(lambda: rt.spmm(A, dB, dC, accumulate=False))
+        seen.append("spmm_heavy_sweep" in rep)
+        assert np.all(np.abs(dC.to_numpy() - want) <= RTOL * bound)
+    assert seen == [False, True, True]
+
+
+def test_spmv_plan_waits_for_the_second_product(monkeypatch):
+    # the same rule for the column-blocked copy an SpMV keeps of a matrix whose x outgrows an L2; with or
+    # without it the additions happen in the checker's order
+    monkeypatch.delenv("COMET_HIP_PLAN_AT_ONCE")
+    n = 600_000
+    pos, crd, val = gen.poisson_csr(n=n, mean=4.0, seed=5)
+    x = gen.dense(n, seed=15)
+    A = rt.CsrMatrix.from_arrays((n, n), pos, crd, val)
+    dx, dy = rt.DeviceArray.from_numpy(x), rt.DeviceArray(n)
+    want = orc.spmv(pos, crd, val, x)
+    seen = []
+    for _ in range(3):
+        rep = _kernels_of(lambda: rt.spmv(A, dx, dy, accumulate=False))
+        seen.append("spmv_csr_blocks" in rep)
+        assert np.array_equal(dy.to_numpy(), want)
+    assert seen == [False, True, True]
+
+
 @pytest.mark.parametrize("groups,held", [(None, 2880), (32, 3840), (16, 1920)])
 def test_spmm_more_long_rows_than_the_sweep_holds(groups, held, monkeypatch):
     """5000 rows of 300 nonzeros: the longest the sweep has room for (ties: lowest row ids) sweep, the others
