@@ -692,10 +692,15 @@ def main():
     ap.add_argument("--masked", action="store_true", help="spgemm: the masked product C<A> = A*A, materialised")
     ap.add_argument("--semiring", default="", help="spgemm: reduce,mult of another semiring, e.g. min,plus")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--plan-at-once", action="store_true",
+                    help="spmm, spmv: build the matrix's plan at its first product instead of its second, so that every "
+                         "launch of a profiled run is a steady-state one")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (every kernel is single-device and no figure at "
                  "several GPUs is produced); rerun with --gpus 1")
+    if args.plan_at_once:
+        os.environ["COMET_HIP_PLAN_AT_ONCE"] = "1"        # read by the library at every product
     from comet_amd import gen, runtime as rt
     from oracle import oracle as orc
     rt.init(0)
