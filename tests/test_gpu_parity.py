@@ -855,6 +855,39 @@ def test_triangle_count_rmat_vs_checker_and_trace(scale, ef, seed):
     assert rt.triangle_count(Ud) == got
 
 
+def test_headline_workloads_at_full_size(monkeypatch):
+    """The benchmark's own SpMM, SpMV and triangle-count inputs at their full sizes, every entry of the results
+    against the checker (the SpGEMM of that size writes 285 GB and is checked by samples in bench.py): the
+    products without a plan (a matrix's first) and with it (its second)."""
+    monkeypatch.delenv("COMET_HIP_PLAN_AT_ONCE")
+    n, K = 500_000, 64
+    pos, crd, val = gen.zipf_csr(n=n, mean=16.0, cap=4096, seed=2)
+    B = gen.dense((n, K), seed=3)
+    A = rt.CsrMatrix.from_arrays((n, n), pos, crd, val)
+    dB, dC = rt.DeviceArray.from_numpy(B), rt.DeviceArray((n, K))
+    want = orc.spmm(pos, crd, val, B)
+    bound = orc.spmm(pos, crd, np.abs(val), np.abs(B))
+    for call in range(2):
+        rep = _kernels_of(lambda: rt.spmm(A, dB, dC, accumulate=False))
+        assert ("spmm_heavy_sweep" in rep) == (call == 1)
+        assert np.all(np.abs(dC.to_numpy() - want) <= RTOL * bound), f"spmm, call {call}"
+    del A, dB, dC, B, want, bound
+    n = 1_000_000
+    pos, crd, val = gen.poisson_csr(n=n, mean=10.0, seed=1)
+    x = gen.dense(n, seed=4)
+    A = rt.CsrMatrix.from_arrays((n, n), pos, crd, val)
+    dx, dy = rt.DeviceArray.from_numpy(x), rt.DeviceArray(n)
+    want = orc.spmv(pos, crd, val, x)
+    for call in range(2):
+        rt.spmv(A, dx, dy, accumulate=False)
+        assert np.array_equal(dy.to_numpy(), want), f"spmv, call {call}"
+    del A, dx, dy
+    pos, crd, val = gen.rmat_symmetric_csr(scale=20, edge_factor=16, seed=20, values="ones")
+    lpos, lcrd, lval = gen.strictly_lower(pos, crd, val)
+    L = rt.CsrMatrix.from_arrays((1 << 20, 1 << 20), lpos, lcrd, lval)
+    assert rt.triangle_count(L) == orc.tricount_masked(lpos, lcrd, lval)
+
+
 def test_masked_sum_general_values():
     rng = np.random.default_rng(3)
     a = _rand_csr(rng, 300, 300, 0.05)
