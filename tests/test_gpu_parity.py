@@ -754,13 +754,15 @@ def test_spgemm_block_by_block_wait_is_bounded(monkeypatch):
     _spgemm_check(a, b, m)
 
 
-def test_spgemm_rmat_scale16_row_blocks_vs_checker():
-    """C = A*A on the benchmark's own generator at scale 16, edge factor 16 (65,536 vertices, 1.8 M entries,
-    1.24e9 products): the symbolic phase over all rows, the numeric phase on sampled blocks of 64 rows - the block
-    with the heaviest row, the hub rows at the low ids, the tail, and random ones - against the checker.  Real
-    R-MAT rows of every class (values in a slab, several column blocks per visit, one block per visit) go through
-    the kernel that serves their class."""
-    scale = 16
+@pytest.mark.parametrize("scale", [16, 20])
+def test_spgemm_rmat_row_blocks_vs_checker(scale):
+    """C = A*A on the benchmark's own generator at edge factor 16 - at scale 16 (65,536 vertices, 1.8 M entries,
+    1.24e9 products) and at the benchmark's scale 20 (31 M entries, 7.0e10 products): the symbolic phase over all
+    rows, the numeric phase on sampled blocks of 64 rows against the checker.  At scale 16 the block with the
+    heaviest row, the hub rows at the low ids, the tail, and random ones; at scale 20, where the hub rows alone
+    would keep the checker busy for minutes, the heaviest block of at most 1.5e8 products, the tail, the middle
+    and random ones of at most 5e7.  Real R-MAT rows of every class (values in a slab, several column blocks per
+    visit, one block per visit) go through the kernel that serves their class."""
     n = 1 << scale
     pos, crd, val = gen.rmat_symmetric_csr(scale=scale, edge_factor=16, seed=20)
     deg = np.diff(pos)
@@ -772,8 +774,14 @@ def test_spgemm_rmat_scale16_row_blocks_vs_checker():
     hpos = dpos.to_numpy()
     assert hpos[0] == 0 and hpos[-1] == nnzC and np.all(np.diff(hpos) >= 0)
     rng = np.random.default_rng(5)
-    starts = {int(np.argmax(rowprod)) // 64 * 64, 0, 64, n - 64, n // 2}
-    starts |= {int(b) * 64 for b in rng.choice(n // 64, 10, replace=False)}
+    if scale == 16:
+        starts = {int(np.argmax(rowprod)) // 64 * 64, 0, 64, n - 64, n // 2}
+        starts |= {int(b) * 64 for b in rng.choice(n // 64, 10, replace=False)}
+    else:
+        blockprod = rowprod.reshape(-1, 64).sum(axis=1)
+        fits = np.flatnonzero(blockprod <= 150_000_000)
+        starts = {int(fits[np.argmax(blockprod[fits])]) * 64, n - 64, n // 2}
+        starts |= {int(b) * 64 for b in rng.choice(np.flatnonzero(blockprod <= 50_000_000), 8, replace=False)}
     rt.profile_reset()
     rt.profile_enable(True)
     checked = 0
@@ -797,7 +805,7 @@ def test_spgemm_rmat_scale16_row_blocks_vs_checker():
     # the masked product C<A> = A*A on the same blocks (structure = mask entries that receive a product)
     mpos, mnnz = rt.spgemm_symbolic(A, A, mask=A)
     hm = mpos.to_numpy()
-    for r0 in sorted(starts)[:6]:
+    for r0 in sorted(starts)[:6 if scale == 16 else 3]:
         r1 = r0 + 64
         cp, cc, cv = orc.spgemm(pos, crd, val, pos, crd, val, n, mask=(pos, crd), rows=(r0, r1))
         assert np.array_equal(cp, hm[r0:r1 + 1] - hm[r0])
@@ -806,6 +814,8 @@ def test_spgemm_rmat_scale16_row_blocks_vs_checker():
         rt.spgemm_numeric(A, A, mpos, r0, r1, dcrd, dval, mask=A)
         assert np.array_equal(dcrd.to_numpy(cnt), cc)
         assert np.all(np.abs(dval.to_numpy(cnt) - cv) <= RTOL * np.abs(cv))
+    if scale > 16:          # (test_headline_workloads_at_full_size counts the triangles of that graph)
+        return
     # and the triangle count of the same graph
     lpos, lcrd, lval = gen.strictly_lower(pos, crd, np.ones_like(val))
     L = rt.CsrMatrix.from_arrays((n, n), lpos, lcrd, lval)
