@@ -866,9 +866,9 @@ def test_triangle_count_rmat_vs_checker_and_trace(scale, ef, seed):
 
 
 def test_headline_workloads_at_full_size(monkeypatch):
-    """The benchmark's own SpMM, SpMV and triangle-count inputs at their full sizes, every entry of the results
-    against the checker (the SpGEMM of that size writes 285 GB and is checked by samples in bench.py): the
-    products without a plan (a matrix's first) and with it (its second)."""
+    """The benchmark's own SpMM, SpMV, triangle-count and TTGT inputs at their full sizes, every entry of the
+    results against the checker (the SpGEMM of that size writes 285 GB: test_spgemm_rmat_row_blocks_vs_checker
+    samples it, and so does bench.py): the products without a plan (a matrix's first) and with it (its second)."""
     monkeypatch.delenv("COMET_HIP_PLAN_AT_ONCE")
     n, K = 500_000, 64
     pos, crd, val = gen.zipf_csr(n=n, mean=16.0, cap=4096, seed=2)
@@ -896,6 +896,14 @@ def test_headline_workloads_at_full_size(monkeypatch):
     lpos, lcrd, lval = gen.strictly_lower(pos, crd, val)
     L = rt.CsrMatrix.from_arrays((1 << 20, 1 << 20), lpos, lcrd, lval)
     assert rt.triangle_count(L) == orc.tricount_masked(lpos, lcrd, lval)
+    del L, lpos, lcrd, lval
+    # the contraction of the TTGT workload, every extent 64 (a 4096^3 GEMM), against the same GEMM by the host's BLAS
+    # (the checker's triple loop would take minutes): |difference| <= 1e-12 * sum |a||b| for every entry
+    A, B = gen.dense((64,) * 4, seed=5), gen.dense((64,) * 4, seed=6)
+    Cm, _ = rt.ttgt_contract("aebf", "dfce", "abcd", rt.DeviceArray.from_numpy(A), rt.DeviceArray.from_numpy(B))
+    A2 = np.ascontiguousarray(A.transpose(0, 2, 1, 3)).reshape(4096, 4096)          # [a b | e f]
+    B2 = np.ascontiguousarray(B.transpose(3, 1, 2, 0)).reshape(4096, 4096)          # [e f | c d]
+    assert np.all(np.abs(Cm.to_numpy().reshape(4096, 4096) - A2 @ B2) <= RTOL * (np.abs(A2) @ np.abs(B2)))
 
 
 def test_masked_sum_general_values():
