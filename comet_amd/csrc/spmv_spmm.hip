@@ -1233,21 +1233,9 @@ static int spmm_heavy_plan(Csr *a)
     uint64_t *k_in = nullptr, *k_out = nullptr;
     uint32_t *i_in = nullptr, *i_out = nullptr;
     Csr *light = new Csr();
+    char *scratch = nullptr;        // everything that does not outlive the planning, in one allocation
     auto cleanup = [&](bool failed) {
-        (void)hipFree(d_cnt);
-        (void)hipFree(d_srow);
-        (void)hipFree(d_hstart);
-        (void)hipFree(d_mstart);
-        (void)hipFree(d_len);
-        (void)hipFree(d_first);
-        (void)hipFree(d_runs);
-        (void)hipFree(d_start);
-        (void)hipFree(d_odd);
-        (void)hipFree(d_pads);
-        (void)hipFree(k_in);
-        (void)hipFree(k_out);
-        (void)hipFree(i_in);
-        (void)hipFree(i_out);
+        (void)hipFree(scratch);
         if (failed) {
             (void)hipFree(a->heavy_seg);
             (void)hipFree(a->heavy_ent);
@@ -1272,19 +1260,40 @@ static int spmm_heavy_plan(Csr *a)
         }                                                                                                     \
     } while (0)
     auto at_least_one = [](int64_t v) { return (size_t)(v > 0 ? v : 1); };
-    HEAVY_TRY(hipMalloc((void **)&d_cnt, 4 * (size_t)(8 * H)));
-    HEAVY_TRY(hipMalloc((void **)&d_srow, 4 * at_least_one(S)));
-    HEAVY_TRY(hipMalloc((void **)&d_hstart, 8 * (size_t)(H + 1)));
-    HEAVY_TRY(hipMalloc((void **)&d_mstart, 8 * (size_t)(M + 1)));
+    {
+        // (an allocation and its release cost about as much as a product each: fourteen arrays, one of each)
+        size_t total = 0;
+        const auto room = [&](size_t bytes) {
+            const size_t at = total;
+            total += (bytes + 255) & ~(size_t)255;
+            return at;
+        };
+        const size_t o_cnt = room(4 * (size_t)(8 * H)), o_srow = room(4 * at_least_one(S)),
+                     o_hstart = room(8 * (size_t)(H + 1)), o_mstart = room(8 * (size_t)(M + 1)),
+                     o_len = room(8 * at_least_one(L)), o_kin = room(8 * (size_t)nent), o_kout = room(8 * (size_t)nent),
+                     o_iin = room(4 * (size_t)nent), o_iout = room(4 * (size_t)nent), o_first = room(8 * (size_t)nent),
+                     o_runs = room(8 * (size_t)(nent + 1)), o_start = room(8 * (size_t)(nent + 1)),
+                     o_odd = room(8 * (size_t)nent), o_pads = room(8 * (size_t)(nent + 1));
+        HEAVY_TRY(hipMalloc((void **)&scratch, total));
+        d_cnt = (int32_t *)(scratch + o_cnt);
+        d_srow = (int32_t *)(scratch + o_srow);
+        d_hstart = (int64_t *)(scratch + o_hstart);
+        d_mstart = (int64_t *)(scratch + o_mstart);
+        d_len = (int64_t *)(scratch + o_len);
+        k_in = (uint64_t *)(scratch + o_kin);
+        k_out = (uint64_t *)(scratch + o_kout);
+        i_in = (uint32_t *)(scratch + o_iin);
+        i_out = (uint32_t *)(scratch + o_iout);
+        d_first = (int64_t *)(scratch + o_first);
+        d_runs = (int64_t *)(scratch + o_runs);
+        d_start = (int64_t *)(scratch + o_start);
+        d_odd = (int64_t *)(scratch + o_odd);
+        d_pads = (int64_t *)(scratch + o_pads);
+    }
     HEAVY_TRY(hipMalloc((void **)&a->medium_row, 4 * at_least_one(M)));
     if (M > 0)
         HEAVY_TRY(hipMemcpyAsync(a->medium_row, mrow.data(), 4 * (size_t)M, hipMemcpyHostToDevice, stream()));
     HEAVY_TRY(hipMemcpyAsync(d_mstart, mstart.data(), 8 * (size_t)(M + 1), hipMemcpyHostToDevice, stream()));
-    HEAVY_TRY(hipMalloc((void **)&d_len, 8 * at_least_one(L)));
-    HEAVY_TRY(hipMalloc((void **)&k_in, 8 * (size_t)nent));
-    HEAVY_TRY(hipMalloc((void **)&k_out, 8 * (size_t)nent));
-    HEAVY_TRY(hipMalloc((void **)&i_in, 4 * (size_t)nent));
-    HEAVY_TRY(hipMalloc((void **)&i_out, 4 * (size_t)nent));
     HEAVY_TRY(hipMalloc((void **)&a->heavy_seg, 8 * (size_t)(8 * hbins + 1)));
     HEAVY_TRY(hipMalloc((void **)&a->heavy_row, 4 * (size_t)H));
     HEAVY_TRY(hipMalloc((void **)&a->heavy_code, 4 * (size_t)(8 * H)));
@@ -1348,11 +1357,6 @@ static int spmm_heavy_plan(Csr *a)
         return COMET_HIP_ERR_HIP;
     }
     // runs (entries of one row inside one column block of one wavefront's list) are padded to even length
-    HEAVY_TRY(hipMalloc((void **)&d_first, 8 * (size_t)nent));
-    HEAVY_TRY(hipMalloc((void **)&d_runs, 8 * (size_t)(nent + 1)));
-    HEAVY_TRY(hipMalloc((void **)&d_start, 8 * (size_t)(nent + 1)));
-    HEAVY_TRY(hipMalloc((void **)&d_odd, 8 * (size_t)nent));
-    HEAVY_TRY(hipMalloc((void **)&d_pads, 8 * (size_t)(nent + 1)));
     const dim3 per_entry((unsigned)ceil_div(nent + 1, 256));
     heavy_mark_runs<<<per_entry, dim3(256), 0, stream()>>>(nent, k_out, d_first);
     if (exclusive_scan_i64(d_first, nent, d_runs) != COMET_HIP_OK) {
