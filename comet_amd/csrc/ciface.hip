@@ -113,7 +113,8 @@ void spmm_ciface(const char *who, comet_memref_1d *pos, comet_memref_1d *crd, co
 template <typename I>
 void spgemm_sizes_ciface(const char *who, int64_t nrowsA, int64_t ncolsB, comet_memref_1d *Apos, comet_memref_1d *Acrd,
                          comet_memref_1d *Aval, comet_memref_1d *Bpos, comet_memref_1d *Bcrd, comet_memref_1d *Bval,
-                         comet_memref_1d *Mpos, comet_memref_1d *Mcrd, comet_memref_1d *sizes)
+                         comet_memref_1d *Mpos, comet_memref_1d *Mcrd, comet_memref_1d *sizes,
+                         int reduce_op = COMET_SR_PLUS, int mult_op = COMET_OP_TIMES)
 {
     const int64_t nrowsB = Bpos->sizes[0] - 1;
     if (Apos->sizes[0] - 1 != nrowsA || !sizes || sizes->sizes[0] < 1) {
@@ -138,7 +139,7 @@ void spgemm_sizes_ciface(const char *who, int64_t nrowsA, int64_t ncolsB, comet_
     }
     if (!a || !b)
         die(who);
-    g_pending_c = comet_hip_spgemm_csr(a, b, m);
+    g_pending_c = comet_hip_spgemm_csr_semiring(a, b, m, reduce_op, mult_op);
     if (!g_pending_c)
         die(who);
     int64_t nnz = 0;
@@ -252,6 +253,190 @@ extern "C" double _mlir_ciface_comet_hip_tricount_f64_i32(int64_t ncols, comet_m
                                                            comet_memref_1d *val)
 {
     return tricount_ciface<int32_t>("comet_hip_tricount_f64_i32", ncols, pos, crd, val);
+}
+
+// The semiring forms of the SpGEMM pair of calls: C[a,c] = A[a,b] @(reduce, mult) B[b,c] with the operator codes of
+// comet_hip_spgemm_csr_semiring (the DSL's names: frontends/comet_dsl/mlir/MLIRGen.cpp:101-147; the nests:
+// lib/Conversion/IndexTreeToSCF/IndexTreeToSCF.cpp:198-360).  The fill call is the plain one under a second name.
+extern "C" void _mlir_ciface_comet_hip_spgemm_csr_sizes_semiring_f64_i64(
+    int64_t nrowsA, int64_t ncolsB, comet_memref_1d *Apos, comet_memref_1d *Acrd, comet_memref_1d *Aval,
+    comet_memref_1d *Bpos, comet_memref_1d *Bcrd, comet_memref_1d *Bval, comet_memref_1d *Mpos,
+    comet_memref_1d *Mcrd, comet_memref_1d *sizes, int32_t reduce_op, int32_t mult_op)
+{
+    spgemm_sizes_ciface<int64_t>("comet_hip_spgemm_csr_sizes_semiring_f64_i64", nrowsA, ncolsB, Apos, Acrd, Aval,
+                                 Bpos, Bcrd, Bval, Mpos, Mcrd, sizes, reduce_op, mult_op);
+}
+extern "C" void _mlir_ciface_comet_hip_spgemm_csr_sizes_semiring_f64_i32(
+    int64_t nrowsA, int64_t ncolsB, comet_memref_1d *Apos, comet_memref_1d *Acrd, comet_memref_1d *Aval,
+    comet_memref_1d *Bpos, comet_memref_1d *Bcrd, comet_memref_1d *Bval, comet_memref_1d *Mpos,
+    comet_memref_1d *Mcrd, comet_memref_1d *sizes, int32_t reduce_op, int32_t mult_op)
+{
+    spgemm_sizes_ciface<int32_t>("comet_hip_spgemm_csr_sizes_semiring_f64_i32", nrowsA, ncolsB, Apos, Acrd, Aval,
+                                 Bpos, Bcrd, Bval, Mpos, Mcrd, sizes, reduce_op, mult_op);
+}
+extern "C" void _mlir_ciface_comet_hip_spgemm_csr_fill_semiring_f64_i64(comet_memref_1d *Cpos, comet_memref_1d *Ccrd,
+                                                                         comet_memref_1d *Cval)
+{
+    spgemm_fill_ciface<int64_t>("comet_hip_spgemm_csr_fill_semiring_f64_i64", Cpos, Ccrd, Cval);
+}
+extern "C" void _mlir_ciface_comet_hip_spgemm_csr_fill_semiring_f64_i32(comet_memref_1d *Cpos, comet_memref_1d *Ccrd,
+                                                                         comet_memref_1d *Cval)
+{
+    spgemm_fill_ciface<int32_t>("comet_hip_spgemm_csr_fill_semiring_f64_i32", Cpos, Ccrd, Cval);
+}
+
+// ---------------------------------------------------------------------------
+// Dense contraction, memref level.  The reference rewrites a contraction into
+// transpose -> collapse -> matmul -> expand -> transpose on host memrefs
+// (lib/Dialect/TensorAlgebra/Transforms/TCtoTTGTDyn.cpp:288-672) and, with
+// -opt-matmul-mkernel, calls _mlir_ciface_linalg_matmul_viewsxs_viewsxs_viewsxs
+// per tile (lib/ExecutionEngine/blis_interface.cpp:143-181).  Here one call
+// takes the three tensors as they are declared and does upload -> plan ->
+// transposes -> GEMM -> download.
+// ---------------------------------------------------------------------------
+namespace {
+
+struct DenseView {
+    double *data;
+    int64_t offset, rank, elems;
+    int64_t shape[8];
+};
+
+// an unranked memref (rank, pointer to StridedMemRefType<double, rank>) that must be contiguous row-major
+DenseView dense_view(int64_t rank, void *desc, const char *who)
+{
+    DenseView v{};
+    if (!desc || rank < 1 || rank > 8) {
+        set_error(COMET_HIP_ERR_ARG, "tensor memref missing or of rank %lld (1..8)", (long long)rank);
+        die(who);
+    }
+    char *p = static_cast<char *>(desc);
+    v.data = *reinterpret_cast<double **>(p + sizeof(double *));
+    v.offset = *reinterpret_cast<int64_t *>(p + 2 * sizeof(double *));
+    const int64_t *sizes = reinterpret_cast<const int64_t *>(p + 2 * sizeof(double *) + sizeof(int64_t));
+    const int64_t *strides = sizes + rank;
+    v.rank = rank;
+    v.elems = 1;
+    for (int64_t d = rank - 1; d >= 0; --d) {
+        if (sizes[d] < 0 || (sizes[d] > 1 && strides[d] != v.elems)) {
+            set_error(COMET_HIP_ERR_ARG, "tensor memref is not contiguous row-major (dimension %lld: size %lld, stride %lld)",
+                      (long long)d, (long long)sizes[d], (long long)strides[d]);
+            die(who);
+        }
+        v.shape[d] = sizes[d];
+        v.elems *= sizes[d];
+    }
+    if (v.elems > 0 && !v.data) {
+        set_error(COMET_HIP_ERR_ARG, "null tensor memref");
+        die(who);
+    }
+    return v;
+}
+
+}  // namespace
+
+// a_lab / b_lab / c_lab: one `index` per dimension, the same number for the same index label
+// (C[a,b,c,d] = A[a,e,b,f] * B[d,f,c,e]: a_lab = 0,4,1,5  b_lab = 3,5,2,4  c_lab = 0,1,2,3); beta 0 or 1.
+extern "C" void _mlir_ciface_comet_hip_ttgt_contract_f64(int64_t rankA, void *A, int64_t rankB, void *B, int64_t rankC,
+                                                          void *C, comet_memref_1d *a_lab, comet_memref_1d *b_lab,
+                                                          comet_memref_1d *c_lab, double beta)
+{
+    const char *who = "comet_hip_ttgt_contract_f64";
+    const DenseView a = dense_view(rankA, A, who), b = dense_view(rankB, B, who), c = dense_view(rankC, C, who);
+    const int64_t *lab[3] = {data1<int64_t>(a_lab, who), data1<int64_t>(b_lab, who), data1<int64_t>(c_lab, who)};
+    const DenseView *view[3] = {&a, &b, &c};
+    const comet_memref_1d *lm[3] = {a_lab, b_lab, c_lab};
+    // labels may be any integers: number them 0, 1, ... in order of first appearance and collect the extents
+    int64_t seen[24], extent[24];
+    int nlab = 0;
+    int32_t ids[3][8];
+    for (int t = 0; t < 3; ++t) {
+        if (lm[t]->sizes[0] != view[t]->rank) {
+            set_error(COMET_HIP_ERR_ARG, "operand %d has rank %lld and %lld labels", t, (long long)view[t]->rank,
+                      (long long)lm[t]->sizes[0]);
+            die(who);
+        }
+        for (int64_t d = 0; d < view[t]->rank; ++d) {
+            int k = 0;
+            while (k < nlab && seen[k] != lab[t][d])
+                ++k;
+            if (k == nlab) {
+                seen[nlab] = lab[t][d];
+                extent[nlab++] = view[t]->shape[d];
+            } else if (extent[k] != view[t]->shape[d]) {
+                set_error(COMET_HIP_ERR_ARG, "index label %lld has extents %lld and %lld", (long long)lab[t][d],
+                          (long long)extent[k], (long long)view[t]->shape[d]);
+                die(who);
+            }
+            ids[t][d] = k;
+        }
+    }
+    comet_ttgt_plan plan;
+    if (comet_hip_ttgt_plan((int32_t)a.rank, ids[0], (int32_t)b.rank, ids[1], (int32_t)c.rank, ids[2], extent, -1, &plan))
+        die(who);
+    DeviceBuf da(a.elems * 8), db(b.elems * 8), dc(c.elems * 8);
+    if ((a.elems && !da.p) || (b.elems && !db.p) || (c.elems && !dc.p))
+        die(who);
+    double *hc = c.data + c.offset;
+    if (comet_hip_memcpy(da.p, a.data + a.offset, a.elems * 8, 0) || comet_hip_memcpy(db.p, b.data + b.offset, b.elems * 8, 0) ||
+        (beta != 0.0 && comet_hip_memcpy(dc.p, hc, c.elems * 8, 0)) ||
+        comet_hip_ttgt_contract(&plan, a.shape, b.shape, c.shape, da.p, db.p, dc.p, beta) ||
+        comet_hip_memcpy(dc.p, hc, c.elems * 8, 1))
+        die(who);
+}
+
+// The reference's own name for the matrix product its TTGT lowering ends in (blis_interface.cpp:143-146):
+// C = alpha * A * B + beta * C on strided 2-D views of host memory.  mr and nr (the micro-kernel's tile) mean
+// nothing here: the whole product runs on the device, so a lowering that calls this once per contraction instead
+// of once per tile is what makes sense with this library.
+extern "C" void _mlir_ciface_linalg_matmul_viewsxs_viewsxs_viewsxs(comet_memref_2d *A, comet_memref_2d *B,
+                                                                    comet_memref_2d *C, int mr, int nr, double alpha,
+                                                                    double beta)
+{
+    const char *who = "linalg_matmul_viewsxs_viewsxs_viewsxs";
+    (void)mr;
+    (void)nr;
+    if (!A || !B || !C || !A->aligned || !B->aligned || !C->aligned) {
+        set_error(COMET_HIP_ERR_ARG, "null memref");
+        die(who);
+    }
+    const int64_t M = A->sizes[0], K = A->sizes[1], N = B->sizes[1];
+    if (B->sizes[0] != K || C->sizes[0] != M || C->sizes[1] != N || M < 0 || N < 0 || K < 0) {
+        set_error(COMET_HIP_ERR_ARG, "matmul shapes do not agree");
+        die(who);
+    }
+    if (M == 0 || N == 0)
+        return;
+    // strided views are packed on the host; alpha goes into A, a beta other than 0 or 1 into C
+    auto pack = [](const comet_memref_2d *m, double scale) {
+        const int64_t r = m->sizes[0], c = m->sizes[1];
+        double *out = (double *)malloc(sizeof(double) * (size_t)(r * c > 0 ? r * c : 1));
+        const double *in = (const double *)m->aligned + m->offset;
+        if (out)
+            for (int64_t i = 0; i < r; ++i)
+                for (int64_t j = 0; j < c; ++j)
+                    out[i * c + j] = scale * in[i * m->strides[0] + j * m->strides[1]];
+        return out;
+    };
+    const bool plain_beta = beta == 0.0 || beta == 1.0;
+    double *ha = pack(A, alpha), *hb = pack(B, 1.0), *hc = pack(C, plain_beta ? 1.0 : beta);
+    DeviceBuf da(M * K * 8), db(K * N * 8), dc(M * N * 8);
+    bool bad = !ha || !hb || !hc || (M * K && !da.p) || (K * N && !db.p) || !dc.p;
+    bad = bad || comet_hip_memcpy(da.p, ha, M * K * 8, 0) || comet_hip_memcpy(db.p, hb, K * N * 8, 0) ||
+          (beta != 0.0 && comet_hip_memcpy(dc.p, hc, M * N * 8, 0)) ||
+          comet_hip_dgemm_f64(M, N, K, da.p, db.p, dc.p, beta == 0.0 ? 0.0 : 1.0) ||
+          comet_hip_memcpy(dc.p, hc, M * N * 8, 1);
+    if (!bad) {
+        double *out = (double *)C->aligned + C->offset;
+        for (int64_t i = 0; i < M; ++i)
+            for (int64_t j = 0; j < N; ++j)
+                out[i * C->strides[0] + j * C->strides[1]] = hc[i * N + j];
+    }
+    free(ha);
+    free(hb);
+    free(hc);
+    if (bad)
+        die(who);
 }
 
 // ---------------------------------------------------------------------------

@@ -67,6 +67,7 @@ struct Csr {
     int32_t *crd = nullptr;
     double *val = nullptr;
     bool owns = false;
+    bool poisoned = false;      // a re-validation after comet_hip_csr_invalidate refused the arrays: no kernel may read them
     // SpMM plan: row that holds the first nonzero of every fixed-size chunk.
     int32_t *spmm_chunk_row = nullptr;
     int64_t spmm_nchunks = 0;
@@ -118,7 +119,7 @@ struct Csr {
     int spmm_uses = 0, spmv_uses = 0;
 };
 
-Csr *csr_from_handle(int64_t h);           // nullptr (and error set) if unknown
+Csr *csr_from_handle(int64_t h, bool allow_poisoned = false);           // nullptr (and error set) if unknown
 int64_t csr_register(Csr *c);              // takes ownership of the struct
 int csr_alloc(Csr *c, int64_t nrows, int64_t ncols, int64_t nnz);   // allocates pos/crd/val, owns = true
 void csr_release(Csr *c);                  // frees the arrays it owns, its plans and the struct

@@ -910,3 +910,39 @@ extern "C" void comet_hip_read_input_2D_f64_i32(int32_t file_id, int32_t a1forma
                                 a2_tile_format, a1pos_desc, a1crd_desc, a1tile_pos_desc, a1tile_crd_desc, a2pos_desc,
                                 a2crd_desc, a2tile_pos_desc, a2tile_crd_desc, aval_desc, read_mode);
 }
+
+// The reader under the names lowered code calls (lib/ExecutionEngine/SparseUtils.cpp:2403-2450, 2562-2568): with
+// this library in -shared-libs in place of libcomet_runner_utils, `ta.read` resolves without a compiler change.
+// Same argument lists, same behaviour as the comet_hip_read_input_* functions above.
+extern "C" void read_input_sizes_2D_f64(int32_t file_id, int32_t a1format, int32_t a1_tile_format, int32_t a2format,
+                                        int32_t a2_tile_format, int sizes_rank, void *sizes_desc, int32_t read_mode)
+{
+    comet_hip_read_input_sizes_2D_f64(file_id, a1format, a1_tile_format, a2format, a2_tile_format, sizes_rank,
+                                      sizes_desc, read_mode);
+}
+
+extern "C" void read_input_2D_f64_i64(int32_t file_id, int32_t a1format, int32_t a1_tile_format, int32_t a2format,
+                                      int32_t a2_tile_format, int a1pos_rank, void *a1pos_desc, int a1crd_rank,
+                                      void *a1crd_desc, int a1tile_pos_rank, void *a1tile_pos_desc, int a1tile_crd_rank,
+                                      void *a1tile_crd_desc, int a2pos_rank, void *a2pos_desc, int a2crd_rank,
+                                      void *a2crd_desc, int a2tile_pos_rank, void *a2tile_pos_desc, int a2tile_crd_rank,
+                                      void *a2tile_crd_desc, int aval_rank, void *aval_desc, int32_t read_mode)
+{
+    comet_hip_read_input_2D_f64_i64(file_id, a1format, a1_tile_format, a2format, a2_tile_format, a1pos_rank, a1pos_desc,
+                                    a1crd_rank, a1crd_desc, a1tile_pos_rank, a1tile_pos_desc, a1tile_crd_rank,
+                                    a1tile_crd_desc, a2pos_rank, a2pos_desc, a2crd_rank, a2crd_desc, a2tile_pos_rank,
+                                    a2tile_pos_desc, a2tile_crd_rank, a2tile_crd_desc, aval_rank, aval_desc, read_mode);
+}
+
+extern "C" void read_input_2D_f64_i32(int32_t file_id, int32_t a1format, int32_t a1_tile_format, int32_t a2format,
+                                      int32_t a2_tile_format, int a1pos_rank, void *a1pos_desc, int a1crd_rank,
+                                      void *a1crd_desc, int a1tile_pos_rank, void *a1tile_pos_desc, int a1tile_crd_rank,
+                                      void *a1tile_crd_desc, int a2pos_rank, void *a2pos_desc, int a2crd_rank,
+                                      void *a2crd_desc, int a2tile_pos_rank, void *a2tile_pos_desc, int a2tile_crd_rank,
+                                      void *a2tile_crd_desc, int aval_rank, void *aval_desc, int32_t read_mode)
+{
+    comet_hip_read_input_2D_f64_i32(file_id, a1format, a1_tile_format, a2format, a2_tile_format, a1pos_rank, a1pos_desc,
+                                    a1crd_rank, a1crd_desc, a1tile_pos_rank, a1tile_pos_desc, a1tile_crd_rank,
+                                    a1tile_crd_desc, a2pos_rank, a2pos_desc, a2crd_rank, a2crd_desc, a2tile_pos_rank,
+                                    a2tile_pos_desc, a2tile_crd_rank, a2tile_crd_desc, aval_rank, aval_desc, read_mode);
+}

@@ -127,12 +127,18 @@ void Workspace::release()
     bytes = 0;
 }
 
-Csr *csr_from_handle(int64_t h)
+Csr *csr_from_handle(int64_t h, bool allow_poisoned)
 {
     Csr *c = reinterpret_cast<Csr *>(h);
     std::lock_guard<std::mutex> lk(g_mu);
     if (!c || !g_live.count(c)) {
         set_error(COMET_HIP_ERR_HANDLE, "unknown CSR handle %lld", (long long)h);
+        return nullptr;
+    }
+    if (c->poisoned && !allow_poisoned) {
+        set_error(COMET_HIP_ERR_HANDLE,
+                  "CSR handle %lld: its arrays failed the check of comet_hip_csr_invalidate; rewrite them and "
+                  "invalidate again, or destroy the handle", (long long)h);
         return nullptr;
     }
     return c;
@@ -309,6 +315,72 @@ __global__ void copy_f64_kernel(double *__restrict__ dst, const double *__restri
     int64_t step = (int64_t)gridDim.x * blockDim.x;
     for (; i < n; i += step)
         dst[i] = src[i];
+}
+
+// Streaming yardsticks, 16 bytes per lane: what the memory system gives a kernel that does nothing but move bytes.
+// Every workgroup walks a contiguous slice so that a DRAM page is opened by one workgroup, not by all of them.
+typedef double stream_v2d __attribute__((ext_vector_type(2)));
+
+__global__ __launch_bounds__(256) void stream_copy16_kernel(stream_v2d *__restrict__ dst, const stream_v2d *__restrict__ src,
+                                                            int64_t n2, int nt)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    if (nt) {
+        for (; i + 3 * step < n2; i += 4 * step) {      // four loads in flight per lane, then four stores
+            const stream_v2d a = __builtin_nontemporal_load(src + i), b = __builtin_nontemporal_load(src + i + step),
+                             c = __builtin_nontemporal_load(src + i + 2 * step),
+                             d = __builtin_nontemporal_load(src + i + 3 * step);
+            __builtin_nontemporal_store(a, dst + i);
+            __builtin_nontemporal_store(b, dst + i + step);
+            __builtin_nontemporal_store(c, dst + i + 2 * step);
+            __builtin_nontemporal_store(d, dst + i + 3 * step);
+        }
+        for (; i < n2; i += step)
+            __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+    } else {
+        for (; i + 3 * step < n2; i += 4 * step) {
+            const stream_v2d a = src[i], b = src[i + step], c = src[i + 2 * step], d = src[i + 3 * step];
+            dst[i] = a;
+            dst[i + step] = b;
+            dst[i + 2 * step] = c;
+            dst[i + 3 * step] = d;
+        }
+        for (; i < n2; i += step)
+            dst[i] = src[i];
+    }
+}
+
+// read-only: every lane sums what it reads, one store per lane at the end
+__global__ __launch_bounds__(256) void stream_read16_kernel(const stream_v2d *__restrict__ src, int64_t n2,
+                                                            double *__restrict__ out)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    stream_v2d s0 = {0.0, 0.0}, s1 = s0, s2 = s0, s3 = s0;
+    for (; i + 3 * step < n2; i += 4 * step) {
+        const stream_v2d a = __builtin_nontemporal_load(src + i), b = __builtin_nontemporal_load(src + i + step),
+                         c = __builtin_nontemporal_load(src + i + 2 * step),
+                         d = __builtin_nontemporal_load(src + i + 3 * step);
+        s0 += a;
+        s1 += b;
+        s2 += c;
+        s3 += d;
+    }
+    for (; i < n2; i += step)
+        s0 += __builtin_nontemporal_load(src + i);
+    s0 += s1 + s2 + s3;
+    out[(int64_t)blockIdx.x * blockDim.x + threadIdx.x] = s0.x + s0.y;
+}
+
+// write-only
+__global__ __launch_bounds__(256) void stream_write16_kernel(stream_v2d *__restrict__ dst, int64_t n2, double v)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    const stream_v2d w = {v, v};
+    for (; i < n2; i += step)
+        __builtin_nontemporal_store(w, dst + i);
 }
 
 // Exclusive scan, three launches: per-block totals, scan of the totals by one
@@ -864,17 +936,21 @@ int comet_hip_csr_download_i32(int64_t csr, int32_t *pos, int32_t *crd, double *
 
 int comet_hip_csr_invalidate(int64_t csr)
 {
-    Csr *c = csr_from_handle(csr);
+    Csr *c = csr_from_handle(csr, true);
     if (!c)
         return COMET_HIP_ERR_HANDLE;
     COMET_HIPCHK(hipStreamSynchronize(stream()));
     csr_drop_plans(c);
-    return validate_device_csr(c);      // the arrays were rewritten: they are looked at again
+    // the arrays were rewritten: they are looked at again, and a handle that fails is refused by every entry
+    // point that would read them (out-of-range columns fault the GPU) until a later call here passes
+    const int rc = validate_device_csr(c);
+    c->poisoned = rc != COMET_HIP_OK;
+    return rc;
 }
 
 int comet_hip_csr_destroy(int64_t csr)
 {
-    Csr *c = csr_from_handle(csr);
+    Csr *c = csr_from_handle(csr, true);
     if (!c)
         return COMET_HIP_ERR_HANDLE;
     COMET_HIPCHK(hipStreamSynchronize(stream()));
@@ -918,6 +994,67 @@ int comet_hip_copy_f64(int64_t dst_dptr, int64_t src_dptr, int64_t n)
         copy_f64_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>((double *)dst_dptr, (const double *)src_dptr, n);
     }
     COMET_HIPCHK(hipGetLastError());
+    return COMET_HIP_OK;
+}
+
+static Workspace g_stream_out;
+
+// mode 0: copy, 16 bytes per lane, ordinary loads and stores; 1: the same with non-temporal loads and stores;
+// 2: read only (src); 3: write only (dst).  n doubles, even; workgroups_per_cu 0 = 8.
+int comet_hip_stream_bench(int mode, int64_t dst_dptr, int64_t src_dptr, int64_t n, int workgroups_per_cu)
+{
+    COMET_CHK(ensure_init());
+    if (n <= 0 || (n & 1) || mode < 0 || mode > 3 || (mode != 2 && !dst_dptr) || (mode != 3 && !src_dptr) ||
+        workgroups_per_cu < 0 || workgroups_per_cu > 64 || ((dst_dptr | src_dptr) & 15))
+        return set_error(COMET_HIP_ERR_ARG, "bad arguments to comet_hip_stream_bench");
+    const int64_t n2 = n / 2;
+    const unsigned blocks =
+        (unsigned)std::min<int64_t>(ceil_div(n2, 256), (int64_t)num_cus() * (workgroups_per_cu ? workgroups_per_cu : 8));
+    if (mode == 2)
+        COMET_CHK(g_stream_out.ensure(sizeof(double) * 256 * (size_t)blocks, false));
+    if (mode <= 1) {
+        KernelTimer t(mode ? "stream_copy16_nt_kernel" : "stream_copy16_kernel");
+        stream_copy16_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>((stream_v2d *)dst_dptr,
+                                                                        (const stream_v2d *)src_dptr, n2, mode);
+    } else if (mode == 2) {
+        KernelTimer t("stream_read16_kernel");
+        stream_read16_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>((const stream_v2d *)src_dptr, n2,
+                                                                        (double *)g_stream_out.ptr);
+    } else {
+        KernelTimer t("stream_write16_kernel");
+        stream_write16_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>((stream_v2d *)dst_dptr, n2, 1.0);
+    }
+    COMET_HIPCHK(hipGetLastError());
+    return COMET_HIP_OK;
+}
+
+// A stream of the caller's own (default priority), for the entry points that take one.
+int64_t comet_hip_stream_create(void)
+{
+    if (ensure_init() != COMET_HIP_OK)
+        return 0;
+    hipStream_t s = nullptr;
+    if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) {
+        (void)hipGetLastError();
+        set_error(COMET_HIP_ERR_HIP, "hipStreamCreateWithFlags failed");
+        return 0;
+    }
+    return (int64_t)s;
+}
+
+int comet_hip_stream_sync(int64_t s)
+{
+    COMET_CHK(ensure_init());
+    COMET_HIPCHK(hipStreamSynchronize(s ? (hipStream_t)s : stream()));
+    return COMET_HIP_OK;
+}
+
+int comet_hip_stream_destroy(int64_t s)
+{
+    COMET_CHK(ensure_init());
+    if (!s)
+        return set_error(COMET_HIP_ERR_ARG, "comet_hip_stream_destroy: null stream");
+    COMET_HIPCHK(hipStreamDestroy((hipStream_t)s));
     return COMET_HIP_OK;
 }
 

@@ -464,9 +464,13 @@ __device__ __forceinline__ double semiring_lds_value(unsigned long long v, int r
         return v < f64_key(0.0) ? 0.0 : key_f64(v);
     return semiring_mult(mult_op, Aval[as + (int64_t)(v >> 32) - 1], Bval[(int64_t)(v & 0xffffffffull)]);
 }
-extern __shared__ uint32_t sg_dyn_lds[];
+// Every kernel here carves its dynamic LDS into 32-bit words and fp64 regions (ds_add_f64 and 64-bit reads fault on
+// an address that is not a multiple of 8): the array itself starts 16-byte aligned, and every fp64 region begins an
+// even number of words into it - asserted where each layout is defined.
+extern __shared__ __align__(16) uint32_t sg_dyn_lds[];
 // Hash table of a masked product's mask row (see spgemm_numeric_kernel): values first (8-byte aligned), keys after.
 constexpr int SG_HASH_LOG = 13, SG_HASH_SLOTS = 1 << SG_HASH_LOG;
+static_assert((2 * SG_HASH_SLOTS) % 2 == 0 && SG_HASH_SLOTS % 2 == 0, "hash table: values at word 0, keys an even number of words in");
 #ifndef COMET_SG_HASH_FILL
 #define COMET_SG_HASH_FILL (SG_HASH_SLOTS * 3 / 4)
 #endif
@@ -945,6 +949,9 @@ constexpr int SG_EMIT = 8192;                                         // entries
 constexpr size_t SG_DENSE_LDS = (size_t)SG_CB * 8 + (size_t)SG_CB / 8 + (size_t)SG_EMIT * sizeof(emit_t) +
                                 2 * (size_t)SG_CB / 8;               // accumulators, bitmap, list of the columns being
                                                                       // written out, the mask row's bits (two blocks)
+// the accumulators (fp64) come first; what follows them is 32- and 16-bit data and starts on a word
+static_assert(((size_t)SG_CB * 8) % 8 == 0 && ((size_t)SG_CB / 8) % 4 == 0 && ((size_t)SG_EMIT * sizeof(emit_t)) % 4 == 0,
+              "the one-block kernel's LDS regions are aligned for their types");
 
 // products[i - row_begin] = sum over k in A_i of nnz(B_k); one wavefront per row.  With Tpos (the dot-product form of
 // a masked product, where row i's pairs k are shared out by which of the two lists is longer) only the k whose row
@@ -1755,6 +1762,8 @@ constexpr int SP_WPT = SP_WORDS / SG_T;                   // consecutive bitmap 
 constexpr int SP_CAP = SG_CB;                             // entries of C per visit at most
 constexpr int SP_CHUNK = 64 * SG_LONG_LOADS;              // entries of a slice that a wavefront takes in one turn
 constexpr size_t SG_SPAN_LDS = (size_t)SP_CAP * 8 + (size_t)SP_WORDS * 4 + (size_t)SP_WORDS * 2;   // values, bitmap, ranks
+static_assert(((size_t)SP_CAP * 8) % 8 == 0 && ((size_t)SP_WORDS * 4) % 4 == 0,
+              "the span kernel's values (fp64) come first in its LDS, bitmap and ranks follow on word boundaries");
 static_assert(SP_WORDS % SG_T == 0 && SP_BLOCK_WORDS % SP_WPT == 0 && SP_CAP >= SG_CB && SP_CAP <= 65535,
               "a thread's words lie in one block, one block fits the value array, ranks fit 16 bits");
 
@@ -2329,6 +2338,18 @@ constexpr size_t dot_lds_bytes(int words)
     return (size_t)dot_table_words(words) * 4 + (size_t)SG_WAVES * 64 * (8 + 4);
 }
 static_assert(dot_lds_bytes(SG_T * DT_WPT) <= 160 * 1024 - 256, "the table of 2^20 columns fits LDS");
+// the fp64 regions of the dot-product kernel: the hash table's values SG_HASH_SLOTS words in, the wavefronts' sums
+// dot_table_words(words) words in, for every table size the host can ask for (a multiple of DT_WPT words)
+constexpr bool dot_fp64_regions_aligned()
+{
+    if (SG_HASH_SLOTS % 2 != 0)
+        return false;
+    for (int w = DT_WPT; w <= SG_T * DT_WPT; w += DT_WPT)
+        if (dot_table_words(w) % 2 != 0)
+            return false;
+    return true;
+}
+static_assert(dot_fp64_regions_aligned(), "an fp64 region of the dot-product kernel's LDS is not 8-byte aligned");
 
 // The pairs [ms, me) of one row of P, dealt to the wavefronts like the entries of a row of A in
 // for_each_product_impl (the walk of a turn and its one-turn-late visits are the same); keep(y, len) says whether
@@ -2958,11 +2979,14 @@ static int sg_plan_blocks(Csr *b)
         b->sg_crd16 = nullptr;
     }
     static_assert(SG_CB <= 65536, "a column inside its block fits 16 bits");
-    if (hipMalloc((void **)&b->sg_crd16, sizeof(uint16_t) * (size_t)(b->nnz > 0 ? b->nnz : 1)) != hipSuccess)
+    if (hipMalloc((void **)&b->sg_crd16, sizeof(uint16_t) * (size_t)(b->nnz > 0 ? b->nnz : 1)) != hipSuccess) {
+        (void)hipGetLastError();        // an allocation that may fail: its error must not reach the next check
         b->sg_crd16 = nullptr;          // the kernel then reads the 32-bit columns
-    else if (b->nnz > 0)
+    } else if (b->nnz > 0) {
         spgemm_block_columns<<<dim3((unsigned)ceil_div(b->nnz, 256)), dim3(256), 0, stream()>>>(b->nnz, b->crd,
                                                                                                  b->sg_crd16);
+        COMET_HIPCHK(hipGetLastError());
+    }
     COMET_HIPCHK(hipMalloc((void **)&b->sg_blkptr,
                            sizeof(int64_t) * (size_t)(nblk + 1) * (size_t)(b->nrows > 0 ? b->nrows : 1)));
     b->sg_nblk = nblk;
@@ -3076,6 +3100,8 @@ static int dot_pairs(const Csr *a, const Csr *b, const Csr *m, int64_t rb, int64
     int words = (int)ceil_div(a->ncols > 0 ? a->ncols : 1, 32);
     words = (int)ceil_div(words, DT_WPT) * DT_WPT;
     const size_t lds = dot_lds_bytes(words);
+    if (dot_table_words(words) % 2 != 0 || words % DT_WPT != 0)        // the wavefronts' fp64 sums follow the table
+        return set_error(COMET_HIP_ERR_SIZE, "dot-product table of %d words leaves its sums misaligned", words);
     const dim3 grid((unsigned)(num_cus() > 0 ? num_cus() : 256)), block(SG_T);
     const int64_t everywhere = 1ll << 62;
     for (int half = 0; half < 2; ++half) {
@@ -3199,6 +3225,9 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
             COMET_CHK(g_sg.dense_rows.ensure(sizeof(DenseRow) * (size_t)nd, false));
             COMET_CHK(g_sg.dense_before.ensure(sizeof(int32_t) * (size_t)nd * (size_t)nblk, false));
             COMET_CHK(g_sg.gave_up.ensure(sizeof(int), true));
+            // cleared before every launch that can set it: a call that fails between the launch and the read
+            // below must not leave it set for the next product
+            COMET_HIPCHK(hipMemsetAsync(g_sg.gave_up.ptr, 0, sizeof(int), stream()));
             COMET_CHK(sg_reset_ticket());
             int patience = DB_PATIENCE;
             if (const char *e = getenv("COMET_HIP_SPGEMM_PATIENCE"))
@@ -3643,4 +3672,14 @@ extern "C" int comet_hip_eltwise_dense_f64(int64_t n, int64_t a_dptr, int64_t b_
                                                                   (double *)c_dptr, op);
     COMET_HIPCHK(hipGetLastError());
     return COMET_HIP_OK;
+}
+
+// Diagnostic: where the fp64 sums of the dot-product kernel begin in its LDS, in 32-bit words, for a bitmap of
+// `words` words (rounded up to what the host would ask for); lets a CPU-side test sweep the invariant "even".
+extern "C" int comet_hip_debug_dot_table_words(int words)
+{
+    if (words < 1)
+        words = 1;
+    words = (int)ceil_div((int64_t)words, (int64_t)DT_WPT) * DT_WPT;
+    return dot_table_words(words);
 }

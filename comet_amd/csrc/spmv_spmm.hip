@@ -347,6 +347,8 @@ static int spmv_plan(Csr *a)
             } else {
                 (void)hipFree(bpos32);
             }
+        } else {
+            (void)hipGetLastError();        // an allocation that may fail: the 64-bit pointers stay in use
         }
     }
     a->spmv_bpos = bpos;
@@ -1740,8 +1742,11 @@ int spmm_static_setup(int device)
 }  // namespace comet
 
 extern "C" int comet_hip_spmm_csr_f64_noalloc(int64_t csr, int64_t K, int64_t b_dptr, int64_t ldb, int64_t c_dptr,
-                                              int64_t ldc, int accumulate)
+                                              int64_t ldc, int accumulate, int64_t on_stream)
 {
+    // on_stream: the hipStream_t the caller wants the kernels on (a stream under graph capture, a serving loop's own
+    // stream), as an integer; 0 = the library's stream, like every other entry point
+    const hipStream_t on = on_stream ? (hipStream_t)on_stream : stream();
     if (!is_initialised())       // bringing the device up creates streams: the caller does that beforehand
         return set_error(COMET_HIP_ERR_ARG, "comet_hip_spmm_csr_f64_noalloc: call comet_hip_init first");
     Csr *a = csr_from_handle(csr);
@@ -1770,7 +1775,7 @@ extern "C" int comet_hip_spmm_csr_f64_noalloc(int64_t csr, int64_t K, int64_t b_
     if (a->nnz == 0) {
         if (!accumulate) {
             const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div(a->nrows * K, 256), 65536);
-            fill_rows_f64<<<dim3(blocks), dim3(256), 0, stream()>>>(C, a->nrows, K, ldc, 0.0);
+            fill_rows_f64<<<dim3(blocks), dim3(256), 0, on>>>(C, a->nrows, K, ldc, 0.0);
             COMET_HIPCHK(hipGetLastError());
         }
         return COMET_HIP_OK;
@@ -1779,19 +1784,19 @@ extern "C" int comet_hip_spmm_csr_f64_noalloc(int64_t csr, int64_t K, int64_t b_
     // slot by the chunk that leaves a piece of a row in it), so nothing has to be cleared between calls.
     int32_t *chunk_row = reinterpret_cast<int32_t *>(scratch);
     double *carry = reinterpret_cast<double *>(scratch + SPMM_STATIC_TABLE_BYTES);
-    spmm_chunk_rows<<<dim3((unsigned)ceil_div(nchunks, 256)), dim3(256), 0, stream()>>>(a->pos, a->nrows, nchunks,
+    spmm_chunk_rows<<<dim3((unsigned)ceil_div(nchunks, 256)), dim3(256), 0, on>>>(a->pos, a->nrows, nchunks,
                                                                                          chunk_row);
     const dim3 grid((unsigned)ceil_div(nchunks, SPMM_WAVES), (unsigned)tiles), block(SPMM_WAVES * 64);
     const double *B = (const double *)b_dptr;
     if (accumulate) {
-        spmm_csr_nnzsplit<true><<<grid, block, 0, stream()>>>(a->pos, a->crd, a->val, a->nnz, a->nrows, chunk_row,
+        spmm_csr_nnzsplit<true><<<grid, block, 0, on>>>(a->pos, a->crd, a->val, a->nnz, a->nrows, chunk_row,
                                                               nchunks, B, ldb, C, ldc, K, carry, nullptr);
-        spmm_csr_fixup<true><<<grid, block, 0, stream()>>>(a->pos, a->nnz, chunk_row, nchunks, C, ldc, K, carry,
+        spmm_csr_fixup<true><<<grid, block, 0, on>>>(a->pos, a->nnz, chunk_row, nchunks, C, ldc, K, carry,
                                                            nullptr);
     } else {
-        spmm_csr_nnzsplit<false><<<grid, block, 0, stream()>>>(a->pos, a->crd, a->val, a->nnz, a->nrows, chunk_row,
+        spmm_csr_nnzsplit<false><<<grid, block, 0, on>>>(a->pos, a->crd, a->val, a->nnz, a->nrows, chunk_row,
                                                                nchunks, B, ldb, C, ldc, K, carry, nullptr);
-        spmm_csr_fixup<false><<<grid, block, 0, stream()>>>(a->pos, a->nnz, chunk_row, nchunks, C, ldc, K, carry,
+        spmm_csr_fixup<false><<<grid, block, 0, on>>>(a->pos, a->nnz, chunk_row, nchunks, C, ldc, K, carry,
                                                             nullptr);
     }
     COMET_HIPCHK(hipGetLastError());

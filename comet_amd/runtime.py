@@ -76,7 +76,7 @@ SIGNATURES = {
     "comet_hip_csr_destroy": (_int, [_i64]),
     "comet_hip_spmv_csr_f64": (_int, [_i64, _i64, _i64, _int]),
     "comet_hip_spmm_csr_f64": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
-    "comet_hip_spmm_csr_f64_noalloc": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
+    "comet_hip_spmm_csr_f64_noalloc": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _int, _i64]),
     "comet_hip_spgemm_csr_symbolic": (_int, [_i64, _i64, _i64, _i64, _pi64]),
     "comet_hip_spgemm_csr_numeric": (_int, [_i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64]),
     "comet_hip_spgemm_csr": (_i64, [_i64, _i64, _i64]),
@@ -124,9 +124,23 @@ SIGNATURES = {
     "comet_hip_profile_query": (_int, [C.c_char_p, _pi64, C.POINTER(_f64)]),
     "comet_hip_profile_name": (_int, [_i32, C.c_char_p, _i64]),
     "comet_hip_copy_f64": (_int, [_i64, _i64, _i64]),
+    "comet_hip_debug_dot_table_words": (_int, [_int]),
+    "comet_hip_stream_create": (_i64, []),
+    "comet_hip_stream_sync": (_int, [_i64]),
+    "comet_hip_stream_destroy": (_int, [_i64]),
+    "comet_hip_stream_bench": (_int, [_int, _i64, _i64, _i64, _int]),
     "comet_hip_mem_info": (_int, [C.POINTER(_i64), C.POINTER(_i64)]),
     "comet_hip_mfma_f64_peak": (_int, [_i64, C.POINTER(C.c_double)]),
     "comet_hip_gather_rows_bench": (_int, [_i64, _i64, _i64, _i64, _i64, _i64]),
+    "_mlir_ciface_comet_hip_spgemm_csr_sizes_semiring_f64_i64": (None, [_i64, _i64, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _i32, _i32]),
+    "_mlir_ciface_comet_hip_spgemm_csr_sizes_semiring_f64_i32": (None, [_i64, _i64, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _i32, _i32]),
+    "_mlir_ciface_comet_hip_spgemm_csr_fill_semiring_f64_i64": (None, [_m1, _m1, _m1]),
+    "_mlir_ciface_comet_hip_spgemm_csr_fill_semiring_f64_i32": (None, [_m1, _m1, _m1]),
+    "_mlir_ciface_comet_hip_ttgt_contract_f64": (None, [_i64, _vp, _i64, _vp, _i64, _vp, _m1, _m1, _m1, _f64]),
+    "_mlir_ciface_linalg_matmul_viewsxs_viewsxs_viewsxs": (None, [_m2, _m2, _m2, _int, _int, _f64, _f64]),
+    "read_input_sizes_2D_f64": (None, [_i32, _i32, _i32, _i32, _i32, _int, _vp, _i32]),
+    "read_input_2D_f64_i64": (None, [_i32, _i32, _i32, _i32, _i32] + [_int, _vp] * 9 + [_i32]),
+    "read_input_2D_f64_i32": (None, [_i32, _i32, _i32, _i32, _i32] + [_int, _vp] * 9 + [_i32]),
     "_mlir_ciface_comet_hip_spmv_csr_f64_i64": (None, [_m1, _m1, _m1, _m1, _m1]),
     "_mlir_ciface_comet_hip_spmm_csr_f64_i64": (None, [_m1, _m1, _m1, _m2, _m2]),
     "_mlir_ciface_comet_hip_spgemm_csr_sizes_f64_i64": (None, [_i64, _i64, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _m1, _m1]),
@@ -668,3 +682,23 @@ def memref2d(a):
     m.sizes[0], m.sizes[1] = a.shape
     m.strides[0], m.strides[1] = a.shape[1], 1
     return m
+
+
+def memref_nd(a):
+    """An unranked-memref descriptor of a contiguous array: (struct, void pointer to it); keep the struct alive
+    while the pointer is in use.  StridedMemRefType<T, N> = {T *allocated; T *aligned; int64 offset;
+    int64 sizes[N]; int64 strides[N]}."""
+    n = a.ndim
+
+    class _M(C.Structure):
+        _fields_ = [("allocated", C.c_void_p), ("aligned", C.c_void_p), ("offset", C.c_int64),
+                    ("sizes", C.c_int64 * n), ("strides", C.c_int64 * n)]
+
+    m = _M()
+    m.allocated = m.aligned = a.ctypes.data
+    m.offset = 0
+    for d in range(n):
+        m.sizes[d] = a.shape[d]
+        m.strides[d] = a.strides[d] // a.itemsize
+    return m, C.cast(C.pointer(m), C.c_void_p)
+

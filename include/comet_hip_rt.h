@@ -54,6 +54,13 @@ int comet_hip_free(int64_t dptr);
 int comet_hip_memcpy(int64_t dptr, void *host, int64_t bytes, int64_t direction);
 int comet_hip_memset(int64_t dptr, int byte_value, int64_t bytes);
 int comet_hip_sync(void);
+/* A stream of the caller's own, as an integer (a hipStream_t, default
+ * priority), for the entry points that take one; 0 on failure.  sync with 0
+ * waits for the library's stream.  No counterpart in the reference, whose
+ * runtime only knows the NULL stream (HipGpuUtils.cpp:21). */
+int64_t comet_hip_stream_create(void);
+int comet_hip_stream_sync(int64_t stream);
+int comet_hip_stream_destroy(int64_t stream);
 int64_t HipMallocF64(int64_t n);
 int64_t HipMallocI64(int64_t n);
 int64_t HipMallocI32(int64_t n);
@@ -68,7 +75,13 @@ void HipMemcpyIndex(int64_t dptr, void *ptr, void *aligned, int64_t offset, int6
  * fill" protocol of read_input_sizes_2D_f64 / read_input_2D_f64,
  * lib/ExecutionEngine/SparseUtils.cpp:1632-1811,1814-2078): upload takes the
  * host arrays the lowered code already owns; dims + download give them back.
- * Returns a handle (> 0) or 0 on failure. */
+ * Returns a handle (> 0) or 0 on failure.
+ * Precondition, checked on the host before anything is copied: pos starts at 0,
+ * never decreases and ends at nnz; every column lies in [0, ncols) and the
+ * columns of a row do not decrease (what the reference's reader produces,
+ * SparseUtils.cpp:421; the kernels bisect rows and index LDS by column).  The
+ * reference's CPU loop nests would also accept rows in any column order; such
+ * arrays are refused here - order them first with comet_hip_csr_from_coo_i64. */
 int64_t comet_hip_csr_upload_i64(int64_t nrows, int64_t ncols, const int64_t *pos,
                                  const int64_t *crd, const double *val);
 int64_t comet_hip_csr_upload_i32(int64_t nrows, int64_t ncols, const int32_t *pos,
@@ -80,7 +93,8 @@ int64_t comet_hip_csr_upload_i32(int64_t nrows, int64_t ncols, const int32_t *po
  * handle is used again.  Both calls look at the arrays once on the device
  * (pos starts at 0, never decreases, ends at nnz; columns inside [0, ncols) and
  * not decreasing inside a row) and refuse anything else: wrap returns 0,
- * invalidate COMET_HIP_ERR_ARG. */
+ * invalidate COMET_HIP_ERR_ARG - and the handle then refuses every product
+ * (COMET_HIP_ERR_HANDLE) until a later invalidate passes or it is destroyed. */
 int64_t comet_hip_csr_wrap(int64_t nrows, int64_t ncols, int64_t nnz,
                            int64_t pos_dptr, int64_t crd_dptr, int64_t val_dptr);
 int comet_hip_csr_dims(int64_t csr, int64_t *nrows, int64_t *ncols, int64_t *nnz);
@@ -104,7 +118,13 @@ int comet_hip_spmv_csr_f64(int64_t csr, int64_t x_dptr, int64_t y_dptr, int accu
  * (elements).  accumulate as for SpMV.
  * Both products keep a plan in the handle (a re-ordered copy of parts of the
  * matrix) that costs tens of products to build: it is built when a handle is
- * multiplied for the second time, the first product runs without it. */
+ * multiplied for the second time, the first product runs without it.
+ * Rounding: a row that lies inside one 256-nonzero chunk is summed in nonzero
+ * order with separate multiply and add, bit for bit as the reference's nest
+ * (IndexTreeToSCF.cpp:203-205); a row cut by a chunk boundary adds its pieces
+ * in chunk order; the long rows a plan takes out (128 nonzeros and more) are
+ * summed with fused multiply-adds from sixteen partial sums, so they agree
+ * with the reference to rounding (1e-12 * sum |a||b|), never bitwise. */
 int comet_hip_spmm_csr_f64(int64_t csr, int64_t K, int64_t b_dptr, int64_t ldb,
                            int64_t c_dptr, int64_t ldc, int accumulate);
 
@@ -116,9 +136,12 @@ int comet_hip_spmm_csr_f64(int64_t csr, int64_t K, int64_t b_dptr, int64_t ldb,
  * ceil(K/64) * ceil(nnz/256) <= 8192 (nnz <= 2,097,152 at K <= 64), larger
  * products return COMET_HIP_ERR_SIZE.  Rows are summed exactly as
  * comet_hip_spmm_csr_f64 sums them for a matrix below its long-row threshold.
- * All calls on one device share the array: calls that overlap in time race. */
+ * All calls on one device share the array: calls that overlap in time race.
+ * on_stream: the hipStream_t (as an integer) the kernels are launched on, so that
+ * a caller that captures a graph or keeps a stream of its own gets them there,
+ * ordered with its other work; 0 = the library's stream, as everywhere else. */
 int comet_hip_spmm_csr_f64_noalloc(int64_t csr, int64_t K, int64_t b_dptr, int64_t ldb,
-                                   int64_t c_dptr, int64_t ldc, int accumulate);
+                                   int64_t c_dptr, int64_t ldc, int accumulate, int64_t on_stream);
 
 /* ---- SpGEMM  C = A * B, CSR x CSR -> CSR, optional structural mask ---------
  * Symbolic phase: per-row count of distinct output columns and the row
@@ -259,6 +282,31 @@ void comet_hip_read_input_2D_f64_i32(int32_t file_id, int32_t a1format, int32_t 
                                      int a2tile_pos_rank, void *a2tile_pos_desc,
                                      int a2tile_crd_rank, void *a2tile_crd_desc,
                                      int aval_rank, void *aval_desc, int32_t read_mode);
+/* The three calls under the names lowered code already calls
+ * (lib/ExecutionEngine/SparseUtils.cpp:2562-2568, 2403-2425, 2427-2450): with this
+ * library in -shared-libs in place of libcomet_runner_utils, `ta.read` resolves
+ * without a compiler change.  Same argument lists and behaviour as above. */
+void read_input_sizes_2D_f64(int32_t file_id, int32_t a1format, int32_t a1_tile_format,
+                             int32_t a2format, int32_t a2_tile_format,
+                             int sizes_rank, void *sizes_desc, int32_t read_mode);
+void read_input_2D_f64_i64(int32_t file_id, int32_t a1format, int32_t a1_tile_format,
+                           int32_t a2format, int32_t a2_tile_format,
+                           int a1pos_rank, void *a1pos_desc, int a1crd_rank, void *a1crd_desc,
+                           int a1tile_pos_rank, void *a1tile_pos_desc,
+                           int a1tile_crd_rank, void *a1tile_crd_desc,
+                           int a2pos_rank, void *a2pos_desc, int a2crd_rank, void *a2crd_desc,
+                           int a2tile_pos_rank, void *a2tile_pos_desc,
+                           int a2tile_crd_rank, void *a2tile_crd_desc,
+                           int aval_rank, void *aval_desc, int32_t read_mode);
+void read_input_2D_f64_i32(int32_t file_id, int32_t a1format, int32_t a1_tile_format,
+                           int32_t a2format, int32_t a2_tile_format,
+                           int a1pos_rank, void *a1pos_desc, int a1crd_rank, void *a1crd_desc,
+                           int a1tile_pos_rank, void *a1tile_pos_desc,
+                           int a1tile_crd_rank, void *a1tile_crd_desc,
+                           int a2pos_rank, void *a2pos_desc, int a2crd_rank, void *a2crd_desc,
+                           int a2tile_pos_rank, void *a2tile_pos_desc,
+                           int a2tile_crd_rank, void *a2tile_crd_desc,
+                           int aval_rank, void *aval_desc, int32_t read_mode);
 /* The same read for lowered code that keeps tensors on the device: the CSR
  * handle itself (0 on failure), no host arrays.  Consumes what a preceding
  * sizes call for the same id and mode built, or reads the file now. */
@@ -359,13 +407,24 @@ int comet_hip_profile_reset(void);
 /* name == NULL: number of distinct kernel names recorded so far. */
 int comet_hip_profile_query(const char *name, int64_t *launches, double *total_ms);
 int comet_hip_profile_name(int32_t index, char *buf, int64_t cap);
-/* Plain device-to-device copy kernel (used to calibrate hardware counters). */
+/* ---- diagnostics: yardsticks the measurements are set against -----------------
+ * None of the functions from here to comet_hip_gather_rows_bench has a
+ * counterpart in the reference and none is on the product path; they exist so
+ * that a roofline fraction can be read against what the machine does on the
+ * simplest kernel of the same kind. */
+/* Plain device-to-device copy kernel, 8 bytes per lane (used to calibrate
+ * hardware counters). */
 int comet_hip_copy_f64(int64_t dst_dptr, int64_t src_dptr, int64_t n);
+/* Streaming kernels with 16 bytes per lane over n doubles (n even, pointers
+ * 16-byte aligned).  mode 0: copy with ordinary loads and stores; 1: copy with
+ * non-temporal loads and stores; 2: read only (src; every lane sums what it
+ * reads); 3: write only (dst).  workgroups_per_cu: 256-lane workgroups per CU in
+ * the grid, 0 = 8. */
+int comet_hip_stream_bench(int mode, int64_t dst_dptr, int64_t src_dptr, int64_t n, int workgroups_per_cu);
 /* Free and total device memory (hipMemGetInfo): lets a caller see what a first
  * call kept (plans cached in a handle, workspaces). */
 int comet_hip_mem_info(int64_t *free_bytes, int64_t *total_bytes);
-/* Two yardsticks the measurements are set against, neither has a counterpart in
- * the reference.  mfma_f64_peak: TFLOP/s of back-to-back v_mfma_f64_16x16x4_f64
+/* Two more diagnostics.  mfma_f64_peak: TFLOP/s of back-to-back v_mfma_f64_16x16x4_f64
  * on registers (`iters` x 16 per wavefront, 8 wavefronts per CU), the rate the
  * TTGT GEMM is compared with.  gather_rows_bench: every wavefront fetches
  * per_wave rows of 64 doubles named by idx (int32, one list per wavefront, 16
@@ -373,6 +432,10 @@ int comet_hip_mem_info(int64_t *free_bytes, int64_t *total_bytes);
  * per lane as the SpMM sweep does, and sums them into out (workgroups x 1024
  * doubles): the rate at which the CUs can take rows out of the L2. */
 int comet_hip_mfma_f64_peak(int64_t iters, double *tflops);
+/* Diagnostic: the word offset at which the fp64 sums of the masked-product
+ * kernel begin in its LDS for a bitmap of `words` 32-bit words; always even (an
+ * odd offset would misalign its 64-bit LDS atomics).  Runs on the host. */
+int comet_hip_debug_dot_table_words(int words);
 int comet_hip_gather_rows_bench(int64_t workgroups, int64_t per_wave, int64_t idx_dptr,
                                 int64_t table_dptr, int64_t table_rows, int64_t out_dptr);
 
@@ -382,7 +445,10 @@ int comet_hip_gather_rows_bench(int64_t workgroups, int64_t per_wave, int64_t id
  * int64 sizes[N]; int64 strides[N]} holding HOST data, exactly as the
  * reference's other runtime calls receive them
  * (lib/ExecutionEngine/StatUtils.cpp:89-113, blis_interface.cpp:143-146).
- * They upload, run the kernel, and copy the result back. */
+ * They upload, run the kernel, and copy the result back.  The CSR operands
+ * must satisfy the precondition stated at comet_hip_csr_upload_* (columns of a
+ * row not decreasing): an operand that does not ends the program with a message,
+ * as every failure of these forms does. */
 typedef struct { void *allocated; void *aligned; int64_t offset; int64_t sizes[1]; int64_t strides[1]; } comet_memref_1d;
 typedef struct { void *allocated; void *aligned; int64_t offset; int64_t sizes[2]; int64_t strides[2]; } comet_memref_2d;
 
@@ -416,6 +482,45 @@ void _mlir_ciface_comet_hip_spgemm_csr_fill_f64_i32(comet_memref_1d *Cpos, comet
                                                     comet_memref_1d *Cval);
 double _mlir_ciface_comet_hip_tricount_f64_i32(int64_t ncols, comet_memref_1d *pos, comet_memref_1d *crd,
                                                comet_memref_1d *val);
+
+/* SpGEMM over a semiring through the same pair of calls: the operator codes of
+ * comet_hip_spgemm_csr_semiring after the sizes memref
+ * (lib/Conversion/IndexTreeToSCF/IndexTreeToSCF.cpp:198-360;
+ * test/integration/semiring/mm_Semiring*_CSRxCSR_oCSR.ta).  The fill call is the
+ * plain one under a second name. */
+void _mlir_ciface_comet_hip_spgemm_csr_sizes_semiring_f64_i64(int64_t nrowsA, int64_t ncolsB,
+        comet_memref_1d *Apos, comet_memref_1d *Acrd, comet_memref_1d *Aval,
+        comet_memref_1d *Bpos, comet_memref_1d *Bcrd, comet_memref_1d *Bval,
+        comet_memref_1d *Mpos, comet_memref_1d *Mcrd, comet_memref_1d *sizes,
+        int32_t reduce_op, int32_t mult_op);
+void _mlir_ciface_comet_hip_spgemm_csr_fill_semiring_f64_i64(comet_memref_1d *Cpos, comet_memref_1d *Ccrd,
+                                                             comet_memref_1d *Cval);
+void _mlir_ciface_comet_hip_spgemm_csr_sizes_semiring_f64_i32(int64_t nrowsA, int64_t ncolsB,
+        comet_memref_1d *Apos, comet_memref_1d *Acrd, comet_memref_1d *Aval,
+        comet_memref_1d *Bpos, comet_memref_1d *Bcrd, comet_memref_1d *Bval,
+        comet_memref_1d *Mpos, comet_memref_1d *Mcrd, comet_memref_1d *sizes,
+        int32_t reduce_op, int32_t mult_op);
+void _mlir_ciface_comet_hip_spgemm_csr_fill_semiring_f64_i32(comet_memref_1d *Cpos, comet_memref_1d *Ccrd,
+                                                             comet_memref_1d *Cval);
+
+/* Dense contraction on host memrefs: upload -> plan -> transposes -> GEMM ->
+ * download in one call, in place of the transpose / collapse / matmul / expand /
+ * transpose chain the reference emits
+ * (lib/Dialect/TensorAlgebra/Transforms/TCtoTTGTDyn.cpp:288-672).  A, B, C are
+ * unranked memrefs (rank, pointer to StridedMemRefType<double, rank>), rank 1..8,
+ * contiguous row-major; x_lab holds one `index` per dimension, the same number
+ * for the same index label (C[a,b,c,d] = A[a,e,b,f] * B[d,f,c,e]: 0,4,1,5 /
+ * 3,5,2,4 / 0,1,2,3); beta 0 overwrites C, 1 adds to it. */
+void _mlir_ciface_comet_hip_ttgt_contract_f64(int64_t rankA, void *A, int64_t rankB, void *B,
+                                              int64_t rankC, void *C, comet_memref_1d *a_lab,
+                                              comet_memref_1d *b_lab, comet_memref_1d *c_lab, double beta);
+/* The reference's own name for the matrix product its TTGT lowering ends in
+ * under -opt-matmul-mkernel (lib/ExecutionEngine/blis_interface.cpp:143-181):
+ * C = alpha * A * B + beta * C on strided 2-D views of host memory.  mr and nr
+ * (the micro-kernel's tile) are ignored: the whole product runs on the device. */
+void _mlir_ciface_linalg_matmul_viewsxs_viewsxs_viewsxs(comet_memref_2d *A, comet_memref_2d *B,
+                                                        comet_memref_2d *C, int mr, int nr,
+                                                        double alpha, double beta);
 
 /* ---- host utilities of the reference's runtime ----------------------------
  * The names and argument lists lowered programs already call

@@ -216,11 +216,100 @@ idx_t oracle_spgemm_symbolic(idx_t row_begin, idx_t row_end, idx_t ncolsB,
     return total;
 }
 
-static int cmp_idx(const void *a, const void *b)
+/* The reference sorts a row's touched columns with std::sort                  */
+/* (lib/ExecutionEngine/SparseUtils.cpp:2600-2626): an introsort - quicksort on */
+/* a median of three, heapsort below a depth limit, one insertion sort at the   */
+/* end - inlined on the element type.  qsort with a comparison callback costs   */
+/* several times as much per element, which would flatter the GPU in the CPU    */
+/* baseline, so the same algorithm is written out here.                         */
+static void sift_down_idx(idx_t *a, size_t root, size_t n)
 {
-    idx_t x = *(const idx_t *)a, y = *(const idx_t *)b;
-    return (x > y) - (x < y);
+    for (;;) {
+        size_t child = 2 * root + 1;
+        if (child >= n)
+            return;
+        if (child + 1 < n && a[child] < a[child + 1])
+            ++child;
+        if (a[root] >= a[child])
+            return;
+        idx_t t = a[root];
+        a[root] = a[child];
+        a[child] = t;
+        root = child;
+    }
 }
+
+static void heapsort_idx(idx_t *a, size_t n)
+{
+    for (size_t i = n / 2; i-- > 0;)
+        sift_down_idx(a, i, n);
+    for (size_t end = n; end-- > 1;) {
+        idx_t t = a[0];
+        a[0] = a[end];
+        a[end] = t;
+        sift_down_idx(a, 0, end);
+    }
+}
+
+static void introsort_loop_idx(idx_t *a, size_t n, int depth)
+{
+    while (n > 16) {
+        if (depth-- == 0) {
+            heapsort_idx(a, n);
+            return;
+        }
+        /* median of first, middle, last to a[0]; Hoare partition around it */
+        idx_t x = a[1], y = a[n / 2], z = a[n - 1], pivot;
+        if (x < y)
+            pivot = y < z ? y : (x < z ? z : x);
+        else
+            pivot = x < z ? x : (y < z ? z : y);
+        size_t i = 0, j = n - 1;
+        for (;;) {
+            while (a[i] < pivot)
+                ++i;
+            while (pivot < a[j])
+                --j;
+            if (i >= j)
+                break;
+            idx_t t = a[i];
+            a[i] = a[j];
+            a[j] = t;
+            ++i;
+            --j;
+        }
+        /* columns of a row are distinct, so i > 0 and i < n: both parts shrink */
+        if (i == 0 || i >= n) {
+            heapsort_idx(a, n);
+            return;
+        }
+        introsort_loop_idx(a + i, n - i, depth);
+        n = i;
+    }
+}
+
+static void sort_idx(idx_t *a, idx_t count)
+{
+    size_t n = (size_t)(count > 0 ? count : 0);
+    if (n < 2)
+        return;
+    int depth = 0;
+    for (size_t m = n; m > 1; m >>= 1)
+        depth += 2;
+    introsort_loop_idx(a, n, depth);
+    for (size_t i = 1; i < n; ++i) {      /* final insertion sort over the nearly sorted array */
+        idx_t v = a[i];
+        size_t j = i;
+        while (j > 0 && v < a[j - 1]) {
+            a[j] = a[j - 1];
+            --j;
+        }
+        a[j] = v;
+    }
+}
+
+/* the sort by itself, for the tests */
+void oracle_sort_idx(idx_t *a, idx_t n) { sort_idx(a, n); }
 
 /* ------------------------------------------------------------------------- */
 /* SpGEMM numeric phase over rows [row_begin,row_end).                         */
@@ -282,7 +371,7 @@ idx_t oracle_spgemm_numeric(idx_t row_begin, idx_t row_end, idx_t ncolsB,
         if (bits)
             for (idx_t t = mpos[i]; t < mpos[i + 1]; ++t)
                 bits[mcrd[t]] = 0;
-        qsort(crds, (size_t)num_crds, sizeof(idx_t), cmp_idx);
+        sort_idx(crds, num_crds);
         for (idx_t t = 0; t < num_crds; ++t) {
             idx_t j = crds[t];
             Ccrd[ipos] = j;
@@ -378,7 +467,7 @@ idx_t oracle_spgemm_numeric_semiring(idx_t row_begin, idx_t row_end, idx_t ncols
         if (bits)
             for (idx_t t = mpos[i]; t < mpos[i + 1]; ++t)
                 bits[mcrd[t]] = 0;
-        qsort(crds, (size_t)num_crds, sizeof(idx_t), cmp_idx);
+        sort_idx(crds, num_crds);
         for (idx_t t = 0; t < num_crds; ++t) {
             idx_t j = crds[t];
             Ccrd[ipos] = j;
@@ -477,7 +566,7 @@ double oracle_tricount_masked(idx_t nrows, idx_t ncols, const idx_t *pos,
         }
         for (idx_t t = pos[i]; t < pos[i + 1]; ++t)
             bits[crd[t]] = 0;
-        qsort(crds, (size_t)num_crds, sizeof(idx_t), cmp_idx);
+        sort_idx(crds, num_crds);
         for (idx_t t = 0; t < num_crds; ++t)
             acc = W[crds[t]] + acc;
     }
@@ -486,6 +575,186 @@ double oracle_tricount_masked(idx_t nrows, idx_t ncols, const idx_t *pos,
     free(crds);
     free(bits);
     return acc;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Row-parallel forms of the numeric phase and of the triangle count: a         */
+/* stronger CPU baseline than the reference itself offers (it never            */
+/* parallelises loops with a sparse output,                                    */
+/* lib/Conversion/TensorAlgebraToIndexTree/TensorAlgebraToIndexTree.cpp:278-   */
+/* 282).  Rows are independent; each thread keeps its own workspace, rows are  */
+/* handed out dynamically in blocks of 16, and a row's entries go where the    */
+/* symbolic phase's row pointer (Cpos, relative to row_begin) says.  A row is   */
+/* computed exactly as in the sequential form, so the output is identical.     */
+/* ------------------------------------------------------------------------- */
+idx_t oracle_spgemm_symbolic_omp(idx_t row_begin, idx_t row_end, idx_t ncolsB,
+                                 const idx_t *Apos, const idx_t *Acrd,
+                                 const idx_t *Bpos, const idx_t *Bcrd,
+                                 const idx_t *mpos, const idx_t *mcrd,
+                                 idx_t *rowcount)
+{
+    size_t n = (size_t)(ncolsB > 0 ? ncolsB : 1);
+    idx_t total = 0;
+#pragma omp parallel reduction(+ : total)
+    {
+        idx_t *mark = (idx_t *)calloc(n, sizeof(idx_t));
+        unsigned char *bits = mpos ? (unsigned char *)calloc(n, 1) : NULL;
+        if (mark && (!mpos || bits)) {
+#pragma omp for schedule(dynamic, 16)
+            for (idx_t i = row_begin; i < row_end; ++i) {
+                idx_t count = 0;
+                if (bits)
+                    for (idx_t t = mpos[i]; t < mpos[i + 1]; ++t)
+                        bits[mcrd[t]] = 1;
+                for (idx_t p = Apos[i]; p < Apos[i + 1]; ++p) {
+                    idx_t k = Acrd[p];
+                    for (idx_t q = Bpos[k]; q < Bpos[k + 1]; ++q) {
+                        idx_t j = Bcrd[q];
+                        if (bits && !bits[j])
+                            continue;
+                        if (mark[j] != i + 1) {
+                            mark[j] = i + 1;
+                            ++count;
+                        }
+                    }
+                }
+                if (bits)
+                    for (idx_t t = mpos[i]; t < mpos[i + 1]; ++t)
+                        bits[mcrd[t]] = 0;
+                rowcount[i - row_begin] = count;
+                total += count;
+            }
+        }
+        free(mark);
+        free(bits);
+    }
+    return total;
+}
+
+idx_t oracle_spgemm_numeric_omp(idx_t row_begin, idx_t row_end, idx_t ncolsB,
+                                const idx_t *Apos, const idx_t *Acrd, const double *Aval,
+                                const idx_t *Bpos, const idx_t *Bcrd, const double *Bval,
+                                const idx_t *mpos, const idx_t *mcrd, const idx_t *Cpos,
+                                idx_t *Ccrd, double *Cval)
+{
+    size_t n = (size_t)(ncolsB > 0 ? ncolsB : 1);
+    int failed = 0;
+#pragma omp parallel
+    {
+        double *W = (double *)malloc(n * sizeof(double));
+        unsigned char *seen = (unsigned char *)calloc(n, 1);
+        idx_t *crds = (idx_t *)malloc(n * sizeof(idx_t));
+        unsigned char *bits = mpos ? (unsigned char *)calloc(n, 1) : NULL;
+        if (!W || !seen || !crds || (mpos && !bits)) {
+#pragma omp atomic write
+            failed = 1;
+        }
+#pragma omp barrier
+        if (!failed) {
+#pragma omp for schedule(dynamic, 16)
+            for (idx_t i = row_begin; i < row_end; ++i) {
+                idx_t num_crds = 0;
+                if (bits)
+                    for (idx_t t = mpos[i]; t < mpos[i + 1]; ++t)
+                        bits[mcrd[t]] = 1;
+                for (idx_t p = Apos[i]; p < Apos[i + 1]; ++p) {
+                    idx_t k = Acrd[p];
+                    double a = Aval[p];
+                    for (idx_t q = Bpos[k]; q < Bpos[k + 1]; ++q) {
+                        idx_t j = Bcrd[q];
+                        if (bits && !bits[j])
+                            continue;
+                        double v = a * Bval[q];
+                        if (seen[j]) {
+                            W[j] = W[j] + v;
+                        } else {
+                            seen[j] = 1;
+                            crds[num_crds++] = j;
+                            W[j] = v;
+                        }
+                    }
+                }
+                if (bits)
+                    for (idx_t t = mpos[i]; t < mpos[i + 1]; ++t)
+                        bits[mcrd[t]] = 0;
+                sort_idx(crds, num_crds);
+                idx_t ipos = Cpos[i - row_begin];
+                for (idx_t t = 0; t < num_crds; ++t) {
+                    idx_t j = crds[t];
+                    Ccrd[ipos] = j;
+                    Cval[ipos] = W[j];
+                    seen[j] = 0;
+                    ++ipos;
+                }
+            }
+        }
+        free(W);
+        free(seen);
+        free(crds);
+        free(bits);
+    }
+    return failed ? -1 : Cpos[row_end - row_begin];
+}
+
+/* per-row sums added in row order afterwards: for unit values (every partial   */
+/* sum an integer below 2^53) this is the sequential result exactly            */
+double oracle_tricount_masked_omp(idx_t nrows, idx_t ncols, const idx_t *pos,
+                                  const idx_t *crd, const double *val)
+{
+    size_t n = (size_t)(ncols > 0 ? ncols : 1);
+    double *rowsum = (double *)calloc((size_t)(nrows > 0 ? nrows : 1), sizeof(double));
+    if (!rowsum)
+        return -1.0;
+#pragma omp parallel
+    {
+        double *W = (double *)malloc(n * sizeof(double));
+        unsigned char *seen = (unsigned char *)calloc(n, 1);
+        idx_t *crds = (idx_t *)malloc(n * sizeof(idx_t));
+        unsigned char *bits = (unsigned char *)calloc(n, 1);
+        if (W && seen && crds && bits) {
+#pragma omp for schedule(dynamic, 16)
+            for (idx_t i = 0; i < nrows; ++i) {
+                idx_t num_crds = 0;
+                for (idx_t t = pos[i]; t < pos[i + 1]; ++t)
+                    bits[crd[t]] = 1;
+                for (idx_t p = pos[i]; p < pos[i + 1]; ++p) {
+                    idx_t k = crd[p];
+                    double a = val[p];
+                    for (idx_t q = pos[k]; q < pos[k + 1]; ++q) {
+                        idx_t j = crd[q];
+                        if (!bits[j])
+                            continue;
+                        double v = a * val[q];
+                        if (seen[j]) {
+                            W[j] = W[j] + v;
+                        } else {
+                            seen[j] = 1;
+                            crds[num_crds++] = j;
+                            W[j] = v;
+                        }
+                    }
+                }
+                for (idx_t t = pos[i]; t < pos[i + 1]; ++t)
+                    bits[crd[t]] = 0;
+                sort_idx(crds, num_crds);
+                double acc = 0.0;
+                for (idx_t t = 0; t < num_crds; ++t) {
+                    acc = W[crds[t]] + acc;
+                    seen[crds[t]] = 0;
+                }
+                rowsum[i] = acc;
+            }
+        }
+        free(W);
+        free(seen);
+        free(crds);
+        free(bits);
+    }
+    double total = 0.0;
+    for (idx_t i = 0; i < nrows; ++i)
+        total = rowsum[i] + total;
+    free(rowsum);
+    return total;
 }
 
 /* ------------------------------------------------------------------------- */

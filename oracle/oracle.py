@@ -65,6 +65,8 @@ def lib():
     L.oracle_eltwise_dense.restype = None
     L.oracle_spgemm_symbolic.argtypes = [C.c_int64, C.c_int64, C.c_int64, i64p, i64p, i64p, i64p, vp, vp, i64p]
     L.oracle_spgemm_symbolic.restype = C.c_int64
+    L.oracle_spgemm_symbolic_omp.argtypes = L.oracle_spgemm_symbolic.argtypes
+    L.oracle_spgemm_symbolic_omp.restype = C.c_int64
     L.oracle_spgemm_numeric.argtypes = [C.c_int64, C.c_int64, C.c_int64, i64p, i64p, f64p, i64p, i64p, f64p,
                                         vp, vp, i64p, f64p]
     L.oracle_spgemm_numeric.restype = C.c_int64
@@ -77,6 +79,13 @@ def lib():
     L.oracle_eltwise_mult_csr.restype = C.c_int64
     L.oracle_tricount_masked.argtypes = [C.c_int64, C.c_int64, i64p, i64p, f64p]
     L.oracle_tricount_masked.restype = C.c_double
+    L.oracle_sort_idx.argtypes = [i64p, C.c_int64]
+    L.oracle_sort_idx.restype = None
+    L.oracle_tricount_masked_omp.argtypes = [C.c_int64, C.c_int64, i64p, i64p, f64p]
+    L.oracle_tricount_masked_omp.restype = C.c_double
+    L.oracle_spgemm_numeric_omp.argtypes = [C.c_int64, C.c_int64, C.c_int64, i64p, i64p, f64p, i64p, i64p, f64p,
+                                            vp, vp, i64p, i64p, f64p]
+    L.oracle_spgemm_numeric_omp.restype = C.c_int64
     L.oracle_coo_to_csr.argtypes = [C.c_int64, C.c_int64, i64p, i64p, f64p, C.c_int, vp, vp, vp]
     L.oracle_coo_to_csr.restype = C.c_int64
     L.oracle_read_mtx_csr.argtypes = [C.c_char_p, C.c_int, i64p, vp, vp, vp]
@@ -171,7 +180,7 @@ def eltwise_dense(a, b, op="times"):
     return out
 
 
-def spgemm_symbolic(Apos, Acrd, Bpos, Bcrd, ncolsB, mask=None, rows=None):
+def spgemm_symbolic(Apos, Acrd, Bpos, Bcrd, ncolsB, mask=None, rows=None, threads=False):
     """Per-row output counts for rows [r0,r1) (default: all rows)."""
     Apos, Acrd, Bpos, Bcrd = _i64(Apos), _i64(Acrd), _i64(Bpos), _i64(Bcrd)
     r0, r1 = (0, len(Apos) - 1) if rows is None else rows
@@ -179,7 +188,8 @@ def spgemm_symbolic(Apos, Acrd, Bpos, Bcrd, ncolsB, mask=None, rows=None):
     if mask is not None:
         mpos, mcrd = _i64(mask[0]), _i64(mask[1])
     cnt = np.zeros(max(r1 - r0, 1), dtype=np.int64)
-    total = lib().oracle_spgemm_symbolic(r0, r1, ncolsB, Apos, Acrd, Bpos, Bcrd, _ptr(mpos), _ptr(mcrd), cnt)
+    fn = lib().oracle_spgemm_symbolic_omp if threads else lib().oracle_spgemm_symbolic
+    total = fn(r0, r1, ncolsB, Apos, Acrd, Bpos, Bcrd, _ptr(mpos), _ptr(mcrd), cnt)
     return cnt[: r1 - r0], int(total)
 
 
@@ -187,13 +197,14 @@ REDUCE_OPS = {"plus": 0, "min": 1, "max": 2, "any": 3}
 MULT_OPS = {"times": 0, "first": 1, "second": 2, "pair": 3, "plus": 4, "minus": 5, "min": 6, "max": 7, "div": 8}
 
 
-def spgemm(Apos, Acrd, Aval, Bpos, Bcrd, Bval, ncolsB, mask=None, rows=None, semiring=None):
+def spgemm(Apos, Acrd, Aval, Bpos, Bcrd, Bval, ncolsB, mask=None, rows=None, semiring=None, threads=False):
     """Symbolic + numeric; returns (pos, crd, val) for rows [r0,r1) with pos starting at 0.
-    semiring = (reduce, mult) names from REDUCE_OPS / MULT_OPS; None is the plain plus-times routine."""
+    semiring = (reduce, mult) names from REDUCE_OPS / MULT_OPS; None is the plain plus-times routine.
+    threads=True: the numeric phase row-parallel over the host's cores (plus-times only; same output)."""
     Apos, Acrd, Aval = _i64(Apos), _i64(Acrd), _f64(Aval)
     Bpos, Bcrd, Bval = _i64(Bpos), _i64(Bcrd), _f64(Bval)
     r0, r1 = (0, len(Apos) - 1) if rows is None else rows
-    cnt, total = spgemm_symbolic(Apos, Acrd, Bpos, Bcrd, ncolsB, mask, (r0, r1))
+    cnt, total = spgemm_symbolic(Apos, Acrd, Bpos, Bcrd, ncolsB, mask, (r0, r1), threads and semiring is None)
     pos = np.zeros(r1 - r0 + 1, dtype=np.int64)
     np.cumsum(cnt, out=pos[1:])
     crd = np.zeros(max(total, 1), dtype=np.int64)
@@ -201,7 +212,10 @@ def spgemm(Apos, Acrd, Aval, Bpos, Bcrd, Bval, ncolsB, mask=None, rows=None, sem
     mpos = mcrd = None
     if mask is not None:
         mpos, mcrd = _i64(mask[0]), _i64(mask[1])
-    if semiring is None:
+    if semiring is None and threads:
+        wrote = lib().oracle_spgemm_numeric_omp(r0, r1, ncolsB, Apos, Acrd, Aval, Bpos, Bcrd, Bval,
+                                                _ptr(mpos), _ptr(mcrd), pos, crd, val)
+    elif semiring is None:
         wrote = lib().oracle_spgemm_numeric(r0, r1, ncolsB, Apos, Acrd, Aval, Bpos, Bcrd, Bval,
                                             _ptr(mpos), _ptr(mcrd), crd, val)
     else:
@@ -229,10 +243,11 @@ def eltwise_mult(Apos, Acrd, Aval, Bpos, Bcrd, Bval):
     return Cpos, Ccrd[:nnz], Cval[:nnz]
 
 
-def tricount_masked(pos, crd, val, ncols=None):
+def tricount_masked(pos, crd, val, ncols=None, threads=False):
     pos, crd, val = _i64(pos), _i64(crd), _f64(val)
     n = len(pos) - 1
-    return float(lib().oracle_tricount_masked(n, n if ncols is None else ncols, pos, crd, val))
+    fn = lib().oracle_tricount_masked_omp if threads else lib().oracle_tricount_masked
+    return float(fn(n, n if ncols is None else ncols, pos, crd, val))
 
 
 def coo_layout(pos, crd, val):

@@ -17,8 +17,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def _declared_symbols():
     text = open(os.path.join(ROOT, "include", "comet_hip_rt.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    names = re.findall(r"\b((?:comet_hip_|_mlir_ciface_comet_hip_|Hip|comet_print_memref_|comet_sort)[A-Za-z0-9_]+|"
-                       r"getTime|printElapsedTime)\s*\(", text)
+    names = re.findall(r"\b((?:comet_hip_|_mlir_ciface_comet_hip_|_mlir_ciface_linalg_|read_input_|Hip|"
+                       r"comet_print_memref_|comet_sort)[A-Za-z0-9_]+|getTime|printElapsedTime)\s*\(", text)
     return sorted(set(names))
 
 
@@ -156,3 +156,14 @@ def test_corrupt_size_lines_and_plans_are_refused_without_a_gpu(tmp_path):
         f.write("%%MatrixMarket matrix coordinate real general\n3 3 4000000000000\n1 1 1.0\n")
     assert L.comet_hip_mtx_read_csr(path.encode(), 1) == 0
     assert b"declares" in L.comet_hip_last_error() or b"HIP device" in L.comet_hip_last_error()
+
+
+def test_lds_fp64_regions_start_on_eight_bytes():
+    """The masked-product kernel puts per-wavefront fp64 sums behind a table whose size depends on the column
+    count; an odd number of 32-bit words in front of them would misalign its 64-bit LDS atomics.  Every size the
+    host can ask for (2^20 columns = 32768 words at most) must give an even offset."""
+    L = rt.lib()
+    for words in list(range(1, 4097)) + list(range(4097, 32769, 7)) + [32768]:
+        off = L.comet_hip_debug_dot_table_words(words)
+        assert off > 0 and off % 2 == 0, (words, off)
+

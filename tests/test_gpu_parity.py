@@ -1031,6 +1031,64 @@ def test_mlir_ciface_entry_points(golden, golden_dir, idt):
     assert cp.tolist() == gm["pos"] and cc.tolist() == gm["crd"] and orc.format_f64(cv) == gm["printed_val"]
     (tr, tc), tpos, tcrd, tval = _mtx(golden_dir, "tc.mtx", 2)
     assert fn("tricount")(tc, rt.memref1d(tpos.astype(idt)), rt.memref1d(tcrd.astype(idt)), rt.memref1d(tval)) == 5.0
+    # two of the reference's semiring goldens through the semiring pair of calls
+    gs = golden["spgemm_csr_semiring"]
+    for name in ("min_plus", "any_pair"):
+        case = gs["cases"][name]
+        r, m = rt.REDUCE_OPS[case["reduce"]], rt.MULT_OPS[case["mult"]]
+        fn("spgemm_csr_sizes_semiring")(nr, nc, rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val),
+                                        rt.memref1d(pos), rt.memref1d(crd), rt.memref1d(val),
+                                        rt.memref1d(empty), rt.memref1d(empty), rt.memref1d(sizes), r, m)
+        assert sizes[0] == len(gs["crd"])
+        cp, cc, cv = np.zeros(nr + 1, dtype=idt), np.zeros(int(sizes[0]), dtype=idt), np.zeros(int(sizes[0]))
+        fn("spgemm_csr_fill_semiring")(rt.memref1d(cp), rt.memref1d(cc), rt.memref1d(cv))
+        assert cp.tolist() == gs["pos"] and cc.tolist() == gs["crd"] and orc.format_f64(cv) == case["printed_val"]
+
+
+def test_mlir_ciface_dense_contraction(golden):
+    """The contraction on host memrefs in one call: the reference's four constant-fill results, a random rank-4
+    case against the checker (overwriting and accumulating), and the reference's matmul entry point by name."""
+    L = rt.lib()
+
+    def contract(a, b, c, A, B, Cm, beta):
+        ids, al, bl, cl = rt.label_ids(a, b, c)
+        labs = [np.array(x, dtype=np.int64) + 10 for x in (al, bl, cl)]       # any integers will do as labels
+        (ma, pa), (mb, pb), (mc, pc) = rt.memref_nd(A), rt.memref_nd(B), rt.memref_nd(Cm)
+        L._mlir_ciface_comet_hip_ttgt_contract_f64(A.ndim, pa, B.ndim, pb, Cm.ndim, pc, rt.memref1d(labs[0]),
+                                                   rt.memref1d(labs[1]), rt.memref1d(labs[2]), beta)
+
+    for g in golden["ttgt"]:
+        A = np.full([g["extent"][ch] for ch in g["A"]], g["A_fill"])
+        B = np.full([g["extent"][ch] for ch in g["B"]], g["B_fill"])
+        Cm = np.full([g["extent"][ch] for ch in g["C"]], 99.0)        # beta = 0 overwrites
+        contract(g["A"], g["B"], g["C"], A, B, Cm, 0.0)
+        assert orc.format_f64(Cm) == g["printed"], g["source"]
+    sizes = {"a": 5, "b": 3, "c": 4, "d": 6, "e": 7, "f": 2}
+    a, b, c = "aebf", "dfce", "abcd"
+    A = gen.dense([sizes[ch] for ch in a], seed=61)
+    B = gen.dense([sizes[ch] for ch in b], seed=62)
+    C0 = gen.dense([sizes[ch] for ch in c], seed=63)
+    bound = np.einsum("aebf,dfce->abcd", np.abs(A), np.abs(B))
+    want0, _, _ = orc.ttgt_contract(a, b, c, A, B)
+    got0 = np.zeros_like(C0)
+    contract(a, b, c, A, B, got0, 0.0)
+    assert np.all(np.abs(got0 - want0) <= RTOL * bound)
+    want1, _, _ = orc.ttgt_contract(a, b, c, A, B, C0=C0, beta=1.0)
+    got1 = C0.copy()
+    contract(a, b, c, A, B, got1, 1.0)
+    assert np.all(np.abs(got1 - want1) <= RTOL * (bound + np.abs(C0)))
+    # _mlir_ciface_linalg_matmul_viewsxs_viewsxs_viewsxs: strided views, alpha and beta as given
+    Am, Bm = gen.dense((37, 29), seed=64), gen.dense((29, 41), seed=65)
+    big = gen.dense((37, 50), seed=66)
+    Cv = big[:, 3:44]                        # a view with row stride 50
+    want = 1.5 * (Am @ Bm) + 0.5 * Cv
+    mc = rt.memref2d(Cv)
+    mc.aligned = mc.allocated = big.ctypes.data
+    mc.offset = 3
+    mc.strides[0], mc.strides[1] = 50, 1
+    L._mlir_ciface_linalg_matmul_viewsxs_viewsxs_viewsxs(rt.memref2d(Am), rt.memref2d(Bm), mc, 6, 8, 1.5, 0.5)
+    assert np.all(np.abs(Cv - want) <= RTOL * (1.5 * (np.abs(Am) @ np.abs(Bm)) + np.abs(want)))
+    assert np.array_equal(big[:, :3], gen.dense((37, 50), seed=66)[:, :3])      # nothing outside the view is touched
 
 
 # ----------------------------------------------------------------- input side and other layouts
@@ -1064,14 +1122,16 @@ def test_reader_file_id_protocol(golden, golden_dir, monkeypatch, layout, idt):
     """The two reader calls with the reference's argument lists, for the three layouts its matrix tests use and
     both index widths (read_input_2D_f64_i64 / _i32, lib/ExecutionEngine/SparseUtils.cpp:2403-2447)."""
     L = rt.lib()
-    read = L.comet_hip_read_input_2D_f64_i64 if idt == np.int64 else L.comet_hip_read_input_2D_f64_i32
+    # the i64 case goes through the names lowered code calls (read_input_*), the i32 case through the prefixed ones
+    read = L.read_input_2D_f64_i64 if idt == np.int64 else L.comet_hip_read_input_2D_f64_i32
+    read_sizes = L.read_input_sizes_2D_f64 if idt == np.int64 else L.comet_hip_read_input_sizes_2D_f64
     monkeypatch.setenv("SPARSE_FILE_NAME3", os.path.join(golden_dir, "test_rank2.mtx"))
     fmt = {"CSR": (0, 0, 1, 0), "COO": (2, 0, 3, 0), "DCSR": (1, 0, 1, 0)}[layout]
     for mode in (1, 3):
         (nr, nc), pos, crd, val = _mtx(golden_dir, "test_rank2.mtx", mode)
         sizes = np.zeros(13, dtype=np.int64)
         sizes_m, sizes_p = _desc(sizes)
-        L.comet_hip_read_input_sizes_2D_f64(3, *fmt, 1, sizes_p, mode)
+        read_sizes(3, *fmt, 1, sizes_p, mode)
         want = {"CSR": (None, pos[:0], pos, crd, val), "COO": orc.coo_layout(pos, crd, val),
                 "DCSR": orc.dcsr_layout(pos, crd, val)}[layout]
         if layout == "CSR":
@@ -1461,8 +1521,17 @@ def test_wrapped_device_arrays_are_checked():
     worse = np.array([0, 3, 1, 7, 2], dtype=np.int32)
     assert L.comet_hip_memcpy(dcrd.ptr, worse.ctypes.data, worse.nbytes, 0) == 0
     assert L.comet_hip_csr_invalidate(h) == 1           # COMET_HIP_ERR_ARG
+    # the handle now refuses every product (nothing is launched on the arrays the check turned down) ...
+    dx, dy = rt.DeviceArray.from_numpy(np.ones(4)), rt.DeviceArray(3)
+    assert L.comet_hip_spmv_csr_f64(h, dx.ptr, dy.ptr, 0) == 3          # COMET_HIP_ERR_HANDLE
+    assert b"failed the check" in L.comet_hip_last_error()
+    assert L.comet_hip_spmm_csr_f64(h, 1, dx.ptr, 1, dy.ptr, 1, 0) == 3
+    assert L.comet_hip_spgemm_csr(h, h, 0) == 0 and b"failed the check" in L.comet_hip_last_error()
+    # ... until the arrays are put right and looked at again
     assert L.comet_hip_memcpy(dcrd.ptr, good[1].ctypes.data, good[1].nbytes, 0) == 0
     assert L.comet_hip_csr_invalidate(h) == 0
+    assert L.comet_hip_spmv_csr_f64(h, dx.ptr, dy.ptr, 0) == 0
+    assert np.array_equal(dy.to_numpy(), np.array([2.0, 0.0, 3.0]))
     assert L.comet_hip_csr_destroy(h) == 0
 
 

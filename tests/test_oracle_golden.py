@@ -543,3 +543,46 @@ def test_sddmm_golden_and_brute_force(golden, golden_dir):
     assert np.allclose(got, A.data * (Cm @ D)[rows, A.indices], rtol=1e-13, atol=1e-15)
     # a dropped term, a transposed operand or B's value left out would all show here
     assert np.array_equal(orc.sddmm(A.indptr, A.indices, A.data, Cm[:, :0], D[:0, :]), A.data * 0.0)
+
+
+def test_checker_sort_is_a_sort():
+    """The checker sorts a row's touched columns with its own introsort (what std::sort is, inlined on the element
+    type); against numpy on the inputs that break a careless quicksort, including ones long enough for the
+    depth limit to send it to heapsort."""
+    rng = np.random.default_rng(7)
+    cases = [np.zeros(0, dtype=np.int64), np.array([5], dtype=np.int64)]
+    for n in (2, 3, 15, 16, 17, 31, 33, 100, 1000, 4097, 70_000):
+        base = rng.permutation(n * 3)[:n].astype(np.int64)          # distinct, as a row's columns are
+        organ = np.concatenate([np.arange(0, n, 2), np.arange(n - 1 - (n % 2 == 0), 0, -2)]).astype(np.int64)
+        cases += [base, np.sort(base), np.sort(base)[::-1].copy(), organ,
+                  np.concatenate([np.sort(base[: n // 2]), np.sort(base[n // 2:])]),
+                  rng.integers(0, 4, n).astype(np.int64)]                # heavy duplicates (never produced by a row, still sorted)
+    # a median-of-three killer for the (first+1, middle, last) sample
+    n = 4096
+    killer = np.arange(n, dtype=np.int64)
+    killer[1::2] = np.arange(n // 2, n)
+    killer[0::2] = np.arange(0, n // 2)
+    cases.append(killer)
+    for a in cases:
+        got = a.copy()
+        orc.lib().oracle_sort_idx(got, len(got))
+        assert np.array_equal(got, np.sort(a)), len(a)
+
+
+def test_row_parallel_checker_equals_sequential():
+    from comet_amd import gen
+    """The OpenMP forms (the stronger CPU baseline of the benchmark) produce what the sequential forms produce."""
+    n = 3000
+    pos, crd, val = gen.zipf_csr(n=n, mean=12.0, cap=1500, seed=41)
+    val = np.abs(val) + 0.1
+    for mask in (None, (pos, crd)):
+        p0, c0, v0 = orc.spgemm(pos, crd, val, pos, crd, val, n, mask=mask)
+        p1, c1, v1 = orc.spgemm(pos, crd, val, pos, crd, val, n, mask=mask, threads=True)
+        assert np.array_equal(p0, p1) and np.array_equal(c0, c1) and np.array_equal(v0, v1)
+        p2, c2, v2 = orc.spgemm(pos, crd, val, pos, crd, val, n, mask=mask, rows=(100, 900), threads=True)
+        assert np.array_equal(c2, c0[p0[100]:p0[900]]) and np.array_equal(v2, v0[p0[100]:p0[900]])
+    apos, acrd, aval = gen.rmat_symmetric_csr(scale=11, edge_factor=8, seed=5, values="ones")
+    lpos, lcrd, _ = gen.strictly_lower(apos, acrd, aval)
+    ones = np.ones(len(lcrd))
+    assert orc.tricount_masked(lpos, lcrd, ones, threads=True) == orc.tricount_masked(lpos, lcrd, ones)
+

@@ -20,7 +20,14 @@ def _device():
     rt.sync()
 
 
-def _product(n, mean, K, seed, accumulate, ld_pad=0):
+def _free_bytes():
+    import ctypes
+    free, total = ctypes.c_int64(0), ctypes.c_int64(0)
+    assert rt.lib().comet_hip_mem_info(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
+def _product(n, mean, K, seed, accumulate, ld_pad=0, stream=0):
     pos, crd, val = gen.zipf_csr(n=n, mean=mean, cap=512, seed=seed)
     B = gen.dense((n, K + ld_pad), seed=seed + 1)
     C0 = gen.dense((n, K + ld_pad), seed=seed + 2)
@@ -30,7 +37,16 @@ def _product(n, mean, K, seed, accumulate, ld_pad=0):
     out = []
     for name in ("comet_hip_spmm_csr_f64", "comet_hip_spmm_csr_f64_noalloc"):
         dC = rt.DeviceArray.from_numpy(C0)
-        rc = getattr(rt.lib(), name)(A.handle, K, dB.ptr, ld, dC.ptr, ld, int(accumulate))
+        if name.endswith("noalloc"):
+            rt.sync()
+            before = _free_bytes()
+            rc = rt.lib().comet_hip_spmm_csr_f64_noalloc(A.handle, K, dB.ptr, ld, dC.ptr, ld, int(accumulate), stream)
+            if stream:
+                assert rt.lib().comet_hip_stream_sync(stream) == 0
+            rt.sync()
+            assert _free_bytes() == before, "the allocation-free entry point changed the free device memory"
+        else:
+            rc = rt.lib().comet_hip_spmm_csr_f64(A.handle, K, dB.ptr, ld, dC.ptr, ld, int(accumulate))
         assert rc == 0, rt.lib().comet_hip_last_error().decode()
         out.append(dC.to_numpy())
     # the ordinary entry point against the checker (tolerance of rows cut by a chunk boundary)
@@ -55,13 +71,24 @@ def test_noalloc_spmm_matches_ordinary_entry_point_twice_in_a_row():
     assert np.array_equal(ref3, got3) and np.array_equal(got3, got1)
 
 
+def test_noalloc_spmm_runs_on_the_callers_stream():
+    # a stream of the caller's own: the kernels go there (and the result is there once that stream is through)
+    s = rt.lib().comet_hip_stream_create()
+    assert s != 0
+    try:
+        (ref, got), _ = _product(6_000, 8.0, 64, seed=21, accumulate=False, stream=s)
+        assert np.array_equal(ref, got)
+    finally:
+        assert rt.lib().comet_hip_stream_destroy(s) == 0
+
+
 def test_noalloc_spmm_refuses_what_the_scratch_cannot_hold():
     n = 4096
     pos = np.arange(n + 1, dtype=np.int64)
     crd = np.zeros(n, dtype=np.int64)
     A = rt.CsrMatrix.from_arrays((n, 1), pos, crd, np.ones(n))
     K = 64 * 600                        # 600 tiles x 16 chunks = 9,600 slots > 8,192
-    rc = rt.lib().comet_hip_spmm_csr_f64_noalloc(A.handle, K, 8, K, 8, K, 0)     # pointers are never touched
+    rc = rt.lib().comet_hip_spmm_csr_f64_noalloc(A.handle, K, 8, K, 8, K, 0, 0)     # pointers are never touched
     assert rc == 4                      # COMET_HIP_ERR_SIZE
     assert "static scratch" in rt.lib().comet_hip_last_error().decode()
 
@@ -72,5 +99,5 @@ def test_noalloc_spmm_empty_matrix_clears_or_keeps_c():
     B = rt.DeviceArray.from_numpy(gen.dense((7, 4), seed=4))
     for acc in (0, 1):
         dC = rt.DeviceArray.from_numpy(C0)
-        assert rt.lib().comet_hip_spmm_csr_f64_noalloc(A.handle, 4, B.ptr, 4, dC.ptr, 4, acc) == 0
+        assert rt.lib().comet_hip_spmm_csr_f64_noalloc(A.handle, 4, B.ptr, 4, dC.ptr, 4, acc, 0) == 0
         assert np.array_equal(dC.to_numpy(), C0 if acc else np.zeros_like(C0))
