@@ -61,7 +61,23 @@ struct HeavyEnt {
     double val;
 };
 
+// A list of the rows of a product that have work, by descending number of products (what the SpGEMM kernels draw
+// their tickets over), kept in the left operand's handle: it depends only on the two structures, the row range and
+// the thresholds, so the seven lists a product of the benchmark takes are built once, not once per product.
+struct RowListEntry {
+    uint64_t b_uid = 0, mask_uid = 0, filter_uid = 0;
+    int64_t rb = 0, re = 0, dense_threshold = 0, wide_threshold = 0, mask_fill = 0, xlo = 0, xhi = 0;
+    int strict = 0;
+    int32_t *rows = nullptr;     // device, re - rb entries
+    int64_t *bounds = nullptr;   // device, 3 entries
+};
+uint64_t next_csr_uid();
+
 struct Csr {
+    // names this state of the matrix: new for every matrix and again whenever its arrays may have changed
+    // (comet_hip_csr_invalidate), so that what other handles keep about it can tell that it is stale
+    uint64_t uid = next_csr_uid();
+    std::vector<RowListEntry> row_lists;
     int64_t nrows = 0, ncols = 0, nnz = 0;
     int64_t *pos = nullptr;
     int32_t *crd = nullptr;

@@ -8,6 +8,7 @@
 #include <string.h>
 
 #include <map>
+#include <atomic>
 #include <mutex>
 #include <unordered_set>
 
@@ -169,8 +170,20 @@ bool plan_at_once()
     return getenv("COMET_HIP_PLAN_AT_ONCE") != nullptr;
 }
 
+uint64_t next_csr_uid()
+{
+    static std::atomic<uint64_t> next{1};
+    return next.fetch_add(1);
+}
+
 static void csr_drop_plans(Csr *c)
 {
+    c->uid = next_csr_uid();
+    for (auto &e : c->row_lists) {
+        (void)hipFree(e.rows);
+        (void)hipFree(e.bounds);
+    }
+    c->row_lists.clear();
     if (c->light)
         csr_release(c->light);
     if (c->transposed)

@@ -2861,15 +2861,43 @@ static SgRowLists g_rl;
 
 // Products per row of rows [rb, re) of A*B and the list of those rows by descending products.
 struct SgPairFilter {          // see spgemm_row_products
-    const int64_t *tpos = nullptr;
+    const Csr *towner = nullptr;        // tpos = towner->pos
     int strict = 0;
     int64_t xlo = 0, xhi = 0;
 };
+// The list depends on the two structures, the range and the thresholds only: it is kept in A's handle and found
+// again by the uids of the matrices it was made from (a matrix gets a new uid when it is invalidated), so a
+// product that is taken again, or taken in row blocks, sorts nothing.  COMET_HIP_SPGEMM_NO_LIST_CACHE turns the
+// keeping off (the tests compare both).
+constexpr size_t SG_ROW_LISTS_KEPT = 24;
 static int sg_row_list(const Csr *a, const Csr *b, int64_t rb, int64_t re, int64_t dense_threshold,
-                       int64_t wide_threshold, RowList *out, const int64_t *long_mask_pos = nullptr,
+                       int64_t wide_threshold, RowList *out, const Csr *long_mask = nullptr,
                        int64_t mask_fill = 0, SgPairFilter filter = SgPairFilter())
 {
     const int64_t n = re - rb;
+    static const bool keep = getenv("COMET_HIP_SPGEMM_NO_LIST_CACHE") == nullptr;
+    Csr *owner = const_cast<Csr *>(a);
+    RowListEntry key;
+    key.b_uid = b->uid;
+    key.mask_uid = long_mask ? long_mask->uid : 0;
+    key.filter_uid = filter.towner ? filter.towner->uid : 0;
+    key.rb = rb;
+    key.re = re;
+    key.dense_threshold = dense_threshold;
+    key.wide_threshold = wide_threshold;
+    key.mask_fill = mask_fill;
+    key.xlo = filter.xlo;
+    key.xhi = filter.xhi;
+    key.strict = filter.strict;
+    if (keep)
+        for (const RowListEntry &e : owner->row_lists)
+            if (e.b_uid == key.b_uid && e.mask_uid == key.mask_uid && e.filter_uid == key.filter_uid && e.rb == rb &&
+                e.re == re && e.dense_threshold == dense_threshold && e.wide_threshold == wide_threshold &&
+                e.mask_fill == mask_fill && e.xlo == key.xlo && e.xhi == key.xhi && e.strict == key.strict) {
+                out->rows = e.rows;
+                out->bounds = e.bounds;
+                return COMET_HIP_OK;
+            }
     COMET_CHK(g_rl.rowprod.ensure(sizeof(int64_t) * (size_t)n, false));
     COMET_CHK(g_rl.keys_in.ensure(8 * (size_t)n, false));
     COMET_CHK(g_rl.keys_out.ensure(8 * (size_t)n, false));
@@ -2880,9 +2908,10 @@ static int sg_row_list(const Csr *a, const Csr *b, int64_t rb, int64_t re, int64
     {
         KernelTimer t("spgemm_row_products");
         spgemm_row_products<<<dim3((unsigned)ceil_div(n, 4)), dim3(256), 0, stream()>>>(
-            rb, re, a->pos, a->crd, b->pos, rowprod, filter.tpos, filter.strict, filter.xlo, filter.xhi);
+            rb, re, a->pos, a->crd, b->pos, rowprod, filter.towner ? filter.towner->pos : nullptr, filter.strict,
+            filter.xlo, filter.xhi);
         sg_row_keys<<<dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, stream()>>>(
-            n, rowprod, long_mask_pos ? long_mask_pos + rb : nullptr, mask_fill, (uint64_t *)g_rl.keys_in.ptr,
+            n, rowprod, long_mask ? long_mask->pos + rb : nullptr, mask_fill, (uint64_t *)g_rl.keys_in.ptr,
             (uint32_t *)g_rl.idx_in.ptr);
     }
     COMET_HIPCHK(hipGetLastError());
@@ -2893,6 +2922,26 @@ static int sg_row_list(const Csr *a, const Csr *b, int64_t rb, int64_t re, int64
     COMET_HIPCHK(hipGetLastError());
     out->rows = (const int32_t *)g_rl.idx_out.ptr;
     out->bounds = (const int64_t *)g_rl.bounds.ptr;
+    if (keep && n > 0) {
+        // a copy of its own; failing to get the memory only means that the list is built again next time
+        if (owner->row_lists.size() >= SG_ROW_LISTS_KEPT) {
+            COMET_HIPCHK(hipStreamSynchronize(stream()));        // a kernel may still be reading the oldest one
+            (void)hipFree(owner->row_lists.front().rows);
+            (void)hipFree(owner->row_lists.front().bounds);
+            owner->row_lists.erase(owner->row_lists.begin());
+        }
+        if (hipMalloc((void **)&key.rows, 4 * (size_t)n) != hipSuccess ||
+            hipMalloc((void **)&key.bounds, 24) != hipSuccess) {
+            (void)hipGetLastError();
+            (void)hipFree(key.rows);
+            return COMET_HIP_OK;
+        }
+        COMET_HIPCHK(hipMemcpyAsync(key.rows, g_rl.idx_out.ptr, 4 * (size_t)n, hipMemcpyDeviceToDevice, stream()));
+        COMET_HIPCHK(hipMemcpyAsync(key.bounds, g_rl.bounds.ptr, 24, hipMemcpyDeviceToDevice, stream()));
+        owner->row_lists.push_back(key);
+        out->rows = key.rows;
+        out->bounds = key.bounds;
+    }
     return COMET_HIP_OK;
 }
 
@@ -3110,7 +3159,7 @@ static int dot_pairs(const Csr *a, const Csr *b, const Csr *m, int64_t rb, int64
         const int64_t first = half == 0 ? rb : 0, last = half == 0 ? re : mt->nrows;
         RowList list;        // the rows that have pairs of this half, by the entries these stream
         SgPairFilter mine;
-        mine.tpos = T->pos;
+        mine.towner = T;
         mine.strict = half;
         mine.xlo = half == 0 ? 0 : rb;
         mine.xhi = half == 0 ? everywhere : re;
@@ -3175,7 +3224,7 @@ static int numeric_rows(const Csr *a, Csr *b, const Csr *m, const int64_t *Cpos,
     RowList list;
     const int64_t wide = sg_wide_threshold(nblk) > dense_threshold ? sg_wide_threshold(nblk) : dense_threshold;
     if (mdense)         // those rows sort in front (sg_row_keys): bounds[0] = bounds[2] = their number
-        COMET_CHK(sg_row_list(a, b, rb, re, 1ll << 61, 1ll << 61, &list, m->pos, SG_HASH_FILL));
+        COMET_CHK(sg_row_list(a, b, rb, re, 1ll << 61, 1ll << 61, &list, m, SG_HASH_FILL));
     else
         COMET_CHK(sg_row_list(a, b, rb, re, dense_threshold, dense ? wide : SG_NO_DENSE, &list));
     uint32_t *gbm = nullptr, *gmask = nullptr;
