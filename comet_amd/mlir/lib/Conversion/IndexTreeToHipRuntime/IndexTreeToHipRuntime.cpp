@@ -22,9 +22,16 @@
 //   C[a,c] = A[a,b] * B[b,c]   all CSR        a, b, c   comet_hip_spgemm_csr_sizes_f64 + comet_hip_spgemm_csr_fill_f64
 //            (+ optional mask operand of the compute op: its pos/crd are passed, else two empty memrefs)
 //
-// Only the plus-times semiring ("plusxy_times") is taken here; the other semirings of the runtime
-// (comet_hip_spgemm_csr_semiring) are reached through the device-handle API, which needs the host rewriting of
-// lib/Conversion/PrepareGpuHost and is left out of this pass.
+//   C[a,c] = A[a,b] @(r,m) B[b,c] all CSR     a, b, c   comet_hip_spgemm_csr_sizes_semiring_f64 + ..._fill_semiring_f64
+//            (the compute op's semiring attribute "<reduce>_<mult>", frontends/comet_dsl/mlir/MLIRGen.cpp:101-147,
+//             turned into the runtime's operator codes; SpMV and SpMM are taken for plus-times only)
+//
+// A second pass in this file, createLowerDenseContractionToHipRuntimePass(), takes ta.mul on dense tensors of
+// rank <= 8 - what --convert-tc-to-ttgt rewrites into transpose/collapse/matmul/expand/transpose
+// (lib/Dialect/TensorAlgebra/Transforms/TCtoTTGTDyn.cpp:153-723) - and emits one call to
+// comet_hip_ttgt_contract_f64 with the three tensors as unranked memrefs and their index labels (the positions of
+// the affine maps' results) as constant index memrefs.  It runs where createLoweringTTGTPass() would
+// (frontends/comet_dsl/comet.cpp:447-470), under the same GpuRuntime == "hip-rt" switch.
 //
 // The callee declarations follow declare_vendor_funcs (lib/Conversion/GpuUtils/GpuUtils.cpp:307-411): private
 // func.func added to the module, here with llvm.emit_c_interface so that the symbol resolved at link time is
@@ -37,11 +44,14 @@
 #include "comet/Dialect/TensorAlgebra/IR/TADialect.h"
 #include "comet/Dialect/Utils/Utils.h"
 
+#include "llvm/ADT/StringSwitch.h"
 #include "mlir/Dialect/Arith/IR/Arith.h"
 #include "mlir/Dialect/Bufferization/IR/Bufferization.h"
 #include "mlir/Dialect/Func/IR/FuncOps.h"
 #include "mlir/Dialect/MemRef/IR/MemRef.h"
 #include "mlir/Dialect/Tensor/IR/Tensor.h"
+#include "mlir/IR/AffineExpr.h"
+#include "mlir/IR/AffineMap.h"
 #include "mlir/IR/BuiltinOps.h"
 #include "mlir/IR/PatternMatch.h"
 #include "mlir/Pass/Pass.h"
@@ -66,7 +76,29 @@ namespace
     Shape shape = Shape::None;
     IndexTreeComputeOp compute;
     Value lhs, a, b, mask;
+    int reduceOp = 0, multOp = 0; /// COMET_SR_* / COMET_OP_* of include/comet_hip_rt.h
   };
+
+  /// "<reduce>_<mult>" with the DSL's operator names -> the runtime's codes; false if either is unknown to it
+  /// (lor, land, noop: those trees stay with the loop lowering).
+  bool semiringCodes(StringRef semiring, int &reduceOp, int &multOp)
+  {
+    auto parts = semiring.split('_');
+    int r = llvm::StringSwitch<int>(parts.first).Case("plusxy", 0).Case("minxy", 1).Case("any", 3).Default(-1);
+    int m = llvm::StringSwitch<int>(parts.second)
+                .Case("times", 0)
+                .Case("first", 1)
+                .Case("second", 2)
+                .Case("pairxy", 3)
+                .Case("plusxy", 4)
+                .Case("minus", 5)
+                .Default(-1);
+    if (r < 0 || m < 0)
+      return false;
+    reduceOp = r;
+    multOp = m;
+    return true;
+  }
 
   bool isCSR(Type t)
   {
@@ -107,8 +139,9 @@ namespace
     if (computes.size() != 1 || tree->getNumResults() != 1)
       return m; /// fused trees and workspace forms go to the loop lowering
     IndexTreeComputeOp c = computes.front();
-    if (c.getSemiring() != "plusxy_times" || c.getRhs().size() != 2 || c.getComputeMissing())
+    if (!semiringCodes(c.getSemiring(), m.reduceOp, m.multOp) || c.getRhs().size() != 2 || c.getComputeMissing())
       return m;
+    const bool plusTimes = m.reduceOp == 0 && m.multOp == 0;
     auto lhsOp = c.getLhs().getDefiningOp<IndexTreeLHSOperandOp>();
     auto aOp = c.getRhs()[0].getDefiningOp<IndexTreeOperandOp>();
     auto bOp = c.getRhs()[1].getDefiningOp<IndexTreeOperandOp>();
@@ -125,9 +158,9 @@ namespace
     Type tl = m.lhs.getType(), ta = m.a.getType(), tb = m.b.getType();
     if (!isCSR(ta))
       return m;
-    if (nIndices == 2 && isDenseOfRank(tb, 1) && isDenseOfRank(tl, 1) && !m.mask)
+    if (nIndices == 2 && isDenseOfRank(tb, 1) && isDenseOfRank(tl, 1) && !m.mask && plusTimes)
       m.shape = Shape::SpMV;
-    else if (nIndices == 3 && isDenseOfRank(tb, 2) && isDenseOfRank(tl, 2) && !m.mask)
+    else if (nIndices == 3 && isDenseOfRank(tb, 2) && isDenseOfRank(tl, 2) && !m.mask && plusTimes)
       m.shape = Shape::SpMM;
     else if (nIndices == 3 && isCSR(tb) && isCSR(tl) && (!m.mask || isCSR(m.mask.getType())))
       m.shape = Shape::SpGEMM;
@@ -200,8 +233,13 @@ namespace
       for (int k = 0; k < 2; ++k)
         sizesArgs.append({idxMemref(), idxMemref(), f64Memref(1)}); /// A, B
       sizesArgs.append({idxMemref(), idxMemref(), indexMemref});       /// mask pos/crd, sizes
-      declare(name("spgemm_csr_sizes"), sizesArgs, {});
-      declare(name("spgemm_csr_fill"), {idxMemref(), idxMemref(), f64Memref(1)}, {});
+      const bool semi = m.reduceOp != 0 || m.multOp != 0;
+      if (semi)
+        sizesArgs.append({b.getI32Type(), b.getI32Type()}); /// reduce and mult operator codes
+      const std::string sizesFn = name(semi ? "spgemm_csr_sizes_semiring" : "spgemm_csr_sizes");
+      const std::string fillFn = name(semi ? "spgemm_csr_fill_semiring" : "spgemm_csr_fill");
+      declare(sizesFn, sizesArgs, {});
+      declare(fillFn, {idxMemref(), idxMemref(), f64Memref(1)}, {});
 
       b.setInsertionPoint(tree);
       Value zero = b.create<arith::ConstantIndexOp>(loc, 0);
@@ -219,15 +257,20 @@ namespace
         mpos = b.create<memref::AllocOp>(loc, idxMemref(), ValueRange{zero});
         mcrd = b.create<memref::AllocOp>(loc, idxMemref(), ValueRange{zero});
       }
-      b.create<func::CallOp>(loc, name("spgemm_csr_sizes"), TypeRange{},
-                             ValueRange{i64(loc, nrows), i64(loc, ncols), pos(loc, m.a), crd(loc, m.a), vals(loc, m.a),
-                                        pos(loc, m.b), crd(loc, m.b), vals(loc, m.b), mpos, mcrd, sizes});
+      SmallVector<Value> sizesOperands = {i64(loc, nrows), i64(loc, ncols), pos(loc, m.a), crd(loc, m.a), vals(loc, m.a),
+                                          pos(loc, m.b), crd(loc, m.b), vals(loc, m.b), mpos, mcrd, sizes};
+      if (semi)
+      {
+        sizesOperands.push_back(b.create<arith::ConstantIntOp>(loc, m.reduceOp, 32));
+        sizesOperands.push_back(b.create<arith::ConstantIntOp>(loc, m.multOp, 32));
+      }
+      b.create<func::CallOp>(loc, sizesFn, TypeRange{}, sizesOperands);
       Value nnz = b.create<memref::LoadOp>(loc, sizes, ValueRange{zero});
       Value npos = b.create<arith::AddIOp>(loc, nrows, one);
       Value cpos = b.create<memref::AllocOp>(loc, idxMemref(), ValueRange{npos});
       Value ccrd = b.create<memref::AllocOp>(loc, idxMemref(), ValueRange{nnz});
       Value cval = b.create<memref::AllocOp>(loc, f64Memref(1), ValueRange{nnz});
-      b.create<func::CallOp>(loc, name("spgemm_csr_fill"), TypeRange{}, ValueRange{cpos, ccrd, cval});
+      b.create<func::CallOp>(loc, fillFn, TypeRange{}, ValueRange{cpos, ccrd, cval});
 
       /// the remaining arrays of the CSR tuple: A1pos = [nrows], A1crd and the tile arrays = [-1]
       /// (what read_input_2D leaves in them, SparseUtils.cpp:1840-1848, 1898-1936)
@@ -304,9 +347,100 @@ namespace
       }
     }
   };
+
+  /// ta.mul on dense f64 tensors -> one call to comet_hip_ttgt_contract_f64.
+  struct LowerDenseContractionToHipRuntimePass
+      : public PassWrapper<LowerDenseContractionToHipRuntimePass, OperationPass<ModuleOp>>
+  {
+    MLIR_DEFINE_EXPLICIT_INTERNAL_INLINE_TYPE_ID(LowerDenseContractionToHipRuntimePass)
+    StringRef getArgument() const final { return "convert-tc-to-hip-runtime"; }
+    StringRef getDescription() const final
+    {
+      return "Replace dense tensor contractions (ta.mul) by a call to comet_hip_ttgt_contract_f64 of libcomet_hip_rt";
+    }
+    void getDependentDialects(DialectRegistry &registry) const override
+    {
+      registry.insert<func::FuncDialect, memref::MemRefDialect, arith::ArithDialect, bufferization::BufferizationDialect>();
+    }
+
+    void runOnOperation() override
+    {
+      ModuleOp module = getOperation();
+      OpBuilder b(module.getContext());
+      const char *fn = "comet_hip_ttgt_contract_f64";
+      auto unrankedF64 = UnrankedMemRefType::get(b.getF64Type(), 0);
+      auto labels = MemRefType::get({ShapedType::kDynamic}, b.getIndexType());
+      SmallVector<TensorMultOp> mults;
+      module.walk([&](TensorMultOp op) { mults.push_back(op); });
+      for (TensorMultOp op : mults)
+      {
+        /// operands as TCtoTTGTDyn.cpp:161-231 reads them: rhs1, rhs2, and the tensor the result is set into
+        Value a = op->getOperand(0), c2 = op->getOperand(1), dst;
+        TensorSetOp set;
+        for (Operation *u : op->getResult(0).getUsers())
+          if ((set = dyn_cast<TensorSetOp>(u)))
+            dst = set->getOperand(1);
+        auto ta = dyn_cast<RankedTensorType>(a.getType()), tb = dyn_cast<RankedTensorType>(c2.getType());
+        auto tc = dst ? dyn_cast<RankedTensorType>(dst.getType()) : RankedTensorType();
+        if (!ta || !tb || !tc || !ta.getElementType().isF64() || ta.getRank() > 8 || tb.getRank() > 8 || tc.getRank() > 8)
+          continue; /// sparse operands and other element types go the reference's way
+        if (!module.lookupSymbol<func::FuncOp>(fn))
+        {
+          OpBuilder::InsertionGuard g(b);
+          b.clearInsertionPoint();
+          auto f = b.create<func::FuncOp>(
+              b.getUnknownLoc(), fn,
+              b.getFunctionType({unrankedF64, unrankedF64, unrankedF64, labels, labels, labels, b.getF64Type()}, {}));
+          f.setVisibility(SymbolTable::Visibility::Private);
+          f->setAttr("llvm.emit_c_interface", b.getUnitAttr());
+          module.push_back(f);
+        }
+        Location loc = op.getLoc();
+        b.setInsertionPoint(op);
+        auto asUnranked = [&](Value tensor)
+        {
+          auto tt = cast<RankedTensorType>(tensor.getType());
+          Value mem = b.create<bufferization::ToMemrefOp>(loc, MemRefType::get(tt.getShape(), tt.getElementType()), tensor);
+          return b.create<memref::CastOp>(loc, unrankedF64, mem).getResult();
+        };
+        /// the labels of an operand: the dimension positions its indexing map names, as index constants
+        auto labelMemref = [&](AffineMap map)
+        {
+          Value n = b.create<arith::ConstantIndexOp>(loc, map.getNumResults());
+          Value mem = b.create<memref::AllocOp>(loc, labels, ValueRange{n});
+          for (unsigned i = 0; i < map.getNumResults(); ++i)
+          {
+            Value at = b.create<arith::ConstantIndexOp>(loc, i);
+            Value lab = b.create<arith::ConstantIndexOp>(loc, cast<AffineDimExpr>(map.getResult(i)).getPosition());
+            b.create<memref::StoreOp>(loc, lab, mem, ValueRange{at});
+          }
+          return mem;
+        };
+        ArrayAttr maps = op.getIndexingMaps();
+        Value la = labelMemref(cast<AffineMapAttr>(maps[0]).getValue());
+        Value lb = labelMemref(cast<AffineMapAttr>(maps[1]).getValue());
+        Value lc = labelMemref(cast<AffineMapAttr>(maps[2]).getValue());
+        double betaValue = 0.0;
+        if (auto betaAttr = op->getAttrOfType<FloatAttr>("__beta__"))
+          betaValue = betaAttr.getValueAsDouble();
+        Value beta = b.create<arith::ConstantFloatOp>(loc, APFloat(betaValue), b.getF64Type());
+        Value cm = asUnranked(dst);
+        b.create<func::CallOp>(loc, fn, TypeRange{}, ValueRange{asUnranked(a), asUnranked(c2), cm, la, lb, lc, beta});
+        /// the call wrote through dst's buffer: the set op that copied the product into it has nothing left to do
+        op->getResult(0).replaceAllUsesWith(dst);
+        set.erase();
+        op.erase();
+      }
+    }
+  };
 } // namespace
 
 std::unique_ptr<Pass> mlir::comet::createLowerIndexTreeToHipRuntimePass(unsigned indexBitwidth)
 {
   return std::make_unique<LowerIndexTreeToHipRuntimePass>(indexBitwidth);
+}
+
+std::unique_ptr<Pass> mlir::comet::createLowerDenseContractionToHipRuntimePass()
+{
+  return std::make_unique<LowerDenseContractionToHipRuntimePass>();
 }
