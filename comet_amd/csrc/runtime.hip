@@ -334,34 +334,28 @@ __global__ void copy_f64_kernel(double *__restrict__ dst, const double *__restri
 // Every workgroup walks a contiguous slice so that a DRAM page is opened by one workgroup, not by all of them.
 typedef double stream_v2d __attribute__((ext_vector_type(2)));
 
+template <bool NT>
 __global__ __launch_bounds__(256) void stream_copy16_kernel(stream_v2d *__restrict__ dst, const stream_v2d *__restrict__ src,
-                                                            int64_t n2, int nt)
+                                                            int64_t n2)
 {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t step = (int64_t)gridDim.x * blockDim.x;
-    if (nt) {
-        for (; i + 3 * step < n2; i += 4 * step) {      // four loads in flight per lane, then four stores
-            const stream_v2d a = __builtin_nontemporal_load(src + i), b = __builtin_nontemporal_load(src + i + step),
-                             c = __builtin_nontemporal_load(src + i + 2 * step),
-                             d = __builtin_nontemporal_load(src + i + 3 * step);
-            __builtin_nontemporal_store(a, dst + i);
-            __builtin_nontemporal_store(b, dst + i + step);
-            __builtin_nontemporal_store(c, dst + i + 2 * step);
-            __builtin_nontemporal_store(d, dst + i + 3 * step);
-        }
-        for (; i < n2; i += step)
-            __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
-    } else {
-        for (; i + 3 * step < n2; i += 4 * step) {
-            const stream_v2d a = src[i], b = src[i + step], c = src[i + 2 * step], d = src[i + 3 * step];
-            dst[i] = a;
-            dst[i + step] = b;
-            dst[i + 2 * step] = c;
-            dst[i + 3 * step] = d;
-        }
-        for (; i < n2; i += step)
-            dst[i] = src[i];
+    const auto ld = [](const stream_v2d *p) { return NT ? __builtin_nontemporal_load(p) : *p; };
+    const auto st = [](stream_v2d v, stream_v2d *p) {
+        if (NT)
+            __builtin_nontemporal_store(v, p);
+        else
+            *p = v;
+    };
+    for (; i + 3 * step < n2; i += 4 * step) {      // four loads in flight per lane, then four stores
+        const stream_v2d a = ld(src + i), b = ld(src + i + step), c = ld(src + i + 2 * step), d = ld(src + i + 3 * step);
+        st(a, dst + i);
+        st(b, dst + i + step);
+        st(c, dst + i + 2 * step);
+        st(d, dst + i + 3 * step);
     }
+    for (; i < n2; i += step)
+        st(ld(src + i), dst + i);
 }
 
 // read-only: every lane sums what it reads, one store per lane at the end
@@ -1025,10 +1019,14 @@ int comet_hip_stream_bench(int mode, int64_t dst_dptr, int64_t src_dptr, int64_t
         (unsigned)std::min<int64_t>(ceil_div(n2, 256), (int64_t)num_cus() * (workgroups_per_cu ? workgroups_per_cu : 8));
     if (mode == 2)
         COMET_CHK(g_stream_out.ensure(sizeof(double) * 256 * (size_t)blocks, false));
-    if (mode <= 1) {
-        KernelTimer t(mode ? "stream_copy16_nt_kernel" : "stream_copy16_kernel");
-        stream_copy16_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>((stream_v2d *)dst_dptr,
-                                                                        (const stream_v2d *)src_dptr, n2, mode);
+    if (mode == 0) {
+        KernelTimer t("stream_copy16_kernel");
+        stream_copy16_kernel<false><<<dim3(blocks), dim3(256), 0, stream()>>>((stream_v2d *)dst_dptr,
+                                                                               (const stream_v2d *)src_dptr, n2);
+    } else if (mode == 1) {
+        KernelTimer t("stream_copy16_nt_kernel");
+        stream_copy16_kernel<true><<<dim3(blocks), dim3(256), 0, stream()>>>((stream_v2d *)dst_dptr,
+                                                                              (const stream_v2d *)src_dptr, n2);
     } else if (mode == 2) {
         KernelTimer t("stream_read16_kernel");
         stream_read16_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>((const stream_v2d *)src_dptr, n2,
