@@ -130,6 +130,10 @@ struct Csr {
     // products taken pair by pair); dup_state: 0 not looked at, 1 no row holds a column twice, 2 some row does
     Csr *transposed_index = nullptr;
     int dup_state = 0;
+    // whether all stored values are the same number (a pattern matrix, as graph kernels use them): 0 not looked
+    // at, 1 they are (iso_value), 2 they are not
+    int iso_state = 0;
+    double iso_value = 0.0;
     // products taken with this matrix on the left so far (0, 1, more): the SpMM and SpMV plans, which cost tens of
     // products, are built when a matrix is multiplied for the second time (plan_at_once() builds them at the first)
     int spmm_uses = 0, spmv_uses = 0;

@@ -192,6 +192,7 @@ static void csr_drop_plans(Csr *c)
         csr_release(c->transposed_index);
     c->light = c->transposed = c->transposed_index = nullptr;
     c->dup_state = 0;
+    c->iso_state = 0;
     (void)hipFree(c->entry_row);
     c->entry_row = nullptr;
     (void)hipFree(c->rowmap);

@@ -26,6 +26,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include <cstring>
 
 namespace comet {
 
@@ -2239,6 +2240,190 @@ __global__ __launch_bounds__(SM_WAVES * 64) void spgemm_masked_sum_small_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// The same sums when every stored value of B is one number b (a pattern matrix): a product that meets the mask
+// adds a * b whatever its place in the row of B, so a row of B only has to be counted - how many of its columns
+// are in the mask row - and the count times a * b is what it contributes.  No value is fetched, nothing is
+// carried from the look-up to a later visit, and the walk shrinks to a load, an LDS read and a bit test per
+// product.  (Sums of whole numbers, as in a triangle count, are the same in either form; otherwise the two differ
+// by rounding, each within the bound the unmasked forms keep.)
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ int bitmap_bit(const uint32_t *bm, int j)
+{
+    return (int)((bm[(uint32_t)j >> 5] >> ((uint32_t)j & 31u)) & 1u);
+}
+__device__ __forceinline__ int bitmap_bits4(const uint32_t *bm, sg_i4u j)
+{
+    const uint32_t w0 = bm[(uint32_t)j.x >> 5], w1 = bm[(uint32_t)j.y >> 5], w2 = bm[(uint32_t)j.z >> 5],
+                   w3 = bm[(uint32_t)j.w >> 5];
+    return (int)(((w0 >> ((uint32_t)j.x & 31u)) & 1u) + ((w1 >> ((uint32_t)j.y & 31u)) & 1u) +
+                 ((w2 >> ((uint32_t)j.z & 31u)) & 1u) + ((w3 >> ((uint32_t)j.w & 31u)) & 1u));
+}
+// how many of the n columns at `row` are set in the bitmap: the whole wavefront on one row, a lane takes four
+// consecutive columns with one 16-byte load, four such loads per lane and turn, and the loads of the next turn
+// are in flight while this turn's bits are looked up.  n is the same in every lane.
+__device__ __forceinline__ int bitmap_row_hits(const uint32_t *bm, const int32_t *__restrict__ row, int n, int lane)
+{
+    const int nq = n >> 2;          // groups of four
+    int hits = 0;
+    sg_i4u cur[4];
+    bool okc[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        const int q = lane + 64 * x;
+        okc[x] = q < nq;
+        cur[x] = sg_i4u{0, 0, 0, 0};
+        if (okc[x])
+            cur[x] = *reinterpret_cast<const sg_i4u *>(row + 4 * q);
+    }
+    for (int tb = 256; tb < nq; tb += 256) {
+        sg_i4u nxt[4];
+        bool okn[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            const int q = tb + lane + 64 * x;
+            okn[x] = q < nq;
+            nxt[x] = sg_i4u{0, 0, 0, 0};
+            if (okn[x])
+                nxt[x] = *reinterpret_cast<const sg_i4u *>(row + 4 * q);
+        }
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+            if (okc[x])
+                hits += bitmap_bits4(bm, cur[x]);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            cur[x] = nxt[x];
+            okc[x] = okn[x];
+        }
+    }
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+        if (okc[x])
+            hits += bitmap_bits4(bm, cur[x]);
+    if (lane < (n & 3))
+        hits += bitmap_bit(bm, row[4 * nq + lane]);
+    return hits;
+}
+
+// The walk of one output row by a team of TEAM wavefronts (this is wavefront `wave` of it): the entries of A's
+// row are dealt to the wavefronts one at a time; a row of B with 64 entries or more takes the whole wavefront,
+// shorter ones go to its four 16-lane quarters, four rows at a time.  Returns the lane's share of the sum.
+template <int TEAM>
+__device__ __forceinline__ double bitmap_walk_iso(int64_t as, int64_t ae, const int32_t *__restrict__ Acrd,
+                                                  const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
+                                                  const int32_t *__restrict__ Bcrd, double biso, const uint32_t *bm,
+                                                  int wave, int lane)
+{
+    double part = 0.0;
+    const int quarter = lane >> 4, sub = lane & 15;
+    for (int64_t base = as + wave; base < ae; base += (int64_t)TEAM * 64) {
+        const int64_t left = (ae - base + TEAM - 1) / TEAM;     // my entries from here on
+        const int cnt = (int)(left < 64 ? left : 64);
+        int64_t bs = 0;
+        int len = 0;
+        double a = 0.0;
+        if (lane < cnt) {
+            const int64_t p = base + (int64_t)lane * TEAM;
+            const int k = Acrd[p];
+            bs = Bpos[k];
+            len = (int)(Bpos[k + 1] - bs);      // a row holds fewer entries than the matrix has columns: < 2^31
+            a = Aval[p] * biso;
+        }
+        unsigned long long big = __ballot(len >= 64);
+        unsigned long long todo = __ballot(len > 0 && len < 64);
+        while (big) {
+            const int t = __builtin_ctzll(big);
+            big &= big - 1;
+            const int64_t s = readlane_i64(bs, t);
+            const int n = __builtin_amdgcn_readlane(len, t);
+            const double at = readlane_d(a, t);
+            const int hits = bitmap_row_hits(bm, Bcrd + s, n, lane);
+            part += (double)hits * at;
+        }
+        while (todo) {
+            int pick = -1;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int t = todo ? __builtin_ctzll(todo) : -1;
+                todo = todo ? (todo & (todo - 1)) : 0;
+                pick = quarter == g ? t : pick;
+            }
+            const int src = pick < 0 ? lane : pick;
+            const int64_t s = ((int64_t)__shfl((int)(bs >> 32), src, 64) << 32) |
+                              (uint32_t)__shfl((int)(bs & 0xffffffff), src, 64);
+            const int n_src = __shfl(len, src, 64);      // by every lane: a lane that sits out may be another's source
+            const int n = pick < 0 ? 0 : n_src;
+            const double at = __hiloint2double(__shfl(__double2hiint(a), src, 64), __shfl(__double2loint(a), src, 64));
+            int j[4];
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+                j[x] = sub + 16 * x < n ? Bcrd[s + sub + 16 * x] : 0;
+            int hits = 0;
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+                if (sub + 16 * x < n)
+                    hits += bitmap_bit(bm, j[x]);
+            part += (double)hits * at;
+        }
+    }
+    return part;
+}
+
+__global__ __launch_bounds__(SG_T) void spgemm_masked_sum_iso_kernel(
+    const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd, const double *__restrict__ Aval,
+    const int64_t *__restrict__ Bpos, const int32_t *__restrict__ Bcrd, double biso,
+    const int64_t *__restrict__ Mpos, const int32_t *__restrict__ Mcrd, int nwords, unsigned long long *ticket,
+    RowList list, double *__restrict__ rowsum)
+{
+    // the workgroup kernel: rows from the heavy end of the list, the mask row as a bitmap of nwords words in LDS
+    __shared__ int64_t row_slot;
+    __shared__ double wave_part[SG_WAVES];
+    uint32_t *bm = sg_dyn_lds;
+    for (int w = threadIdx.x; w < nwords; w += SG_T)
+        bm[w] = 0;
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int64_t t_first, t_end;
+    list_range(list, 2, &t_first, &t_end);
+    int64_t tk = draw_front(ticket, t_end, &row_slot);
+    while (tk < t_end) {
+        const int64_t i = list.rows[tk];      // rows outside the list keep the zero the host put there
+        const int64_t as = Apos[i], ae = Apos[i + 1];
+        const int64_t ms = Mpos[i], me = Mpos[i + 1];
+        const bool work = as != ae && ms != me;
+        if (work) {
+            for (int64_t t = ms + threadIdx.x; t < me; t += SG_T) {
+                const uint32_t j = (uint32_t)Mcrd[t];
+                atomicOr(&bm[j >> 5], 1u << (j & 31u));
+            }
+            __syncthreads();
+            double part = bitmap_walk_iso<SG_WAVES>(as, ae, Acrd, Aval, Bpos, Bcrd, biso, bm, wave, lane);
+            part = wave_sum_f64(part);
+            if (lane == 0)
+                wave_part[wave] = part;
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                double total = 0.0;
+                for (int w = 0; w < SG_WAVES; ++w)
+                    total += wave_part[w];
+                rowsum[i] = total;
+            }
+            for (int64_t t = ms + threadIdx.x; t < me; t += SG_T)
+                bm[(uint32_t)Mcrd[t] >> 5] = 0;
+        }   // work
+        tk = draw_front(ticket, t_end, &row_slot);     // its barriers also close this row's bitmap clean-up
+    }
+}
+
+// whether all stored values of a matrix are one number (looked at once per matrix)
+__global__ void csr_values_differ(int64_t nnz, const double *__restrict__ val, int *__restrict__ flag)
+{
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p < nnz && val[p] != val[0])
+        *flag = 1;
+}
+
+// ---------------------------------------------------------------------------
 // CSR .* CSR -> CSR, one lane per row, two-pointer merge of the sorted rows
 // (lib/Conversion/IndexTreeToSCF/IndexTreeToSCF.cpp:864-1053).
 // ---------------------------------------------------------------------------
@@ -3521,6 +3706,27 @@ extern "C" int64_t comet_hip_spgemm_csr_semiring(int64_t ah, int64_t bh, int64_t
     return csr_register(c);
 }
 
+static int csr_is_iso(const Csr *x, bool *iso)
+{
+    Csr *m = const_cast<Csr *>(x);
+    if (m->iso_state == 0) {
+        int flag = 1;
+        if (m->nnz > 0) {
+            COMET_CHK(g_dot_flag.ensure(sizeof(int), false));
+            COMET_HIPCHK(hipMemsetAsync(g_dot_flag.ptr, 0, sizeof(int), stream()));
+            csr_values_differ<<<dim3((unsigned)ceil_div(m->nnz, 256)), dim3(256), 0, stream()>>>(m->nnz, m->val,
+                                                                                                (int *)g_dot_flag.ptr);
+            COMET_HIPCHK(hipGetLastError());
+            COMET_HIPCHK(hipMemcpyAsync(&flag, g_dot_flag.ptr, sizeof(int), hipMemcpyDeviceToHost, stream()));
+            COMET_HIPCHK(hipMemcpyAsync(&m->iso_value, m->val, sizeof(double), hipMemcpyDeviceToHost, stream()));
+            COMET_HIPCHK(hipStreamSynchronize(stream()));
+        }
+        m->iso_state = flag ? 2 : 1;
+    }
+    *iso = m->iso_state == 1;
+    return COMET_HIP_OK;
+}
+
 extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, double *out)
 {
     COMET_CHK(ensure_init());
@@ -3545,7 +3751,10 @@ extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, d
     }
     double *rowsum = (double *)g_sg.rowcount.ptr;
     RowList list;
-    COMET_CHK(sg_row_list(a, b, 0, a->nrows, SG_NO_DENSE, SG_NO_DENSE, &list));
+    // rows whose mask row is too long for the wavefront kernel's table sort to the front, whatever their products:
+    // the workgroup kernel, which starts there, looks a column up in one LDS read; the wavefront kernel would
+    // bisect the mask row in memory for every product
+    COMET_CHK(sg_row_list(a, b, 0, a->nrows, SG_NO_DENSE, SG_NO_DENSE, &list, m, SM_MASK_MAX));
     COMET_HIPCHK(hipMemsetAsync(rowsum, 0, sizeof(double) * (size_t)a->nrows, stream()));
     const dim3 grid((unsigned)g.groups), block(SG_T);
     // Two kernels side by side, the second on the auxiliary stream: a workgroup per row from the heavy end of
@@ -3556,8 +3765,23 @@ extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, d
     // the best fixed split (49152 products), 18.9 ms with the two ends meeting by themselves (the difference is
     // the last wavefront-rows near the meeting point; looking at the ticket word before drawing from it, to keep
     // the wavefronts away from those rows, or drawing 16 rows at a time, costs more on that one word than it saves).
+    bool iso = false;
+    if (g.lds)
+        COMET_CHK(csr_is_iso(b, &iso));
+    // COMET_HIP_MASKED_SUM_ONLY=workgroup|wavefront launches one of the two kernels only, which then takes every
+    // row: the tests send each class of rows through both
+    const char *only = getenv("COMET_HIP_MASKED_SUM_ONLY");
+    const bool run_wg = !only || strcmp(only, "wavefront") != 0, run_wave = !only || strcmp(only, "workgroup") != 0;
     COMET_CHK(aux_fork());
-    if (g.lds) {
+    if (!run_wg) {
+    } else if (iso) {
+        const int nwords = (int)ceil_div(b->ncols, 32);
+        COMET_CHK(sg_allow_lds(spgemm_masked_sum_iso_kernel, sizeof(uint32_t) * (size_t)nwords));
+        KernelTimer t("spgemm_masked_sum");
+        spgemm_masked_sum_iso_kernel<<<grid, block, sizeof(uint32_t) * (size_t)nwords, stream()>>>(
+            a->pos, a->crd, a->val, b->pos, b->crd, b->iso_value, m->pos, m->crd, nwords,
+            (unsigned long long *)g_sg.ticket.ptr, list, rowsum);
+    } else if (g.lds) {
         COMET_CHK(sg_allow_lds(spgemm_masked_sum_kernel<true>, g.lds_bytes));
         KernelTimer t("spgemm_masked_sum");
         spgemm_masked_sum_kernel<true><<<grid, block, g.lds_bytes, stream()>>>(
@@ -3569,7 +3793,7 @@ extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, d
             a->nrows, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m->pos, m->crd, g.logW, gbm,
             (unsigned long long *)g_sg.ticket.ptr, list, rowsum);
     }
-    {   // eight workgroups of four wavefronts per CU: four fit beside the kernel above, the rest follow it
+    if (run_wave) {   // eight workgroups of four wavefronts per CU: four fit beside the kernel above, the rest follow it
         KernelTimer t("spgemm_masked_sum_small", aux_stream());
         spgemm_masked_sum_small_kernel<<<dim3((unsigned)(num_cus() * 8)), dim3(SM_WAVES * 64), 0, aux_stream()>>>(
             a->pos, a->crd, a->val, b->pos, b->crd, b->val, m->pos, m->crd,
