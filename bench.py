@@ -381,7 +381,7 @@ def bench_tricount(rt, orc, gen, args):
     # rows with many products take a workgroup each, the others a wavefront each: two kernels that run side by side
     # on two streams, so their durations overlap and the span of both is what counts
     dom = "spgemm_masked_sum || spgemm_masked_sum_small"
-    dom_ms = max(kt["spgemm_masked_sum"]["avg_ms"], kt["spgemm_masked_sum_small"]["avg_ms"])
+    dom_ms = max(kt[k]["avg_ms"] for k in ("spgemm_masked_sum", "spgemm_masked_sum_small") if k in kt)
     flops = 2.0 * nprod
     ib = 4
     alg_bytes = nnzL * (ib + 8) + (n + 1) * ib + 8

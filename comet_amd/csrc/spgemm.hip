@@ -2258,64 +2258,89 @@ __device__ __forceinline__ int bitmap_bits4(const uint32_t *bm, sg_i4u j)
     return (int)(((w0 >> ((uint32_t)j.x & 31u)) & 1u) + ((w1 >> ((uint32_t)j.y & 31u)) & 1u) +
                  ((w2 >> ((uint32_t)j.z & 31u)) & 1u) + ((w3 >> ((uint32_t)j.w & 31u)) & 1u));
 }
-// how many of the n columns at `row` are set in the bitmap: the whole wavefront on one row, a lane takes four
-// consecutive columns with one 16-byte load, four such loads per lane and turn, and the loads of the next turn
-// are in flight while this turn's bits are looked up.  n is the same in every lane.
-__device__ __forceinline__ int bitmap_row_hits(const uint32_t *bm, const int32_t *__restrict__ row, int n, int lane)
+// What a lane holds of a turn in flight: up to four 16-byte loads (four consecutive columns each) of the row of
+// B its group of lanes is on, one more column if the row's length is not a multiple of four, and the value
+// a * b every hit of this row is worth.
+struct IsoTurn {
+    sg_i4u q[4];
+    int tail;
+    uint32_t ok;        // bit x: q[x] holds columns; bit 4: tail does
+    double at;
+};
+// The loads of a turn.  `row` is the lane's row of B, `first` the first group of four columns the lane takes and
+// `stride` the distance to its next one, nq the number of full groups of four in the row; rest = the columns
+// beyond them if this is the row's last turn (else 0), taken by the first lanes of the group (sub = the lane's
+// number inside it).
+__device__ __forceinline__ void iso_issue(IsoTurn &t, const int32_t *__restrict__ row, int first, int stride, int nq,
+                                          int rest, int sub, double at)
 {
-    const int nq = n >> 2;          // groups of four
-    int hits = 0;
-    sg_i4u cur[4];
-    bool okc[4];
+    t.ok = 0;
+    t.at = at;
+    t.tail = 0;
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
-        const int q = lane + 64 * x;
-        okc[x] = q < nq;
-        cur[x] = sg_i4u{0, 0, 0, 0};
-        if (okc[x])
-            cur[x] = *reinterpret_cast<const sg_i4u *>(row + 4 * q);
-    }
-    for (int tb = 256; tb < nq; tb += 256) {
-        sg_i4u nxt[4];
-        bool okn[4];
-#pragma unroll
-        for (int x = 0; x < 4; ++x) {
-            const int q = tb + lane + 64 * x;
-            okn[x] = q < nq;
-            nxt[x] = sg_i4u{0, 0, 0, 0};
-            if (okn[x])
-                nxt[x] = *reinterpret_cast<const sg_i4u *>(row + 4 * q);
-        }
-#pragma unroll
-        for (int x = 0; x < 4; ++x)
-            if (okc[x])
-                hits += bitmap_bits4(bm, cur[x]);
-#pragma unroll
-        for (int x = 0; x < 4; ++x) {
-            cur[x] = nxt[x];
-            okc[x] = okn[x];
+        const int qi = first + stride * x;
+        t.q[x] = sg_i4u{0, 0, 0, 0};
+        if (qi < nq) {
+            t.q[x] = *reinterpret_cast<const sg_i4u *>(row + 4 * qi);
+            t.ok |= 1u << x;
         }
     }
+    if (sub < rest) {
+        t.tail = row[4 * nq + sub];
+        t.ok |= 16u;
+    }
+}
+template <typename PROBE>
+__device__ __forceinline__ void iso_consume(const IsoTurn &t, const PROBE &probe, double &part)
+{
+    int hits = 0;
 #pragma unroll
     for (int x = 0; x < 4; ++x)
-        if (okc[x])
-            hits += bitmap_bits4(bm, cur[x]);
-    if (lane < (n & 3))
-        hits += bitmap_bit(bm, row[4 * nq + lane]);
-    return hits;
+        if (t.ok & (1u << x))
+            hits += probe.four(t.q[x]);
+    if (t.ok & 16u)
+        hits += probe.one(t.tail);
+    if (hits)                   // a row without hits adds nothing, whatever its value (0 * inf would be NaN)
+        part += (double)hits * t.at;
+}
+// `todo` names lanes that hold a row of B each; the next G of them go to the G groups of 64 / G lanes of the
+// wavefront.  Returns the lane whose row this lane's group takes, or -1.
+template <int G>
+__device__ __forceinline__ int iso_pick(unsigned long long &todo, int lane)
+{
+    int pick = -1;
+    const int group = lane / (64 / G);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int t = todo ? __builtin_ctzll(todo) : -1;
+        todo = todo ? (todo & (todo - 1)) : 0;
+        pick = group == g ? t : pick;
+    }
+    return pick;
 }
 
-// The walk of one output row by a team of TEAM wavefronts (this is wavefront `wave` of it): the entries of A's
-// row are dealt to the wavefronts one at a time; a row of B with 64 entries or more takes the whole wavefront,
-// shorter ones go to its four 16-lane quarters, four rows at a time.  Returns the lane's share of the sum.
-template <int TEAM>
-__device__ __forceinline__ double bitmap_walk_iso(int64_t as, int64_t ae, const int32_t *__restrict__ Acrd,
-                                                  const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
-                                                  const int32_t *__restrict__ Bcrd, double biso, const uint32_t *bm,
-                                                  int wave, int lane)
+// The walk of one output row by a team of TEAM wavefronts (this is wavefront `wave` of it).  The entries of A's
+// row are dealt to the wavefronts one at a time, 64 per wavefront and pass.  What bounds a walk like this is
+// not the look-ups but the wait for a row of B to arrive, so rows are taken several at a time and a turn
+// ahead: rows of 512 entries and more by the whole wavefront, 1024 columns per turn; rows of 256 and more two at
+// a time, one per half; shorter ones four at a time, one per 16-lane quarter; and the loads of a turn are issued
+// before the look-ups of the turn before it, across rows.  probe.four(j4) / probe.one(j) say how many of the
+// columns are in the mask row.  Returns the lane's share of the sum.
+template <int TEAM, typename PROBE>
+__device__ __forceinline__ double iso_walk(int64_t as, int64_t ae, const int32_t *__restrict__ Acrd,
+                                           const double *__restrict__ Aval, const int64_t *__restrict__ Bpos,
+                                           const int32_t *__restrict__ Bcrd, double biso, const PROBE &probe, int wave,
+                                           int lane)
 {
     double part = 0.0;
-    const int quarter = lane >> 4, sub = lane & 15;
+    IsoTurn pend;
+    pend.ok = 0;
+    pend.at = 0.0;
+    pend.tail = 0;
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+        pend.q[x] = sg_i4u{0, 0, 0, 0};
     for (int64_t base = as + wave; base < ae; base += (int64_t)TEAM * 64) {
         const int64_t left = (ae - base + TEAM - 1) / TEAM;     // my entries from here on
         const int cnt = (int)(left < 64 ? left : 64);
@@ -2329,45 +2354,60 @@ __device__ __forceinline__ double bitmap_walk_iso(int64_t as, int64_t ae, const 
             len = (int)(Bpos[k + 1] - bs);      // a row holds fewer entries than the matrix has columns: < 2^31
             a = Aval[p] * biso;
         }
-        unsigned long long big = __ballot(len >= 64);
-        unsigned long long todo = __ballot(len > 0 && len < 64);
+        unsigned long long big = __ballot(len >= 512);
+        unsigned long long mid = __ballot(len >= 256 && len < 512);
+        unsigned long long small = __ballot(len > 0 && len < 256);
         while (big) {
             const int t = __builtin_ctzll(big);
             big &= big - 1;
-            const int64_t s = readlane_i64(bs, t);
+            const int32_t *row = Bcrd + readlane_i64(bs, t);
             const int n = __builtin_amdgcn_readlane(len, t);
             const double at = readlane_d(a, t);
-            const int hits = bitmap_row_hits(bm, Bcrd + s, n, lane);
-            part += (double)hits * at;
-        }
-        while (todo) {
-            int pick = -1;
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int t = todo ? __builtin_ctzll(todo) : -1;
-                todo = todo ? (todo & (todo - 1)) : 0;
-                pick = quarter == g ? t : pick;
+            const int nq = n >> 2;
+            for (int tb = 0; tb == 0 || tb < nq; tb += 256) {
+                IsoTurn now;
+                iso_issue(now, row, tb + lane, 64, nq, tb + 256 >= nq ? (n & 3) : 0, lane, at);
+                iso_consume(pend, probe, part);
+                pend = now;
             }
+        }
+        while (mid) {
+            const int pick = iso_pick<2>(mid, lane);
+            const int src = pick < 0 ? lane : pick;
+            // by every lane: a lane whose group sits this round out may be another's source
+            const int64_t s = ((int64_t)__shfl((int)(bs >> 32), src, 64) << 32) |
+                              (uint32_t)__shfl((int)(bs & 0xffffffff), src, 64);
+            const int n_src = __shfl(len, src, 64);
+            const double at = __hiloint2double(__shfl(__double2hiint(a), src, 64), __shfl(__double2loint(a), src, 64));
+            const int n = pick < 0 ? 0 : n_src;
+            IsoTurn now;
+            iso_issue(now, Bcrd + s, lane & 31, 32, n >> 2, n & 3, lane & 31, at);
+            iso_consume(pend, probe, part);
+            pend = now;
+        }
+        while (small) {
+            const int pick = iso_pick<4>(small, lane);
             const int src = pick < 0 ? lane : pick;
             const int64_t s = ((int64_t)__shfl((int)(bs >> 32), src, 64) << 32) |
                               (uint32_t)__shfl((int)(bs & 0xffffffff), src, 64);
-            const int n_src = __shfl(len, src, 64);      // by every lane: a lane that sits out may be another's source
-            const int n = pick < 0 ? 0 : n_src;
+            const int n_src = __shfl(len, src, 64);
             const double at = __hiloint2double(__shfl(__double2hiint(a), src, 64), __shfl(__double2loint(a), src, 64));
-            int j[4];
-#pragma unroll
-            for (int x = 0; x < 4; ++x)
-                j[x] = sub + 16 * x < n ? Bcrd[s + sub + 16 * x] : 0;
-            int hits = 0;
-#pragma unroll
-            for (int x = 0; x < 4; ++x)
-                if (sub + 16 * x < n)
-                    hits += bitmap_bit(bm, j[x]);
-            part += (double)hits * at;
+            const int n = pick < 0 ? 0 : n_src;
+            IsoTurn now;
+            iso_issue(now, Bcrd + s, lane & 15, 16, n >> 2, n & 3, lane & 15, at);
+            iso_consume(pend, probe, part);
+            pend = now;
         }
     }
+    iso_consume(pend, probe, part);
     return part;
 }
+
+struct BitmapProbe {
+    const uint32_t *bm;
+    __device__ __forceinline__ int one(int j) const { return bitmap_bit(bm, j); }
+    __device__ __forceinline__ int four(sg_i4u j) const { return bitmap_bits4(bm, j); }
+};
 
 __global__ __launch_bounds__(SG_T) void spgemm_masked_sum_iso_kernel(
     const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd, const double *__restrict__ Aval,
@@ -2397,7 +2437,7 @@ __global__ __launch_bounds__(SG_T) void spgemm_masked_sum_iso_kernel(
                 atomicOr(&bm[j >> 5], 1u << (j & 31u));
             }
             __syncthreads();
-            double part = bitmap_walk_iso<SG_WAVES>(as, ae, Acrd, Aval, Bpos, Bcrd, biso, bm, wave, lane);
+            double part = iso_walk<SG_WAVES>(as, ae, Acrd, Aval, Bpos, Bcrd, biso, BitmapProbe{bm}, wave, lane);
             part = wave_sum_f64(part);
             if (lane == 0)
                 wave_part[wave] = part;
