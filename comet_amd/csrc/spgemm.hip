@@ -2455,6 +2455,125 @@ __global__ __launch_bounds__(SG_T) void spgemm_masked_sum_iso_kernel(
     }
 }
 
+// The wavefront kernel for a pattern matrix B: the walk above with the mask row in a table of the wavefront's own.
+// The table is 64 buckets of four columns, the bucket a multiplicative hash of the column, so a look-up is one
+// 16-byte LDS read and four compares, without a loop.  A mask row goes in if no bucket overflows; three more
+// multipliers are tried before the row is searched by bisection in memory instead, as are mask rows of more than
+// SI_MASK_MAX entries (which sort to the other kernel's end of the list and only come here when this kernel gets
+// that far).
+constexpr int SI_MASK_MAX = 48;
+constexpr int SI_TRIES = 4;
+// a bucket read or cleared as one 16-byte access; may_alias, because the same words are also written one at a
+// time by atomicCAS through an int pointer, and without it the compiler is free to reorder the two kinds
+typedef int si_bucket __attribute__((ext_vector_type(4), may_alias));
+struct BucketProbe {
+    const int *tab;
+    uint32_t mult;
+    __device__ __forceinline__ static int bucket(int j, uint32_t mult)
+    {
+        return (int)((uint32_t)__umul24((uint32_t)j, mult) >> 26);      // __umul24 returns int: shift it as unsigned
+    }
+    __device__ __forceinline__ int one(int j) const
+    {
+        const si_bucket b = *reinterpret_cast<const si_bucket *>(tab + 4 * bucket(j, mult));
+        return (b.x == j) | (b.y == j) | (b.z == j) | (b.w == j);
+    }
+    __device__ __forceinline__ int four(sg_i4u j) const { return one(j.x) + one(j.y) + one(j.z) + one(j.w); }
+};
+struct BisectProbe {
+    const int32_t *m;       // the mask row, ascending
+    int n;
+    __device__ __forceinline__ int one(int j) const
+    {
+        int lo = 0, hi = n;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (m[mid] < j)
+                lo = mid + 1;
+            else
+                hi = mid;
+        }
+        return lo < n && m[lo] == j;
+    }
+    __device__ __forceinline__ int four(sg_i4u j) const { return one(j.x) + one(j.y) + one(j.z) + one(j.w); }
+};
+
+__global__ __launch_bounds__(SM_WAVES * 64) void spgemm_masked_sum_small_iso_kernel(
+    const int64_t *__restrict__ Apos, const int32_t *__restrict__ Acrd, const double *__restrict__ Aval,
+    const int64_t *__restrict__ Bpos, const int32_t *__restrict__ Bcrd, double biso,
+    const int64_t *__restrict__ Mpos, const int32_t *__restrict__ Mcrd, unsigned long long *ticket, RowList list,
+    double *__restrict__ rowsum)
+{
+    __shared__ __align__(16) int table[SM_WAVES][SM_SLOTS];
+    const int lane = threadIdx.x & 63;
+    int *tab = table[threadIdx.x >> 6];
+    reinterpret_cast<si_bucket *>(tab)[lane] = si_bucket{-1, -1, -1, -1};
+    int64_t t_first, t_end;
+    list_range(list, 2, &t_first, &t_end);
+    int take = SM_BATCH;
+    for (;;) {
+        // rows from the light end of the list, as spgemm_masked_sum_small_kernel draws them
+        unsigned long long drawn = 0;
+        if (lane == 0)
+            drawn = atomicAdd(ticket, (unsigned long long)take << 32);
+        const int64_t f = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(drawn & 0xffffffffu));
+        const int64_t b = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(drawn >> 32));
+        if (f + b >= t_end)
+            break;
+        const int nb = (int)(b + take < t_end - f ? take : t_end - f - b);      // what the front had not reached
+        const int64_t taken = b + take;
+        take = taken < t_end / 2 ? SM_BATCH : taken < t_end - t_end / 4 ? SM_BATCH / 4 : 1;
+        // the rows of the batch and where they start and end in A and in the mask: one round trip for all of them
+        int bi = 0;
+        int64_t bas = 0, bae = 0, bms = 0, bme = 0;
+        if (lane < nb) {
+            bi = list.rows[t_end - 1 - (b + lane)];
+            bas = Apos[bi];
+            bae = Apos[bi + 1];
+            bms = Mpos[bi];
+            bme = Mpos[bi + 1];
+        }
+        for (int r = 0; r < nb; ++r) {
+            const int i = __builtin_amdgcn_readlane(bi, r);
+            const int64_t as = readlane_i64(bas, r), ae = readlane_i64(bae, r);
+            const int64_t ms = readlane_i64(bms, r), me = readlane_i64(bme, r);
+            if (as == ae || ms == me)
+                continue;               // rowsum[i] keeps the zero the host put there
+            const int mlen = (int)(me - ms < (int64_t)SI_MASK_MAX + 1 ? me - ms : SI_MASK_MAX + 1);
+            bool hashed = false;
+            uint32_t mult = 0;
+            if (mlen <= SI_MASK_MAX) {
+                const int j = lane < mlen ? Mcrd[ms + lane] : -1;
+                static_assert(SI_MASK_MAX <= 64, "a lane holds one column of the mask row");
+                for (int attempt = 0; attempt < SI_TRIES && !hashed; ++attempt) {
+                    mult = attempt == 0 ? 0x9E3779u : attempt == 1 ? 0x85EBCBu : attempt == 2 ? 0xC2B2AFu : 0x27D4EBu;
+                    bool placed = j < 0;
+                    if (j >= 0) {
+                        int *bk = tab + 4 * BucketProbe::bucket(j, mult);
+#pragma unroll
+                        for (int x = 0; x < 4; ++x)
+                            if (!placed)
+                                placed = atomicCAS(&bk[x], -1, j) == -1;
+                    }
+                    hashed = !__any(!placed);
+                    if (!hashed)
+                        reinterpret_cast<si_bucket *>(tab)[lane] = si_bucket{-1, -1, -1, -1};
+                }
+            }
+            double part;
+            if (hashed)
+                part = iso_walk<1>(as, ae, Acrd, Aval, Bpos, Bcrd, biso, BucketProbe{tab, mult}, 0, lane);
+            else
+                part = iso_walk<1>(as, ae, Acrd, Aval, Bpos, Bcrd, biso, BisectProbe{Mcrd + ms, (int)(me - ms)}, 0, lane);
+            part = wave_sum_f64(part);
+            if (lane == 0)
+                rowsum[i] = part;
+            if (hashed)
+                reinterpret_cast<si_bucket *>(tab)[lane] = si_bucket{-1, -1, -1, -1};
+        }
+    }
+}
+
 // whether all stored values of a matrix are one number (looked at once per matrix)
 __global__ void csr_values_differ(int64_t nnz, const double *__restrict__ val, int *__restrict__ flag)
 {
@@ -3794,7 +3913,10 @@ extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, d
     // rows whose mask row is too long for the wavefront kernel's table sort to the front, whatever their products:
     // the workgroup kernel, which starts there, looks a column up in one LDS read; the wavefront kernel would
     // bisect the mask row in memory for every product
-    COMET_CHK(sg_row_list(a, b, 0, a->nrows, SG_NO_DENSE, SG_NO_DENSE, &list, m, SM_MASK_MAX));
+    bool iso = false;
+    if (g.lds)
+        COMET_CHK(csr_is_iso(b, &iso));
+    COMET_CHK(sg_row_list(a, b, 0, a->nrows, SG_NO_DENSE, SG_NO_DENSE, &list, m, iso ? SI_MASK_MAX : SM_MASK_MAX));
     COMET_HIPCHK(hipMemsetAsync(rowsum, 0, sizeof(double) * (size_t)a->nrows, stream()));
     const dim3 grid((unsigned)g.groups), block(SG_T);
     // Two kernels side by side, the second on the auxiliary stream: a workgroup per row from the heavy end of
@@ -3805,9 +3927,6 @@ extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, d
     // the best fixed split (49152 products), 18.9 ms with the two ends meeting by themselves (the difference is
     // the last wavefront-rows near the meeting point; looking at the ticket word before drawing from it, to keep
     // the wavefronts away from those rows, or drawing 16 rows at a time, costs more on that one word than it saves).
-    bool iso = false;
-    if (g.lds)
-        COMET_CHK(csr_is_iso(b, &iso));
     // COMET_HIP_MASKED_SUM_ONLY=workgroup|wavefront launches one of the two kernels only, which then takes every
     // row: the tests send each class of rows through both
     const char *only = getenv("COMET_HIP_MASKED_SUM_ONLY");
@@ -3833,7 +3952,12 @@ extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, d
             a->nrows, a->pos, a->crd, a->val, b->pos, b->crd, b->val, m->pos, m->crd, g.logW, gbm,
             (unsigned long long *)g_sg.ticket.ptr, list, rowsum);
     }
-    if (run_wave) {   // eight workgroups of four wavefronts per CU: four fit beside the kernel above, the rest follow it
+    if (run_wave && iso) {
+        KernelTimer t("spgemm_masked_sum_small", aux_stream());
+        spgemm_masked_sum_small_iso_kernel<<<dim3((unsigned)(num_cus() * 8)), dim3(SM_WAVES * 64), 0, aux_stream()>>>(
+            a->pos, a->crd, a->val, b->pos, b->crd, b->iso_value, m->pos, m->crd,
+            (unsigned long long *)g_sg.ticket.ptr, list, rowsum);
+    } else if (run_wave) {   // eight workgroups of four wavefronts per CU: four fit beside the kernel above, the rest follow it
         KernelTimer t("spgemm_masked_sum_small", aux_stream());
         spgemm_masked_sum_small_kernel<<<dim3((unsigned)(num_cus() * 8)), dim3(SM_WAVES * 64), 0, aux_stream()>>>(
             a->pos, a->crd, a->val, b->pos, b->crd, b->val, m->pos, m->crd,
