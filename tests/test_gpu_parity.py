@@ -918,6 +918,68 @@ def test_masked_sum_general_values():
     assert abs(got - orc.reduce_sum(wv)) <= RTOL * bound.sum()
 
 
+def _pattern_case(rng, ncols, entries, blen, mlen, nrows, bvalue):
+    """`nrows` output rows with `entries` stored entries each (random values), every one naming a row of B with
+    `blen` columns and the one value `bvalue`; a mask row of `mlen` columns, half of them taken from the columns B
+    uses so that products do meet the mask."""
+    rows = [np.sort(rng.choice(ncols, blen, replace=False)) for _ in range(entries)]
+    bpos = np.zeros(ncols + 1, np.int64)
+    bpos[1:entries + 1] = np.cumsum([blen] * entries)
+    bpos[entries + 1:] = bpos[entries]
+    bcrd = np.concatenate(rows).astype(np.int32)
+    b = (bpos, bcrd, np.full(len(bcrd), bvalue))
+    apos = np.zeros(ncols + 1, np.int64)
+    apos[ncols - nrows + 1:] = np.arange(1, nrows + 1) * entries
+    a = (apos, np.tile(np.arange(entries, dtype=np.int32), nrows), rng.uniform(0.5, 1.5, entries * nrows))
+    used = np.unique(bcrd)
+    masks = [np.unique(np.concatenate([rng.choice(used, min(mlen // 2, len(used)), replace=False),
+                                       rng.choice(ncols, mlen - mlen // 2, replace=False)])) for _ in range(nrows)]
+    mpos = np.zeros(ncols + 1, np.int64)
+    mpos[ncols - nrows + 1:] = np.cumsum([len(m) for m in masks])
+    mcrd = np.concatenate(masks).astype(np.int32)
+    return a, b, (mpos, mcrd, np.ones(len(mcrd)))
+
+
+@pytest.mark.parametrize("only", [None, "workgroup", "wavefront"])
+def test_masked_sum_pattern_matrix(only, monkeypatch):
+    """B with one value for all its entries takes kernels of its own that count the hits of a row of B instead of
+    fetching values.  Every class of rows - few and many entries in A's row (more than a wavefront's 64 and a
+    workgroup's 1024 lanes), rows of B below and above the lengths at which four, two and one of them share a
+    wavefront and longer than one turn, mask rows that fit the wavefront's table (up to 48 columns), that do not,
+    and empty ones - through both kernels together and through each alone."""
+    if only:
+        monkeypatch.setenv("COMET_HIP_MASKED_SUM_ONLY", only)
+    rng = np.random.default_rng(11)
+    ncols = 1 << 13
+    cases = [(e, bl, ml, nr) for e in (1, 17, 70, 257, 1100) for bl in (3, 63, 64, 255, 256, 511, 512, 1027, 2500)
+             for ml in (0, 4, 48, 49, 300) for nr in (1, 7)]
+    for k, (e, bl, ml, nr) in enumerate(cases):
+        if k % 3 != (0 if only is None else 1 if only == "workgroup" else 2) and (e, bl) != (257, 63):
+            continue            # a third of the grid per mode, and the round with one row left over in all of them
+        a, b, m = _pattern_case(rng, ncols, e, bl, ml, nr, 0.75)
+        A, B, M = (rt.CsrMatrix.from_arrays((ncols, ncols), *x) for x in (a, b, m))
+        got = rt.spgemm_masked_sum(A, B, M)
+        wp, wc, wv = orc.spgemm(*a, *b, ncols, mask=(m[0], m[1]))
+        want = orc.reduce_sum(wv)
+        assert abs(got - want) <= RTOL * abs(want), (e, bl, ml, nr)
+    # the same kernels on a graph, whole numbers: exact
+    pos, crd, val = gen.rmat_symmetric_csr(scale=13, edge_factor=16, seed=5, values="ones")
+    lpos, lcrd, lval = gen.strictly_lower(pos, crd, val)
+    L = rt.CsrMatrix.from_arrays((1 << 13, 1 << 13), lpos, lcrd, lval)
+    rep = _kernels_of(lambda: rt.triangle_count(L))
+    assert ("spgemm_masked_sum" in rep) == (only != "wavefront")
+    assert ("spgemm_masked_sum_small" in rep) == (only != "workgroup")
+    assert rt.triangle_count(L) == orc.tricount_masked(lpos, lcrd, lval)
+    # an infinite value in a row of A whose products all miss the mask adds nothing
+    a, b, m = _pattern_case(rng, ncols, 5, 100, 10, 1, 1.0)
+    mpos = np.zeros(ncols + 1, np.int64)
+    mpos[ncols] = 10
+    m = (mpos, np.setdiff1d(np.arange(ncols, dtype=np.int32), b[1])[:10].astype(np.int32), np.ones(10))
+    a[2][:] = np.inf
+    A, B, M = (rt.CsrMatrix.from_arrays((ncols, ncols), *x) for x in (a, b, m))
+    assert rt.spgemm_masked_sum(A, B, M) == 0.0
+
+
 def test_eltwise_golden_and_random(golden, golden_dir):
     g = golden["eltwise_mult_csr"]
     (nr, nc), pos, crd, val = _mtx(golden_dir, g["A"])
