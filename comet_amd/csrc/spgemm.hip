@@ -3937,7 +3937,12 @@ extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, d
         const int nwords = (int)ceil_div(b->ncols, 32);
         COMET_CHK(sg_allow_lds(spgemm_masked_sum_iso_kernel, sizeof(uint32_t) * (size_t)nwords));
         KernelTimer t("spgemm_masked_sum");
-        spgemm_masked_sum_iso_kernel<<<grid, block, sizeof(uint32_t) * (size_t)nwords, stream()>>>(
+        // Not a workgroup for every CU: beside one, a CU's registers hold a single wavefront of the other kernel per
+        // SIMD, and the half million light rows that kernel takes each wait on memory four times in a row.  The
+        // CUs left free hold sixteen of its wavefronts (triangle count of the scale-20 graph: 5.2 ms with a
+        // workgroup on every CU, 4.76 ms on 208 to 224 of 256, 5.7 ms on 192).
+        const dim3 igrid(g.groups == num_cus() ? (unsigned)(g.groups - 3 * (g.groups / 16)) : (unsigned)g.groups);
+        spgemm_masked_sum_iso_kernel<<<igrid, block, sizeof(uint32_t) * (size_t)nwords, stream()>>>(
             a->pos, a->crd, a->val, b->pos, b->crd, b->iso_value, m->pos, m->crd, nwords,
             (unsigned long long *)g_sg.ticket.ptr, list, rowsum);
     } else if (g.lds) {
