@@ -87,6 +87,7 @@ struct BmAddr {
 // turn costs about one trip to memory, so each turn issues all of its loads (up
 // to four per lane; a load no lane needs is skipped) before the visitor runs.
 constexpr int FEP_SHORT = 32, FEP_SHORT_LOADS = FEP_SHORT / 16, FEP_LONG_LOADS = 4;
+constexpr int FEP_WIDE_DEPTH = 4;       // turns of a long row a wavefront takes at a time (WIDE walks)
 // what the look-up and fetch steps of a masked product's visitor hand to the visit itself: where the column's
 // value lives (negative: the mask does not hold the column) and B's value, fetched for hits only
 struct MaskHit {
@@ -182,9 +183,46 @@ __device__ inline void for_each_product_impl(int64_t as, int64_t ae, const int32
                 // 16-byte load, and the loads of the next turn are in flight while the visitor works on this one.
                 static_assert(FEP_LONG_LOADS == 4, "a lane's entries of a full turn are one 16-byte load");
                 int64_t c = s + 4 * (int64_t)lane;
-                sg_i4u j = *reinterpret_cast<const sg_i4u *>(Bcrd + c);
                 int64_t done = 0;
-                for (int64_t full = 64 * FEP_LONG_LOADS; full + 64 * FEP_LONG_LOADS <= len;
+                // A wavefront with one or two kilobytes on their way from memory waits most of the time (a row of
+                // B comes from beyond the L2 as a rule, two microseconds away): rows long enough are taken
+                // FEP_WIDE_DEPTH turns at a time with as many again in flight behind them, then two at a time
+                // (symbolic phase of A*A on an R-MAT graph of scale 20: 64.7 -> 46.8 ms; eight at a time gains
+                // nothing over four).
+                constexpr int64_t TURN = 64 * FEP_LONG_LOADS;
+                const auto deep = [&](auto dtag) {
+                    constexpr int D = decltype(dtag)::value;
+                    if (len - done < 2 * D * TURN)
+                        return;
+                    sg_i4u jd[D];
+#pragma unroll
+                    for (int d = 0; d < D; ++d)
+                        jd[d] = *reinterpret_cast<const sg_i4u *>(Bcrd + c + d * TURN);
+                    for (int64_t full = done + D * TURN; full + D * TURN <= len; full += D * TURN) {
+                        sg_i4u jn[D];
+#pragma unroll
+                        for (int d = 0; d < D; ++d)
+                            jn[d] = *reinterpret_cast<const sg_i4u *>(Bcrd + c + (D + d) * TURN);
+#pragma unroll
+                        for (int d = 0; d < D; ++d)
+                            f4(jd[d], c + d * TURN, at, p, s);
+#pragma unroll
+                        for (int d = 0; d < D; ++d)
+                            jd[d] = jn[d];
+                        c += D * TURN;
+                        done += D * TURN;
+                    }
+#pragma unroll
+                    for (int d = 0; d < D; ++d)
+                        f4(jd[d], c + d * TURN, at, p, s);
+                    c += D * TURN;
+                    done += D * TURN;
+                };
+                deep(std::integral_constant<int, FEP_WIDE_DEPTH>());
+                deep(std::integral_constant<int, 2>());
+                if (len - done >= TURN) {
+                sg_i4u j = *reinterpret_cast<const sg_i4u *>(Bcrd + c);
+                for (int64_t full = done + 64 * FEP_LONG_LOADS; full + 64 * FEP_LONG_LOADS <= len;
                      full += 64 * FEP_LONG_LOADS) {
                     const sg_i4u jn = *reinterpret_cast<const sg_i4u *>(Bcrd + c + 64 * FEP_LONG_LOADS);
                     f4(j, c, at, p, s);
@@ -193,7 +231,9 @@ __device__ inline void for_each_product_impl(int64_t as, int64_t ae, const int32
                     done += 64 * FEP_LONG_LOADS;
                 }
                 f4(j, c, at, p, s);
-                o += done + 64 * FEP_LONG_LOADS;
+                done += 64 * FEP_LONG_LOADS;
+                }
+                o += done;
             }
             if (!WIDE && len >= 64 * FEP_LONG_LOADS) {
                 // Turns in which every lane has all its entries: no predicates, and the loads of the next such
