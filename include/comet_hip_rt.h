@@ -344,7 +344,13 @@ int64_t comet_hip_csr_transpose(int64_t csr);
  * test/integration/kernels/triangleCount_SandiaLL_wMasking.ta:18-39, i.e. the
  * masked numeric phase followed by ReduceOpLowering
  * (lib/Conversion/TensorAlgebraToSCF/TensorAlgebraToSCF.cpp:417-529), without
- * materialising C.  a, b, mask may all be the same handle. */
+ * materialising C.  a, b, mask may all be the same handle.
+ * When every stored value of b is one number (a pattern matrix, looked at once per
+ * handle), the kernels count per row of b how many of its columns the mask row
+ * holds and add count * (a's entry * that number): sums of whole numbers, such as
+ * a triangle count, are exact; other values agree with the product-by-product sum
+ * to rounding.  COMET_HIP_MASKED_SUM_ONLY=workgroup|wavefront in the environment
+ * sends every row through one of the two kernels (a diagnostic: the tests use it). */
 int comet_hip_spgemm_masked_sum(int64_t a, int64_t b, int64_t mask, double *out);
 
 /* ---- SUM over a device float64 array (ReduceOpLowering, as above) --------- */
