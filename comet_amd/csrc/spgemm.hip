@@ -3981,6 +3981,9 @@ extern "C" int comet_hip_spgemm_masked_sum(int64_t ah, int64_t bh, int64_t mh, d
         // SIMD, and the half million light rows that kernel takes each wait on memory four times in a row.  The
         // CUs left free hold sixteen of its wavefronts (triangle count of the scale-20 graph: 5.2 ms with a
         // workgroup on every CU, 4.76 ms on 208 to 224 of 256, 5.7 ms on 192).
+        // That single wavefront per SIMD is there only as long as this kernel keeps to 96 vector registers (four
+        // wavefronts of 96 and one of the other kernel's 112 make 496 of a SIMD's 512): with 97 it is allotted 104,
+        // the other kernel is left with the free CUs alone and the count takes 6.6 ms.
         const dim3 igrid(g.groups == num_cus() ? (unsigned)(g.groups - 3 * (g.groups / 16)) : (unsigned)g.groups);
         spgemm_masked_sum_iso_kernel<<<igrid, block, sizeof(uint32_t) * (size_t)nwords, stream()>>>(
             a->pos, a->crd, a->val, b->pos, b->crd, b->iso_value, m->pos, m->crd, nwords,
@@ -4153,6 +4156,22 @@ extern "C" int comet_hip_eltwise_dense_f64(int64_t n, int64_t a_dptr, int64_t b_
     eltwise_dense_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(n, (const double *)a_dptr, (const double *)b_dptr,
                                                                   (double *)c_dptr, op);
     COMET_HIPCHK(hipGetLastError());
+    return COMET_HIP_OK;
+}
+
+// Diagnostic: the vector registers per lane of the two kernels of the pattern-matrix masked sum, as the loaded code
+// object has them.  The workgroup kernel (16 wavefronts, four to a SIMD) and one wavefront of the other kernel
+// share a SIMD's 512 registers, allotted in eights: what a test holds them to.
+extern "C" int comet_hip_debug_masked_sum_registers(int *workgroup_kernel, int *wavefront_kernel)
+{
+    COMET_CHK(ensure_init());
+    if (!workgroup_kernel || !wavefront_kernel)
+        return set_error(COMET_HIP_ERR_ARG, "null result pointer");
+    hipFuncAttributes at;
+    COMET_HIPCHK(hipFuncGetAttributes(&at, reinterpret_cast<const void *>(spgemm_masked_sum_iso_kernel)));
+    *workgroup_kernel = at.numRegs;
+    COMET_HIPCHK(hipFuncGetAttributes(&at, reinterpret_cast<const void *>(spgemm_masked_sum_small_iso_kernel)));
+    *wavefront_kernel = at.numRegs;
     return COMET_HIP_OK;
 }
 

@@ -125,6 +125,7 @@ SIGNATURES = {
     "comet_hip_profile_name": (_int, [_i32, C.c_char_p, _i64]),
     "comet_hip_copy_f64": (_int, [_i64, _i64, _i64]),
     "comet_hip_debug_dot_table_words": (_int, [_int]),
+    "comet_hip_debug_masked_sum_registers": (_int, [C.POINTER(_int), C.POINTER(_int)]),
     "comet_hip_stream_create": (_i64, []),
     "comet_hip_stream_sync": (_int, [_i64]),
     "comet_hip_stream_destroy": (_int, [_i64]),

@@ -442,6 +442,11 @@ int comet_hip_mfma_f64_peak(int64_t iters, double *tflops);
  * kernel begin in its LDS for a bitmap of `words` 32-bit words; always even (an
  * odd offset would misalign its 64-bit LDS atomics).  Runs on the host. */
 int comet_hip_debug_dot_table_words(int words);
+/* Diagnostic: vector registers per lane of the two kernels of the pattern-matrix
+ * masked sum (comet_hip_spgemm_masked_sum) in the loaded code object.  They share
+ * the CUs, and do so only while four wavefronts of the first and one of the second
+ * fit a SIMD's 512 registers. */
+int comet_hip_debug_masked_sum_registers(int *workgroup_kernel, int *wavefront_kernel);
 int comet_hip_gather_rows_bench(int64_t workgroups, int64_t per_wave, int64_t idx_dptr,
                                 int64_t table_dptr, int64_t table_rows, int64_t out_dptr);
 

@@ -980,6 +980,17 @@ def test_masked_sum_pattern_matrix(only, monkeypatch):
     assert rt.spgemm_masked_sum(A, B, M) == 0.0
 
 
+def test_masked_sum_kernels_share_a_simd():
+    """The two kernels of the pattern-matrix masked sum run side by side on the same CUs only while four wavefronts
+    of the workgroup kernel and one of the wavefront kernel fit the 512 vector registers of a SIMD (allotted in
+    eights): one register more in the first and the triangle count takes 40 % longer."""
+    import ctypes as C
+    wg, wave = C.c_int(), C.c_int()
+    rt._check(rt.lib().comet_hip_debug_masked_sum_registers(C.byref(wg), C.byref(wave)), "registers")
+    up8 = lambda r: (r + 7) // 8 * 8
+    assert 4 * up8(wg.value) + up8(wave.value) <= 512, (wg.value, wave.value)
+
+
 def test_eltwise_golden_and_random(golden, golden_dir):
     g = golden["eltwise_mult_csr"]
     (nr, nc), pos, crd, val = _mtx(golden_dir, g["A"])
